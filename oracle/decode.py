@@ -1,0 +1,164 @@
+"""Token-recurrence oracle for k-last decode, MTP verify and accepted-prefix commit.
+
+Test infrastructure only; see ``oracle/__init__.py``.
+
+State layout is k-last: ``S[hv, v, k]``.  One step, per value head
+(scripts/decode/kda_mtp_sglang/private/_reference.py:44-50)::
+
+    S[v,k] *= exp(g[k]);  d[v] = sum_k S[v,k] k[k];  u[v] = (v[v] - d[v]) * beta
+    S[v,k] += u[v] k[k];  o[v] = sum_k S[v,k] q[k]        (q carries ``scale``)
+"""
+
+import torch
+
+from .gates import softplus_gate, lower_bound_gate, sigmoid_beta, l2norm
+
+
+def recurrent_step(S, q, k, v, log_decay, beta):
+    """One gated delta-rule step on ``S [HV,V,K]`` (updated copy returned).
+
+    ``q,k [HV,K]`` (already normalised / scaled / head-expanded), ``v [HV,V]``,
+    ``log_decay [HV,K]`` or ``[HV,1]``, ``beta [HV]``.  Returns ``(S_new, o [HV,V])``.
+    Follows tests/test_k_last_state_dtype.py:146-149.
+    """
+    S = S * log_decay.exp()[:, None, :]
+    d = torch.einsum("hvk,hk->hv", S, k)
+    u = (v - d) * beta[:, None]
+    S = S + u[:, :, None] * k[:, None, :]
+    o = torch.einsum("hvk,hk->hv", S, q)
+    return S, o
+
+
+def _invalid_slot(slot, is_sglang):
+    # sglang: pad id is negative, slot 0 is real; vLLM: block 0 is the null block
+    # (src/decode/k-last/fused_sigmoid_gating_k_last_kernel.cuh:232-248).
+    return slot < 0 if is_sglang else slot <= 0
+
+
+def k_last_reference(q, k, v, a, b, A_log, dt_bias, state, state_indices, lengths, *,
+                     scale=None, use_qk_l2norm=True, is_kda=False,
+                     disable_state_update=False,
+                     cache=None, cache_indices=None, num_accepted=None, parents=None,
+                     lower_bound=None, is_sglang=True,
+                     softplus_beta=1.0, softplus_threshold=20.0,
+                     log_decay=None, beta_activated=None, compute_dtype=torch.float32):
+    """Reference for ``fused_sigmoid_gating_delta_rule_forward_k_last{,_packed}``.
+
+    Restates tests/test_k_last_state_dtype.py:108-156 (``reference``) and adds
+    the vLLM 2-D slot-table mode of
+    src/decode/k-last/fused_sigmoid_gating_k_last_kernel.cuh:215-229, 847-863.
+
+    Token tensors are flat over requests: ``q,k [ntok,H,K]``, ``v [ntok,HV,V]``,
+    ``a [ntok,HV]`` (GDN) or ``[ntok,HV,K]`` (KDA), ``b [ntok,HV]``;
+    ``lengths[n]`` tokens belong to request ``n``.  ``state [slots,HV,V,K]``.
+    ``state_indices``: list ``[B]`` or nested list ``[B][S]`` (vLLM, requires
+    ``is_sglang=False``).  ``log_decay`` (same shape as ``a``, float) replaces
+    the gate computed from ``a/A_log/dt_bias``; ``beta_activated`` replaces
+    ``sigmoid(b)``.
+
+    Returns ``(out [ntok,HV,V] in v.dtype, state_after, cache_after)``; inputs
+    are not modified.
+    """
+    cd = compute_dtype
+    K = q.shape[-1]
+    HV = v.shape[1]
+    if scale is None:
+        scale = K ** -0.5
+    qf, kf = q.float(), k.float()
+    if use_qk_l2norm:
+        qf, kf = l2norm(qf), l2norm(kf)
+    qf = qf * scale
+    rep = HV // q.shape[1]
+    qf = qf.repeat_interleave(rep, dim=1).to(cd)
+    kf = kf.repeat_interleave(rep, dim=1).to(cd)
+    vf = v.to(cd)
+    if log_decay is None:
+        if lower_bound is not None:
+            g = lower_bound_gate(a, dt_bias, A_log, lower_bound, per_channel=is_kda)
+        else:
+            g = softplus_gate(a, dt_bias, A_log, softplus_beta, softplus_threshold,
+                              per_channel=is_kda)
+    else:
+        g = log_decay.float()
+    g = g.to(cd)
+    if not is_kda:
+        g = g[..., None]
+    beta = (sigmoid_beta(b) if beta_activated is None else beta_activated.float()).to(cd)
+
+    state = state.clone()
+    cache = None if cache is None else cache.clone()
+    out = torch.zeros_like(vf)
+    two_d = len(state_indices) > 0 and isinstance(state_indices[0], (list, tuple))
+    bos = 0
+    for n, length in enumerate(lengths):
+        if length == 0:                      # empty request: nothing is read or written
+            continue
+        if two_d:
+            acc = 1 if num_accepted is None else int(num_accepted[n])
+            col = acc - 1 if acc > 0 else 0
+            slot = int(state_indices[n][col])
+        else:
+            slot = int(state_indices[n])
+        if _invalid_slot(slot, is_sglang):   # zeros in o, no state / cache access
+            bos += length
+            continue
+        cidx = -1
+        if cache is not None and cache_indices is not None:
+            cidx = int(cache_indices[n])
+        h = state[slot].to(cd)
+        for t in range(length):
+            if parents is not None and t > 0 and cidx >= 0:
+                parent = int(parents[n][t])
+                if parent >= 0 and parent != t - 1:
+                    h = cache[cidx, parent].to(cd)
+            i = bos + t
+            h, o = recurrent_step(h, qf[i], kf[i], vf[i], g[i], beta[i])
+            out[i] = o
+            if is_sglang:
+                if cache is not None and cidx >= 0:
+                    cache[cidx, t] = h.to(cache.dtype)
+            elif two_d:
+                step_slot = int(state_indices[n][t])
+                if step_slot > 0:
+                    state[step_slot] = h.to(state.dtype)
+        if not disable_state_update:
+            state[slot] = h.to(state.dtype)
+        bos += length
+    return out.to(v.dtype), state, cache
+
+
+def fold_reference(state, rawk, rawv, g, beta, slot_indices, accept_lens, *,
+                   null_block_id=-1, compute_dtype=torch.float32):
+    """Accepted-prefix commit: replay ``accept_lens[n]`` recorded tokens into the state.
+
+    Restates scripts/decode/kda_mtp_sglang/private/_reference.py:183-216
+    (``fold_reference``; one layer): raw k is L2-normalised in division form
+    with eps inside the square root, then decay -> delta -> rank-1.  A request
+    whose slot is ``<= null_block_id`` or whose accepted length is ``<= 0``
+    leaves its slot untouched (src/decode/kda_replayssm/kda_mtp_fold.cu:306).
+
+    ``state [slots,HV,V,K]``; records are indexed by slot: ``rawk [slots,H,L,K]``,
+    ``rawv [slots,HV,L,V]``, ``g [slots,HV,L,K]`` (log-decay), ``beta [slots,HV,L]``.
+    Returns the folded copy of ``state``.
+    """
+    cd = compute_dtype
+    state = state.clone()
+    HV = state.shape[1]
+    H = rawk.shape[1]
+    rep = HV // H
+    for n, slot in enumerate(slot_indices):
+        slot = int(slot)
+        n_acc = int(accept_lens[n])
+        if slot <= null_block_id or n_acc <= 0:
+            continue
+        h = state[slot].to(cd)
+        for t in range(n_acc):
+            kk = rawk[slot, :, t].to(cd)
+            kk = kk / torch.sqrt((kk * kk).sum(-1, keepdim=True) + 1e-6)
+            kk = kk.repeat_interleave(rep, dim=0)
+            h = h * g[slot, :, t].to(cd).exp()[:, None, :]
+            d = torch.einsum("hvk,hk->hv", h, kk)
+            u = (rawv[slot, :, t].to(cd) - d) * beta[slot, :, t].to(cd)[:, None]
+            h = h + u[:, :, None] * kk[:, None, :]
+        state[slot] = h.to(state.dtype)
+    return state
