@@ -1,0 +1,153 @@
+#!/usr/bin/env python3
+"""Headline benchmark: packed GDN decode at batch 256 over an indexed FP32 k-last pool.
+
+One step = one call of ``fused_sigmoid_gating_delta_rule_forward_k_last_packed`` on the
+benchmark configuration (B=256, H=16, HV=32, K=V=128, pool of 4096 slots, 5 % of the
+entries padded with -1).  Inputs are resident in HBM before the timed region.  To keep the
+256 MB last-level cache from serving the state, consecutive steps use disjoint slot sets
+drawn from one seeded permutation of the pool (16 sets of 256 slots = 8.6 GB between two
+uses of a slot), which is what a model with many layers does to the cache.
+
+Prints ONE JSON line (see README / DESIGN for the fields).  ``value`` is the state
+traffic rate: n_active * HV * 131072 bytes per step / step time.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+BF16_PEAK_TFLOPS = 2500.0
+
+
+def build_decode_sets(w, n_sets, pool_slots, B, pad_frac, seed, device):
+    """Disjoint slot sets for consecutive steps, each with the same number of padded entries."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(pool_slots, generator=g).to(torch.int32)
+    n_pad = int(round(B * pad_frac))
+    pad_pos = torch.randperm(B, generator=g)[:n_pad]
+    sets = []
+    for i in range(n_sets):
+        idx = perm[i * B:(i + 1) * B].clone()
+        idx[pad_pos] = -1
+        sets.append(idx.to(device))
+    return sets, B - n_pad
+
+
+def bench_decode(steps, warmup, device):
+    import torch
+    from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
+    from pla_amd.workloads import gdn_decode_packed
+
+    B, H, HV, slots, pad = 256, 16, 32, 4096, 0.05
+    w = gdn_decode_packed(B, H=H, HV=HV, pool_slots=slots, pad_frac=pad, seed=101, device=device)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    sets, n_active = build_decode_sets(w, slots // B, slots, B, pad, 11, device)
+    bytes_state = n_active * HV * 131072
+
+    def step(i):
+        call["initial_state_indices"] = sets[i % len(sets)]
+        packed(**call)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        step(i)
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    kernel_ms = [s.elapsed_time(e) for s, e in zip(starts, ends)]
+    avg_kernel_s = statistics.mean(kernel_ms) * 1e-3
+    return dict(
+        wall_s=wall, ms_per_step=wall / steps * 1e3, bytes_state=bytes_state, n_active=n_active,
+        kernel_us_avg=avg_kernel_s * 1e6, kernel_us_median=statistics.median(kernel_ms) * 1e3,
+        achieved_gbps=bytes_state / avg_kernel_s / 1e9,
+        value_gbps=bytes_state * steps / wall / 1e9, workload=w)
+
+
+def cpu_baseline_decode(w, sample_requests=32, reps=5):
+    """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
+    sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
+    import torch
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from oracle import k_last_reference
+    meta = w["_meta"]
+    H, HV = meta["H"], meta["HV"]
+    n = sample_requests
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    mixed = w["mixed_qkv"][:n].cpu()
+    q = mixed[:, : H * 128].reshape(n, H, 128)
+    k = mixed[:, H * 128: 2 * H * 128].reshape(n, H, 128)
+    v = mixed[:, 2 * H * 128:].reshape(n, HV, 128)
+    a, b = w["a"][:n].cpu(), w["b"][:n].cpu()
+    state = w["initial_state_source"][:n].cpu()
+    idx = list(range(n))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        k_last_reference(q, k, v, a, b, w["A_log"].cpu(), w["dt_bias"].cpu(), state, idx, [1] * n,
+                         scale=w["scale"], use_qk_l2norm=True, is_kda=False)
+        times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    return dict(value=n * HV * 131072 / t / 1e9, unit="GB/s", cores=threads, kind="port",
+                sample="first %d of the 256 requests, one step, median of %d runs (%.1f ms/step for the "
+                       "sample; %.0f us per request)" % (n, reps, t * 1e3, t / n * 1e6),
+                threads_torch=torch.get_num_threads())
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the decode and prefill "
+              "kernels shard by request / head without communication); run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (MI355X)", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    d = bench_decode(args.steps, args.warmup, device)
+    result = {
+        "metric": "gdn_packed_decode_state_hbm_GBps@B=256",
+        "value": round(d["value_gbps"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(d["ms_per_step"], 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "configs[1]: GDN packed-QKV decode, 1 step, B=256 (243 active, 13 padded), "
+                               "H=16, HV=32, K=V=128, FP32 k-last pool of 4096 slots, bf16 activations",
+                   "batch": 256, "n_active": d["n_active"], "pool_slots": 4096,
+                   "slot_rotation": "16 disjoint slot sets, one per consecutive step"},
+        "decode_us_per_step": round(d["kernel_us_avg"], 2),
+        "roofline": {"bound": "hbm", "achieved": round(d["achieved_gbps"], 1), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(d["achieved_gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "k_last_kernel<bf16,GDN,T=1,rows_per_wave=32>",
+                     "bytes_per_launch": d["bytes_state"], "launch_us_avg": round(d["kernel_us_avg"], 2),
+                     "launch_us_median": round(d["kernel_us_median"], 2)},
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_decode(d["workload"])
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,130 @@
+/*
+ * C ABI of libpla_gfx950.so: gated delta-rule (GDN / KDA) decode, MTP verify,
+ * accepted-prefix commit and chunk-64 prefill for AMD MI355X (gfx950).
+ *
+ * Every entry point takes plain device pointers, sizes and element strides and
+ * a hipStream_t (as void*); nothing is retained after the call returns, no
+ * entry point allocates, synchronises or copies to the host, so every call is
+ * hipGraph-capturable.  Return value: 0 on success, non-zero on a rejected
+ * argument or a launch error; pla_last_error() then describes it.  Argument
+ * rejections happen before any kernel is launched, so no state is written.
+ *
+ * Each declaration cites the interface of the reference (t-head/pla) that it
+ * replaces.
+ */
+#ifndef PLA_GFX950_H
+#define PLA_GFX950_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type codes */
+enum {
+  PLA_F32 = 0,
+  PLA_BF16 = 1,
+  PLA_F16 = 2
+};
+
+/* gate_mode of the k-last entry points */
+enum {
+  PLA_GATE_SOFTPLUS = 0,    /* g = -exp(A_log) * softplus_{beta,threshold}(a + dt_bias)           */
+  PLA_GATE_LOWER_BOUND = 1, /* g = lower_bound * sigmoid(exp(A_log) * (a + dt_bias)), KDA only     */
+  PLA_GATE_LOG_DECAY = 2    /* `a` already holds the float32 log-decay g; A_log/dt_bias ignored    */
+};
+
+/* Library identification: "pla_gfx950 <version> gfx950". */
+const char* pla_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* pla_last_error(void);
+
+/*
+ * Packed one-token decode over an indexed FP32 k-last state pool.
+ * Replaces k_last_packed_launcher_t
+ * (src/decode/k-last/fused_sigmoid_gating_cuda_k_last_packed.cpp:53-80) and the
+ * kernel fused_sigmoid_gating_delta_kernel_packed
+ * (src/decode/k-last/fused_sigmoid_gating_k_last_packed_kernel.cuh:59-384).
+ *
+ *   mixed_qkv  [tokens, 2*H*128 + HV*128] act dtype, row pitch stride_qkv elements
+ *   a          [tokens, HV] (GDN) or [tokens, HV*128] (KDA), pitch stride_a
+ *   b          [tokens, HV], pitch stride_b
+ *   A_log      [HV] of alog_dtype;  dt_bias [HV] or [HV*128] act dtype
+ *   o          [tokens, HV, 128] act dtype, dense
+ *   h0         state pool, slot pitch h0_slot_stride floats, slot = [HV,128(V),128(K)]
+ *   cu_seqlens [B+1] int32 or NULL (then request n owns token n)
+ *   h0_indices [B] int32; invalid slot (<0 when is_sglang, <=0 otherwise) => zeros in o,
+ *              no state access;  a request of length 0 touches nothing.
+ * rows_per_wave: 0 = pick from the gfx950 tuning table, else 8, 16 or 32.
+ */
+int pla_k_last_packed_launch(
+    const void* A_log, int alog_dtype, const void* a, const void* dt_bias,
+    float softplus_beta, float softplus_threshold,
+    const void* mixed_qkv, const void* b, void* o, float* h0,
+    const int32_t* cu_seqlens, const int32_t* h0_indices,
+    float scale, int T_max,
+    int64_t stride_a, int64_t stride_qkv, int64_t stride_b, int64_t h0_slot_stride,
+    int B, int H, int HV, int K, int V,
+    int use_qk_l2norm, int is_sglang, int is_kda, int act_dtype,
+    int rows_per_wave, void* stream);
+
+/*
+ * Non-packed decode and MTP / speculative verify.
+ * Replaces k_last_launcher_t
+ * (src/decode/k-last/fused_sigmoid_gating_cuda_k_last.cpp:161-199) and the kernel
+ * fused_sigmoid_gating_delta_kernel
+ * (src/decode/k-last/fused_sigmoid_gating_k_last_kernel.cuh:131-1058).
+ *
+ *   q,k [tokens,H,128], v [tokens,HV,128] act dtype with token pitches stride_q/k/v
+ *   a: gate input (see gate_mode); with PLA_GATE_LOG_DECAY it is float32
+ *   b: raw beta logits (act dtype), or float32 activated beta when beta_is_activated
+ *   dt_bias: float32 when dt_bias_is_f32 else act dtype
+ *   cache: SGLang intermediate-state buffer [rows, cache_steps, HV,128,128] float32 or NULL;
+ *          step t of request n is written to cache[cache_indices[n]*cache_steps + t]
+ *          when is_sglang and cache_indices[n] >= 0
+ *   parents: int64 [B, >=T] eagle-tree parent steps (needs cache), or NULL
+ *   h0_indices: [B] (stride_h0_indices_seq == 0) or a 2-D [B,S] table with row pitch
+ *          stride_h0_indices_seq (vLLM; requires !is_sglang): the start slot is column
+ *          max(num_accepted[n]-1, 0) and step t is written to slot table[n][t] when > 0
+ *   disable_state_update: do not write the final state back to the start slot
+ */
+int pla_k_last_launch(
+    const void* A_log, int alog_dtype, const void* a, const void* dt_bias, int dt_bias_is_f32,
+    float softplus_beta_or_lower_bound, float softplus_threshold, int gate_mode,
+    const void* q, const void* k, const void* v, const void* b, int beta_is_activated,
+    void* o, float* h0, const int32_t* cu_seqlens, float* cache,
+    const int32_t* h0_indices, const int32_t* cache_indices, int cache_steps,
+    const int64_t* parents, int64_t stride_parent_seq, int64_t stride_parent_token,
+    float scale, int T_max,
+    int64_t stride_a, int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_b,
+    int64_t h0_slot_stride,
+    int B, int H, int HV, int K, int V,
+    int use_qk_l2norm, int disable_state_update,
+    const int32_t* num_accepted, int64_t stride_h0_indices_seq, int is_sglang,
+    int is_kda, int act_dtype, int rows_per_wave, void* stream);
+
+/*
+ * Accepted-prefix commit: replays accept_lens[n] recorded tokens of request n into
+ * its FP32 state, in place.  Replaces launch_fold
+ * (src/decode/kda_replayssm/kda_mtp_abi.h:165-176; kernel
+ * src/decode/kda_replayssm/kda_mtp_fold.cu:256-545), single layer per call.
+ *
+ *   h0    [slots,HV,128,128] float32, slot pitch h0_slot_stride
+ *   rawk  [slots,H,L,128]  act dtype (pre-normalisation; L2-normalised inside)
+ *   rawv  [slots,HV,L,128] act dtype
+ *   gk    [slots,HV,L,128] float32 log-decay;  beta [slots,HV,L] float32
+ *   slot_idx, accept_lens [B] int32.  slot <= null_block_id or accept_len <= 0 => untouched.
+ */
+int pla_kda_fold_launch(
+    float* h0, const void* rawv, const void* rawk, const float* gk, const float* beta,
+    const int32_t* slot_idx, const int32_t* accept_lens,
+    int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
+    int64_t gk_slot_stride, int64_t beta_slot_stride,
+    int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PLA_GFX950_H */

@@ -1,0 +1,82 @@
+// Shared host/device helpers for the gfx950 gated delta-rule kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/pla_gfx950.h"
+
+namespace pla {
+
+// ---- error reporting (host) -------------------------------------------------
+char* error_buffer();   // thread-local, 512 bytes
+inline int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(error_buffer(), 512, fmt, ap);
+  va_end(ap);
+  return 1;
+}
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail("%s: %s", what, hipGetErrorString(e));
+  return 0;
+}
+#define PLA_REQUIRE(cond, ...) \
+  do { if (!(cond)) return ::pla::fail(__VA_ARGS__); } while (0)
+
+// ---- 16-bit activation types -------------------------------------------------
+struct bf16_t { uint16_t bits; };
+struct f16_t  { uint16_t bits; };
+
+__device__ __forceinline__ float to_float(bf16_t x) {
+  return __builtin_bit_cast(float, (uint32_t)x.bits << 16);
+}
+__device__ __forceinline__ float to_float(f16_t x) {
+  return (float)__builtin_bit_cast(_Float16, x.bits);
+}
+template <typename T> __device__ __forceinline__ T from_float(float f);
+template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
+  uint32_t u = __builtin_bit_cast(uint32_t, f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40)};  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                                   // round to nearest even
+  return bf16_t{(uint16_t)(u >> 16)};
+}
+template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) {
+  return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
+}
+
+// Low / high half of a packed pair of 16-bit activations.
+template <typename T> __device__ __forceinline__ float lo16(uint32_t w) { return to_float(T{(uint16_t)(w & 0xffffu)}); }
+template <typename T> __device__ __forceinline__ float hi16(uint32_t w) { return to_float(T{(uint16_t)(w >> 16)}); }
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
+  return (uint32_t)from_float<T>(a).bits | ((uint32_t)from_float<T>(b).bits << 16);
+}
+
+// ---- DPP cross-lane sums -----------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float x) {
+  return __builtin_bit_cast(float,
+      __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+// Sum over each aligned group of 16 lanes; every lane of the group gets the total.
+__device__ __forceinline__ float row16_allreduce(float x) {
+  x += dpp_mov<0xB1>(x);    // quad_perm [1,0,3,2]
+  x += dpp_mov<0x4E>(x);    // quad_perm [2,3,0,1]
+  x += dpp_mov<0x141>(x);   // row_half_mirror
+  x += dpp_mov<0x140>(x);   // row_mirror
+  return x;
+}
+// Sum over the whole 64-lane wavefront; every lane gets the total.
+__device__ __forceinline__ float wave64_allreduce(float x) {
+  x = row16_allreduce(x);
+  x += __shfl_xor(x, 16, 64);
+  x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+__device__ __forceinline__ float fast_sigmoid(float x) { return 1.0f / (1.0f + __expf(-x)); }
+
+}  // namespace pla

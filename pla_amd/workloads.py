@@ -1,0 +1,179 @@
+"""Seeded synthetic workloads of the five benchmark configurations.
+
+Used by ``bench.py``, the smoke run and the parity tests so that all of them see
+identical inputs.  Small tensors are drawn on the CPU with a seeded
+``torch.Generator`` and copied to the device; state pools (up to 8.6 GB) are
+drawn on the device with a seeded device generator.
+
+Distributions: q, k ~ N(0,1) rounded to bf16, L2-normalised per head in float32
+and stored as bf16; v ~ N(0,1); b ~ N(0,1) (beta = sigmoid(b)); A_log ~
+U(0, ln 16); a ~ N(0,1); dt_bias ~ U(-1,1); state ~ N(0, 0.1); scale = 128^-0.5.
+"""
+
+import math
+
+import torch
+
+D = 128
+
+
+def _gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def _normalised(shape, g, dtype):
+    x = torch.randn(*shape, generator=g).to(dtype).float()
+    x = x * torch.rsqrt(x.square().sum(-1, keepdim=True) + 1e-6)
+    return x.to(dtype)
+
+
+def _pool(slots, HV, device, seed, pitch_pad=0):
+    """FP32 k-last pool [slots, HV, 128, 128] ~ N(0, 0.1); optional padded slot pitch."""
+    width = HV * D * D
+    if device.type == "cuda":
+        g = torch.Generator(device=device).manual_seed(seed)
+        backing = torch.empty(slots, width + pitch_pad, dtype=torch.float32, device=device)
+        backing.normal_(0.0, 0.1, generator=g)
+    else:
+        backing = torch.randn(slots, width + pitch_pad, generator=_gen(seed)) * 0.1
+    return backing, backing[:, :width].view(slots, HV, D, D)
+
+
+def slot_subset(slots, B, pad_frac, g, pad_value=-1):
+    """First B entries of a seeded permutation (never arange), pad_frac of them set to pad_value."""
+    perm = torch.randperm(slots, generator=g)[:B].to(torch.int32)
+    n_pad = int(round(B * pad_frac))
+    if n_pad:
+        pos = torch.randperm(B, generator=g)[:n_pad]
+        perm[pos] = pad_value
+    return perm
+
+
+def gdn_decode_packed(B, H=16, HV=32, pool_slots=None, pad_frac=0.0, seed=0, device="cuda",
+                      dtype=torch.bfloat16, is_kda=False, pitch_pad=0):
+    """Configs 0/1: packed one-token decode. Returns a dict of call arguments + metadata."""
+    device = torch.device(device)
+    g = _gen(seed)
+    pool_slots = pool_slots or B
+    q = _normalised((B, H, D), g, dtype)
+    k = _normalised((B, H, D), g, dtype)
+    v = torch.randn(B, HV, D, generator=g).to(dtype)
+    mixed = torch.cat([q.reshape(B, -1), k.reshape(B, -1), v.reshape(B, -1)], dim=1)
+    a = torch.randn(B, HV * D if is_kda else HV, generator=g).to(dtype)
+    b = torch.randn(B, HV, generator=g).to(dtype)
+    A_log = torch.rand(HV, generator=g) * math.log(16.0)
+    dt_bias = (torch.rand(HV * D if is_kda else HV, generator=g) * 2 - 1).to(dtype)
+    if pool_slots == B and pad_frac == 0.0:
+        indices = torch.arange(B, dtype=torch.int32)
+    else:
+        indices = slot_subset(pool_slots, B, pad_frac, g)
+    backing, state = _pool(pool_slots, HV, device, seed + 1, pitch_pad)
+    to = lambda t: t.to(device)
+    return dict(
+        mixed_qkv=to(mixed), a=to(a), b=to(b), A_log=to(A_log), dt_bias=to(dt_bias),
+        softplus_beta=1.0, softplus_threshold=20.0, scale=D ** -0.5,
+        initial_state_source=state, initial_state_indices=to(indices),
+        out=torch.empty(B, 1, HV, D, dtype=dtype, device=device),
+        use_qk_l2norm_in_kernel=True,
+        cu_seqlens=to(torch.arange(B + 1, dtype=torch.int32)),
+        is_kda=is_kda, is_sglang=True,
+        _meta=dict(B=B, H=H, HV=HV, backing=backing, n_active=int((indices >= 0).sum()),
+                   state_bytes=int((indices >= 0).sum()) * HV * D * D * 4 * 2),
+    )
+
+
+def kda_mtp_verify(B=64, HV=32, T=4, pool_slots=1024, seed=0, device="cuda", dtype=torch.bfloat16):
+    """Config 2: KDA MTP verify with a supplied per-channel log-decay and accepted-prefix commit.
+
+    g = -softplus(N(0,1)) * U(0.01, 1) float32 [B*T, HV, 128]; num_accepted ~ U{0..T}.
+    Records for the commit are laid out per slot: rawk/rawv [slots, HV, T, 128] bf16,
+    gk [slots, HV, T, 128] float32, beta [slots, HV, T] float32.
+    """
+    device = torch.device(device)
+    g = _gen(seed)
+    H = HV
+    nt = B * T
+    q = _normalised((nt, H, D), g, dtype)
+    k = _normalised((nt, H, D), g, dtype)
+    v = torch.randn(nt, HV, D, generator=g).to(dtype)
+    log_decay = -torch.nn.functional.softplus(torch.randn(nt, HV, D, generator=g)) * \
+        (torch.rand(nt, HV, D, generator=g) * 0.99 + 0.01)
+    beta = torch.sigmoid(torch.randn(nt, HV, generator=g))
+    indices = slot_subset(pool_slots, B, 0.0, g)
+    num_accepted = torch.randint(0, T + 1, (B,), generator=g).to(torch.int32)
+    backing, state = _pool(pool_slots, HV, device, seed + 1)
+    to = lambda t: t.to(device)
+    return dict(
+        q=to(q.view(1, nt, H, D)), k=to(k.view(1, nt, H, D)), v=to(v.view(1, nt, HV, D)),
+        log_decay=to(log_decay), beta=to(beta), state=state, indices=to(indices),
+        num_accepted=to(num_accepted), cu_seqlens=to(torch.arange(0, nt + 1, T, dtype=torch.int32)),
+        scale=D ** -0.5, _meta=dict(B=B, H=H, HV=HV, T=T, backing=backing),
+    )
+
+
+def ragged_lengths(n_seq, lo, hi, seed):
+    g = _gen(seed)
+    return torch.randint(lo, hi + 1, (n_seq,), generator=g).tolist()
+
+
+def gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=64, seed=0, device="cuda", dtype=torch.bfloat16,
+                       tail_pad=0):
+    """Config 3: packed varlen GDN prefill with raw gating and an indexed FP32 pool."""
+    device = torch.device(device)
+    g = _gen(seed)
+    T = sum(lengths) + tail_pad
+    N = len(lengths)
+    q = torch.randn(T, H, D, generator=g).to(dtype)
+    k = torch.randn(T, H, D, generator=g).to(dtype)
+    v = torch.randn(T, HV, D, generator=g).to(dtype)
+    packed = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], dim=1)
+    a = torch.randn(T, HV, generator=g).to(dtype)
+    b = torch.randn(T, HV, generator=g).to(dtype)
+    A_log = torch.rand(HV, generator=g) * math.log(16.0)
+    dt_bias = torch.rand(HV, generator=g) * 2 - 1
+    offs = [0]
+    for n in lengths:
+        offs.append(offs[-1] + n)
+    indices = slot_subset(pool_slots, N, 0.0, g)
+    backing, state = _pool(pool_slots, HV, device, seed + 1)
+    to = lambda t: t.to(device)
+    return dict(
+        packed_qkv=to(packed), raw_gate_a=to(a), raw_beta_b=to(b), A_log=to(A_log), dt_bias=to(dt_bias),
+        cu_seqlens=to(torch.tensor(offs, dtype=torch.int32)), num_qk_heads=H, num_v_heads=HV,
+        scale=D ** -0.5, initial_state=state, initial_state_indices=to(indices),
+        raw_cu_seqlens=tuple(offs),
+        _meta=dict(T=T, N=N, H=H, HV=HV, offsets=offs, backing=backing),
+    )
+
+
+def kda_prefill(T=65536, H=32, seed=0, device="cuda", dtype=torch.bfloat16, lower_bound=-5.0):
+    """Config 4: one long KDA sequence; heads [0, H/2) decay strongly (g ~ -U(0.5, 2) per token
+    and channel), heads [H/2, H) weakly (g ~ -U(1e-4, 1e-2)).
+
+    The operator takes the RAW gate: with A_log = 0 and dt_bias = 0 the lower-bound gate is
+    g = lower_bound * sigmoid(raw), so raw = logit(g / lower_bound), stored in bf16.
+    """
+    device = torch.device(device)
+    g = _gen(seed)
+    q = torch.randn(T, H, D, generator=g).to(dtype)
+    k = torch.randn(T, H, D, generator=g).to(dtype)
+    v = torch.randn(T, H, D, generator=g).to(dtype)
+    u = torch.rand(T, H, D, generator=g)
+    strong = -(0.5 + 1.5 * u)
+    weak = -(1e-4 + (1e-2 - 1e-4) * u)
+    target = torch.where((torch.arange(H) < H // 2)[None, :, None], strong, weak)
+    frac = (target / lower_bound).clamp(1e-7, 1 - 1e-7)
+    raw = torch.log(frac) - torch.log1p(-frac)
+    beta_raw = torch.randn(T, H, generator=g).to(dtype)
+    g2 = torch.Generator().manual_seed(seed + 1)
+    state = torch.randn(1, H, D, D, generator=g2) * 0.1
+    to = lambda t: t.to(device)
+    return dict(
+        q=to(q), k=to(k), v=to(v), g=to(raw.to(dtype)), beta=to(beta_raw),
+        A_log=to(torch.zeros(H)), dt_bias=to(torch.zeros(H, D)),
+        out=torch.empty(T, H, D, dtype=dtype, device=device),
+        scale=D ** -0.5, lower_bound=lower_bound, initial_state=to(state),
+        final_state=torch.empty(1, H, D, D, dtype=torch.float32, device=device),
+        cu_seqlens=to(torch.tensor([0, T], dtype=torch.int32)), raw_cu_seqlens=(0, T),
+        _meta=dict(T=T, H=H),
+    )
