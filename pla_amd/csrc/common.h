@@ -39,10 +39,7 @@ __device__ __forceinline__ float to_float(f16_t x) {
 }
 template <typename T> __device__ __forceinline__ T from_float(float f);
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float f) {
-  uint32_t u = __builtin_bit_cast(uint32_t, f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t{(uint16_t)((u >> 16) | 0x40)};  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                                   // round to nearest even
-  return bf16_t{(uint16_t)(u >> 16)};
+  return bf16_t{__builtin_bit_cast(uint16_t, (__bf16)f)};   // v_cvt_pk_bf16_f32, round to nearest even
 }
 template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) {
   return f16_t{__builtin_bit_cast(uint16_t, (_Float16)f)};
@@ -51,8 +48,18 @@ template <> __device__ __forceinline__ f16_t from_float<f16_t>(float f) {
 // Low / high half of a packed pair of 16-bit activations.
 template <typename T> __device__ __forceinline__ float lo16(uint32_t w) { return to_float(T{(uint16_t)(w & 0xffffu)}); }
 template <typename T> __device__ __forceinline__ float hi16(uint32_t w) { return to_float(T{(uint16_t)(w >> 16)}); }
-template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b) {
-  return (uint32_t)from_float<T>(a).bits | ((uint32_t)from_float<T>(b).bits << 16);
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+// Two floats rounded (nearest even) and packed, `a` in the low half.
+template <typename T> __device__ __forceinline__ uint32_t pack2(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2<bf16_t>(float a, float b) {
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));   // one v_cvt_pk_bf16_f32
+}
+template <> __device__ __forceinline__ uint32_t pack2<f16_t>(float a, float b) {
+  const f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2_t));
 }
 
 // ---- DPP cross-lane sums -----------------------------------------------------
@@ -77,6 +84,8 @@ __device__ __forceinline__ float wave64_allreduce(float x) {
   return x;
 }
 
-__device__ __forceinline__ float fast_sigmoid(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }     // v_rcp_f32, 1 ulp
+__device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }  // v_rsq_f32, 1 ulp
+__device__ __forceinline__ float fast_sigmoid(float x) { return fast_rcp(1.0f + __expf(-x)); }
 
 }  // namespace pla
