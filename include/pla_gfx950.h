@@ -124,6 +124,43 @@ int pla_kda_fold_launch(
     int64_t gk_slot_stride, int64_t beta_slot_stride,
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
 
+/*
+ * Workspace size in bytes (256-byte aligned buffer) needed by pla_gdn_prefill_launch for T physical
+ * tokens in N sequences.  Chunk metadata is sized for the worst case T/64 + N chunks so that no
+ * host copy of cu_seqlens is needed.
+ */
+int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV);
+
+/*
+ * GDN chunk-64 prefill over packed variable-length sequences (scalar gate per value head).
+ * Replaces the FlashQLA stage launchers launch_*_cute
+ * (src/prefill/flashqla/host/torch_extension_cute.cc:60-148: chunk_local_cumsum_qk_norm_gated,
+ * kkt_solve, fused_fwd) with one call that runs all stages on `stream`.
+ *
+ *   q,k [T,H,128], v [T,HV,128] bf16 with token pitches stride_q/k/v (views into a packed
+ *       Q|K|V row are fine); a,b [T,HV] raw gate / beta logits (pitches stride_a/b) with
+ *       A_log, dt_bias [HV] float32:  g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b);
+ *       or g_in, beta_in [T,HV] float32 (log-decay per token, activated beta) instead.
+ *   normalize_qk: L2-normalise q and k (eps 1e-6 inside the root) and round to bf16 first.
+ *   cu_seqlens [N+1] int32; tokens at and beyond cu_seqlens[N] are padding: their rows of o
+ *       are set to zero and they never touch a state.  Empty sequences keep their state.
+ *   h0 / ht: k-last FP32 state [slots,HV,128,128] read at h0_indices[n] (or n when the index
+ *       array is NULL; zero state when h0 is NULL) and written at ht_indices[n].  h0 == ht with
+ *       the same indices updates an indexed pool in place.
+ *   o [T,HV,128] bf16 dense.   gcum_out / beta_out: optional [T,HV] float32 copies of the
+ *       chunk-local cumulative log-decay and of beta (NULL keeps them in the workspace).
+ */
+int pla_gdn_prefill_launch(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,6 +33,14 @@ SIGNATURES = {
         _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
         _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_gdn_prefill_launch": [
+        _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64,
+        _c_p, _c_p, _c_i64, _c_i64,
+        _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_int, _c_int, _c_f, _c_int,
+        _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
+        _c_p, _c_p, _c_i64, _c_p, _c_p,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
 }
 
 _lib = None
@@ -52,6 +60,8 @@ def load():
     lib.pla_version.argtypes = []
     lib.pla_last_error.restype = ctypes.c_char_p
     lib.pla_last_error.argtypes = []
+    lib.pla_gdn_prefill_workspace_bytes.restype = _c_i64
+    lib.pla_gdn_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int, _c_int]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _c_int

@@ -1,0 +1,637 @@
+// Chunk-64 gated delta-rule prefill for GDN (scalar gate per value head) on gfx950.
+//
+// Per chunk of C = 64 tokens (G = inclusive cumulative log-decay inside the chunk, S the
+// FP32 state, k-last):
+//     L   = I + strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
+//     W   = L^-1 diag(beta)                                   (parallel over chunks)
+//     P   = scale * tril(q_i . k_j e^{G_i - G_j})             (parallel over chunks)
+//     X   = V - e^{G} (.) (K S^T)         U = W X             (sequential)
+//     O   = scale e^{G} (.) (Q S^T) + P U
+//     S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
+// which is the WY/UT form of the token recurrence (reference algebra:
+// scripts/prefill/flashqla/private/ref_gdr.py:78-298; kernels
+// src/prefill/flashqla/kernels/chunk_cumsum_cute.cu:232-330, kkt_solve_cute_impl.cuh:34-60,
+// fused_fwd_cute.cu:34-66).  Because the gate is a scalar per (token, head) every decay is a
+// row or column scaling of a GEMM result, so the bf16 MFMA operands q, k, v stay exact;
+// the FP32 quantities that feed the state (S, X, W, U) are split into bf16 hi + lo parts
+// (16 mantissa bits), which keeps the FP32 final state within 1e-5 of a float64 evaluation.
+//
+// Kernels:
+//   gdn_chunk_map_kernel     chunk table from cu_seqlens (device side, graph-capturable)
+//   gdn_prep_kernel          gate, beta, chunk-local cumsum, q/k L2 norm (rounded to bf16), K^T tiles
+//   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
+//                            forward substitution in LDS, W (hi/lo) and P to the workspace
+//   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), 8 wavefronts each owning a
+//                            16-wide V slice of S^T in MFMA accumulator layout; the chain
+//                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_bf16 with every
+//                            intermediate staying in registers (an accumulator tile is already a
+//                            valid B operand of the next product), A operands staged through LDS.
+
+#include "common.h"
+
+namespace pla {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x8_t __attribute__((ext_vector_type(8)));
+
+constexpr int CHUNK = 64;
+
+__device__ __forceinline__ f32x4_t mfma16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// hi = bf16(x), lo = bf16(x - hi) for two accumulator quads (eight contraction elements).
+struct HiLo { bf16x8_t hi, lo; };
+__device__ __forceinline__ HiLo split8(f32x4_t a, f32x4_t b) {
+  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  HiLo r;
+  r.hi = __builtin_convertvector(x, bf16x8_t);
+  const f32x8_t back = __builtin_convertvector(r.hi, f32x8_t);
+  r.lo = __builtin_convertvector(x - back, bf16x8_t);
+  return r;
+}
+__device__ __forceinline__ bf16x8_t round8(f32x4_t a, f32x4_t b) {
+  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  return __builtin_convertvector(x, bf16x8_t);
+}
+
+// A (or B) operand of one 16x16x32 MFMA step from a row-major bf16 tile: lane (r = lane%16,
+// kb = lane/16) takes columns [32s+4kb, +4) and [32s+16+4kb, +4) of row r, which is the
+// contraction order in which an accumulator tile pair (row blocks 2s, 2s+1) presents its rows.
+__device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s, int kb) {
+  const uint2 p0 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 4 * kb);
+  const uint2 p1 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 16 + 4 * kb);
+  const uint4 u = make_uint4(p0.x, p0.y, p1.x, p1.y);
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
+struct GdnPrefillParams {
+  // inputs
+  const void* q; const void* k; const void* v;        // activation dtype, token strides below
+  int64_t stride_q, stride_k, stride_v;               // elements
+  const void* a; const void* b; int64_t stride_a, stride_b;   // raw gate / beta logits [T, HV]
+  const float* A_log; const float* dt_bias;           // [HV]
+  const float* g_in; const float* beta_in;            // optional precomputed log-decay / beta [T, HV]
+  const int32_t* cu_seqlens; int N; int T;            // packed offsets, sequences, physical tokens
+  float scale; int normalize_qk;
+  // state
+  const float* h0; const int32_t* h0_indices; int64_t h0_slot_stride;   // read (may be null)
+  float* ht; const int32_t* ht_indices; int64_t ht_slot_stride;         // written (may be null)
+  // output
+  void* o;                                            // [T, HV, 128] dense
+  // workspace
+  int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
+  uint16_t* qn; uint16_t* kn; uint16_t* knT;
+  float* gcum; float* beta;
+  uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
+  int H, HV, NC_max;
+};
+
+// ---------------------------------------------------------------------------------------------
+__global__ void gdn_chunk_map_kernel(const GdnPrefillParams p) {
+  // Single workgroup: exclusive scan of chunks per sequence, then the per-chunk table.
+  __shared__ int total;
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int n = 0; n < p.N; ++n) {
+      p.seq_chunk_off[n] = acc;
+      const int len = max(p.cu_seqlens[n + 1] - p.cu_seqlens[n], 0);
+      acc += (len + CHUNK - 1) / CHUNK;
+    }
+    p.seq_chunk_off[p.N] = acc;
+    total = acc;
+  }
+  __syncthreads();
+  for (int n = threadIdx.x; n < p.N; n += blockDim.x) {
+    const int start = p.cu_seqlens[n];
+    const int len = max(p.cu_seqlens[n + 1] - start, 0);
+    const int c0 = p.seq_chunk_off[n];
+    const int nc = (len + CHUNK - 1) / CHUNK;
+    for (int c = 0; c < nc; ++c) {
+      if (c0 + c >= p.NC_max) break;
+      p.chunk_seq[c0 + c] = n;
+      p.chunk_tok[c0 + c] = start + c * CHUNK;
+      p.chunk_len[c0 + c] = min(CHUNK, len - c * CHUNK);
+    }
+  }
+  (void)total;
+}
+
+// ---------------------------------------------------------------------------------------------
+// One workgroup (256 threads) per chunk.
+template <typename act_t>
+__global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
+  const int cb = blockIdx.x;
+  if (cb >= p.seq_chunk_off[p.N]) return;
+  const int t0 = p.chunk_tok[cb];
+  const int len = p.chunk_len[cb];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  __shared__ uint16_t tile[CHUNK][130];     // normalised k of one head, for the transposed copy
+
+  // gate, beta, chunk-local cumulative log-decay: one thread per value head
+  for (int hv = threadIdx.x; hv < p.HV; hv += blockDim.x) {
+    float cum = 0.f;
+    const float eA = p.g_in ? 0.f : expf(p.A_log[hv]);
+    const float dt = p.g_in ? 0.f : p.dt_bias[hv];
+    for (int j = 0; j < len; ++j) {
+      const int64_t t = t0 + j;
+      float g, bt;
+      if (p.g_in) {
+        g = p.g_in[t * p.HV + hv];
+        bt = p.beta_in[t * p.HV + hv];
+      } else {
+        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + dt;
+        const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
+        g = -eA * sp;
+        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
+        bt = 1.0f / (1.0f + expf(-braw));
+      }
+      cum += g;
+      p.gcum[t * p.HV + hv] = cum;
+      p.beta[t * p.HV + hv] = bt;
+    }
+  }
+
+  // q / k L2 normalisation (float32, eps inside the root), rounded to bf16
+  for (int h = 0; h < p.H; ++h) {
+    for (int j = wave; j < CHUNK; j += 4) {
+      uint32_t kw = 0;
+      if (j < len) {
+        const int64_t t = t0 + j;
+        const uint32_t qw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.q) + t * p.stride_q + h * 128 + 2 * lane);
+        kw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.k) + t * p.stride_k + h * 128 + 2 * lane);
+        float q0 = lo16<act_t>(qw), q1 = hi16<act_t>(qw), k0 = lo16<act_t>(kw), k1 = hi16<act_t>(kw);
+        if (p.normalize_qk) {
+          const float qs = wave64_allreduce(q0 * q0 + q1 * q1);
+          const float ks = wave64_allreduce(k0 * k0 + k1 * k1);
+          const float qi = rsqrtf(qs + 1e-6f), ki = rsqrtf(ks + 1e-6f);
+          q0 *= qi; q1 *= qi; k0 *= ki; k1 *= ki;
+        }
+        const uint32_t qo = pack2<bf16_t>(q0, q1);
+        kw = pack2<bf16_t>(k0, k1);
+        *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = qo;
+        *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = kw;
+      }
+      *reinterpret_cast<uint32_t*>(&tile[j][2 * lane]) = kw;       // zero rows beyond the chunk
+    }
+    __syncthreads();
+    // K^T tile [128][64]: thread (c, half) gathers 32 tokens of column c
+    {
+      const int c = threadIdx.x >> 1, half = threadIdx.x & 1;
+      uint16_t* dst = p.knT + (((int64_t)cb * p.H + h) * 128 + c) * CHUNK + 32 * half;
+#pragma unroll
+      for (int jj = 0; jj < 32; jj += 2) {
+        const uint32_t w = (uint32_t)tile[32 * half + jj][c] | ((uint32_t)tile[32 * half + jj + 1][c] << 16);
+        *reinterpret_cast<uint32_t*>(dst + jj) = w;
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// One wavefront per (chunk, value head).
+__global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillParams p) {
+  const int cb = blockIdx.x / p.HV;
+  const int hv = blockIdx.x - cb * p.HV;
+  if (cb >= p.seq_chunk_off[p.N]) return;
+  const int h = hv / (p.HV / p.H);
+  const int t0 = p.chunk_tok[cb];
+  const int len = p.chunk_len[cb];
+  const int lane = threadIdx.x;
+  const int r16 = lane & 15, kb = lane >> 4;
+
+  __shared__ float Lm[CHUNK][68];
+  __shared__ float Gs[CHUNK];
+  __shared__ float Bs[CHUNK];
+
+  {
+    const bool ok = lane < len;
+    const float glast = p.gcum[(int64_t)(t0 + len - 1) * p.HV + hv];
+    Gs[lane] = ok ? p.gcum[(int64_t)(t0 + lane) * p.HV + hv] : glast;
+    Bs[lane] = ok ? p.beta[(int64_t)(t0 + lane) * p.HV + hv] : 0.f;
+  }
+
+  // operands of K and Q: 4 row blocks x 4 contraction steps
+  bf16x8_t Kop[4][4], Qop[4][4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const int row = 16 * mb + r16;
+    const bool ok = row < len;
+    const uint16_t* kr = p.kn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
+    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      bf16x8_t kz = operand_from(kr, s, kb), qz = operand_from(qr, s, kb);
+      if (!ok) {
+        const uint4 z = make_uint4(0, 0, 0, 0);
+        kz = __builtin_bit_cast(bf16x8_t, z);
+        qz = kz;
+      }
+      Kop[mb][s] = kz;
+      Qop[mb][s] = qz;
+    }
+  }
+  __syncthreads();
+
+  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      if (ni > mi) {
+        // strictly upper blocks: L is not read there, P is zero
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Pt[(16 * mi + 4 * kb + r) * 64 + 16 * ni + r16] = 0;
+        continue;
+      }
+      f32x4_t kk = {0.f, 0.f, 0.f, 0.f}, qk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        kk = mfma16(Kop[mi][s], Kop[ni][s], kk);
+        qk = mfma16(Qop[mi][s], Kop[ni][s], qk);
+      }
+      const int j = 16 * ni + r16;
+      const float Gj = Gs[j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * mi + 4 * kb + r;
+        const float gam = i >= j ? __expf(Gs[i] - Gj) : 0.f;
+        Lm[i][j] = i > j ? Bs[i] * kk[r] * gam : 0.f;
+        Pt[i * 64 + j] = from_float<bf16_t>(p.scale * qk[r] * gam).bits;
+      }
+    }
+  }
+  __syncthreads();
+
+  // forward substitution, one column per lane: x_i = beta_j [i == j] - sum_{l < i} L[i][l] x_l
+  float x[CHUNK];
+  const float bj = Bs[lane];
+#pragma unroll
+  for (int i = 0; i < CHUNK; ++i) {
+    float acc = (i == lane) ? bj : 0.f;
+#pragma unroll
+    for (int l4 = 0; l4 < i; l4 += 4) {
+      const float4 row = *reinterpret_cast<const float4*>(&Lm[i][l4]);
+      acc = fmaf(-row.x, x[l4], acc);
+      if (l4 + 1 < i) acc = fmaf(-row.y, x[l4 + 1], acc);
+      if (l4 + 2 < i) acc = fmaf(-row.z, x[l4 + 2], acc);
+      if (l4 + 3 < i) acc = fmaf(-row.w, x[l4 + 3], acc);
+    }
+    x[i] = acc;
+  }
+  uint16_t* const Wh = p.Whi + ((int64_t)cb * p.HV + hv) * 4096;
+  uint16_t* const Wl = p.Wlo + ((int64_t)cb * p.HV + hv) * 4096;
+#pragma unroll
+  for (int i = 0; i < CHUNK; ++i) {
+    const bf16_t hi = from_float<bf16_t>(x[i]);
+    Wh[i * 64 + lane] = hi.bits;
+    Wl[i * 64 + lane] = from_float<bf16_t>(x[i] - to_float(hi)).bits;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// LDS tiles of the sequential kernel (bf16 elements, padded pitches keep 16-byte row alignment
+// and spread rows over banks).
+constexpr int PITCH128 = 136;
+constexpr int PITCH64 = 72;
+struct SeqTiles {
+  uint16_t K[CHUNK][PITCH128];
+  uint16_t Q[CHUNK][PITCH128];
+  uint16_t Kt[128][PITCH64];
+  uint16_t Whi[CHUNK][PITCH64];
+  uint16_t Wlo[CHUNK][PITCH64];
+  uint16_t P[CHUNK][PITCH64];
+  float sQ[CHUNK];     // scale * e^{G_i}
+  float eG[CHUNK];     // e^{G_i}
+  float dG[CHUNK];     // e^{G_last - G_i}
+  float eGlast;
+};
+
+// Registers holding the next chunk's tiles while the current chunk is being processed.
+struct SeqPrefetch {
+  uint4 k[2], q[2], kt[2], whi, wlo, pp;
+  float g;
+};
+
+template <typename act_t>
+__global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
+  const int n = blockIdx.x / p.HV;
+  const int hv = blockIdx.x - n * p.HV;
+  const int h = hv / (p.HV / p.H);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int vcol = 16 * wave + r16;                  // this lane's V column
+  const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
+  if (c_begin >= c_end) return;                      // empty sequence: state untouched, no output
+
+  __shared__ SeqTiles T;
+
+  // S^T slice in accumulator layout: St[mc][r] = S[v = vcol][c = 16 mc + 4 kb + r]
+  f32x4_t St[8];
+  {
+    const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
+    if (slot >= 0) {
+      const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)hv * 128 + vcol) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+        St[mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+      }
+    } else {
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+
+  // cooperative tile fetch: 512 threads x 16 bytes
+  auto fetch = [&](int cb) {
+    SeqPrefetch f;
+    const int t0 = p.chunk_tok[cb];
+    const int len = p.chunk_len[cb];
+    const uint4 z = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int vec = tid + 512 * u;                 // 1024 vectors of 8 elements: 64 rows x 16
+      const int row = vec >> 4, cv = vec & 15;
+      const bool ok = row < len;
+      const int64_t tok = t0 + (ok ? row : 0);
+      const uint4 kx = *reinterpret_cast<const uint4*>(p.kn + (tok * p.H + h) * 128 + 8 * cv);
+      const uint4 qx = *reinterpret_cast<const uint4*>(p.qn + (tok * p.H + h) * 128 + 8 * cv);
+      f.k[u] = ok ? kx : z;
+      f.q[u] = ok ? qx : z;
+      // K^T: 128 rows x 8 vectors
+      f.kt[u] = *reinterpret_cast<const uint4*>(p.knT + ((int64_t)cb * p.H + h) * 8192 + 8 * vec);
+    }
+    {
+      const int64_t tb = ((int64_t)cb * p.HV + hv) * 4096 + 8 * tid;   // 512 vectors: 64 rows x 8
+      f.whi = *reinterpret_cast<const uint4*>(p.Whi + tb);
+      f.wlo = *reinterpret_cast<const uint4*>(p.Wlo + tb);
+      f.pp = *reinterpret_cast<const uint4*>(p.P + tb);
+    }
+    f.g = 0.f;
+    if (tid < CHUNK) {
+      const int j = tid < len ? tid : len - 1;
+      f.g = p.gcum[(int64_t)(t0 + j) * p.HV + hv];
+    }
+    return f;
+  };
+  auto stash = [&](const SeqPrefetch& f, int len) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int vec = tid + 512 * u;
+      const int row = vec >> 4, cv = vec & 15;
+      *reinterpret_cast<uint4*>(&T.K[row][8 * cv]) = f.k[u];
+      *reinterpret_cast<uint4*>(&T.Q[row][8 * cv]) = f.q[u];
+      const int trow = vec >> 3, tcv = vec & 7;
+      *reinterpret_cast<uint4*>(&T.Kt[trow][8 * tcv]) = f.kt[u];
+    }
+    {
+      const int row = tid >> 3, cv = tid & 7;
+      *reinterpret_cast<uint4*>(&T.Whi[row][8 * cv]) = f.whi;
+      *reinterpret_cast<uint4*>(&T.Wlo[row][8 * cv]) = f.wlo;
+      *reinterpret_cast<uint4*>(&T.P[row][8 * cv]) = f.pp;
+    }
+    if (tid < CHUNK) {
+      // every lane of wave 0 holds G_j; the last valid row's value is G_last
+      const float glast = __shfl(f.g, len - 1, 64);
+      const float e = __expf(f.g);
+      T.eG[tid] = e;
+      T.sQ[tid] = p.scale * e;
+      T.dG[tid] = __expf(glast - f.g);
+      if (tid == 0) T.eGlast = __expf(glast);
+    }
+  };
+
+  SeqPrefetch nxt = fetch(c_begin);
+  for (int cb = c_begin; cb < c_end; ++cb) {
+    const int t0 = p.chunk_tok[cb];
+    const int len = p.chunk_len[cb];
+    __syncthreads();                 // everyone finished reading the previous chunk's tiles
+    stash(nxt, len);
+    __syncthreads();
+    if (cb + 1 < c_end) nxt = fetch(cb + 1);
+
+    // V of this lane's column for the 16 rows it owns in accumulator layout
+    float vreg[4][4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * mi + 4 * kb + r;
+        vreg[mi][r] = i < len
+            ? to_float(reinterpret_cast<const act_t*>(p.v)[(int64_t)(t0 + i) * p.stride_v + hv * 128 + vcol])
+            : 0.f;
+      }
+
+    // (1) KS = K S^T and (3a) QS = Q S^T : contraction over the 128 K channels
+    f32x4_t KS[4], QS[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) { KS[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[mi] = KS[mi]; }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const HiLo sb = split8(St[2 * s], St[2 * s + 1]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        const bf16x8_t ka = operand_from(&T.K[16 * mi + r16][0], s, kb);
+        const bf16x8_t qa = operand_from(&T.Q[16 * mi + r16][0], s, kb);
+        KS[mi] = mfma16(ka, sb.hi, KS[mi]);
+        KS[mi] = mfma16(ka, sb.lo, KS[mi]);
+        QS[mi] = mfma16(qa, sb.hi, QS[mi]);
+      }
+    }
+
+    // X = V - e^{G} (.) KS   (rows of the accumulator are tokens)
+    f32x4_t X[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) X[mi][r] = vreg[mi][r] - T.eG[16 * mi + 4 * kb + r] * KS[mi][r];
+
+    // (2) U = W X : contraction over the 64 tokens, W and X both split
+    f32x4_t U[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) U[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const HiLo xb = split8(X[2 * s], X[2 * s + 1]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        const bf16x8_t wh = operand_from(&T.Whi[16 * mi + r16][0], s, kb);
+        const bf16x8_t wl = operand_from(&T.Wlo[16 * mi + r16][0], s, kb);
+        U[mi] = mfma16(wh, xb.hi, U[mi]);
+        U[mi] = mfma16(wl, xb.hi, U[mi]);
+        U[mi] = mfma16(wh, xb.lo, U[mi]);
+      }
+    }
+
+    // (3b) O = scale e^{G} (.) QS + P U
+    f32x4_t O[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) O[mi][r] = T.sQ[16 * mi + 4 * kb + r] * QS[mi][r];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const bf16x8_t ub = round8(U[2 * s], U[2 * s + 1]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+        O[mi] = mfma16(operand_from(&T.P[16 * mi + r16][0], s, kb), ub, O[mi]);
+    }
+    {
+      act_t* const orow = reinterpret_cast<act_t*>(p.o) + ((int64_t)t0 * p.HV + hv) * 128 + vcol;
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int i = 16 * mi + 4 * kb + r;
+          if (i < len) orow[(int64_t)i * p.HV * 128] = from_float<act_t>(O[mi][r]);
+        }
+    }
+
+    // (4) S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
+    const float egl = T.eGlast;
+#pragma unroll
+    for (int mc = 0; mc < 8; ++mc) St[mc] *= egl;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      f32x4_t u0 = U[2 * s], u1 = U[2 * s + 1];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        u0[r] *= T.dG[32 * s + 4 * kb + r];
+        u1[r] *= T.dG[32 * s + 16 + 4 * kb + r];
+      }
+      const HiLo ub = split8(u0, u1);
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const bf16x8_t ka = operand_from(&T.Kt[16 * mc + r16][0], s, kb);
+        St[mc] = mfma16(ka, ub.hi, St[mc]);
+        St[mc] = mfma16(ka, ub.lo, St[mc]);
+      }
+    }
+  }
+
+  if (p.ht != nullptr) {
+    const int slot = p.ht_indices ? p.ht_indices[n] : n;
+    if (slot >= 0) {
+      float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)hv * 128 + vcol) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[mc].x, St[mc].y, St[mc].z, St[mc].w);
+    }
+  }
+}
+
+// Zero the output rows that lie beyond the last sequence (physical padding).
+template <typename act_t>
+__global__ void gdn_zero_tail_kernel(const GdnPrefillParams p) {
+  const int64_t first = (int64_t)p.cu_seqlens[p.N] * p.HV * 128;
+  const int64_t total = (int64_t)p.T * p.HV * 128;
+  uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
+  for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    o[i] = 0;
+}
+
+static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
+
+struct GdnWorkspaceLayout {
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, Whi, Wlo, P, total;
+  int NC_max;
+};
+static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
+  GdnWorkspaceLayout L;
+  L.NC_max = T / CHUNK + N;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { const size_t at = off; off = align_up(off + bytes); return at; };
+  L.seq_chunk_off = take((size_t)(N + 1) * 4);
+  L.chunk_seq = take((size_t)L.NC_max * 4);
+  L.chunk_tok = take((size_t)L.NC_max * 4);
+  L.chunk_len = take((size_t)L.NC_max * 4);
+  L.qn = take((size_t)T * H * 128 * 2);
+  L.kn = take((size_t)T * H * 128 * 2);
+  L.knT = take((size_t)L.NC_max * H * 128 * CHUNK * 2);
+  L.gcum = take((size_t)T * HV * 4);
+  L.beta = take((size_t)T * HV * 4);
+  L.Whi = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.Wlo = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.P = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.total = off;
+  return L;
+}
+
+}  // namespace pla
+
+using namespace pla;
+
+extern "C" int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV) {
+  if (T <= 0 || N <= 0 || H <= 0 || HV <= 0) return 0;
+  return (int64_t)gdn_layout(T, N, H, HV).total;
+}
+
+extern "C" int pla_gdn_prefill_launch(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream) {
+  PLA_REQUIRE(K == 128 && V == 128, "GDN prefill requires head_dim K == V == 128, got K=%d, V=%d", K, V);
+  PLA_REQUIRE(T > 0 && N > 0, "GDN prefill needs at least one token and one sequence");
+  PLA_REQUIRE(H > 0 && HV >= H && HV % H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", H, HV);
+  PLA_REQUIRE(act_dtype == PLA_BF16, "GDN prefill takes bf16 activations (the MFMA operands are bf16)");
+  PLA_REQUIRE(q && k && v && o && cu_seqlens && workspace, "null tensor pointer");
+  PLA_REQUIRE((g_in != nullptr) == (beta_in != nullptr), "g and beta must be given together");
+  PLA_REQUIRE(g_in != nullptr || (a && b && A_log && dt_bias), "raw gating needs a, b, A_log and dt_bias");
+  PLA_REQUIRE(((uintptr_t)q % 4 == 0) && ((uintptr_t)k % 4 == 0) && stride_q % 2 == 0 && stride_k % 2 == 0,
+              "q/k rows require 4-byte alignment");
+  const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV);
+  PLA_REQUIRE(workspace_bytes >= (int64_t)L.total, "workspace too small: need %zu bytes", L.total);
+  PLA_REQUIRE((uintptr_t)workspace % 256 == 0, "workspace requires 256-byte alignment");
+  if (h0) PLA_REQUIRE((uintptr_t)h0 % 16 == 0 && h0_slot_stride % 4 == 0, "state requires 16-byte alignment");
+  if (ht) PLA_REQUIRE((uintptr_t)ht % 16 == 0 && ht_slot_stride % 4 == 0, "state requires 16-byte alignment");
+
+  char* ws = reinterpret_cast<char*>(workspace);
+  GdnPrefillParams p{};
+  p.q = q; p.k = k; p.v = v; p.stride_q = stride_q; p.stride_k = stride_k; p.stride_v = stride_v;
+  p.a = a; p.b = b; p.stride_a = stride_a; p.stride_b = stride_b;
+  p.A_log = A_log; p.dt_bias = dt_bias; p.g_in = g_in; p.beta_in = beta_in;
+  p.cu_seqlens = cu_seqlens; p.N = N; p.T = T; p.scale = scale; p.normalize_qk = normalize_qk;
+  p.h0 = h0; p.h0_indices = h0_indices; p.h0_slot_stride = h0_slot_stride;
+  p.ht = ht; p.ht_indices = ht_indices; p.ht_slot_stride = ht_slot_stride;
+  p.o = o;
+  p.seq_chunk_off = reinterpret_cast<int32_t*>(ws + L.seq_chunk_off);
+  p.chunk_seq = reinterpret_cast<int32_t*>(ws + L.chunk_seq);
+  p.chunk_tok = reinterpret_cast<int32_t*>(ws + L.chunk_tok);
+  p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
+  p.qn = reinterpret_cast<uint16_t*>(ws + L.qn);
+  p.kn = reinterpret_cast<uint16_t*>(ws + L.kn);
+  p.knT = reinterpret_cast<uint16_t*>(ws + L.knT);
+  p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
+  p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
+  p.Whi = reinterpret_cast<uint16_t*>(ws + L.Whi);
+  p.Wlo = reinterpret_cast<uint16_t*>(ws + L.Wlo);
+  p.P = reinterpret_cast<uint16_t*>(ws + L.P);
+  p.H = H; p.HV = HV; p.NC_max = L.NC_max;
+
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(gdn_chunk_map_kernel, dim3(1), dim3(256), 0, s, p);
+  if (act_dtype == PLA_BF16) {
+    hipLaunchKernelGGL(gdn_zero_tail_kernel<bf16_t>, dim3(64), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max), dim3(256), 0, s, p);
+  } else {
+    hipLaunchKernelGGL(gdn_zero_tail_kernel<f16_t>, dim3(64), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max), dim3(256), 0, s, p);
+  }
+  hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
+  if (act_dtype == PLA_BF16)
+    hipLaunchKernelGGL(gdn_chunk_seq_kernel<bf16_t>, dim3((unsigned)N * HV), dim3(512), 0, s, p);
+  else
+    hipLaunchKernelGGL(gdn_chunk_seq_kernel<f16_t>, dim3((unsigned)N * HV), dim3(512), 0, s, p);
+  return check_launch("gdn prefill launch");
+}

@@ -1,0 +1,139 @@
+"""GPU parity of the GDN chunk-64 prefill against the CPU oracle (token recurrence / float64
+chunked evaluation).  Tolerances: bf16 o atol 2e-2 / rtol 2e-2, FP32 final state rel-L2 <= 1e-3;
+untouched pool slots and the padded output suffix bit-exact."""
+import pytest
+import torch
+
+from helpers import rel_l2
+from oracle import gdn_prefill_reference, chunked_delta_rule_fp64, softplus_gate, sigmoid_beta, l2norm
+
+pytestmark = pytest.mark.gpu
+
+
+def _run_workload(w, output_final_state=True):
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    packed = call.pop("packed_qkv")
+    a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+    return gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, output_final_state=output_final_state, **call)
+
+
+def _oracle_workload(w, fast=False):
+    m = w["_meta"]
+    T, H, HV = m["T"], m["H"], m["HV"]
+    packed = w["packed_qkv"].cpu()
+    q = packed[:, : H * 128].reshape(T, H, 128)
+    k = packed[:, H * 128: 2 * H * 128].reshape(T, H, 128)
+    v = packed[:, 2 * H * 128:].reshape(T, HV, 128)
+    idx = w["initial_state_indices"].cpu().long()
+    S0 = w["initial_state"][idx.to(w["initial_state"].device)].cpu()
+    a, b = w["raw_gate_a"].cpu(), w["raw_beta_b"].cpu()
+    A, dt = w["A_log"].cpu(), w["dt_bias"].cpu()
+    if not fast:
+        return gdn_prefill_reference(q, k, v, a, b, A, dt, m["offsets"], S0, scale=w["scale"])
+    # float64 chunked evaluation of the same definition (validated against the token recurrence)
+    qn, kn = l2norm(q).to(q.dtype), l2norm(k).to(k.dtype)
+    g = softplus_gate(a, dt, A)
+    beta = sigmoid_beta(b)
+    o = torch.zeros(T, HV, 128, dtype=torch.float64)
+    final = S0.double().clone()
+    offs = m["offsets"]
+    for n in range(len(offs) - 1):
+        lo, hi = offs[n], offs[n + 1]
+        if hi > lo:
+            o[lo:hi], final[n] = chunked_delta_rule_fp64(qn[lo:hi], kn[lo:hi], v[lo:hi], g[lo:hi], beta[lo:hi],
+                                                         S0[n], scale=w["scale"])
+    return o, final
+
+
+def _check(w, fast=False):
+    m = w["_meta"]
+    backing = m["backing"]
+    before = backing.clone()
+    exp_o, exp_final = _oracle_workload(w, fast)
+    g_cum, A, o, none, final = _run_workload(w)
+    torch.cuda.synchronize()
+    assert none is None and o.shape == (1, m["T"], m["HV"], 128) and o.dtype == torch.bfloat16
+    torch.testing.assert_close(o[0].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
+    idx = w["initial_state_indices"].cpu().tolist()
+    worst = max(rel_l2(final[n], exp_final[n]) for n in range(len(idx)))
+    assert worst <= 1e-3, worst
+    pool = w["initial_state"]
+    for n, slot in enumerate(idx):
+        assert torch.equal(pool[slot], final[n])               # final_state is the gathered pool rows
+    untouched = torch.ones(pool.shape[0], dtype=torch.bool, device=pool.device)
+    untouched[torch.tensor(idx, device=pool.device)] = False
+    assert torch.equal(backing[untouched], before[untouched])
+    tail = m["offsets"][-1]
+    assert torch.count_nonzero(o[0, tail:]) == 0
+    return worst
+
+
+@pytest.mark.parametrize("lengths,tail_pad", [([64], 0), ([1], 0), ([17], 3), ([63, 65, 128], 0),
+                                              ([200, 0, 33, 2049], 5), ([5555], 0)])
+@pytest.mark.parametrize("H,HV", [(2, 4), (4, 4)])
+def test_gdn_prefill_small(lengths, tail_pad, H, HV):
+    from pla_amd.workloads import gdn_prefill_packed
+    w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=sum(lengths) + H, tail_pad=tail_pad)
+    _check(w, fast=sum(lengths) > 3000)
+
+
+def test_gdn_prefill_no_final_state_still_updates_pool_and_chained_calls():
+    from pla_amd.workloads import gdn_prefill_packed
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    w = gdn_prefill_packed([300], H=2, HV=4, pool_slots=4, seed=5)
+    pool0 = w["initial_state"].clone()
+    _, _, o_full, _, final_full = _run_workload(w)
+    pool_full = w["initial_state"].clone()
+    # output_final_state=False: same pool contents, no returned state
+    w["initial_state"].copy_(pool0)
+    _, _, o2, _, final2 = _run_workload(w, output_final_state=False)
+    torch.cuda.synchronize()
+    assert final2 is None and torch.equal(o2, o_full) and torch.equal(w["initial_state"], pool_full)
+    # two chained calls (192 + 108 tokens, chunk aligned) == one call, bit for bit per chunk schedule
+    w["initial_state"].copy_(pool0)
+    parts = []
+    for lo, hi in ((0, 192), (192, 300)):
+        cu = torch.tensor([0, hi - lo], dtype=torch.int32, device="cuda")
+        r = gdn_prefill_packed_qkv_fwd(w["packed_qkv"][lo:hi], w["raw_gate_a"][lo:hi], w["raw_beta_b"][lo:hi],
+                                       w["A_log"], w["dt_bias"], cu, num_qk_heads=2, num_v_heads=4,
+                                       scale=w["scale"], initial_state=w["initial_state"],
+                                       initial_state_indices=w["initial_state_indices"])
+        parts.append(r[2])
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat(parts, dim=1), o_full)
+    assert torch.equal(w["initial_state"], pool_full)
+
+
+def test_gdn_prefill_split_inputs_and_compact_state():
+    """g / beta given explicitly, q/k already normalised, compact (non-indexed) state."""
+    from pla_amd.prefill.flashqla import chunk_gated_delta_rule_fwd
+    from oracle.prefill import token_recurrence
+    g = torch.Generator().manual_seed(3)
+    T, H, HV = 150, 2, 4
+    q = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
+    k = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
+    v = torch.randn(T, HV, 128, generator=g).bfloat16()
+    gate = -torch.rand(T, HV, generator=g) * 0.3
+    beta = torch.rand(T, HV, generator=g)
+    S0 = torch.randn(2, HV, 128, 128, generator=g) * 0.1
+    offs = [0, 50, 150]
+    exp_o, exp_final = token_recurrence(q, k, v, gate, beta, offs, S0, scale=128 ** -0.5)
+    dev = "cuda"
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    g_cum, A, o, _, final = chunk_gated_delta_rule_fwd(
+        q[None].to(dev), k[None].to(dev), v[None].to(dev), gate[None].to(dev), beta[None].to(dev),
+        initial_state=S0.to(dev), cu_seqlens=cu)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(o[0].cpu().float(), exp_o, atol=2e-2, rtol=2e-2)
+    assert max(rel_l2(final[n], exp_final[n]) for n in range(2)) <= 1e-3
+    # chunk-local cumulative gate resets at every chunk and sequence start
+    want = torch.cat([gate[0:50].cumsum(0), gate[50:114].cumsum(0), gate[114:150].cumsum(0)])
+    torch.testing.assert_close(g_cum[0].cpu(), want, rtol=1e-5, atol=1e-6)
+
+
+def test_config3_gdn_prefill_32k_varlen():
+    from pla_amd.workloads import gdn_prefill_packed, ragged_lengths
+    lengths = ragged_lengths(8, 512, 8192, seed=303)
+    w = gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=64, seed=303)
+    _check(w, fast=True)
