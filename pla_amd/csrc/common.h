@@ -76,12 +76,34 @@ __device__ __forceinline__ float row16_allreduce(float x) {
   x += dpp_mov<0x140>(x);   // row_mirror
   return x;
 }
+// Cross-row exchanges use the gfx950 lane-swap instructions through inline asm
+// (inline asm keeps both results of the swap in plain scalar registers).  The s_nop pairs cover the VALU -> lane-swap
+// and lane-swap -> VALU wait states that the hazard recogniser cannot see
+// inside an asm statement.
+struct LanePair { float lo, hi; };
+// lo: the value held by lanes 0-31 (replicated to all lanes), hi: by lanes 32-63.
+__device__ __forceinline__ LanePair swap_halves(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return LanePair{a, b};
+}
+// lo: the value of the even DPP row of each row pair, hi: of the odd DPP row.
+__device__ __forceinline__ LanePair swap_rows16(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return LanePair{a, b};
+}
+
+// Sum over each aligned group of 32 lanes (one state row); every lane gets the total.
+__device__ __forceinline__ float row32_allreduce(float x) {
+  const LanePair r = swap_rows16(row16_allreduce(x));
+  return r.lo + r.hi;
+}
+
 // Sum over the whole 64-lane wavefront; every lane gets the total.
 __device__ __forceinline__ float wave64_allreduce(float x) {
-  x = row16_allreduce(x);
-  x += __shfl_xor(x, 16, 64);
-  x += __shfl_xor(x, 32, 64);
-  return x;
+  const LanePair r = swap_halves(row32_allreduce(x));
+  return r.lo + r.hi;
 }
 
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }     // v_rcp_f32, 1 ulp

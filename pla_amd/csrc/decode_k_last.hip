@@ -111,24 +111,6 @@ __device__ __forceinline__ void row_scalars(const uint32_t (&w)[RPW / 2], int ha
   for (int j = 0; j < RPW / 2; ++j) x[j] = to_float(act_t{(uint16_t)(w[j] >> sh)});
 }
 
-// Cross-row exchanges use the gfx950 lane-swap instructions through inline asm
-// (inline asm keeps both results of the swap in plain scalar registers).  The s_nop pairs cover the VALU -> lane-swap
-// and lane-swap -> VALU wait states that the hazard recogniser cannot see
-// inside an asm statement.
-struct LanePair { float lo, hi; };
-// lo: the value held by lanes 0-31 (replicated to all lanes), hi: by lanes 32-63.
-__device__ __forceinline__ LanePair swap_halves(float x) {
-  float a = x, b = x;
-  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-  return LanePair{a, b};
-}
-// lo: the value of the even DPP row of each row pair, hi: of the odd DPP row.
-__device__ __forceinline__ LanePair swap_rows16(float x) {
-  float a = x, b = x;
-  asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-  return LanePair{a, b};
-}
-
 // Lane 0 receives the odd rows' values from lane 32 and writes the wave's RPW
 // outputs as one contiguous run.
 template <typename act_t, int RPW>
@@ -144,12 +126,6 @@ __device__ __forceinline__ void store_row_scalars(act_t* p, int lane, const floa
     for (int i = 0; i < RPW / 8; ++i)
       reinterpret_cast<uint4*>(p)[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
   }
-}
-
-// Sum over each aligned group of 32 lanes (one state row); every lane gets the total.
-__device__ __forceinline__ float row32_allreduce(float x) {
-  const LanePair r = swap_rows16(row16_allreduce(x));
-  return r.lo + r.hi;
 }
 
 // State tiles are streamed exactly once per call, so they are moved with raw

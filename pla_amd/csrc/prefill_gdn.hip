@@ -119,7 +119,9 @@ __global__ void gdn_chunk_map_kernel(const GdnPrefillParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// One workgroup (256 threads) per chunk.
+// grid (chunk, H + 1), 256 threads.  blockIdx.y < H: L2 norm of q and k of one head for the
+// chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing) and
+// the transposed K tile; blockIdx.y == H: gate, beta and the chunk-local cumulative log-decay.
 template <typename act_t>
 __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
   const int cb = blockIdx.x;
@@ -127,66 +129,87 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  __shared__ uint16_t tile[CHUNK][130];     // normalised k of one head, for the transposed copy
+  __shared__ union {
+    uint16_t tile[CHUNK][130];        // normalised k of one head, for the transposed copy
+    float g[CHUNK][129];              // per-token log-decay of up to 128 value heads
+  } sh;
 
-  // gate, beta, chunk-local cumulative log-decay: one thread per value head
-  for (int hv = threadIdx.x; hv < p.HV; hv += blockDim.x) {
-    float cum = 0.f;
-    const float eA = p.g_in ? 0.f : expf(p.A_log[hv]);
-    const float dt = p.g_in ? 0.f : p.dt_bias[hv];
-    for (int j = 0; j < len; ++j) {
-      const int64_t t = t0 + j;
-      float g, bt;
-      if (p.g_in) {
-        g = p.g_in[t * p.HV + hv];
-        bt = p.beta_in[t * p.HV + hv];
-      } else {
-        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + dt;
-        const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
-        g = -eA * sp;
-        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
-        bt = 1.0f / (1.0f + expf(-braw));
+  if ((int)blockIdx.y == p.H) {
+    for (int hv0 = 0; hv0 < p.HV; hv0 += 128) {
+      const int nh = min(128, p.HV - hv0);
+      for (int idx = threadIdx.x; idx < CHUNK * nh; idx += 256) {
+        const int j = idx / nh, hv = hv0 + idx - j * nh;
+        float g = 0.f;
+        if (j < len) {
+          const int64_t t = t0 + j;
+          float bt;
+          if (p.g_in) {
+            g = p.g_in[t * p.HV + hv];
+            bt = p.beta_in[t * p.HV + hv];
+          } else {
+            const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
+            const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
+            g = -expf(p.A_log[hv]) * sp;
+            const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
+            bt = 1.0f / (1.0f + expf(-braw));
+          }
+          p.beta[t * p.HV + hv] = bt;
+        }
+        sh.g[j][hv - hv0] = g;
       }
-      cum += g;
-      p.gcum[t * p.HV + hv] = cum;
-      p.beta[t * p.HV + hv] = bt;
+      __syncthreads();
+      if ((int)threadIdx.x < nh) {
+        float cum = 0.f;
+        for (int j = 0; j < len; ++j) {
+          cum += sh.g[j][threadIdx.x];
+          p.gcum[(int64_t)(t0 + j) * p.HV + hv0 + threadIdx.x] = cum;
+        }
+      }
+      __syncthreads();
     }
+    return;
   }
 
-  // q / k L2 normalisation (float32, eps inside the root), rounded to bf16
-  for (int h = 0; h < p.H; ++h) {
-    for (int j = wave; j < CHUNK; j += 4) {
-      uint32_t kw = 0;
-      if (j < len) {
-        const int64_t t = t0 + j;
-        const uint32_t qw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.q) + t * p.stride_q + h * 128 + 2 * lane);
-        kw = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.k) + t * p.stride_k + h * 128 + 2 * lane);
-        float q0 = lo16<act_t>(qw), q1 = hi16<act_t>(qw), k0 = lo16<act_t>(kw), k1 = hi16<act_t>(kw);
-        if (p.normalize_qk) {
-          const float qs = wave64_allreduce(q0 * q0 + q1 * q1);
-          const float ks = wave64_allreduce(k0 * k0 + k1 * k1);
-          const float qi = rsqrtf(qs + 1e-6f), ki = rsqrtf(ks + 1e-6f);
-          q0 *= qi; q1 *= qi; k0 *= ki; k1 *= ki;
-        }
-        const uint32_t qo = pack2<bf16_t>(q0, q1);
-        kw = pack2<bf16_t>(k0, k1);
-        *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = qo;
-        *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = kw;
-      }
-      *reinterpret_cast<uint32_t*>(&tile[j][2 * lane]) = kw;       // zero rows beyond the chunk
-    }
-    __syncthreads();
-    // K^T tile [128][64]: thread (c, half) gathers 32 tokens of column c
-    {
-      const int c = threadIdx.x >> 1, half = threadIdx.x & 1;
-      uint16_t* dst = p.knT + (((int64_t)cb * p.H + h) * 128 + c) * CHUNK + 32 * half;
+  const int h = blockIdx.y;
+  uint32_t qw[16], kw[16];
 #pragma unroll
-      for (int jj = 0; jj < 32; jj += 2) {
-        const uint32_t w = (uint32_t)tile[32 * half + jj][c] | ((uint32_t)tile[32 * half + jj + 1][c] << 16);
-        *reinterpret_cast<uint32_t*>(dst + jj) = w;
-      }
+  for (int x = 0; x < 16; ++x) {
+    const int j = 16 * wave + x;
+    const int64_t t = t0 + (j < len ? j : 0);
+    qw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.q) + t * p.stride_q + h * 128 + 2 * lane);
+    kw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.k) + t * p.stride_k + h * 128 + 2 * lane);
+  }
+#pragma unroll
+  for (int x = 0; x < 16; ++x) {
+    const int j = 16 * wave + x;
+    float q0 = lo16<act_t>(qw[x]), q1 = hi16<act_t>(qw[x]), k0 = lo16<act_t>(kw[x]), k1 = hi16<act_t>(kw[x]);
+    if (p.normalize_qk) {
+      const float qs = wave64_allreduce(q0 * q0 + q1 * q1);
+      const float ks = wave64_allreduce(k0 * k0 + k1 * k1);
+      const float qi = rsqrtf(qs + 1e-6f), ki = rsqrtf(ks + 1e-6f);
+      q0 *= qi; q1 *= qi; k0 *= ki; k1 *= ki;
     }
-    __syncthreads();
+    uint32_t ko = 0;
+    if (j < len) {
+      ko = pack2<bf16_t>(k0, k1);
+      const int64_t t = t0 + j;
+      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2<bf16_t>(q0, q1);
+      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = ko;
+    }
+    *reinterpret_cast<uint32_t*>(&sh.tile[j][2 * lane]) = ko;       // zero rows beyond the chunk
+  }
+  __syncthreads();
+  // K^T tile [128][64]: thread (c, half) gathers 32 tokens of column c
+  {
+    const int c = threadIdx.x >> 1, half = threadIdx.x & 1;
+    uint16_t* dst = p.knT + (((int64_t)cb * p.H + h) * 128 + c) * CHUNK + 32 * half;
+    uint32_t w[16];
+#pragma unroll
+    for (int jj = 0; jj < 16; ++jj)
+      w[jj] = (uint32_t)sh.tile[32 * half + 2 * jj][c] | ((uint32_t)sh.tile[32 * half + 2 * jj + 1][c] << 16);
+#pragma unroll
+    for (int x = 0; x < 4; ++x)
+      reinterpret_cast<uint4*>(dst)[x] = make_uint4(w[4 * x], w[4 * x + 1], w[4 * x + 2], w[4 * x + 3]);
   }
 }
 
@@ -213,52 +236,69 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
     Bs[lane] = ok ? p.beta[(int64_t)(t0 + lane) * p.HV + hv] : 0.f;
   }
 
-  // operands of K and Q: 4 row blocks x 4 contraction steps
-  bf16x8_t Kop[4][4], Qop[4][4];
+  // K operands: 4 row blocks x 4 contraction steps (rows beyond the chunk are zero)
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+  bf16x8_t Kop[4][4];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
     const int row = 16 * mb + r16;
     const bool ok = row < len;
     const uint16_t* kr = p.kn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
-    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      bf16x8_t kz = operand_from(kr, s, kb), qz = operand_from(qr, s, kb);
-      if (!ok) {
-        const uint4 z = make_uint4(0, 0, 0, 0);
-        kz = __builtin_bit_cast(bf16x8_t, z);
-        qz = kz;
-      }
-      Kop[mb][s] = kz;
-      Qop[mb][s] = qz;
+      const bf16x8_t kz = operand_from(kr, s, kb);
+      Kop[mb][s] = ok ? kz : __builtin_bit_cast(bf16x8_t, zero4);
     }
   }
   __syncthreads();
 
-  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
+  // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi) {
 #pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
-      if (ni > mi) {
-        // strictly upper blocks: L is not read there, P is zero
+    for (int ni = 0; ni <= mi; ++ni) {
+      f32x4_t kk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Pt[(16 * mi + 4 * kb + r) * 64 + 16 * ni + r16] = 0;
-        continue;
-      }
-      f32x4_t kk = {0.f, 0.f, 0.f, 0.f}, qk = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        kk = mfma16(Kop[mi][s], Kop[ni][s], kk);
-        qk = mfma16(Qop[mi][s], Kop[ni][s], qk);
-      }
+      for (int s = 0; s < 4; ++s) kk = mfma16(Kop[mi][s], Kop[ni][s], kk);
       const int j = 16 * ni + r16;
       const float Gj = Gs[j];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * mi + 4 * kb + r;
+        Lm[i][j] = i > j ? Bs[i] * kk[r] * __expf(Gs[i] - Gj) : 0.f;
+      }
+    }
+  }
+
+  // P = scale * tril(q_i . k_j e^{G_i - G_j}); one row block of Q at a time keeps registers low
+  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) {
+    const int row = 16 * mi + r16;
+    const bool ok = row < len;
+    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
+    bf16x8_t Qop[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bf16x8_t qz = operand_from(qr, s, kb);
+      Qop[s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
+    }
+#pragma unroll
+    for (int ni = 0; ni < 4; ++ni) {
+      const int j = 16 * ni + r16;
+      if (ni > mi) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) Pt[(16 * mi + 4 * kb + r) * 64 + j] = 0;
+        continue;
+      }
+      f32x4_t qk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) qk = mfma16(Qop[s], Kop[ni][s], qk);
+      const float Gj = Gs[j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * mi + 4 * kb + r;
         const float gam = i >= j ? __expf(Gs[i] - Gj) : 0.f;
-        Lm[i][j] = i > j ? Bs[i] * kk[r] * gam : 0.f;
         Pt[i * 64 + j] = from_float<bf16_t>(p.scale * qk[r] * gam).bits;
       }
     }
@@ -270,16 +310,17 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
   const float bj = Bs[lane];
 #pragma unroll
   for (int i = 0; i < CHUNK; ++i) {
-    float acc = (i == lane) ? bj : 0.f;
+    // four independent partial sums keep the FMA pipeline full
+    float a0 = (i == lane) ? bj : 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
 #pragma unroll
     for (int l4 = 0; l4 < i; l4 += 4) {
       const float4 row = *reinterpret_cast<const float4*>(&Lm[i][l4]);
-      acc = fmaf(-row.x, x[l4], acc);
-      if (l4 + 1 < i) acc = fmaf(-row.y, x[l4 + 1], acc);
-      if (l4 + 2 < i) acc = fmaf(-row.z, x[l4 + 2], acc);
-      if (l4 + 3 < i) acc = fmaf(-row.w, x[l4 + 3], acc);
+      a0 = fmaf(-row.x, x[l4], a0);
+      if (l4 + 1 < i) a1 = fmaf(-row.y, x[l4 + 1], a1);
+      if (l4 + 2 < i) a2 = fmaf(-row.z, x[l4 + 2], a2);
+      if (l4 + 3 < i) a3 = fmaf(-row.w, x[l4 + 3], a3);
     }
-    x[i] = acc;
+    x[i] = (a0 + a1) + (a2 + a3);
   }
   uint16_t* const Wh = p.Whi + ((int64_t)cb * p.HV + hv) * 4096;
   uint16_t* const Wl = p.Wlo + ((int64_t)cb * p.HV + hv) * 4096;
@@ -296,9 +337,11 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 // and spread rows over banks).
 constexpr int PITCH128 = 136;
 constexpr int PITCH64 = 72;
-struct SeqTiles {
+struct __align__(16) SeqTiles {
   uint16_t K[CHUNK][PITCH128];
   uint16_t Q[CHUNK][PITCH128];
+  uint16_t V[CHUNK][PITCH128];
+  uint16_t O[CHUNK][PITCH128];
   uint16_t Kt[128][PITCH64];
   uint16_t Whi[CHUNK][PITCH64];
   uint16_t Wlo[CHUNK][PITCH64];
@@ -309,12 +352,10 @@ struct SeqTiles {
   float eGlast;
 };
 
-// Registers holding the next chunk's tiles while the current chunk is being processed.
-struct SeqPrefetch {
-  uint4 k[2], q[2], kt[2], whi, wlo, pp;
-  float g;
-};
-
+// Everything the next chunk needs is requested from global memory one chunk ahead and parked
+// in registers (eleven 16-byte vectors per thread), every per-chunk address is a running
+// pointer, V and O travel through LDS tiles (coalesced 16-byte global accesses, immediate-offset
+// LDS accesses), so the chunk-to-chunk critical path holds only LDS reads, conversions and MFMAs.
 template <typename act_t>
 __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
   const int n = blockIdx.x / p.HV;
@@ -326,6 +367,8 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
   const int vcol = 16 * wave + r16;                  // this lane's V column
   const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
   if (c_begin >= c_end) return;                      // empty sequence: state untouched, no output
+  const int seq_start = p.cu_seqlens[n];
+  const int seq_len = p.cu_seqlens[n + 1] - seq_start;
 
   __shared__ SeqTiles T;
 
@@ -346,85 +389,91 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
     }
   }
 
-  // cooperative tile fetch: 512 threads x 16 bytes
-  auto fetch = [&](int cb) {
-    SeqPrefetch f;
-    const int t0 = p.chunk_tok[cb];
-    const int len = p.chunk_len[cb];
-    const uint4 z = make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int vec = tid + 512 * u;                 // 1024 vectors of 8 elements: 64 rows x 16
-      const int row = vec >> 4, cv = vec & 15;
-      const bool ok = row < len;
-      const int64_t tok = t0 + (ok ? row : 0);
-      const uint4 kx = *reinterpret_cast<const uint4*>(p.kn + (tok * p.H + h) * 128 + 8 * cv);
-      const uint4 qx = *reinterpret_cast<const uint4*>(p.qn + (tok * p.H + h) * 128 + 8 * cv);
-      f.k[u] = ok ? kx : z;
-      f.q[u] = ok ? qx : z;
-      // K^T: 128 rows x 8 vectors
-      f.kt[u] = *reinterpret_cast<const uint4*>(p.knT + ((int64_t)cb * p.H + h) * 8192 + 8 * vec);
-    }
-    {
-      const int64_t tb = ((int64_t)cb * p.HV + hv) * 4096 + 8 * tid;   // 512 vectors: 64 rows x 8
-      f.whi = *reinterpret_cast<const uint4*>(p.Whi + tb);
-      f.wlo = *reinterpret_cast<const uint4*>(p.Wlo + tb);
-      f.pp = *reinterpret_cast<const uint4*>(p.P + tb);
-    }
-    f.g = 0.f;
-    if (tid < CHUNK) {
-      const int j = tid < len ? tid : len - 1;
-      f.g = p.gcum[(int64_t)(t0 + j) * p.HV + hv];
-    }
-    return f;
+  // cooperative copy coordinates: 64-row x 128-column tiles are 1024 16-byte vectors (two per
+  // thread: rows krow and krow + 32), 64 x 64 and the 128 x 64 K^T tiles 512 / 1024 vectors.
+  const int krow = tid >> 4, kcv = tid & 15;
+  const int srow = tid >> 3, scv = tid & 7;
+  const int64_t tok_pitch = (int64_t)p.H * 128;                // elements between tokens of kn / qn
+  const int64_t half_k = 32 * tok_pitch, half_v = 32 * p.stride_v;
+  const uint16_t* kptr = p.kn + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
+  const uint16_t* qptr = p.qn + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
+  const uint16_t* vptr = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)(seq_start + krow) * p.stride_v + hv * 128 + 8 * kcv;
+  const uint16_t* ktptr = p.knT + ((int64_t)c_begin * p.H + h) * 8192 + 8 * tid;
+  const uint16_t* whptr = p.Whi + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
+  const uint16_t* wlptr = p.Wlo + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
+  const uint16_t* ppptr = p.P + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
+  const float* gptr = p.gcum + (int64_t)seq_start * p.HV + hv;
+  uint16_t* optr = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
+  const int64_t o_half = (int64_t)32 * p.HV * 128;
+  const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+  uint4 pk0, pk1, pq0, pq1, pv0, pv1, pt0, pt1, pwh, pwl, ppp;
+  float pg;
+  // `len` rows of the chunk are real; rows beyond are read from row 0 of the chunk and zeroed.
+  auto prefetch = [&](int len) {
+    const bool ok0 = krow < len, ok1 = krow + 32 < len;
+    const int64_t back0 = ok0 ? 0 : -(int64_t)krow, back1 = ok1 ? 32 : -(int64_t)krow;
+    pk0 = *reinterpret_cast<const uint4*>(kptr + back0 * tok_pitch);
+    pq0 = *reinterpret_cast<const uint4*>(qptr + back0 * tok_pitch);
+    pv0 = *reinterpret_cast<const uint4*>(vptr + back0 * p.stride_v);
+    pk1 = *reinterpret_cast<const uint4*>(kptr + back1 * tok_pitch);
+    pq1 = *reinterpret_cast<const uint4*>(qptr + back1 * tok_pitch);
+    pv1 = *reinterpret_cast<const uint4*>(vptr + back1 * p.stride_v);
+    pt0 = *reinterpret_cast<const uint4*>(ktptr);
+    pt1 = *reinterpret_cast<const uint4*>(ktptr + 4096);
+    pwh = *reinterpret_cast<const uint4*>(whptr);
+    pwl = *reinterpret_cast<const uint4*>(wlptr);
+    ppp = *reinterpret_cast<const uint4*>(ppptr);
+    pg = gptr[(int64_t)(lane < len ? lane : len - 1) * p.HV];
+    if (!ok0) { pk0 = zero4; pq0 = zero4; pv0 = zero4; }
+    if (!ok1) { pk1 = zero4; pq1 = zero4; pv1 = zero4; }
+    (void)half_k; (void)half_v;
   };
-  auto stash = [&](const SeqPrefetch& f, int len) {
-#pragma unroll
-    for (int u = 0; u < 2; ++u) {
-      const int vec = tid + 512 * u;
-      const int row = vec >> 4, cv = vec & 15;
-      *reinterpret_cast<uint4*>(&T.K[row][8 * cv]) = f.k[u];
-      *reinterpret_cast<uint4*>(&T.Q[row][8 * cv]) = f.q[u];
-      const int trow = vec >> 3, tcv = vec & 7;
-      *reinterpret_cast<uint4*>(&T.Kt[trow][8 * tcv]) = f.kt[u];
-    }
-    {
-      const int row = tid >> 3, cv = tid & 7;
-      *reinterpret_cast<uint4*>(&T.Whi[row][8 * cv]) = f.whi;
-      *reinterpret_cast<uint4*>(&T.Wlo[row][8 * cv]) = f.wlo;
-      *reinterpret_cast<uint4*>(&T.P[row][8 * cv]) = f.pp;
-    }
-    if (tid < CHUNK) {
-      // every lane of wave 0 holds G_j; the last valid row's value is G_last
-      const float glast = __shfl(f.g, len - 1, 64);
-      const float e = __expf(f.g);
-      T.eG[tid] = e;
-      T.sQ[tid] = p.scale * e;
-      T.dG[tid] = __expf(glast - f.g);
-      if (tid == 0) T.eGlast = __expf(glast);
-    }
+  auto advance = [&]() {
+    kptr += CHUNK * tok_pitch; qptr += CHUNK * tok_pitch; vptr += CHUNK * p.stride_v;
+    ktptr += (int64_t)p.H * 8192; whptr += (int64_t)p.HV * 4096; wlptr += (int64_t)p.HV * 4096;
+    ppptr += (int64_t)p.HV * 4096; gptr += (int64_t)CHUNK * p.HV;
+  };
+  // coalesced write of the previous chunk's output tile
+  auto flush_output = [&](int len) {
+    if (krow < len) *reinterpret_cast<uint4*>(optr) = *reinterpret_cast<const uint4*>(&T.O[krow][8 * kcv]);
+    if (krow + 32 < len) *reinterpret_cast<uint4*>(optr + o_half) = *reinterpret_cast<const uint4*>(&T.O[krow + 32][8 * kcv]);
+    optr += (int64_t)CHUNK * p.HV * 128;
   };
 
-  SeqPrefetch nxt = fetch(c_begin);
-  for (int cb = c_begin; cb < c_end; ++cb) {
-    const int t0 = p.chunk_tok[cb];
-    const int len = p.chunk_len[cb];
-    __syncthreads();                 // everyone finished reading the previous chunk's tiles
-    stash(nxt, len);
+  const int n_chunks = c_end - c_begin;
+  prefetch(min(CHUNK, seq_len));
+  advance();
+  int prev_len = 0;
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int len = min(CHUNK, seq_len - ci * CHUNK);
+
+    __syncthreads();                 // everyone finished with the previous chunk's tiles
+    if (ci > 0) flush_output(prev_len);
+    *reinterpret_cast<uint4*>(&T.K[krow][8 * kcv]) = pk0;
+    *reinterpret_cast<uint4*>(&T.K[krow + 32][8 * kcv]) = pk1;
+    *reinterpret_cast<uint4*>(&T.Q[krow][8 * kcv]) = pq0;
+    *reinterpret_cast<uint4*>(&T.Q[krow + 32][8 * kcv]) = pq1;
+    *reinterpret_cast<uint4*>(&T.V[krow][8 * kcv]) = pv0;
+    *reinterpret_cast<uint4*>(&T.V[krow + 32][8 * kcv]) = pv1;
+    *reinterpret_cast<uint4*>(&T.Kt[srow][8 * scv]) = pt0;
+    *reinterpret_cast<uint4*>(&T.Kt[64 + srow][8 * scv]) = pt1;
+    *reinterpret_cast<uint4*>(&T.Whi[srow][8 * scv]) = pwh;
+    *reinterpret_cast<uint4*>(&T.Wlo[srow][8 * scv]) = pwl;
+    *reinterpret_cast<uint4*>(&T.P[srow][8 * scv]) = ppp;
+    if (wave == 0) {
+      const float glast = __shfl(pg, len - 1, 64);
+      const float e = __expf(pg);
+      T.eG[lane] = e;
+      T.sQ[lane] = p.scale * e;
+      T.dG[lane] = __expf(glast - pg);
+      if (lane == 0) T.eGlast = __expf(glast);
+    }
     __syncthreads();
-    if (cb + 1 < c_end) nxt = fetch(cb + 1);
-
-    // V of this lane's column for the 16 rows it owns in accumulator layout
-    float vreg[4][4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * mi + 4 * kb + r;
-        vreg[mi][r] = i < len
-            ? to_float(reinterpret_cast<const act_t*>(p.v)[(int64_t)(t0 + i) * p.stride_v + hv * 128 + vcol])
-            : 0.f;
-      }
+    if (ci + 1 < n_chunks) {
+      prefetch(min(CHUNK, seq_len - (ci + 1) * CHUNK));
+      advance();
+    }
 
     // (1) KS = K S^T and (3a) QS = Q S^T : contraction over the 128 K channels
     f32x4_t KS[4], QS[4];
@@ -438,17 +487,22 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
         const bf16x8_t ka = operand_from(&T.K[16 * mi + r16][0], s, kb);
         const bf16x8_t qa = operand_from(&T.Q[16 * mi + r16][0], s, kb);
         KS[mi] = mfma16(ka, sb.hi, KS[mi]);
-        KS[mi] = mfma16(ka, sb.lo, KS[mi]);
         QS[mi] = mfma16(qa, sb.hi, QS[mi]);
+        KS[mi] = mfma16(ka, sb.lo, KS[mi]);
       }
     }
 
     // X = V - e^{G} (.) KS   (rows of the accumulator are tokens)
     f32x4_t X[4];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) X[mi][r] = vreg[mi][r] - T.eG[16 * mi + 4 * kb + r] * KS[mi][r];
+    for (int mi = 0; mi < 4; ++mi) {
+      const float4 eg = *reinterpret_cast<const float4*>(&T.eG[16 * mi + 4 * kb]);
+      const uint16_t* vr = &T.V[16 * mi + 4 * kb][vcol];
+      X[mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[mi][0];
+      X[mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[mi][1];
+      X[mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[mi][2];
+      X[mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[mi][3];
+    }
 
     // (2) U = W X : contraction over the 64 tokens, W and X both split
     f32x4_t U[4];
@@ -467,42 +521,16 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
       }
     }
 
-    // (3b) O = scale e^{G} (.) QS + P U
-    f32x4_t O[4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) O[mi][r] = T.sQ[16 * mi + 4 * kb + r] * QS[mi][r];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const bf16x8_t ub = round8(U[2 * s], U[2 * s + 1]);
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-        O[mi] = mfma16(operand_from(&T.P[16 * mi + r16][0], s, kb), ub, O[mi]);
-    }
-    {
-      act_t* const orow = reinterpret_cast<act_t*>(p.o) + ((int64_t)t0 * p.HV + hv) * 128 + vcol;
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int i = 16 * mi + 4 * kb + r;
-          if (i < len) orow[(int64_t)i * p.HV * 128] = from_float<act_t>(O[mi][r]);
-        }
-    }
-
-    // (4) S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
+    // (4) S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)   -- the next chunk waits for this
     const float egl = T.eGlast;
 #pragma unroll
     for (int mc = 0; mc < 8; ++mc) St[mc] *= egl;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      f32x4_t u0 = U[2 * s], u1 = U[2 * s + 1];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        u0[r] *= T.dG[32 * s + 4 * kb + r];
-        u1[r] *= T.dG[32 * s + 16 + 4 * kb + r];
-      }
+      const float4 d0 = *reinterpret_cast<const float4*>(&T.dG[32 * s + 4 * kb]);
+      const float4 d1 = *reinterpret_cast<const float4*>(&T.dG[32 * s + 16 + 4 * kb]);
+      const f32x4_t u0 = {U[2 * s][0] * d0.x, U[2 * s][1] * d0.y, U[2 * s][2] * d0.z, U[2 * s][3] * d0.w};
+      const f32x4_t u1 = {U[2 * s + 1][0] * d1.x, U[2 * s + 1][1] * d1.y, U[2 * s + 1][2] * d1.z, U[2 * s + 1][3] * d1.w};
       const HiLo ub = split8(u0, u1);
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
@@ -511,7 +539,33 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
         St[mc] = mfma16(ka, ub.lo, St[mc]);
       }
     }
+
+    // (3b) O = scale e^{G} (.) QS + P U   -- off the state's critical path
+    f32x4_t O[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      const float4 sq = *reinterpret_cast<const float4*>(&T.sQ[16 * mi + 4 * kb]);
+      O[mi] = f32x4_t{sq.x * QS[mi][0], sq.y * QS[mi][1], sq.z * QS[mi][2], sq.w * QS[mi][3]};
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const bf16x8_t ub = round8(U[2 * s], U[2 * s + 1]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+        O[mi] = mfma16(operand_from(&T.P[16 * mi + r16][0], s, kb), ub, O[mi]);
+    }
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      uint16_t* orow = &T.O[16 * mi + 4 * kb][vcol];
+      orow[0] = from_float<act_t>(O[mi][0]).bits;
+      orow[PITCH128] = from_float<act_t>(O[mi][1]).bits;
+      orow[2 * PITCH128] = from_float<act_t>(O[mi][2]).bits;
+      orow[3 * PITCH128] = from_float<act_t>(O[mi][3]).bits;
+    }
+    prev_len = len;
   }
+  __syncthreads();
+  flush_output(prev_len);
 
   if (p.ht != nullptr) {
     const int slot = p.ht_indices ? p.ht_indices[n] : n;
@@ -623,10 +677,10 @@ extern "C" int pla_gdn_prefill_launch(
   hipLaunchKernelGGL(gdn_chunk_map_kernel, dim3(1), dim3(256), 0, s, p);
   if (act_dtype == PLA_BF16) {
     hipLaunchKernelGGL(gdn_zero_tail_kernel<bf16_t>, dim3(64), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   } else {
     hipLaunchKernelGGL(gdn_zero_tail_kernel<f16_t>, dim3(64), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   }
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
   if (act_dtype == PLA_BF16)
