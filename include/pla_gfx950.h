@@ -161,6 +161,31 @@ int pla_gdn_prefill_launch(
     float* gcum_out, float* beta_out,
     int H, int HV, int K, int V, int act_dtype, void* stream);
 
+/* Workspace bytes (256-byte aligned) needed by pla_kda_prefill_launch. */
+int64_t pla_kda_prefill_workspace_bytes(int T, int N, int H);
+
+/*
+ * KDA chunk-64 prefill over packed variable-length sequences (per-channel lower-bound gate).
+ * Replaces _C.flashkda_fwd (pla/prefill/flashkdapro/ops.py:215-219) and the tc01 FLA stage
+ * launchers fla_runtime::Launchers (src/prefill/flashkdapro/tc01/fla/launchers.h:38-78).
+ *
+ *   q,k,v,g [T,H,128] bf16 (token pitches stride_*; heads and channels contiguous), g the RAW gate;
+ *   beta [T,H] bf16 raw logits (token pitch stride_beta); A_log [H], dt_bias [H*128] float32:
+ *       log-decay = lower_bound * sigmoid(exp(A_log) * (g + dt_bias)),  beta = sigmoid(beta).
+ *   q and k are L2-normalised (eps 1e-6 inside the root) and rounded to bf16 first.
+ *   cu_seqlens [N+1] int32; rows of o at and beyond cu_seqlens[N] are zeroed.
+ *   h0 / ht as in pla_gdn_prefill_launch (k-last FP32 [slots,H,128,128]).
+ */
+int pla_kda_prefill_launch(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_g, int64_t stride_beta,
+    const float* A_log, const float* dt_bias, float lower_bound, float scale,
+    const int32_t* cu_seqlens, int N, int T,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    int H, int K, int V, int act_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

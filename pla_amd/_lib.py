@@ -41,6 +41,14 @@ SIGNATURES = {
         _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
         _c_p, _c_p, _c_i64, _c_p, _c_p,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_kda_prefill_launch": [
+        _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
+        _c_p, _c_p, _c_f, _c_f,
+        _c_p, _c_int, _c_int,
+        _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
+        _c_p, _c_p, _c_i64,
+        _c_int, _c_int, _c_int, _c_int, _c_p],
 }
 
 _lib = None
@@ -62,6 +70,8 @@ def load():
     lib.pla_last_error.argtypes = []
     lib.pla_gdn_prefill_workspace_bytes.restype = _c_i64
     lib.pla_gdn_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int, _c_int]
+    lib.pla_kda_prefill_workspace_bytes.restype = _c_i64
+    lib.pla_kda_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int]
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _c_int

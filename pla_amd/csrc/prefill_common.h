@@ -1,0 +1,88 @@
+// Pieces shared by the GDN and KDA chunk-64 prefill kernels: MFMA wrappers, bf16 hi/lo
+// splitting, operand access for v_mfma_f32_16x16x32_bf16 and the device-side chunk table.
+#pragma once
+
+#include "common.h"
+
+namespace pla {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x8_t __attribute__((ext_vector_type(8)));
+
+constexpr int CHUNK = 64;
+
+__device__ __forceinline__ f32x4_t mfma16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// hi = bf16(x), lo = bf16(x - hi) for two accumulator quads (eight contraction elements).
+struct HiLo { bf16x8_t hi, lo; };
+__device__ __forceinline__ HiLo split8(f32x4_t a, f32x4_t b) {
+  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  HiLo r;
+  r.hi = __builtin_convertvector(x, bf16x8_t);
+  const f32x8_t back = __builtin_convertvector(r.hi, f32x8_t);
+  r.lo = __builtin_convertvector(x - back, bf16x8_t);
+  return r;
+}
+__device__ __forceinline__ bf16x8_t round8(f32x4_t a, f32x4_t b) {
+  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  return __builtin_convertvector(x, bf16x8_t);
+}
+
+// A (or B) operand of one 16x16x32 MFMA step from a row-major bf16 tile: lane (r = lane%16,
+// kb = lane/16) takes columns [32s+4kb, +4) and [32s+16+4kb, +4) of row r, which is the
+// contraction order in which an accumulator tile pair (row blocks 2s, 2s+1) presents its rows.
+__device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s, int kb) {
+  const uint2 p0 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 4 * kb);
+  const uint2 p1 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 16 + 4 * kb);
+  const uint4 u = make_uint4(p0.x, p0.y, p1.x, p1.y);
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
+// LDS tile pitches (bf16 elements): rows stay 16-byte aligned and consecutive rows start 4 (128-wide)
+// or 36 (64-wide) banks apart, which keeps the 8-byte operand reads of a wavefront conflict free.
+constexpr int PITCH128 = 136;
+constexpr int PITCH64 = 72;
+
+// Chunk table from cu_seqlens, built on the device so that no call reads offsets back to the host.
+// Single workgroup.  seq_chunk_off[n] = first chunk of sequence n (seq_chunk_off[N] = total).
+static __global__ void chunk_map_kernel(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,
+                                        int32_t* chunk_seq, int32_t* chunk_tok, int32_t* chunk_len) {
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int n = 0; n < N; ++n) {
+      seq_chunk_off[n] = acc;
+      const int len = max(cu_seqlens[n + 1] - cu_seqlens[n], 0);
+      acc += (len + CHUNK - 1) / CHUNK;
+    }
+    seq_chunk_off[N] = acc;
+  }
+  __syncthreads();
+  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+    const int start = cu_seqlens[n];
+    const int len = max(cu_seqlens[n + 1] - start, 0);
+    const int c0 = seq_chunk_off[n];
+    const int nc = (len + CHUNK - 1) / CHUNK;
+    for (int c = 0; c < nc; ++c) {
+      if (c0 + c >= NC_max) break;
+      chunk_seq[c0 + c] = n;
+      chunk_tok[c0 + c] = start + c * CHUNK;
+      chunk_len[c0 + c] = min(CHUNK, len - c * CHUNK);
+    }
+  }
+}
+
+// Zero the rows of a dense [T, heads, 128] 16-bit output that lie beyond the last sequence.
+static __global__ void zero_tail_kernel(uint16_t* o, const int32_t* cu_seqlens, int N, int T, int heads) {
+  const int64_t first = (int64_t)cu_seqlens[N] * heads * 128;
+  const int64_t total = (int64_t)T * heads * 128;
+  for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+       i += (int64_t)gridDim.x * blockDim.x)
+    o[i] = 0;
+}
+
+inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+}  // namespace pla

@@ -17,7 +17,7 @@
 // (16 mantissa bits), which keeps the FP32 final state within 1e-5 of a float64 evaluation.
 //
 // Kernels:
-//   gdn_chunk_map_kernel     chunk table from cu_seqlens (device side, graph-capturable)
+//   chunk_map_kernel         chunk table from cu_seqlens (device side, graph-capturable)
 //   gdn_prep_kernel          gate, beta, chunk-local cumsum, q/k L2 norm (rounded to bf16), K^T tiles
 //   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
 //                            forward substitution in LDS, W (hi/lo) and P to the workspace
@@ -27,44 +27,9 @@
 //                            intermediate staying in registers (an accumulator tile is already a
 //                            valid B operand of the next product), A operands staged through LDS.
 
-#include "common.h"
+#include "prefill_common.h"
 
 namespace pla {
-
-typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-typedef float f32x8_t __attribute__((ext_vector_type(8)));
-
-constexpr int CHUNK = 64;
-
-__device__ __forceinline__ f32x4_t mfma16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
-}
-
-// hi = bf16(x), lo = bf16(x - hi) for two accumulator quads (eight contraction elements).
-struct HiLo { bf16x8_t hi, lo; };
-__device__ __forceinline__ HiLo split8(f32x4_t a, f32x4_t b) {
-  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-  HiLo r;
-  r.hi = __builtin_convertvector(x, bf16x8_t);
-  const f32x8_t back = __builtin_convertvector(r.hi, f32x8_t);
-  r.lo = __builtin_convertvector(x - back, bf16x8_t);
-  return r;
-}
-__device__ __forceinline__ bf16x8_t round8(f32x4_t a, f32x4_t b) {
-  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
-  return __builtin_convertvector(x, bf16x8_t);
-}
-
-// A (or B) operand of one 16x16x32 MFMA step from a row-major bf16 tile: lane (r = lane%16,
-// kb = lane/16) takes columns [32s+4kb, +4) and [32s+16+4kb, +4) of row r, which is the
-// contraction order in which an accumulator tile pair (row blocks 2s, 2s+1) presents its rows.
-__device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s, int kb) {
-  const uint2 p0 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 4 * kb);
-  const uint2 p1 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 16 + 4 * kb);
-  const uint4 u = make_uint4(p0.x, p0.y, p1.x, p1.y);
-  return __builtin_bit_cast(bf16x8_t, u);
-}
 
 struct GdnPrefillParams {
   // inputs
@@ -87,36 +52,6 @@ struct GdnPrefillParams {
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
   int H, HV, NC_max;
 };
-
-// ---------------------------------------------------------------------------------------------
-__global__ void gdn_chunk_map_kernel(const GdnPrefillParams p) {
-  // Single workgroup: exclusive scan of chunks per sequence, then the per-chunk table.
-  __shared__ int total;
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int n = 0; n < p.N; ++n) {
-      p.seq_chunk_off[n] = acc;
-      const int len = max(p.cu_seqlens[n + 1] - p.cu_seqlens[n], 0);
-      acc += (len + CHUNK - 1) / CHUNK;
-    }
-    p.seq_chunk_off[p.N] = acc;
-    total = acc;
-  }
-  __syncthreads();
-  for (int n = threadIdx.x; n < p.N; n += blockDim.x) {
-    const int start = p.cu_seqlens[n];
-    const int len = max(p.cu_seqlens[n + 1] - start, 0);
-    const int c0 = p.seq_chunk_off[n];
-    const int nc = (len + CHUNK - 1) / CHUNK;
-    for (int c = 0; c < nc; ++c) {
-      if (c0 + c >= p.NC_max) break;
-      p.chunk_seq[c0 + c] = n;
-      p.chunk_tok[c0 + c] = start + c * CHUNK;
-      p.chunk_len[c0 + c] = min(CHUNK, len - c * CHUNK);
-    }
-  }
-  (void)total;
-}
 
 // ---------------------------------------------------------------------------------------------
 // grid (chunk, H + 1), 256 threads.  blockIdx.y < H: L2 norm of q and k of one head for the
@@ -335,8 +270,6 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 // ---------------------------------------------------------------------------------------------
 // LDS tiles of the sequential kernel (bf16 elements, padded pitches keep 16-byte row alignment
 // and spread rows over banks).
-constexpr int PITCH128 = 136;
-constexpr int PITCH64 = 72;
 struct __align__(16) SeqTiles {
   uint16_t K[CHUNK][PITCH128];
   uint16_t Q[CHUNK][PITCH128];
@@ -578,18 +511,6 @@ __global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillPara
   }
 }
 
-// Zero the output rows that lie beyond the last sequence (physical padding).
-template <typename act_t>
-__global__ void gdn_zero_tail_kernel(const GdnPrefillParams p) {
-  const int64_t first = (int64_t)p.cu_seqlens[p.N] * p.HV * 128;
-  const int64_t total = (int64_t)p.T * p.HV * 128;
-  uint16_t* o = reinterpret_cast<uint16_t*>(p.o);
-  for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x)
-    o[i] = 0;
-}
-
-static size_t align_up(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, Whi, Wlo, P, total;
@@ -599,7 +520,7 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   GdnWorkspaceLayout L;
   L.NC_max = T / CHUNK + N;
   size_t off = 0;
-  auto take = [&](size_t bytes) { const size_t at = off; off = align_up(off + bytes); return at; };
+  auto take = [&](size_t bytes) { const size_t at = off; off = align_up256(off + bytes); return at; };
   L.seq_chunk_off = take((size_t)(N + 1) * 4);
   L.chunk_seq = take((size_t)L.NC_max * 4);
   L.chunk_tok = take((size_t)L.NC_max * 4);
@@ -674,12 +595,12 @@ extern "C" int pla_gdn_prefill_launch(
   p.H = H; p.HV = HV; p.NC_max = L.NC_max;
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(gdn_chunk_map_kernel, dim3(1), dim3(256), 0, s, p);
+  hipLaunchKernelGGL(chunk_map_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, N, L.NC_max, p.seq_chunk_off,
+                     p.chunk_seq, p.chunk_tok, p.chunk_len);
+  hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, HV);
   if (act_dtype == PLA_BF16) {
-    hipLaunchKernelGGL(gdn_zero_tail_kernel<bf16_t>, dim3(64), dim3(256), 0, s, p);
     hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   } else {
-    hipLaunchKernelGGL(gdn_zero_tail_kernel<f16_t>, dim3(64), dim3(256), 0, s, p);
     hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   }
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
