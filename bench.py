@@ -78,6 +78,77 @@ def bench_decode(steps, warmup, device):
         value_gbps=bytes_state * steps / wall / 1e9, workload=w)
 
 
+PREFILL_SEED = 348      # ragged_lengths(8, 512, 8192, 348) sums to 32 810 tokens
+GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64, K = V = 128, HV = 32, H = 16
+
+
+def bench_prefill(steps, warmup, device):
+    """Config 3: GDN chunk-64 prefill, 8 ragged sequences (about 32K tokens), indexed FP32 pool."""
+    import torch
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from pla_amd.workloads import gdn_prefill_packed, ragged_lengths
+    lengths = ragged_lengths(8, 512, 8192, PREFILL_SEED)
+    w = gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=64, seed=PREFILL_SEED, device=device)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    packed = call.pop("packed_qkv")
+    a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+
+    def run():
+        return gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, output_final_state=False, **call)
+
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / steps
+    T = sum(lengths)
+    tflops = GDN_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
+    return dict(tokens=T, lengths=lengths, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
+                roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=None,
+                              flop_per_token=GDN_FLOP_PER_TOKEN,
+                              note="algorithmic flops (dense, no hi/lo passes) over the whole call: "
+                                   "chunk map + prep + gram/solve + sequential kernels"))
+
+
+def bench_small_decode(device, steps=200):
+    """Config 0 (B=8 packed GDN decode) and config 2 (KDA MTP verify T=4, B=64 + commit): kernel times."""
+    import torch
+    from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
+    from pla_amd.decode.kda_replayssm_sglang import kda_mtp_verify
+    from pla_amd.workloads import gdn_decode_packed, kda_mtp_verify as make_verify
+    out = {}
+    w = gdn_decode_packed(8, seed=100, device=device)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+
+    def timed(fn):
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / steps * 1e3
+
+    us = timed(lambda: packed(**call))
+    out["config0_gdn_decode_b8_us"] = round(us, 2)
+    out["config0_state_GBps"] = round(8 * 32 * 131072 / us / 1e3, 1)
+    v = make_verify(B=64, pool_slots=1024, seed=202, device=device)
+    us = timed(lambda: kda_mtp_verify(v["q"], v["k"], v["v"], v["log_decay"], v["beta"], v["state"], v["indices"],
+                                      v["cu_seqlens"], scale=v["scale"]))
+    out["config2_kda_verify_t4_b64_us"] = round(us, 2)
+    out["config2_verify_state_read_GBps"] = round(64 * 32 * 65536 / us / 1e3, 1)
+    return out
+
+
 def cpu_baseline_decode(w, sample_requests=32, reps=5):
     """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
     sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
@@ -115,6 +186,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--decode-only", action="store_true", help="skip the secondary decode / prefill measurements")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the decode and prefill "
@@ -147,6 +219,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_decode(d["workload"])
+    del d
+    torch.cuda.empty_cache()
+    if not args.decode_only:
+        result["other_decode"] = bench_small_decode(device)
+        result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
     print(json.dumps(result))
 
 

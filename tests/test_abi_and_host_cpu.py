@@ -1,0 +1,99 @@
+"""CPU-only checks: the C-ABI library loads and exports every symbol the header declares, the
+ctypes signatures have the header's arity, and host-side argument validation rejects bad calls
+before anything native runs (no compute call is made here)."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pla_gfx950.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(pla_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        args = m.group(2).strip()
+        out[m.group(1)] = 0 if args in ("", "void") else len(args.split(","))
+    return out
+
+
+def test_library_exports_every_declared_symbol():
+    from pla_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python -m pla_amd.build"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    declared = _declared()
+    assert {"pla_version", "pla_last_error", "pla_k_last_packed_launch", "pla_k_last_launch",
+            "pla_kda_fold_launch", "pla_gdn_prefill_launch", "pla_gdn_prefill_workspace_bytes",
+            "pla_kda_prefill_launch", "pla_kda_prefill_workspace_bytes"} <= set(declared)
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.pla_version.restype = ctypes.c_char_p
+    assert b"gfx950" in lib.pla_version()
+
+
+def test_ctypes_signatures_match_header_arity():
+    from pla_amd import _lib
+    declared = _declared()
+    for name, argtypes in _lib.SIGNATURES.items():
+        assert declared[name] == len(argtypes), name
+
+
+def test_workspace_sizes_are_monotone_and_aligned():
+    from pla_amd import _lib
+    lib = _lib.load()
+    a = lib.pla_gdn_prefill_workspace_bytes(4096, 2, 16, 32)
+    b = lib.pla_gdn_prefill_workspace_bytes(8192, 2, 16, 32)
+    assert 0 < a < b and a % 256 == 0 and b % 256 == 0
+    assert lib.pla_gdn_prefill_workspace_bytes(0, 1, 1, 1) == 0
+    c = lib.pla_kda_prefill_workspace_bytes(4096, 1, 32)
+    assert c > 0 and c % 256 == 0
+
+
+def test_native_entry_points_reject_bad_arguments_without_a_gpu():
+    """Argument checks run before any launch, so they are testable on a CPU-only host."""
+    from pla_amd import _lib
+    lib = _lib.load()
+    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, None, None,
+                                      0.1, 1, 0, 0, 0, 0, 4, 2, 4, 64, 64, 1, 1, 0, _lib.BF16, 0, None)
+    assert rc != 0 and b"K == V == 128" in lib.pla_last_error()
+    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, None, None,
+                                      0.1, 1, 0, 0, 0, 0, 4, 3, 4, 128, 128, 1, 1, 0, _lib.BF16, 0, None)
+    assert rc != 0 and b"multiple of H" in lib.pla_last_error()
+    rc = lib.pla_kda_prefill_launch(None, None, None, None, None, 0, 0, 0, 0, 0, None, None, -7.0, 1.0,
+                                    None, 1, 64, None, None, 0, None, None, 0, None, None, 0, 4, 128, 128,
+                                    _lib.BF16, None)
+    assert rc != 0
+
+
+def test_facade_validation_raises_before_native_code():
+    from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    HV, H = 4, 2
+    state = torch.zeros(3, HV, 128, 128)
+    mixed = torch.zeros(2, (2 * H + HV) * 128 - 1, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="packed QKV width"):
+        packed(mixed, torch.zeros(2, HV, dtype=torch.bfloat16), torch.zeros(2, HV, dtype=torch.bfloat16),
+               torch.zeros(HV), torch.zeros(HV, dtype=torch.bfloat16), 1.0, 20.0, None, state,
+               torch.zeros(2, dtype=torch.int32), torch.zeros(2, 1, HV, 128, dtype=torch.bfloat16), True, None, False)
+    with pytest.raises(RuntimeError, match="initial_state_source is required"):
+        packed(mixed, None, None, None, None, 1.0, 20.0, None, None, None, None, True, None, False)
+    with pytest.raises(ValueError, match="CUDA tensor"):
+        gdn_prefill_packed_qkv_fwd(torch.zeros(4, 1024, dtype=torch.bfloat16), None, None, None, None, None,
+                                   num_qk_heads=2, num_v_heads=4)
+    with pytest.raises(ValueError, match="CUDA tensor"):
+        flashkda_fwd(*([torch.zeros(4, 2, 128, dtype=torch.bfloat16)] * 4), torch.zeros(4, 2), torch.zeros(2),
+                     torch.zeros(2, 128), torch.zeros(4, 2, 128, dtype=torch.bfloat16))
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    from pla_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libpla_gfx950.so")
+    with pytest.raises(RuntimeError, match="there is no fallback path"):
+        _lib.load()
