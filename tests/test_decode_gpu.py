@@ -342,3 +342,24 @@ def test_kda_packed_decode_b64_pool_with_padded_pitch():
     from pla_amd.workloads import gdn_decode_packed
     _check_packed_workload(gdn_decode_packed(64, H=32, HV=32, pool_slots=256, pad_frac=0.05, seed=102,
                                              is_kda=True, pitch_pad=256))
+
+
+def test_sanity_mode_rejects_before_launch_and_bypass_flag(monkeypatch):
+    forward, packed = _ops()[:2]
+    args, backing, lengths, state_ids, cache_ids = make_k_last_case(False, "decode", H=4, HV=8, B=3, padded=False)
+    monkeypatch.setenv("PLA_SANITY_CHECK", "1")
+    out = forward(**args)                                   # a valid call passes the diagnostic checks
+    torch.cuda.synchronize()
+    before = backing.clone()
+    bad = dict(args, initial_state_indices=torch.tensor([1, 1, 2], dtype=torch.int32, device="cuda"))
+    with pytest.raises(RuntimeError, match=r"PLA_SANITY_CHECK \[k_last\].*alias"):
+        forward(**bad)
+    bad = dict(args, initial_state_indices=torch.tensor([1, 99, 2], dtype=torch.int32, device="cuda"))
+    with pytest.raises(RuntimeError, match=r"PLA_SANITY_CHECK \[k_last\].*out of range"):
+        forward(**bad)
+    kw = packed_from(args)
+    kw["cu_seqlens"] = torch.tensor([0, 2, 2, 3], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match=r"PLA_SANITY_CHECK \[k_last_packed\]"):
+        packed(**kw)
+    torch.cuda.synchronize()
+    assert torch.equal(backing, before)
