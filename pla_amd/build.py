@@ -20,7 +20,7 @@ OBJ_DIR = os.path.join(HERE, "build")
 SOURCES = ["api.hip", "decode_k_last.hip", "prefill_gdn.hip", "prefill_kda.hip"]
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-inline-asm",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
@@ -49,7 +49,7 @@ def build_library(verbose=True):
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     tmp = LIB_PATH + ".tmp"
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wno-inline-asm", "-o", tmp, *objs]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (proc.stdout, proc.stderr))

@@ -46,6 +46,69 @@ __device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s,
 constexpr int PITCH128 = 136;
 constexpr int PITCH64 = 72;
 
+// ---------------------------------------------------------------------------------------------
+// Asynchronous global -> LDS tile copies (global_load_lds_dwordx4: no registers, no LDS store
+// instructions).  Lane i of a wavefront writes its 16 bytes at (wave-uniform LDS base) + 16 i, so
+// a padded tile is filled as linear memory in 1 KiB pieces; a lane whose slot falls into a row's
+// padding re-reads the last 16 data bytes of that row (the padding is never read back).
+//
+// The copy is issued from inline assembly so that the compiler's wait-count bookkeeping does not
+// see it (it would drain every outstanding copy before each LDS read).  Kernels wait by hand with
+// wait_vmcnt<N>(), N = number of copies this wavefront issued after the one it needs: vector
+// memory operations complete in issue order, and other memory operations issued in between only
+// make such a wait longer than necessary, never shorter.
+__device__ __forceinline__ void dma16(const char* gbase, uint32_t byte_offset, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :: "s"(lds_wave_base), "v"(byte_offset), "s"(gbase) : "memory", "m0");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+__device__ __forceinline__ uint32_t lds_address(const void* ptr) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)ptr;
+}
+
+// Copy plan for one padded LDS tile: ROWS rows of PITCH_B bytes whose first VALID_B bytes are data,
+// filled from rows `row_pitch_b` apart in global memory by the four wavefronts of a workgroup.
+// Each wavefront issues PIECES / 4 copies, wavefront 0 also the PIECES % 4 left over, so the copy
+// counts per wavefront are compile-time constants (EACH, FIRST).  The per-lane source offsets are
+// computed once; rows beyond `last_row` re-read that row.
+template <int ROWS, int PITCH_B, int VALID_B>
+struct TileCopy {
+  static constexpr int BYTES = ROWS * PITCH_B;
+  static_assert(BYTES % 1024 == 0 && PITCH_B % 16 == 0 && VALID_B % 16 == 0, "tiles are filled in 1 KiB pieces");
+  static constexpr int PIECES = BYTES / 1024;
+  static constexpr int EACH = PIECES / 4;
+  static constexpr int REST = PIECES % 4;
+  static constexpr int FIRST = EACH + REST;
+  uint32_t off[EACH];
+  uint32_t off_rest[REST > 0 ? REST : 1];
+
+  static __device__ __forceinline__ uint32_t source_offset(int piece, int lane, uint32_t row_pitch_b, int last_row) {
+    const int at = 1024 * piece + 16 * lane;
+    const int row = at / PITCH_B, cb = at - row * PITCH_B;
+    return (uint32_t)min(row, last_row) * row_pitch_b + (uint32_t)min(cb, VALID_B - 16);
+  }
+  __device__ __forceinline__ void plan(uint32_t row_pitch_b, int last_row, int wave, int lane) {
+#pragma unroll
+    for (int j0 = 0; j0 < EACH; ++j0) off[j0] = source_offset(4 * j0 + wave, lane, row_pitch_b, last_row);
+#pragma unroll
+    for (int j = 0; j < REST; ++j) off_rest[j] = source_offset(4 * EACH + j, lane, row_pitch_b, last_row);
+  }
+  // `gbase` (wave-uniform) addresses row 0 of the source tile.
+  __device__ __forceinline__ void issue(const void* tile, const char* gbase, int wave) const {
+    const uint32_t base = lds_address(tile) + 1024u * wave;
+#pragma unroll
+    for (int j0 = 0; j0 < EACH; ++j0) dma16(gbase, off[j0], base + 4096u * j0);
+    if (wave == 0) {
+#pragma unroll
+      for (int j = 0; j < REST; ++j) dma16(gbase, off_rest[j], base + 1024u * (4 * EACH + j));
+    }
+  }
+};
+
 // Chunk table from cu_seqlens, built on the device so that no call reads offsets back to the host.
 // Single workgroup.  seq_chunk_off[n] = first chunk of sequence n (seq_chunk_off[N] = total).
 static __global__ void chunk_map_kernel(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,

@@ -50,6 +50,7 @@ struct GdnPrefillParams {
   uint16_t* qn; uint16_t* kn; uint16_t* knT;
   float* gcum; float* beta;
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
+  float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
   int H, HV, NC_max;
 };
 
@@ -97,8 +98,21 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
         float cum = 0.f;
         for (int j = 0; j < len; ++j) {
           cum += sh.g[j][threadIdx.x];
+          sh.g[j][threadIdx.x] = cum;
           p.gcum[(int64_t)(t0 + j) * p.HV + hv0 + threadIdx.x] = cum;
         }
+      }
+      __syncthreads();
+      // per-chunk decay factors, one 1 KiB tile per value head (rows past the chunk repeat its last row)
+      for (int idx = threadIdx.x; idx < CHUNK * nh; idx += 256) {
+        const int hl = idx >> 6, j = idx & 63;
+        const float g = sh.g[min(j, len - 1)][hl], glast = sh.g[len - 1][hl];
+        float* gt = p.gtile + ((int64_t)cb * p.HV + hv0 + hl) * 256;
+        const float e = __expf(g);
+        gt[j] = p.scale * e;
+        gt[64 + j] = e;
+        gt[128 + j] = __expf(glast - g);
+        gt[192 + j] = __expf(glast);
       }
       __syncthreads();
     }
@@ -268,252 +282,302 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 }
 
 // ---------------------------------------------------------------------------------------------
-// LDS tiles of the sequential kernel (bf16 elements, padded pitches keep 16-byte row alignment
-// and spread rows over banks).
-struct __align__(16) SeqTiles {
-  uint16_t K[CHUNK][PITCH128];
-  uint16_t Q[CHUNK][PITCH128];
-  uint16_t V[CHUNK][PITCH128];
-  uint16_t O[CHUNK][PITCH128];
-  uint16_t Kt[128][PITCH64];
-  uint16_t Whi[CHUNK][PITCH64];
-  uint16_t Wlo[CHUNK][PITCH64];
-  uint16_t P[CHUNK][PITCH64];
-  float sQ[CHUNK];     // scale * e^{G_i}
-  float eG[CHUNK];     // e^{G_i}
-  float dG[CHUNK];     // e^{G_last - G_i}
-  float eGlast;
-};
+// Sequential kernel: one workgroup per (sequence, value head), four wavefronts (one per SIMD),
+// each owning two 16-column blocks of V that share every A operand.  S^T stays in MFMA
+// accumulator layout (an accumulator tile pair is already a valid B operand of the next product),
+// A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  Every tile
+// is single buffered, and the copy of chunk c+1's version of a tile is issued at the first barrier
+// after the last use of chunk c's version, so each copy has most of a chunk's compute time to land:
+//
+//   barrier 1   K, Q, V, decay factors of chunk c landed    flush O(c-1), issue P(c), factors of c+1
+//               KS = K S^T, QS = Q S^T, X = V - e^G (.) KS
+//   barrier 2   W landed                                     issue K, Q, V of chunk c+1
+//               U = W X
+//   barrier 3   K^T landed                                   issue W of chunk c+1
+//               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
+//   barrier 4   P landed                                     issue K^T of chunk c+1
+//               O = scale e^G (.) QS + P U  -> O tile
+using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256>;     // 64 x 128 tile
+using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128>;    // 64 x 64 tile
+using CopyKt = TileCopy<128, 2 * PITCH64, 128>;          // 128 x 64 tile
 
-// Everything the next chunk needs is requested from global memory one chunk ahead and parked
-// in registers (eleven 16-byte vectors per thread), every per-chunk address is a running
-// pointer, V and O travel through LDS tiles (coalesced 16-byte global accesses, immediate-offset
-// LDS accesses), so the chunk-to-chunk critical path holds only LDS reads, conversions and MFMAs.
 template <typename act_t>
-__global__ __launch_bounds__(512) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
+__global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
   const int n = blockIdx.x / p.HV;
   const int hv = blockIdx.x - n * p.HV;
   const int h = hv / (p.HV / p.H);
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int vcol = 16 * wave + r16;                  // this lane's V column
+  const int vcol = 32 * wave + r16;                  // first of this lane's two V columns (second: +16)
   const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
-  if (c_begin >= c_end) return;                      // empty sequence: state untouched, no output
+  if (c_begin >= c_end) return;
   const int seq_start = p.cu_seqlens[n];
   const int seq_len = p.cu_seqlens[n + 1] - seq_start;
+  const int n_chunks = c_end - c_begin;
 
-  __shared__ SeqTiles T;
+  // distinct LDS objects: the compiler tracks outstanding direct-to-LDS loads per object
+  __shared__ __align__(16) uint16_t tK[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tKt[128 * PITCH64];
+  __shared__ __align__(16) uint16_t tWh[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tWl[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  // decay factors by chunk parity: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
+  __shared__ __align__(16) float tG[2][256];
 
-  // S^T slice in accumulator layout: St[mc][r] = S[v = vcol][c = 16 mc + 4 kb + r]
-  f32x4_t St[8];
+  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
+  f32x4_t St[2][8];
   {
     const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
-    if (slot >= 0) {
-      const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)hv * 128 + vcol) * 128 + 4 * kb;
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) {
-        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
-        St[mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+    for (int nb = 0; nb < 2; ++nb)
+      if (slot >= 0) {
+        const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) {
+          const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+          St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+        }
+      } else {
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       }
-    } else {
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) St[mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
   }
 
-  // cooperative copy coordinates: 64-row x 128-column tiles are 1024 16-byte vectors (two per
-  // thread: rows krow and krow + 32), 64 x 64 and the 128 x 64 K^T tiles 512 / 1024 vectors.
+  const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
+  const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
+  const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
+  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
+  const char* const kt_b = reinterpret_cast<const char*>(p.knT) + ((int64_t)c_begin * p.H + h) * 16384;
+  const char* const wh_b = reinterpret_cast<const char*>(p.Whi) + ((int64_t)c_begin * p.HV + hv) * 8192;
+  const char* const wl_b = reinterpret_cast<const char*>(p.Wlo) + ((int64_t)c_begin * p.HV + hv) * 8192;
+  const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
+  const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
+
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+  // Copy plans.  K and Q share one (same pitch); the last chunk of a sequence gets plans of its own
+  // that keep rows past the sequence end inside it.
+  CopyWide plan_kq, plan_v;
+  CopyNarrow plan_w;
+  CopyKt plan_kt;
+  plan_kq.plan((uint32_t)tok_pitch_b, CHUNK - 1, wave, lane);
+  plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
+  plan_w.plan(128, CHUNK - 1, wave, lane);
+  plan_kt.plan(128, 127, wave, lane);
+  auto issue_kqv = [&](int c) {
+    const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
+    const char* qs = qn_b + (int64_t)c * CHUNK * tok_pitch_b;
+    const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+    const int len = chunk_len(c);
+    if (len == CHUNK) {
+      plan_kq.issue(tK, ks, wave);
+      plan_kq.issue(tQ, qs, wave);
+      plan_v.issue(tV, vs, wave);
+    } else {
+      CopyWide tail_kq, tail_v;
+      tail_kq.plan((uint32_t)tok_pitch_b, len - 1, wave, lane);
+      tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
+      tail_kq.issue(tK, ks, wave);
+      tail_kq.issue(tQ, qs, wave);
+      tail_v.issue(tV, vs, wave);
+    }
+  };
+  auto issue_w = [&](int c) {
+    plan_w.issue(tWh, wh_b + (int64_t)c * p.HV * 8192, wave);
+    plan_w.issue(tWl, wl_b + (int64_t)c * p.HV * 8192, wave);
+  };
+  auto issue_kt = [&](int c) { plan_kt.issue(tKt, kt_b + (int64_t)c * p.H * 16384, wave); };
+  auto issue_p = [&](int c) { plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave); };
+  auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
+    if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
+  };
+  // Copies issued after the one a barrier waits for (wavefronts 1..3 / wavefront 0); the gate piece
+  // is left out of wavefront 0's counts where it is conditional, which only makes the wait longer.
+  constexpr int KQV_O = 3 * CopyWide::EACH, KQV_0 = 3 * CopyWide::FIRST;
+  constexpr int W_O = 2 * CopyNarrow::EACH, W_0 = 2 * CopyNarrow::FIRST;
+  constexpr int KT_O = CopyKt::EACH, KT_0 = CopyKt::FIRST;
+  constexpr int P_O = CopyNarrow::EACH, P_0 = CopyNarrow::FIRST;
+  // coalesced write of a finished output tile
   const int krow = tid >> 4, kcv = tid & 15;
-  const int srow = tid >> 3, scv = tid & 7;
-  const int64_t tok_pitch = (int64_t)p.H * 128;                // elements between tokens of kn / qn
-  const int64_t half_k = 32 * tok_pitch, half_v = 32 * p.stride_v;
-  const uint16_t* kptr = p.kn + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
-  const uint16_t* qptr = p.qn + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
-  const uint16_t* vptr = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)(seq_start + krow) * p.stride_v + hv * 128 + 8 * kcv;
-  const uint16_t* ktptr = p.knT + ((int64_t)c_begin * p.H + h) * 8192 + 8 * tid;
-  const uint16_t* whptr = p.Whi + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
-  const uint16_t* wlptr = p.Wlo + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
-  const uint16_t* ppptr = p.P + ((int64_t)c_begin * p.HV + hv) * 4096 + 8 * tid;
-  const float* gptr = p.gcum + (int64_t)seq_start * p.HV + hv;
-  uint16_t* optr = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
-  const int64_t o_half = (int64_t)32 * p.HV * 128;
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
-
-  uint4 pk0, pk1, pq0, pq1, pv0, pv1, pt0, pt1, pwh, pwl, ppp;
-  float pg;
-  // `len` rows of the chunk are real; rows beyond are read from row 0 of the chunk and zeroed.
-  auto prefetch = [&](int len) {
-    const bool ok0 = krow < len, ok1 = krow + 32 < len;
-    const int64_t back0 = ok0 ? 0 : -(int64_t)krow, back1 = ok1 ? 32 : -(int64_t)krow;
-    pk0 = *reinterpret_cast<const uint4*>(kptr + back0 * tok_pitch);
-    pq0 = *reinterpret_cast<const uint4*>(qptr + back0 * tok_pitch);
-    pv0 = *reinterpret_cast<const uint4*>(vptr + back0 * p.stride_v);
-    pk1 = *reinterpret_cast<const uint4*>(kptr + back1 * tok_pitch);
-    pq1 = *reinterpret_cast<const uint4*>(qptr + back1 * tok_pitch);
-    pv1 = *reinterpret_cast<const uint4*>(vptr + back1 * p.stride_v);
-    pt0 = *reinterpret_cast<const uint4*>(ktptr);
-    pt1 = *reinterpret_cast<const uint4*>(ktptr + 4096);
-    pwh = *reinterpret_cast<const uint4*>(whptr);
-    pwl = *reinterpret_cast<const uint4*>(wlptr);
-    ppp = *reinterpret_cast<const uint4*>(ppptr);
-    pg = gptr[(int64_t)(lane < len ? lane : len - 1) * p.HV];
-    if (!ok0) { pk0 = zero4; pq0 = zero4; pv0 = zero4; }
-    if (!ok1) { pk1 = zero4; pq1 = zero4; pv1 = zero4; }
-    (void)half_k; (void)half_v;
-  };
-  auto advance = [&]() {
-    kptr += CHUNK * tok_pitch; qptr += CHUNK * tok_pitch; vptr += CHUNK * p.stride_v;
-    ktptr += (int64_t)p.H * 8192; whptr += (int64_t)p.HV * 4096; wlptr += (int64_t)p.HV * 4096;
-    ppptr += (int64_t)p.HV * 4096; gptr += (int64_t)CHUNK * p.HV;
-  };
-  // coalesced write of the previous chunk's output tile
-  auto flush_output = [&](int len) {
-    if (krow < len) *reinterpret_cast<uint4*>(optr) = *reinterpret_cast<const uint4*>(&T.O[krow][8 * kcv]);
-    if (krow + 32 < len) *reinterpret_cast<uint4*>(optr + o_half) = *reinterpret_cast<const uint4*>(&T.O[krow + 32][8 * kcv]);
-    optr += (int64_t)CHUNK * p.HV * 128;
-  };
-
-  const int n_chunks = c_end - c_begin;
-  prefetch(min(CHUNK, seq_len));
-  advance();
-  int prev_len = 0;
-  for (int ci = 0; ci < n_chunks; ++ci) {
-    const int len = min(CHUNK, seq_len - ci * CHUNK);
-
-    __syncthreads();                 // everyone finished with the previous chunk's tiles
-    if (ci > 0) flush_output(prev_len);
-    *reinterpret_cast<uint4*>(&T.K[krow][8 * kcv]) = pk0;
-    *reinterpret_cast<uint4*>(&T.K[krow + 32][8 * kcv]) = pk1;
-    *reinterpret_cast<uint4*>(&T.Q[krow][8 * kcv]) = pq0;
-    *reinterpret_cast<uint4*>(&T.Q[krow + 32][8 * kcv]) = pq1;
-    *reinterpret_cast<uint4*>(&T.V[krow][8 * kcv]) = pv0;
-    *reinterpret_cast<uint4*>(&T.V[krow + 32][8 * kcv]) = pv1;
-    *reinterpret_cast<uint4*>(&T.Kt[srow][8 * scv]) = pt0;
-    *reinterpret_cast<uint4*>(&T.Kt[64 + srow][8 * scv]) = pt1;
-    *reinterpret_cast<uint4*>(&T.Whi[srow][8 * scv]) = pwh;
-    *reinterpret_cast<uint4*>(&T.Wlo[srow][8 * scv]) = pwl;
-    *reinterpret_cast<uint4*>(&T.P[srow][8 * scv]) = ppp;
-    if (wave == 0) {
-      const float glast = __shfl(pg, len - 1, 64);
-      const float e = __expf(pg);
-      T.eG[lane] = e;
-      T.sQ[lane] = p.scale * e;
-      T.dG[lane] = __expf(glast - pg);
-      if (lane == 0) T.eGlast = __expf(glast);
-    }
-    __syncthreads();
-    if (ci + 1 < n_chunks) {
-      prefetch(min(CHUNK, seq_len - (ci + 1) * CHUNK));
-      advance();
-    }
-
-    // (1) KS = K S^T and (3a) QS = Q S^T : contraction over the 128 K channels
-    f32x4_t KS[4], QS[4];
+  uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
+  auto flush_output = [&](int c) {
+    const int len = chunk_len(c);
+    uint16_t* dst = o_b + (int64_t)c * CHUNK * p.HV * 128;
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) { KS[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[mi] = KS[mi]; }
+    for (int i = 0; i < 4; ++i)
+      if (krow + 16 * i < len)
+        *reinterpret_cast<uint4*>(dst + (int64_t)16 * i * p.HV * 128) =
+            *reinterpret_cast<const uint4*>(&tO[(krow + 16 * i) * PITCH128 + 8 * kcv]);
+  };
+
+  issue_gates(0);
+  issue_kqv(0);
+  issue_w(0);
+  issue_kt(0);
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int par = ci & 1;
+    const bool more = ci + 1 < n_chunks;
+
+    // barrier 1: K, Q, V (and the decay factors) of this chunk; W and K^T were issued after them
+    if (wave == 0) wait_vmcnt<W_0 + KT_0>(); else wait_vmcnt<W_O + KT_O>();
+    __syncthreads();
+    if (ci > 0) flush_output(ci - 1);
+    issue_p(ci);
+    if (more) issue_gates(ci + 1);
+
+    f32x4_t KS[2][4], QS[2][4];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const HiLo sb = split8(St[2 * s], St[2 * s + 1]);
+      const HiLo sb0 = split8(St[0][2 * s], St[0][2 * s + 1]);
+      const HiLo sb1 = split8(St[1][2 * s], St[1][2 * s + 1]);
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t ka = operand_from(&T.K[16 * mi + r16][0], s, kb);
-        const bf16x8_t qa = operand_from(&T.Q[16 * mi + r16][0], s, kb);
-        KS[mi] = mfma16(ka, sb.hi, KS[mi]);
-        QS[mi] = mfma16(qa, sb.hi, QS[mi]);
-        KS[mi] = mfma16(ka, sb.lo, KS[mi]);
+        const bf16x8_t ka = operand_from(&tK[(16 * mi + r16) * PITCH128], s, kb);
+        const bf16x8_t qa = operand_from(&tQ[(16 * mi + r16) * PITCH128], s, kb);
+        KS[0][mi] = mfma16(ka, sb0.hi, KS[0][mi]);
+        KS[1][mi] = mfma16(ka, sb1.hi, KS[1][mi]);
+        QS[0][mi] = mfma16(qa, sb0.hi, QS[0][mi]);
+        QS[1][mi] = mfma16(qa, sb1.hi, QS[1][mi]);
+        KS[0][mi] = mfma16(ka, sb0.lo, KS[0][mi]);
+        KS[1][mi] = mfma16(ka, sb1.lo, KS[1][mi]);
       }
     }
-
-    // X = V - e^{G} (.) KS   (rows of the accumulator are tokens)
-    f32x4_t X[4];
+    // X = V - e^{G} (.) KS
+    f32x4_t X[2][4];
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
-      const float4 eg = *reinterpret_cast<const float4*>(&T.eG[16 * mi + 4 * kb]);
-      const uint16_t* vr = &T.V[16 * mi + 4 * kb][vcol];
-      X[mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[mi][0];
-      X[mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[mi][1];
-      X[mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[mi][2];
-      X[mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[mi][3];
-    }
-
-    // (2) U = W X : contraction over the 64 tokens, W and X both split
-    f32x4_t U[4];
+      const float4 eg = *reinterpret_cast<const float4*>(&tG[par][64 + 16 * mi + 4 * kb]);
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) U[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const HiLo xb = split8(X[2 * s], X[2 * s + 1]);
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t wh = operand_from(&T.Whi[16 * mi + r16][0], s, kb);
-        const bf16x8_t wl = operand_from(&T.Wlo[16 * mi + r16][0], s, kb);
-        U[mi] = mfma16(wh, xb.hi, U[mi]);
-        U[mi] = mfma16(wl, xb.hi, U[mi]);
-        U[mi] = mfma16(wh, xb.lo, U[mi]);
+      for (int nb = 0; nb < 2; ++nb) {
+        const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+        X[nb][mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[nb][mi][0];
+        X[nb][mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[nb][mi][1];
+        X[nb][mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[nb][mi][2];
+        X[nb][mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[nb][mi][3];
       }
     }
 
-    // (4) S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)   -- the next chunk waits for this
-    const float egl = T.eGlast;
+    // barrier 2: W; K^T and P were issued after it
+    if (wave == 0) wait_vmcnt<KT_0 + P_0>(); else wait_vmcnt<KT_O + P_O>();
+    __syncthreads();
+    if (more) issue_kqv(ci + 1);
+    f32x4_t U[2][4];
 #pragma unroll
-    for (int mc = 0; mc < 8; ++mc) St[mc] *= egl;
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const float4 d0 = *reinterpret_cast<const float4*>(&T.dG[32 * s + 4 * kb]);
-      const float4 d1 = *reinterpret_cast<const float4*>(&T.dG[32 * s + 16 + 4 * kb]);
-      const f32x4_t u0 = {U[2 * s][0] * d0.x, U[2 * s][1] * d0.y, U[2 * s][2] * d0.z, U[2 * s][3] * d0.w};
-      const f32x4_t u1 = {U[2 * s + 1][0] * d1.x, U[2 * s + 1][1] * d1.y, U[2 * s + 1][2] * d1.z, U[2 * s + 1][3] * d1.w};
-      const HiLo ub = split8(u0, u1);
+      const HiLo xb0 = split8(X[0][2 * s], X[0][2 * s + 1]);
+      const HiLo xb1 = split8(X[1][2 * s], X[1][2 * s + 1]);
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        const bf16x8_t wh = operand_from(&tWh[(16 * mi + r16) * PITCH64], s, kb);
+        const bf16x8_t wl = operand_from(&tWl[(16 * mi + r16) * PITCH64], s, kb);
+        U[0][mi] = mfma16(wh, xb0.hi, U[0][mi]);
+        U[1][mi] = mfma16(wh, xb1.hi, U[1][mi]);
+        U[0][mi] = mfma16(wl, xb0.hi, U[0][mi]);
+        U[1][mi] = mfma16(wl, xb1.hi, U[1][mi]);
+        U[0][mi] = mfma16(wh, xb0.lo, U[0][mi]);
+        U[1][mi] = mfma16(wh, xb1.lo, U[1][mi]);
+      }
+    }
+
+    // barrier 3: K^T; P and (unless this is the last chunk) the next K, Q, V were issued after it
+    if (!more) { if (wave == 0) wait_vmcnt<P_0>(); else wait_vmcnt<P_O>(); }
+    else if (wave == 0) wait_vmcnt<P_0 + KQV_0>(); else wait_vmcnt<P_O + KQV_O>();
+    __syncthreads();
+    if (more) issue_w(ci + 1);
+    const float egl = tG[par][192];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const float4 d0 = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 4 * kb]);
+      const float4 d1 = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 16 + 4 * kb]);
+      HiLo ub[2];
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        const f32x4_t u0 = {U[nb][2 * s][0] * d0.x, U[nb][2 * s][1] * d0.y, U[nb][2 * s][2] * d0.z, U[nb][2 * s][3] * d0.w};
+        const f32x4_t u1 = {U[nb][2 * s + 1][0] * d1.x, U[nb][2 * s + 1][1] * d1.y, U[nb][2 * s + 1][2] * d1.z,
+                            U[nb][2 * s + 1][3] * d1.w};
+        ub[nb] = split8(u0, u1);
+      }
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
-        const bf16x8_t ka = operand_from(&T.Kt[16 * mc + r16][0], s, kb);
-        St[mc] = mfma16(ka, ub.hi, St[mc]);
-        St[mc] = mfma16(ka, ub.lo, St[mc]);
+        const bf16x8_t ka = operand_from(&tKt[(16 * mc + r16) * PITCH64], s, kb);
+        St[0][mc] = mfma16(ka, ub[0].hi, St[0][mc]);
+        St[1][mc] = mfma16(ka, ub[1].hi, St[1][mc]);
+        St[0][mc] = mfma16(ka, ub[0].lo, St[0][mc]);
+        St[1][mc] = mfma16(ka, ub[1].lo, St[1][mc]);
       }
     }
 
-    // (3b) O = scale e^{G} (.) QS + P U   -- off the state's critical path
-    f32x4_t O[4];
+    // barrier 4: P; the next K, Q, V and W were issued after it
+    if (!more) wait_vmcnt<0>();
+    else if (wave == 0) wait_vmcnt<KQV_0 + W_0>(); else wait_vmcnt<KQV_O + W_O>();
+    __syncthreads();
+    if (more) issue_kt(ci + 1);
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
-      const float4 sq = *reinterpret_cast<const float4*>(&T.sQ[16 * mi + 4 * kb]);
-      O[mi] = f32x4_t{sq.x * QS[mi][0], sq.y * QS[mi][1], sq.z * QS[mi][2], sq.w * QS[mi][3]};
+      const float4 sq = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        QS[nb][mi][0] *= sq.x; QS[nb][mi][1] *= sq.y; QS[nb][mi][2] *= sq.z; QS[nb][mi][3] *= sq.w;
+      }
     }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const bf16x8_t ub = round8(U[2 * s], U[2 * s + 1]);
+      const bf16x8_t ur0 = round8(U[0][2 * s], U[0][2 * s + 1]);
+      const bf16x8_t ur1 = round8(U[1][2 * s], U[1][2 * s + 1]);
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-        O[mi] = mfma16(operand_from(&T.P[16 * mi + r16][0], s, kb), ub, O[mi]);
+      for (int mi = 0; mi < 4; ++mi) {
+        const bf16x8_t pa = operand_from(&tP[(16 * mi + r16) * PITCH64], s, kb);
+        QS[0][mi] = mfma16(pa, ur0, QS[0][mi]);
+        QS[1][mi] = mfma16(pa, ur1, QS[1][mi]);
+      }
     }
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      uint16_t* orow = &T.O[16 * mi + 4 * kb][vcol];
-      orow[0] = from_float<act_t>(O[mi][0]).bits;
-      orow[PITCH128] = from_float<act_t>(O[mi][1]).bits;
-      orow[2 * PITCH128] = from_float<act_t>(O[mi][2]).bits;
-      orow[3 * PITCH128] = from_float<act_t>(O[mi][3]).bits;
-    }
-    prev_len = len;
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+        orow[0] = from_float<act_t>(QS[nb][mi][0]).bits;
+        orow[PITCH128] = from_float<act_t>(QS[nb][mi][1]).bits;
+        orow[2 * PITCH128] = from_float<act_t>(QS[nb][mi][2]).bits;
+        orow[3 * PITCH128] = from_float<act_t>(QS[nb][mi][3]).bits;
+      }
   }
   __syncthreads();
-  flush_output(prev_len);
+  flush_output(n_chunks - 1);
 
   if (p.ht != nullptr) {
     const int slot = p.ht_indices ? p.ht_indices[n] : n;
     if (slot >= 0) {
-      float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)hv * 128 + vcol) * 128 + 4 * kb;
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[mc].x, St[mc].y, St[mc].z, St[mc].w);
+      for (int nb = 0; nb < 2; ++nb) {
+        float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc)
+          *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+      }
     }
   }
 }
 
-
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, Whi, Wlo, P, total;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P, total;
   int NC_max;
 };
 static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
@@ -530,6 +594,7 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   L.knT = take((size_t)L.NC_max * H * 128 * CHUNK * 2);
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
+  L.gtile = take((size_t)L.NC_max * HV * 256 * 4);
   L.Whi = take((size_t)L.NC_max * HV * 4096 * 2);
   L.Wlo = take((size_t)L.NC_max * HV * 4096 * 2);
   L.P = take((size_t)L.NC_max * HV * 4096 * 2);
@@ -589,6 +654,7 @@ extern "C" int pla_gdn_prefill_launch(
   p.knT = reinterpret_cast<uint16_t*>(ws + L.knT);
   p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
   p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
+  p.gtile = reinterpret_cast<float*>(ws + L.gtile);
   p.Whi = reinterpret_cast<uint16_t*>(ws + L.Whi);
   p.Wlo = reinterpret_cast<uint16_t*>(ws + L.Wlo);
   p.P = reinterpret_cast<uint16_t*>(ws + L.P);
@@ -604,9 +670,6 @@ extern "C" int pla_gdn_prefill_launch(
     hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   }
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
-  if (act_dtype == PLA_BF16)
-    hipLaunchKernelGGL(gdn_chunk_seq_kernel<bf16_t>, dim3((unsigned)N * HV), dim3(512), 0, s, p);
-  else
-    hipLaunchKernelGGL(gdn_chunk_seq_kernel<f16_t>, dim3((unsigned)N * HV), dim3(512), 0, s, p);
+  hipLaunchKernelGGL(gdn_chunk_seq_kernel<bf16_t>, dim3((unsigned)N * HV), dim3(256), 0, s, p);
   return check_launch("gdn prefill launch");
 }
