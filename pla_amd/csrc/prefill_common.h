@@ -9,6 +9,8 @@ namespace pla {
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x8_t __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned u32x8_t __attribute__((ext_vector_type(8)));
 
 constexpr int CHUNK = 64;
 
@@ -22,7 +24,11 @@ __device__ __forceinline__ HiLo split8(f32x4_t a, f32x4_t b) {
   const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
   HiLo r;
   r.hi = __builtin_convertvector(x, bf16x8_t);
-  const f32x8_t back = __builtin_convertvector(r.hi, f32x8_t);
+  // widen the packed pairs back with one shift or mask each
+  const u32x4_t w = __builtin_bit_cast(u32x4_t, r.hi);
+  const u32x8_t wide = {w[0] << 16, w[0] & 0xffff0000u, w[1] << 16, w[1] & 0xffff0000u,
+                        w[2] << 16, w[2] & 0xffff0000u, w[3] << 16, w[3] & 0xffff0000u};
+  const f32x8_t back = __builtin_bit_cast(f32x8_t, wide);
   r.lo = __builtin_convertvector(x - back, bf16x8_t);
   return r;
 }
@@ -71,19 +77,19 @@ __device__ __forceinline__ uint32_t lds_address(const void* ptr) {
 }
 
 // Copy plan for one padded LDS tile: ROWS rows of PITCH_B bytes whose first VALID_B bytes are data,
-// filled from rows `row_pitch_b` apart in global memory by the four wavefronts of a workgroup.
-// Each wavefront issues PIECES / 4 copies, wavefront 0 also the PIECES % 4 left over, so the copy
+// filled from rows `row_pitch_b` apart in global memory by the WAVES wavefronts of a workgroup.
+// Each wavefront issues PIECES / WAVES copies, wavefront 0 also the PIECES % WAVES left over, so the copy
 // counts per wavefront are compile-time constants (EACH, FIRST).  The per-lane source offsets are
 // computed once; rows beyond `last_row` re-read that row.
-template <int ROWS, int PITCH_B, int VALID_B>
+template <int ROWS, int PITCH_B, int VALID_B, int WAVES>
 struct TileCopy {
   static constexpr int BYTES = ROWS * PITCH_B;
   static_assert(BYTES % 1024 == 0 && PITCH_B % 16 == 0 && VALID_B % 16 == 0, "tiles are filled in 1 KiB pieces");
   static constexpr int PIECES = BYTES / 1024;
-  static constexpr int EACH = PIECES / 4;
-  static constexpr int REST = PIECES % 4;
+  static constexpr int EACH = PIECES / WAVES;
+  static constexpr int REST = PIECES % WAVES;
   static constexpr int FIRST = EACH + REST;
-  uint32_t off[EACH];
+  uint32_t off[EACH > 0 ? EACH : 1];
   uint32_t off_rest[REST > 0 ? REST : 1];
 
   static __device__ __forceinline__ uint32_t source_offset(int piece, int lane, uint32_t row_pitch_b, int last_row) {
@@ -93,18 +99,18 @@ struct TileCopy {
   }
   __device__ __forceinline__ void plan(uint32_t row_pitch_b, int last_row, int wave, int lane) {
 #pragma unroll
-    for (int j0 = 0; j0 < EACH; ++j0) off[j0] = source_offset(4 * j0 + wave, lane, row_pitch_b, last_row);
+    for (int j0 = 0; j0 < EACH; ++j0) off[j0] = source_offset(WAVES * j0 + wave, lane, row_pitch_b, last_row);
 #pragma unroll
-    for (int j = 0; j < REST; ++j) off_rest[j] = source_offset(4 * EACH + j, lane, row_pitch_b, last_row);
+    for (int j = 0; j < REST; ++j) off_rest[j] = source_offset(WAVES * EACH + j, lane, row_pitch_b, last_row);
   }
   // `gbase` (wave-uniform) addresses row 0 of the source tile.
   __device__ __forceinline__ void issue(const void* tile, const char* gbase, int wave) const {
     const uint32_t base = lds_address(tile) + 1024u * wave;
 #pragma unroll
-    for (int j0 = 0; j0 < EACH; ++j0) dma16(gbase, off[j0], base + 4096u * j0);
+    for (int j0 = 0; j0 < EACH; ++j0) dma16(gbase, off[j0], base + 1024u * WAVES * j0);
     if (wave == 0) {
 #pragma unroll
-      for (int j = 0; j < REST; ++j) dma16(gbase, off_rest[j], base + 1024u * (4 * EACH + j));
+      for (int j = 0; j < REST; ++j) dma16(gbase, off_rest[j], base + 1024u * (WAVES * EACH + j));
     }
   }
 };

@@ -18,14 +18,16 @@
 //
 // Kernels:
 //   chunk_map_kernel         chunk table from cu_seqlens (device side, graph-capturable)
-//   gdn_prep_kernel          gate, beta, chunk-local cumsum, q/k L2 norm (rounded to bf16), K^T tiles
+//   gdn_prep_kernel          gate, beta, chunk-local cumsum and per-chunk decay-factor tiles, q/k L2
+//                            norm (rounded to bf16), K^T tiles
 //   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
 //                            forward substitution in LDS, W (hi/lo) and P to the workspace
-//   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), 8 wavefronts each owning a
-//                            16-wide V slice of S^T in MFMA accumulator layout; the chain
+//   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), four wavefronts each owning a
+//                            32-wide V slice of S^T in MFMA accumulator layout; the chain
 //                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_bf16 with every
 //                            intermediate staying in registers (an accumulator tile is already a
-//                            valid B operand of the next product), A operands staged through LDS.
+//                            valid B operand of the next product); A operands come from LDS tiles
+//                            filled by asynchronous global -> LDS copies one chunk ahead.
 
 #include "prefill_common.h"
 
@@ -282,8 +284,10 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sequential kernel: one workgroup per (sequence, value head), four wavefronts (one per SIMD),
-// each owning two 16-column blocks of V that share every A operand.  S^T stays in MFMA
+// Sequential kernel: one workgroup per (sequence, value head), 8 / NB wavefronts, each owning NB
+// 16-column blocks of V that share every A operand (NB = 2: four wavefronts, one per SIMD; every
+// wavefront reads every A tile once per chunk, so fewer, wider wavefronts halve the LDS traffic,
+// which is what bounds this kernel).  S^T stays in MFMA
 // accumulator layout (an accumulator tile pair is already a valid B operand of the next product),
 // A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  Every tile
 // is single buffered, and the copy of chunk c+1's version of a tile is issued at the first barrier
@@ -297,12 +301,12 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 //               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
 //   barrier 4   P landed                                     issue K^T of chunk c+1
 //               O = scale e^G (.) QS + P U  -> O tile
-using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256>;     // 64 x 128 tile
-using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128>;    // 64 x 64 tile
-using CopyKt = TileCopy<128, 2 * PITCH64, 128>;          // 128 x 64 tile
-
-template <typename act_t>
-__global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
+template <typename act_t, int NB>
+__global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
+  constexpr int WAVES = 8 / NB;                            // NB 16-column blocks of V per wavefront
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
+  using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
   const int n = blockIdx.x / p.HV;
   const int hv = blockIdx.x - n * p.HV;
   const int h = hv / (p.HV / p.H);
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillPara
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int vcol = 32 * wave + r16;                  // first of this lane's two V columns (second: +16)
+  const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the others: +16 each)
   const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
   if (c_begin >= c_end) return;
   const int seq_start = p.cu_seqlens[n];
@@ -330,11 +334,11 @@ __global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillPara
   __shared__ __align__(16) float tG[2][256];
 
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
-  f32x4_t St[2][8];
+  f32x4_t St[NB][8];
   {
     const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
       if (slot >= 0) {
         const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
@@ -402,16 +406,17 @@ __global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillPara
   constexpr int KT_O = CopyKt::EACH, KT_0 = CopyKt::FIRST;
   constexpr int P_O = CopyNarrow::EACH, P_0 = CopyNarrow::FIRST;
   // coalesced write of a finished output tile
+  constexpr int FLUSH_ROWS = 32 / NB;                       // rows covered by one pass of the workgroup
   const int krow = tid >> 4, kcv = tid & 15;
   uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
   auto flush_output = [&](int c) {
     const int len = chunk_len(c);
     uint16_t* dst = o_b + (int64_t)c * CHUNK * p.HV * 128;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (krow + 16 * i < len)
-        *reinterpret_cast<uint4*>(dst + (int64_t)16 * i * p.HV * 128) =
-            *reinterpret_cast<const uint4*>(&tO[(krow + 16 * i) * PITCH128 + 8 * kcv]);
+    for (int i = 0; i < CHUNK / FLUSH_ROWS; ++i)
+      if (krow + FLUSH_ROWS * i < len)
+        *reinterpret_cast<uint4*>(dst + (int64_t)FLUSH_ROWS * i * p.HV * 128) =
+            *reinterpret_cast<const uint4*>(&tO[(krow + FLUSH_ROWS * i) * PITCH128 + 8 * kcv]);
   };
 
   issue_gates(0);
@@ -423,135 +428,194 @@ __global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillPara
     const int par = ci & 1;
     const bool more = ci + 1 < n_chunks;
 
+    // Within a phase the LDS operands are requested ahead of the MFMAs that use them (scheduling
+    // fences keep that order), so a wavefront waits for LDS once per phase, not once per MFMA.
+
     // barrier 1: K, Q, V (and the decay factors) of this chunk; W and K^T were issued after them
     if (wave == 0) wait_vmcnt<W_0 + KT_0>(); else wait_vmcnt<W_O + KT_O>();
     __syncthreads();
+    bf16x8_t ka[2][4], qa[2][4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) {
+      ka[0][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], 0, kb);
+      qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (ci > 0) flush_output(ci - 1);
     issue_p(ci);
     if (more) issue_gates(ci + 1);
 
-    f32x4_t KS[2][4], QS[2][4];
+    f32x4_t KS[NB][4], QS[NB][4];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
+    float4 eg[4];
+    uint16_t vraw[NB][16];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const HiLo sb0 = split8(St[0][2 * s], St[0][2 * s + 1]);
-      const HiLo sb1 = split8(St[1][2 * s], St[1][2 * s + 1]);
+      if (s < 3) {
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t ka = operand_from(&tK[(16 * mi + r16) * PITCH128], s, kb);
-        const bf16x8_t qa = operand_from(&tQ[(16 * mi + r16) * PITCH128], s, kb);
-        KS[0][mi] = mfma16(ka, sb0.hi, KS[0][mi]);
-        KS[1][mi] = mfma16(ka, sb1.hi, KS[1][mi]);
-        QS[0][mi] = mfma16(qa, sb0.hi, QS[0][mi]);
-        QS[1][mi] = mfma16(qa, sb1.hi, QS[1][mi]);
-        KS[0][mi] = mfma16(ka, sb0.lo, KS[0][mi]);
-        KS[1][mi] = mfma16(ka, sb1.lo, KS[1][mi]);
+        for (int mi = 0; mi < 4; ++mi) {
+          ka[(s + 1) & 1][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], s + 1, kb);
+          qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
+        }
+      } else {
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+          eg[mi] = *reinterpret_cast<const float4*>(&tG[par][64 + 16 * mi + 4 * kb]);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+          }
+        }
       }
+      __builtin_amdgcn_sched_barrier(0);
+      HiLo sb[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[nb] = split8(St[nb][2 * s], St[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[nb].hi, KS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[nb].hi, QS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[nb].lo, KS[nb][mi]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - e^{G} (.) KS
-    f32x4_t X[2][4];
+    f32x4_t X[NB][4];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      const float4 eg = *reinterpret_cast<const float4*>(&tG[par][64 + 16 * mi + 4 * kb]);
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-        X[nb][mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[nb][mi][0];
-        X[nb][mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[nb][mi][1];
-        X[nb][mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[nb][mi][2];
-        X[nb][mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[nb][mi][3];
+      for (int mi = 0; mi < 4; ++mi) {
+        X[nb][mi][0] = to_float(act_t{vraw[nb][4 * mi + 0]}) - eg[mi].x * KS[nb][mi][0];
+        X[nb][mi][1] = to_float(act_t{vraw[nb][4 * mi + 1]}) - eg[mi].y * KS[nb][mi][1];
+        X[nb][mi][2] = to_float(act_t{vraw[nb][4 * mi + 2]}) - eg[mi].z * KS[nb][mi][2];
+        X[nb][mi][3] = to_float(act_t{vraw[nb][4 * mi + 3]}) - eg[mi].w * KS[nb][mi][3];
       }
-    }
 
     // barrier 2: W; K^T and P were issued after it
     if (wave == 0) wait_vmcnt<KT_0 + P_0>(); else wait_vmcnt<KT_O + P_O>();
     __syncthreads();
-    if (more) issue_kqv(ci + 1);
-    f32x4_t U[2][4];
+    bf16x8_t wh[2][4], wl[2][4];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        wh[s][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s, kb);
+        wl[s][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s, kb);
+      }
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) issue_kqv(ci + 1);
+    f32x4_t U[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const HiLo xb0 = split8(X[0][2 * s], X[0][2 * s + 1]);
-      const HiLo xb1 = split8(X[1][2 * s], X[1][2 * s + 1]);
+      HiLo xb[NB];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t wh = operand_from(&tWh[(16 * mi + r16) * PITCH64], s, kb);
-        const bf16x8_t wl = operand_from(&tWl[(16 * mi + r16) * PITCH64], s, kb);
-        U[0][mi] = mfma16(wh, xb0.hi, U[0][mi]);
-        U[1][mi] = mfma16(wh, xb1.hi, U[1][mi]);
-        U[0][mi] = mfma16(wl, xb0.hi, U[0][mi]);
-        U[1][mi] = mfma16(wl, xb1.hi, U[1][mi]);
-        U[0][mi] = mfma16(wh, xb0.lo, U[0][mi]);
-        U[1][mi] = mfma16(wh, xb1.lo, U[1][mi]);
-      }
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = split8(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].hi, U[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wl[s][mi], xb[nb].hi, U[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
     }
 
     // barrier 3: K^T; P and (unless this is the last chunk) the next K, Q, V were issued after it
     if (!more) { if (wave == 0) wait_vmcnt<P_0>(); else wait_vmcnt<P_O>(); }
     else if (wave == 0) wait_vmcnt<P_0 + KQV_0>(); else wait_vmcnt<P_O + KQV_O>();
     __syncthreads();
-    if (more) issue_w(ci + 1);
-    const float egl = tG[par][192];
+    bf16x8_t kt[2][8];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_from(&tKt[(16 * mc + r16) * PITCH64], s, kb);
+    float4 dg[2][2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      dg[s][0] = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 4 * kb]);
+      dg[s][1] = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 16 + 4 * kb]);
+    }
+    const float egl = tG[par][192];
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) issue_w(ci + 1);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const float4 d0 = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 4 * kb]);
-      const float4 d1 = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 16 + 4 * kb]);
-      HiLo ub[2];
+      HiLo ub[NB];
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        const f32x4_t u0 = {U[nb][2 * s][0] * d0.x, U[nb][2 * s][1] * d0.y, U[nb][2 * s][2] * d0.z, U[nb][2 * s][3] * d0.w};
-        const f32x4_t u1 = {U[nb][2 * s + 1][0] * d1.x, U[nb][2 * s + 1][1] * d1.y, U[nb][2 * s + 1][2] * d1.z,
-                            U[nb][2 * s + 1][3] * d1.w};
+      for (int nb = 0; nb < NB; ++nb) {
+        const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
+                            U[nb][2 * s][3] * dg[s][0].w};
+        const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
+                            U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
         ub[nb] = split8(u0, u1);
       }
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) {
-        const bf16x8_t ka = operand_from(&tKt[(16 * mc + r16) * PITCH64], s, kb);
-        St[0][mc] = mfma16(ka, ub[0].hi, St[0][mc]);
-        St[1][mc] = mfma16(ka, ub[1].hi, St[1][mc]);
-        St[0][mc] = mfma16(ka, ub[0].lo, St[0][mc]);
-        St[1][mc] = mfma16(ka, ub[1].lo, St[1][mc]);
-      }
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(kt[s][mc], ub[nb].hi, St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(kt[s][mc], ub[nb].lo, St[nb][mc]);
     }
 
     // barrier 4: P; the next K, Q, V and W were issued after it
     if (!more) wait_vmcnt<0>();
     else if (wave == 0) wait_vmcnt<KQV_0 + W_0>(); else wait_vmcnt<KQV_O + W_O>();
     __syncthreads();
+    bf16x8_t pa[2][4];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) pa[s][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s, kb);
+    float4 sq[4];
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
+    __builtin_amdgcn_sched_barrier(0);
     if (more) issue_kt(ci + 1);
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      const float4 sq = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
+    for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
-        QS[nb][mi][0] *= sq.x; QS[nb][mi][1] *= sq.y; QS[nb][mi][2] *= sq.z; QS[nb][mi][3] *= sq.w;
+      for (int nb = 0; nb < NB; ++nb) {
+        QS[nb][mi][0] *= sq[mi].x; QS[nb][mi][1] *= sq[mi].y; QS[nb][mi][2] *= sq[mi].z; QS[nb][mi][3] *= sq[mi].w;
       }
-    }
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const bf16x8_t ur0 = round8(U[0][2 * s], U[0][2 * s + 1]);
-      const bf16x8_t ur1 = round8(U[1][2 * s], U[1][2 * s + 1]);
+      bf16x8_t ur[NB];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t pa = operand_from(&tP[(16 * mi + r16) * PITCH64], s, kb);
-        QS[0][mi] = mfma16(pa, ur0, QS[0][mi]);
-        QS[1][mi] = mfma16(pa, ur1, QS[1][mi]);
-      }
+      for (int nb = 0; nb < NB; ++nb) ur[nb] = round8(U[nb][2 * s], U[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(pa[s][mi], ur[nb], QS[nb][mi]);
     }
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
+      for (int nb = 0; nb < NB; ++nb) {
         uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
         orow[0] = from_float<act_t>(QS[nb][mi][0]).bits;
         orow[PITCH128] = from_float<act_t>(QS[nb][mi][1]).bits;
@@ -566,7 +630,7 @@ __global__ __launch_bounds__(256) void gdn_chunk_seq_kernel(const GdnPrefillPara
     const int slot = p.ht_indices ? p.ht_indices[n] : n;
     if (slot >= 0) {
 #pragma unroll
-      for (int nb = 0; nb < 2; ++nb) {
+      for (int nb = 0; nb < NB; ++nb) {
         float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
         for (int mc = 0; mc < 8; ++mc)
@@ -670,6 +734,6 @@ extern "C" int pla_gdn_prefill_launch(
     hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   }
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
-  hipLaunchKernelGGL(gdn_chunk_seq_kernel<bf16_t>, dim3((unsigned)N * HV), dim3(256), 0, s, p);
+  hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
   return check_launch("gdn prefill launch");
 }
