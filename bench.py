@@ -80,6 +80,7 @@ def bench_decode(steps, warmup, device):
 
 PREFILL_SEED = 348      # ragged_lengths(8, 512, 8192, 348) sums to 32 810 tokens
 GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64, K = V = 128, HV = 32, H = 16
+KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
 
 
 def bench_prefill(steps, warmup, device):
@@ -114,6 +115,48 @@ def bench_prefill(steps, warmup, device):
                               flop_per_token=GDN_FLOP_PER_TOKEN,
                               note="algorithmic flops (dense, no hi/lo passes) over the whole call: "
                                    "chunk map + prep + gram/solve + sequential kernels"))
+
+
+def bench_prefill_kda(steps, device):
+    """Config 4: KDA chunk-64 prefill of one 65 536-token sequence, 32 heads (32 independent chains)."""
+    import torch
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    from pla_amd.workloads import kda_prefill
+    T = 65536
+    c = {k: v for k, v in kda_prefill(T=T, H=32, seed=4, device=device).items() if not k.startswith("_")}
+
+    def run():
+        flashkda_fwd(c["q"], c["k"], c["v"], c["g"], c["beta"], c["A_log"], c["dt_bias"], c["out"], scale=c["scale"],
+                     lower_bound=c["lower_bound"], initial_state=c["initial_state"], final_state=c["final_state"],
+                     cu_seqlens=c["cu_seqlens"])
+
+    for _ in range(2):
+        run()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / steps
+    tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
+    return dict(tokens=T, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
+                roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
+                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=None,
+                              flop_per_token=KDA_FLOP_PER_TOKEN))
+
+
+def copy_calibration(device, reps=5):
+    """A plain device-to-device copy of known size (1 GiB read + 1 GiB written per launch): the
+    reference point that scales the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run."""
+    import torch
+    src = torch.empty(1 << 28, dtype=torch.float32, device=device).normal_()
+    dst = torch.empty_like(src)
+    for _ in range(reps):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    return dict(bytes_read=src.numel() * 4, bytes_written=src.numel() * 4, launches=reps)
 
 
 def bench_small_decode(device, steps=200):
@@ -187,6 +230,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-only", action="store_true", help="skip the secondary decode / prefill measurements")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch a 1 GiB device copy (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the decode and prefill "
@@ -224,6 +269,10 @@ def main():
     if not args.decode_only:
         result["other_decode"] = bench_small_decode(device)
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
+        torch.cuda.empty_cache()
+        result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+    if args.copy_calibration:
+        result["copy_calibration"] = copy_calibration(device)
     print(json.dumps(result))
 
 

@@ -183,3 +183,45 @@ def test_config4_kda_prefill_strong_and_weak_decay_prefix():
     torch.testing.assert_close(call["out"].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
     for head in range(8):
         assert rel_l2(call["final_state"][0, head], exp_final[0, head]) <= 1e-3, head
+
+
+def test_config4_kda_prefill_full_size():
+    """Config 4 at its full size (one sequence of 65536 tokens, 32 heads).  Three heads (strong
+    decay, first weak-decay head, last head) are checked against the float64 chunked oracle over
+    the whole sequence; every head is checked through the chained-calls invariant: two calls
+    that split the sequence at a chunk boundary and pass the state on give bit-identical o and
+    final state."""
+    from pla_amd.workloads import kda_prefill
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    T, H = 65536, 32
+    w = kda_prefill(T=T, H=H, seed=4)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+
+    def run(lo, hi, init, out, final):
+        cu = torch.tensor([0, hi - lo], dtype=torch.int32, device="cuda")
+        flashkda_fwd(call["q"][lo:hi], call["k"][lo:hi], call["v"][lo:hi], call["g"][lo:hi], call["beta"][lo:hi],
+                     call["A_log"], call["dt_bias"], out, scale=call["scale"], lower_bound=call["lower_bound"],
+                     initial_state=init, final_state=final, cu_seqlens=cu)
+
+    run(0, T, call["initial_state"], call["out"], call["final_state"])
+    torch.cuda.synchronize()
+    assert torch.isfinite(call["out"].float()).all() and torch.isfinite(call["final_state"]).all()
+
+    split = 40 * 64 * 16                                    # chunk-aligned, not the middle
+    o2 = torch.empty_like(call["out"])
+    mid = torch.empty_like(call["final_state"])
+    fin = torch.empty_like(call["final_state"])
+    run(0, split, call["initial_state"], o2[:split], mid)
+    run(split, T, mid, o2[split:], fin)
+    torch.cuda.synchronize()
+    assert torch.equal(o2, call["out"])
+    assert torch.equal(fin, call["final_state"])
+
+    heads = [0, H // 2, H - 1]
+    cpu = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in call.items()}
+    sel = lambda t: t[:, heads].contiguous()
+    exp_o, exp_final = _oracle(sel(cpu["q"]), sel(cpu["k"]), sel(cpu["v"]), sel(cpu["g"]), sel(cpu["beta"]),
+                               cpu["A_log"][heads], cpu["dt_bias"][heads], [0, T], cpu["initial_state"][:, heads], fast=True)
+    torch.testing.assert_close(call["out"][:, heads].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
+    for i, head in enumerate(heads):
+        assert rel_l2(call["final_state"][0, head], exp_final[0, i]) <= 1e-3, head
