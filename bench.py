@@ -22,6 +22,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per launch of the headline decode kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, then
+# WRITE_SIZE, KiB per dispatch) scaled by the same counters of a 1 GiB device copy (x2.00 and x1.00);
+# the runs and figures are in profiles/k_last_decode_kernel_gdn_b256.txt.
+DECODE_TRAFFIC_BYTES_PER_LAUNCH = 1027728285
 BF16_PEAK_TFLOPS = 2500.0
 
 
@@ -258,7 +262,8 @@ def main():
                    "slot_rotation": "16 disjoint slot sets, one per consecutive step"},
         "decode_us_per_step": round(d["kernel_us_avg"], 2),
         "roofline": {"bound": "hbm", "achieved": round(d["achieved_gbps"], 1), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(d["achieved_gbps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "unit": "GB/s", "frac": round(d["achieved_gbps"] / HBM_PEAK_GBPS, 4),
+                     "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
                      "kernel": "k_last_decode_kernel<bf16,GDN,rows_per_wave=32>",
                      "bytes_per_launch": d["bytes_state"], "launch_us_avg": round(d["kernel_us_avg"], 2)},
     }
