@@ -45,13 +45,22 @@ struct KdaPrefillParams {
   int H, NC_max;
 };
 
+// 69 KB, so that two workgroups share a CU.  L takes over Qn's storage once every wavefront has
+// formed its q operands (a barrier in phase 3 separates the two uses).
 struct __align__(16) KdaPrepShared {
   float G[CHUNK][132];
-  float L[CHUNK][68];
   uint16_t Kn[CHUNK][PITCH128];
-  uint16_t Qn[CHUNK][PITCH128];
+  union {
+    uint16_t Qn[CHUNK][PITCH128];
+    float L[CHUNK][68];
+  };
   float B[CHUNK];
 };
+static_assert(sizeof(float[CHUNK][68]) <= sizeof(uint16_t[CHUNK][PITCH128]), "L must fit into Qn's storage");
+
+// Column j of L is stored at slot 16 (j % 4) + 4 (j / 16) + (j / 4) % 4, which makes the columns
+// l = 16 m + 4 e + p (e = 0..3) of one lane part p contiguous for the quad-split forward substitution.
+__device__ __forceinline__ int solve_slot(int j) { return 16 * (j & 3) + 4 * (j >> 4) + ((j >> 2) & 3); }
 
 // Eight decayed elements of a bf16 row: x[c] * exp(sign * (G[c] - R[c])) for the lane's two
 // channel quads of contraction step s.
@@ -81,6 +90,9 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   __shared__ KdaPrepShared sh;
   const int64_t tile = (int64_t)cb * p.H + h;
 
+#ifdef PLA_PROF
+  long long tk[6]; tk[0] = clock64();
+#endif
   // ---- phase 1: normalised q / k, per-channel log-decay, beta ---------------------------------
   {
     uint32_t qw[16], kw[16];
@@ -101,15 +113,30 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       *reinterpret_cast<uint32_t*>(&sh.Qn[j][2 * lane]) = ok ? pack2<bf16_t>(q0 * qi, q1 * qi) : 0u;
       *reinterpret_cast<uint32_t*>(&sh.Kn[j][2 * lane]) = ok ? pack2<bf16_t>(k0 * ki, k1 * ki) : 0u;
     }
+    // gate: thread handles eight channels of rows tid / 16 + 16 u; all four 16-byte loads are in flight at once
     const float eA = expf(p.A_log[h]);
-    for (int idx = tid; idx < CHUNK * 128; idx += 256) {
-      const int j = idx >> 7, c = idx & 127;
-      float g = 0.f;
-      if (j < len) {
-        const float raw = to_float(reinterpret_cast<const bf16_t*>(p.g)[(int64_t)(t0 + j) * p.stride_g + h * 128 + c]);
-        g = p.lower_bound / (1.0f + expf(-eA * (raw + p.dt_bias[h * 128 + c])));
+    const int gc0 = 8 * (tid & 15);
+    uint4 graw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = (tid >> 4) + 16 * u;
+      graw[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.g) +
+                                                (int64_t)(t0 + (j < len ? j : 0)) * p.stride_g + h * 128 + gc0);
+    }
+    float dtb[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dtb[e] = p.dt_bias[h * 128 + gc0 + e];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = (tid >> 4) + 16 * u;
+      const uint32_t w[4] = {graw[u].x, graw[u].y, graw[u].z, graw[u].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float g0 = p.lower_bound * fast_rcp(1.0f + __expf(-eA * (lo16<bf16_t>(w[e]) + dtb[2 * e])));
+        const float g1 = p.lower_bound * fast_rcp(1.0f + __expf(-eA * (hi16<bf16_t>(w[e]) + dtb[2 * e + 1])));
+        sh.G[j][gc0 + 2 * e] = j < len ? g0 : 0.f;
+        sh.G[j][gc0 + 2 * e + 1] = j < len ? g1 : 0.f;
       }
-      sh.G[j][c] = g;
     }
     if (tid < CHUNK) {
       float bt = 0.f;
@@ -121,16 +148,22 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
     }
   }
   __syncthreads();
+#ifdef PLA_PROF
+  tk[1] = clock64();
+#endif
   if (tid < 128) {
     float cum = 0.f;
     for (int j = 0; j < CHUNK; ++j) {
       cum += sh.G[j][tid];
       sh.G[j][tid] = cum;                 // rows beyond the chunk repeat G_last (their g is zero)
     }
-    p.eGlast[tile * 128 + tid] = expf(cum);
+    p.eGlast[tile * 128 + tid] = __expf(cum);
   }
   __syncthreads();
 
+#ifdef PLA_PROF
+  tk[2] = clock64();
+#endif
   // ---- phase 2: decayed operand tiles for the sequential kernel -------------------------------
   {
     // row-major tiles: thread handles row j, eight channels, twice
@@ -144,7 +177,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       uint32_t khi[4], klo[4], qh[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float e0 = expf(sh.G[j][c0 + 2 * e]), e1 = expf(sh.G[j][c0 + 2 * e + 1]);
+        const float e0 = __expf(sh.G[j][c0 + 2 * e]), e1 = __expf(sh.G[j][c0 + 2 * e + 1]);
         const float a0 = lo16<bf16_t>(kwv[e]) * e0, a1 = hi16<bf16_t>(kwv[e]) * e1;
         khi[e] = pack2<bf16_t>(a0, a1);
         klo[e] = pack2<bf16_t>(a0 - lo16<bf16_t>(khi[e]), a1 - hi16<bf16_t>(khi[e]));
@@ -162,8 +195,8 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #pragma unroll
     for (int jj = 0; jj < 16; ++jj) {
       const int j0 = 32 * half + 2 * jj;
-      const float a0 = to_float(bf16_t{sh.Kn[j0][c]}) * expf(gl - sh.G[j0][c]);
-      const float a1 = to_float(bf16_t{sh.Kn[j0 + 1][c]}) * expf(gl - sh.G[j0 + 1][c]);
+      const float a0 = to_float(bf16_t{sh.Kn[j0][c]}) * __expf(gl - sh.G[j0][c]);
+      const float a1 = to_float(bf16_t{sh.Kn[j0 + 1][c]}) * __expf(gl - sh.G[j0 + 1][c]);
       th[jj] = pack2<bf16_t>(a0, a1);
       tl[jj] = pack2<bf16_t>(a0 - lo16<bf16_t>(th[jj]), a1 - hi16<bf16_t>(th[jj]));
     }
@@ -175,6 +208,9 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
     }
   }
 
+#ifdef PLA_PROF
+  tk[3] = clock64();
+#endif
   // ---- phase 3: M and P, wavefront w owns row block w (reference row = first row of the block) --
   {
     const int bi = wave;
@@ -190,6 +226,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       decayed8(&sh.Qn[i_row][0], &sh.G[i_row][0], R, 1.0f, s, kb, a, b);
       Ql[s] = round8(a, b);
     }
+    __syncthreads();                     // Qn is dead from here on: L reuses its storage
     uint16_t* const Pt = p.P + tile * 4096;
     for (int bj = 0; bj < 4; ++bj) {
       const int j = 16 * bj + r16;
@@ -212,39 +249,70 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * bi + 4 * kb + r;
-        sh.L[i][j] = i > j ? sh.B[i] * m[r] : 0.f;
+        sh.L[i][solve_slot(j)] = i > j ? sh.B[i] * m[r] : 0.f;
         Pt[i * 64 + j] = from_float<bf16_t>(i >= j ? p.scale * pq[r] : 0.f).bits;
       }
     }
   }
   __syncthreads();
 
-  // ---- phase 4: W = L^-1 diag(beta), one column per lane of wavefront 0 -----------------------
-  if (wave == 0) {
-    float x[CHUNK];
-    const float bj = sh.B[lane];
+#ifdef PLA_PROF
+  tk[4] = clock64();
+#endif
+  // ---- phase 4: W = L^-1 diag(beta) by forward substitution ------------------------------------
+  // Wavefront w owns columns 16 w .. 16 w + 15; the four lanes of a quad share one column and split
+  // each row's dot product by l mod 4 (lane part p keeps x_l for l = 16 m + 4 e + p in xs[4 m + e],
+  // and L is stored with those columns contiguous), so a row costs ceil(i / 16) float4 reads and
+  // 4 ceil(i / 16) FMAs per lane plus a two-step quad reduction.
+  {
+    const int col = 16 * wave + (lane >> 2), part = lane & 3;
+    const float bcol = sh.B[col];
+    float xs[16];
+#pragma unroll
+    for (int t = 0; t < 16; ++t) xs[t] = 0.f;
+    // the L values of row i + 2 are requested while row i is reduced: they do not depend on x
+    float4 ahead[2][4];
+#pragma unroll
+    for (int i = 1; i < 3; ++i) ahead[i & 1][0] = *reinterpret_cast<const float4*>(&sh.L[i][16 * part]);
 #pragma unroll
     for (int i = 0; i < CHUNK; ++i) {
-      float a0 = (i == lane) ? bj : 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+      float4 row[4];
 #pragma unroll
-      for (int l4 = 0; l4 < i; l4 += 4) {
-        const float4 row = *reinterpret_cast<const float4*>(&sh.L[i][l4]);
-        a0 = fmaf(-row.x, x[l4], a0);
-        if (l4 + 1 < i) a1 = fmaf(-row.y, x[l4 + 1], a1);
-        if (l4 + 2 < i) a2 = fmaf(-row.z, x[l4 + 2], a2);
-        if (l4 + 3 < i) a3 = fmaf(-row.w, x[l4 + 3], a3);
+      for (int m = 0; 16 * m < i; ++m) row[m] = ahead[i & 1][m];
+      if (i + 2 < CHUNK) {
+#pragma unroll
+        for (int m = 0; 16 * m < i + 2; ++m)
+          ahead[i & 1][m] = *reinterpret_cast<const float4*>(&sh.L[i + 2][16 * part + 4 * m]);
       }
-      x[i] = (a0 + a1) + (a2 + a3);
-    }
-    uint16_t* const Wh = p.Whi + tile * 4096;
-    uint16_t* const Wl = p.Wlo + tile * 4096;
+      float acc = 0.f, acc2 = 0.f;
 #pragma unroll
-    for (int i = 0; i < CHUNK; ++i) {
-      const bf16_t hi = from_float<bf16_t>(x[i]);
-      Wh[i * 64 + lane] = hi.bits;
-      Wl[i * 64 + lane] = from_float<bf16_t>(x[i] - to_float(hi)).bits;
+      for (int m = 0; 16 * m < i; ++m) {
+        acc = fmaf(row[m].x, xs[4 * m + 0], acc);
+        acc2 = fmaf(row[m].y, xs[4 * m + 1], acc2);
+        acc = fmaf(row[m].z, xs[4 * m + 2], acc);
+        acc2 = fmaf(row[m].w, xs[4 * m + 3], acc2);
+      }
+      acc += acc2;
+      acc += dpp_mov<0xB1>(acc);    // quad_perm [1,0,3,2]
+      acc += dpp_mov<0x4E>(acc);    // quad_perm [2,3,0,1]
+      const float xi = (i == col ? bcol : 0.f) - acc;
+      if (part == (i & 3)) xs[4 * (i >> 4) + ((i & 15) >> 2)] = xi;
+    }
+    uint16_t* const Wh = p.Whi + tile * 4096 + col;
+    uint16_t* const Wl = p.Wlo + tile * 4096 + col;
+#pragma unroll
+    for (int t = 0; t < 16; ++t) {
+      const int l = 16 * (t >> 2) + 4 * (t & 3) + part;
+      const bf16_t hi = from_float<bf16_t>(xs[t]);
+      Wh[l * 64] = hi.bits;
+      Wl[l * 64] = from_float<bf16_t>(xs[t] - to_float(hi)).bits;
     }
   }
+#ifdef PLA_PROF
+  tk[5] = clock64();
+  if (blockIdx.x == 100 && blockIdx.y == 3 && lane == 0)
+    printf("prep wave %d: p1 %lld cumsum %lld p2 %lld p3 %lld p4 %lld\n", wave, tk[1] - tk[0], tk[2] - tk[1], tk[3] - tk[2], tk[4] - tk[3], tk[5] - tk[4]);
+#endif
 }
 
 // ---------------------------------------------------------------------------------------------
