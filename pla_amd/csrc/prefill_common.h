@@ -143,6 +143,126 @@ static __global__ void chunk_map_kernel(const int32_t* cu_seqlens, int N, int NC
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Splitting long sequences into segments, for calls with too few (sequence, head) chains to fill the
+// chip.  The per-token recurrence is affine in the state, S_out = S_in M + B, where for one segment
+// B is the state the segment produces from a zero state and M (K x K) is what it produces from the
+// identity with all values v = 0 (rows of the k-last state transform independently).  So:
+//   pass 1   every segment after the first of its sequence runs twice, from zero (-> B) and from the
+//            identity with v = 0 (-> M), without writing o; first segments run normally
+//   combine  per (sequence, head): S_in of every later segment, S <- S M + B in FP32, final state
+//   pass 2   the later segments run again from their true S_in and write o
+// which costs three sweeps over a later segment instead of one but runs them all concurrently.
+struct SegmentTable {
+  int32_t* seq_seg_off;   // [N + 1] first segment of each sequence
+  int32_t* seg_seq;       // [segments] sequence of a segment
+  int32_t* seg_c0;        // first chunk (global chunk index)
+  int32_t* seg_nc;        // number of chunks
+  float* M;               // [segment, head, 128, 128] transition matrices
+  float* B;               // [segment, head, V, K] zero-state results (first segments: the state they end in)
+  float* S;               // [segment, head, V, K] state entering the segment
+  float* identity;        // [128, 128]
+  int seg_chunks;         // chunks per segment (0: sequences are not split)
+  int max_segments;
+};
+
+// Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map_kernel.
+static __global__ void segment_map_kernel(const int32_t* seq_chunk_off, int N, SegmentTable t) {
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int n = 0; n < N; ++n) {
+      t.seq_seg_off[n] = acc;
+      const int nc = seq_chunk_off[n + 1] - seq_chunk_off[n];
+      acc += (nc + t.seg_chunks - 1) / t.seg_chunks;
+    }
+    t.seq_seg_off[N] = acc;
+  }
+  for (int i = threadIdx.x; i < 128 * 128; i += blockDim.x) t.identity[i] = (i >> 7) == (i & 127) ? 1.f : 0.f;
+  __syncthreads();
+  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+    const int c0 = seq_chunk_off[n], nc = seq_chunk_off[n + 1] - c0, s0 = t.seq_seg_off[n];
+    const int ns = (nc + t.seg_chunks - 1) / t.seg_chunks;
+    for (int i = 0; i < ns; ++i) {
+      if (s0 + i >= t.max_segments) break;
+      t.seg_seq[s0 + i] = n;
+      t.seg_c0[s0 + i] = c0 + i * t.seg_chunks;
+      t.seg_nc[s0 + i] = min(t.seg_chunks, nc - i * t.seg_chunks);
+    }
+  }
+}
+
+// One workgroup of 256 threads per (sequence, head): walks the sequence's segments, stores the state
+// entering each later segment and the final state.  Thread (tv, tk) owns the 8 x 8 block of S at rows
+// 8 tv, columns 8 tk; S lives in LDS between steps, M and B are streamed from global memory.
+static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads, float* ht,
+                                                                     const int32_t* ht_indices, int64_t ht_slot_stride) {
+  const int n = blockIdx.x / heads, h = blockIdx.x - n * heads;
+  const int first = t.seq_seg_off[n], end = t.seq_seg_off[n + 1];
+  if (end - first < 2) return;                 // a single segment wrote its final state itself
+  __shared__ float S[128][129];
+  const int tv = threadIdx.x >> 4, tk = threadIdx.x & 15;
+  float acc[8][8];
+  {
+    const float* src = t.B + ((int64_t)first * heads + h) * 16384;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc[r][c] = src[(8 * tv + r) * 128 + 8 * tk + c];
+  }
+  for (int seg = first + 1; seg < end; ++seg) {
+    const int64_t tile = ((int64_t)seg * heads + h) * 16384;
+    float* sin = t.S + tile;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c) S[8 * tv + r][8 * tk + c] = acc[r][c];
+      *reinterpret_cast<float4*>(sin + (8 * tv + r) * 128 + 8 * tk) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+      *reinterpret_cast<float4*>(sin + (8 * tv + r) * 128 + 8 * tk + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
+    }
+    __syncthreads();
+    const float* Mt = t.M + tile;
+    const float* Bt = t.B + tile;
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc[r][c] = Bt[(8 * tv + r) * 128 + 8 * tk + c];
+    for (int j = 0; j < 128; ++j) {
+      const float4 m0 = *reinterpret_cast<const float4*>(Mt + j * 128 + 8 * tk);
+      const float4 m1 = *reinterpret_cast<const float4*>(Mt + j * 128 + 8 * tk + 4);
+      const float mrow[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        const float sv = S[8 * tv + r][j];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[r][c] = fmaf(sv, mrow[c], acc[r][c]);
+      }
+    }
+    __syncthreads();
+  }
+  if (ht != nullptr) {
+    const int slot = ht_indices ? ht_indices[n] : n;
+    if (slot >= 0) {
+      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384;
+#pragma unroll
+      for (int r = 0; r < 8; ++r) {
+        *reinterpret_cast<float4*>(dst + (8 * tv + r) * 128 + 8 * tk) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+        *reinterpret_cast<float4*>(dst + (8 * tv + r) * 128 + 8 * tk + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
+      }
+    }
+  }
+}
+
+// Chunks per segment for a call of T tokens, N sequences and `heads` value heads: 0 (no split) unless
+// the call has at most 64 chains and the segments would be at least 16 chunks long and at least two.
+inline int pick_segment_chunks(int T, int N, int heads) {
+  if ((int64_t)N * heads > 64) return 0;
+  const int nc = T / CHUNK;
+  int seg = (int)(((int64_t)nc * heads + 255) / 256);
+  if (seg < 16) seg = 16;
+  return 2 * seg > nc ? 0 : seg;
+}
+inline int max_segments(int T, int N, int seg_chunks) { return seg_chunks > 0 ? T / CHUNK / seg_chunks + N + 1 : 0; }
+
 // Zero the rows of a dense [T, heads, 128] 16-bit output that lie beyond the last sequence.
 static __global__ void zero_tail_kernel(uint16_t* o, const int32_t* cu_seqlens, int N, int T, int heads) {
   const int64_t first = (int64_t)cu_seqlens[N] * heads * 128;

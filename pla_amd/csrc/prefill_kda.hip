@@ -42,6 +42,8 @@ struct KdaPrefillParams {
   uint16_t* KtH; uint16_t* KtL;                    // [chunk, H, 128, 64]: (k e^{G_last - G})^T (hi, lo)
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;       // [chunk, H, 64, 64]
   float* eGlast;                                   // [chunk, H, 128]: e^{G_last}
+  SegmentTable seg;                                // split long sequences (seg.seg_chunks > 0)
+  int pass;                                        // 0: whole sequences; 1, 2: the two sweeps over segments
   int H, NC_max;
 };
 
@@ -330,24 +332,68 @@ struct __align__(16) KdaSeqTiles {
 };
 
 __global__ __launch_bounds__(512) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
-  const int n = blockIdx.x / p.H;
-  const int h = blockIdx.x - n * p.H;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int r16 = lane & 15, kb = lane >> 4;
   const int vcol = 16 * wave + r16;
-  const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
-  if (c_begin >= c_end) return;
-  const int seq_start = p.cu_seqlens[n];
-  const int seq_len = p.cu_seqlens[n + 1] - seq_start;
+
+  // What this workgroup sweeps: a whole sequence, or one segment of it in one of three roles.
+  int n, h, c_begin, c_end;
+  const float* init = nullptr;        // [V, K] tile the state starts from (nullptr: zero)
+  float* fin = nullptr;               // [V, K] tile that receives the state at the end (nullptr: none)
+  bool zero_v = false, write_o = true;
+  if (p.pass == 0) {
+    n = blockIdx.x / p.H;
+    h = blockIdx.x - n * p.H;
+    c_begin = p.seq_chunk_off[n];
+    c_end = p.seq_chunk_off[n + 1];
+    if (c_begin >= c_end) return;
+    const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
+    if (slot >= 0) init = p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)h * 16384;
+    const int oslot = (p.ht != nullptr) ? (p.ht_indices ? p.ht_indices[n] : n) : -1;
+    if (oslot >= 0) fin = p.ht + (int64_t)oslot * p.ht_slot_stride + (int64_t)h * 16384;
+  } else {
+    const int item = p.pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+    const int from_identity = p.pass == 1 ? (int)(blockIdx.x & 1) : 0;
+    const int seg = item / p.H;
+    h = item - seg * p.H;
+    if (seg >= p.seg.seq_seg_off[p.N]) return;
+    n = p.seg.seg_seq[seg];
+    const bool first = seg == p.seg.seq_seg_off[n], last = seg + 1 == p.seg.seq_seg_off[n + 1];
+    c_begin = p.seg.seg_c0[seg];
+    c_end = c_begin + p.seg.seg_nc[seg];
+    const int64_t tile = ((int64_t)seg * p.H + h) * 16384;
+    if (p.pass == 1) {
+      if (first) {
+        if (from_identity) return;
+        const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
+        if (slot >= 0) init = p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)h * 16384;
+        if (!last) {
+          fin = p.seg.B + tile;                       // the state that enters the second segment
+        } else {
+          const int oslot = (p.ht != nullptr) ? (p.ht_indices ? p.ht_indices[n] : n) : -1;
+          if (oslot >= 0) fin = p.ht + (int64_t)oslot * p.ht_slot_stride + (int64_t)h * 16384;
+        }
+      } else {
+        write_o = false;
+        if (from_identity) { init = p.seg.identity; zero_v = true; fin = p.seg.M + tile; }
+        else fin = p.seg.B + tile;
+      }
+    } else {
+      if (first) return;
+      init = p.seg.S + tile;                          // the final state came out of the combine step
+    }
+  }
+  const int chunk_in_seq = c_begin - p.seq_chunk_off[n];
+  const int seq_start = p.cu_seqlens[n] + chunk_in_seq * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
 
   __shared__ KdaSeqTiles T;
 
   f32x4_t St[8];
   {
-    const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
-    if (slot >= 0) {
-      const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)h * 128 + vcol) * 128 + 4 * kb;
+    if (init != nullptr) {
+      const float* src = init + (int64_t)vcol * 128 + 4 * kb;
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
         const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
@@ -391,11 +437,12 @@ __global__ __launch_bounds__(512) void kda_chunk_seq_kernel(const KdaPrefillPara
     const int64_t back0 = ok0 ? 0 : -(int64_t)krow, back1 = ok1 ? 32 : -(int64_t)krow;
     pv0 = *reinterpret_cast<const uint4*>(vptr + back0 * p.stride_v);
     pv1 = *reinterpret_cast<const uint4*>(vptr + back1 * p.stride_v);
-    if (!ok0) pv0 = zero4;
-    if (!ok1) pv1 = zero4;
+    if (!ok0 || zero_v) pv0 = zero4;
+    if (!ok1 || zero_v) pv1 = zero4;
     big += tile_stride; small += small_stride; vptr += CHUNK * p.stride_v;
   };
   auto flush_output = [&](int len) {
+    if (!write_o) return;
     if (krow < len) *reinterpret_cast<uint4*>(optr) = *reinterpret_cast<const uint4*>(&T.V[krow][8 * kcv]);
     if (krow + 32 < len) *reinterpret_cast<uint4*>(optr + o_half) = *reinterpret_cast<const uint4*>(&T.V[krow + 32][8 * kcv]);
     optr += (int64_t)CHUNK * p.H * 128;
@@ -515,20 +562,18 @@ __global__ __launch_bounds__(512) void kda_chunk_seq_kernel(const KdaPrefillPara
   __syncthreads();
   flush_output(prev_len);
 
-  if (p.ht != nullptr) {
-    const int slot = p.ht_indices ? p.ht_indices[n] : n;
-    if (slot >= 0) {
-      float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)h * 128 + vcol) * 128 + 4 * kb;
+  if (fin != nullptr) {
+    float* dst = fin + (int64_t)vcol * 128 + 4 * kb;
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[mc].x, St[mc].y, St[mc].z, St[mc].w);
-    }
+    for (int mc = 0; mc < 8; ++mc)
+      *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[mc].x, St[mc].y, St[mc].z, St[mc].w);
   }
 }
 
 struct KdaWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Khi, Klo, Qh, KtH, KtL, Whi, Wlo, P, eGlast, total;
-  int NC_max;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Khi, Klo, Qh, KtH, KtL, Whi, Wlo, P, eGlast;
+  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity, total;
+  int NC_max, seg_chunks, max_segments;
 };
 static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   KdaWorkspaceLayout L;
@@ -543,6 +588,17 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   L.Khi = take(big); L.Klo = take(big); L.Qh = take(big); L.KtH = take(big); L.KtL = take(big);
   L.Whi = take(small); L.Wlo = take(small); L.P = take(small);
   L.eGlast = take((size_t)L.NC_max * H * 128 * 4);
+  L.seg_chunks = pick_segment_chunks(T, N, H);
+  L.max_segments = max_segments(T, N, L.seg_chunks);
+  if (L.seg_chunks > 0) {
+    L.seq_seg_off = take((size_t)(N + 1) * 4);
+    L.seg_seq = take((size_t)L.max_segments * 4);
+    L.seg_c0 = take((size_t)L.max_segments * 4);
+    L.seg_nc = take((size_t)L.max_segments * 4);
+    const size_t states = (size_t)L.max_segments * H * 16384 * 4;
+    L.segM = take(states); L.segB = take(states); L.segS = take(states);
+    L.identity = take(16384 * 4);
+  }
   L.total = off;
   return L;
 }
@@ -606,6 +662,27 @@ extern "C" int pla_kda_prefill_launch(
                      p.chunk_seq, p.chunk_tok, p.chunk_len);
   hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, H);
   hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, s, p);
-  hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)N * H), dim3(512), 0, s, p);
+  if (L.seg_chunks == 0) {
+    p.pass = 0;
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)N * H), dim3(512), 0, s, p);
+  } else {
+    // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
+    p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
+    p.seg.seg_seq = reinterpret_cast<int32_t*>(ws + L.seg_seq);
+    p.seg.seg_c0 = reinterpret_cast<int32_t*>(ws + L.seg_c0);
+    p.seg.seg_nc = reinterpret_cast<int32_t*>(ws + L.seg_nc);
+    p.seg.M = reinterpret_cast<float*>(ws + L.segM);
+    p.seg.B = reinterpret_cast<float*>(ws + L.segB);
+    p.seg.S = reinterpret_cast<float*>(ws + L.segS);
+    p.seg.identity = reinterpret_cast<float*>(ws + L.identity);
+    p.seg.seg_chunks = L.seg_chunks;
+    p.seg.max_segments = L.max_segments;
+    hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
+    p.pass = 1;
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H * 2), dim3(512), 0, s, p);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H), dim3(256), 0, s, p.seg, H, ht, ht_indices, ht_slot_stride);
+    p.pass = 2;
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(512), 0, s, p);
+  }
   return check_launch("kda prefill launch");
 }

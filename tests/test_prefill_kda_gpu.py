@@ -189,8 +189,8 @@ def test_config4_kda_prefill_full_size():
     """Config 4 at its full size (one sequence of 65536 tokens, 32 heads).  Three heads (strong
     decay, first weak-decay head, last head) are checked against the float64 chunked oracle over
     the whole sequence; every head is checked through the chained-calls invariant: two calls
-    that split the sequence at a chunk boundary and pass the state on give bit-identical o and
-    final state."""
+    that split the sequence at a chunk boundary and pass the state on give the same o and final
+    state."""
     from pla_amd.workloads import kda_prefill
     from pla_amd.prefill.flashkdapro import flashkda_fwd
     T, H = 65536, 32
@@ -214,8 +214,12 @@ def test_config4_kda_prefill_full_size():
     run(0, split, call["initial_state"], o2[:split], mid)
     run(split, T, mid, o2[split:], fin)
     torch.cuda.synchronize()
-    assert torch.equal(o2, call["out"])
-    assert torch.equal(fin, call["final_state"])
+    # A call with this few chains splits the sequence into concurrently swept segments, and the two
+    # shorter calls split differently, so the results agree to rounding rather than bit for bit.
+    torch.testing.assert_close(o2.float(), call["out"].float(), atol=2e-2, rtol=2e-2)
+    assert (o2 != call["out"]).float().mean().item() < 0.05
+    for head in range(H):
+        assert rel_l2(fin[0, head], call["final_state"][0, head]) <= 1e-4, head
 
     heads = [0, H // 2, H - 1]
     cpu = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in call.items()}
@@ -225,3 +229,34 @@ def test_config4_kda_prefill_full_size():
     torch.testing.assert_close(call["out"][:, heads].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
     for i, head in enumerate(heads):
         assert rel_l2(call["final_state"][0, head], exp_final[0, i]) <= 1e-3, head
+
+
+@pytest.mark.parametrize("lengths,pad,H", [([2500, 0, 1111, 40], 5, 2), ([4096], 0, 1), ([1030, 2049], 0, 3)])
+def test_kda_prefill_split_sequences_match_oracle(lengths, pad, H):
+    """Few, long sequences are split into 16-chunk segments that are swept concurrently (zero-state
+    and identity sweeps, a combine step, a second sweep).  Ragged lengths, an empty sequence, a
+    sequence shorter than one segment, initial and final states, against the float64 oracle."""
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    from pla_amd import _lib
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=515, pad=pad)
+    T, N = q.shape[0], len(lengths)
+    size = _lib.load().pla_kda_prefill_workspace_bytes
+    unsplit_per_head = size(T, N, 65 * H) / (65 * H)          # more than 64 chains are never split
+    assert size(T, N, H) > 1.1 * H * unsplit_per_head           # so this call carries the segment buffers
+    dev = "cuda"
+    out = torch.full((T, H, 128), float("nan"), dtype=torch.bfloat16, device=dev)
+    final = torch.full((N, H, 128, 128), float("nan"), device=dev)
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    flashkda_fwd(q.to(dev), k.to(dev), v.to(dev), raw.to(dev), beta.to(dev), A_log.to(dev), dt_bias.to(dev), out,
+                 initial_state=S0.to(dev), final_state=final, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    exp_o, exp_final = _oracle(q, k, v, raw, beta, A_log, dt_bias, offs, S0, fast=True)
+    real = offs[-1]
+    torch.testing.assert_close(out[:real].cpu().float(), exp_o[:real].float(), atol=2e-2, rtol=2e-2)
+    assert (out[real:] == 0).all()
+    for n, length in enumerate(lengths):
+        for head in range(H):
+            if length == 0:
+                assert torch.equal(final[n, head].cpu(), S0[n, head])   # an empty sequence publishes its incoming state
+            else:
+                assert rel_l2(final[n, head], exp_final[n, head]) <= 1e-3, (n, head)
