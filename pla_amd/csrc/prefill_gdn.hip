@@ -290,17 +290,16 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 // which is what bounds this kernel).  S^T stays in MFMA
 // accumulator layout (an accumulator tile pair is already a valid B operand of the next product),
 // A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  Every tile
-// is single buffered, and the copy of chunk c+1's version of a tile is issued at the first barrier
-// after the last use of chunk c's version, so each copy has most of a chunk's compute time to land:
+// is single buffered and there are two barriers per chunk; a tile's next version is requested at the
+// barrier after its last use and has half a chunk of compute time to land:
 //
-//   barrier 1   K, Q, V, decay factors of chunk c landed    flush O(c-1), issue P(c), factors of c+1
-//               KS = K S^T, QS = Q S^T, X = V - e^G (.) KS
-//   barrier 2   W landed                                     issue K, Q, V of chunk c+1
-//               U = W X
-//   barrier 3   K^T landed                                   issue W of chunk c+1
-//               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)
-//   barrier 4   P landed                                     issue K^T of chunk c+1
-//               O = scale e^G (.) QS + P U  -> O tile
+//   barrier A   K, Q, V, W, decay factors of chunk c landed   flush O(c-1); issue K^T(c), P(c), factors of c+1
+//               KS = K S^T, QS = Q S^T, X = V - e^G (.) KS, U = W X
+//   barrier B   K^T, P of chunk c landed                      issue K, Q, V, W of chunk c+1
+//               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U),  O = scale e^G (.) QS + P U -> O tile
+//
+// Every wait is for all outstanding copies (s_waitcnt vmcnt(0)): whatever is in flight at a barrier is
+// exactly what the next half needs.
 template <typename act_t, int NB>
 __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
   constexpr int WAVES = 8 / NB;                            // NB 16-column blocks of V per wavefront
@@ -399,12 +398,6 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
     if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
   };
-  // Copies issued after the one a barrier waits for (wavefronts 1..3 / wavefront 0); the gate piece
-  // is left out of wavefront 0's counts where it is conditional, which only makes the wait longer.
-  constexpr int KQV_O = 3 * CopyWide::EACH, KQV_0 = 3 * CopyWide::FIRST;
-  constexpr int W_O = 2 * CopyNarrow::EACH, W_0 = 2 * CopyNarrow::FIRST;
-  constexpr int KT_O = CopyKt::EACH, KT_0 = CopyKt::FIRST;
-  constexpr int P_O = CopyNarrow::EACH, P_0 = CopyNarrow::FIRST;
   // coalesced write of a finished output tile
   constexpr int FLUSH_ROWS = 32 / NB;                       // rows covered by one pass of the workgroup
   const int krow = tid >> 4, kcv = tid & 15;
@@ -422,17 +415,15 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   issue_gates(0);
   issue_kqv(0);
   issue_w(0);
-  issue_kt(0);
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
     const bool more = ci + 1 < n_chunks;
+    // Within a half the LDS operands are requested ahead of the MFMAs that use them (scheduling
+    // fences keep that order), so a wavefront waits for LDS once per product, not once per MFMA.
 
-    // Within a phase the LDS operands are requested ahead of the MFMAs that use them (scheduling
-    // fences keep that order), so a wavefront waits for LDS once per phase, not once per MFMA.
-
-    // barrier 1: K, Q, V (and the decay factors) of this chunk; W and K^T were issued after them
-    if (wave == 0) wait_vmcnt<W_0 + KT_0>(); else wait_vmcnt<W_O + KT_O>();
+    // barrier A: K, Q, V, W and the decay factors of this chunk have landed (nothing younger is in flight)
+    wait_vmcnt<0>();
     __syncthreads();
     bf16x8_t ka[2][4], qa[2][4];
 #pragma unroll
@@ -442,6 +433,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     }
     __builtin_amdgcn_sched_barrier(0);
     if (ci > 0) flush_output(ci - 1);
+    issue_kt(ci);
     issue_p(ci);
     if (more) issue_gates(ci + 1);
 
@@ -452,6 +444,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
     float4 eg[4];
     uint16_t vraw[NB][16];
+    bf16x8_t wh[2][4], wl[2][4];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
@@ -461,6 +454,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
           qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
         }
       } else {
+        // the last step's MFMAs cover the reads for X and for U = W X
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
           eg[mi] = *reinterpret_cast<const float4*>(&tG[par][64 + 16 * mi + 4 * kb]);
@@ -471,6 +465,13 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
             for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
           }
         }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            wh[s2][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s2, kb);
+            wl[s2][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s2, kb);
+          }
       }
       __builtin_amdgcn_sched_barrier(0);
       HiLo sb[NB];
@@ -501,20 +502,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         X[nb][mi][2] = to_float(act_t{vraw[nb][4 * mi + 2]}) - eg[mi].z * KS[nb][mi][2];
         X[nb][mi][3] = to_float(act_t{vraw[nb][4 * mi + 3]}) - eg[mi].w * KS[nb][mi][3];
       }
-
-    // barrier 2: W; K^T and P were issued after it
-    if (wave == 0) wait_vmcnt<KT_0 + P_0>(); else wait_vmcnt<KT_O + P_O>();
-    __syncthreads();
-    bf16x8_t wh[2][4], wl[2][4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        wh[s][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s, kb);
-        wl[s][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s, kb);
-      }
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) issue_kqv(ci + 1);
+    // U = W X
     f32x4_t U[NB][4];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
@@ -539,9 +527,8 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
     }
 
-    // barrier 3: K^T; P and (unless this is the last chunk) the next K, Q, V were issued after it
-    if (!more) { if (wave == 0) wait_vmcnt<P_0>(); else wait_vmcnt<P_O>(); }
-    else if (wave == 0) wait_vmcnt<P_0 + KQV_0>(); else wait_vmcnt<P_O + KQV_O>();
+    // barrier B: K^T and P of this chunk have landed; K, Q, V, W are free for the next chunk
+    wait_vmcnt<0>();
     __syncthreads();
     bf16x8_t kt[2][8];
 #pragma unroll
@@ -556,13 +543,28 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     }
     const float egl = tG[par][192];
     __builtin_amdgcn_sched_barrier(0);
-    if (more) issue_w(ci + 1);
+    if (more) {
+      issue_kqv(ci + 1);
+      issue_w(ci + 1);
+    }
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
+    bf16x8_t pa[2][4];
+    float4 sq[4];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
+      if (s == 1) {
+        // the last step's MFMAs cover the reads for the output product
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
       HiLo ub[NB];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
@@ -582,20 +584,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(kt[s][mc], ub[nb].lo, St[nb][mc]);
     }
 
-    // barrier 4: P; the next K, Q, V and W were issued after it
-    if (!more) wait_vmcnt<0>();
-    else if (wave == 0) wait_vmcnt<KQV_0 + W_0>(); else wait_vmcnt<KQV_O + W_O>();
-    __syncthreads();
-    bf16x8_t pa[2][4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) pa[s][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s, kb);
-    float4 sq[4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) issue_kt(ci + 1);
+    // O = scale e^{G} (.) QS + P U -> O tile
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
