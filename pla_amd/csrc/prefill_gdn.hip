@@ -445,6 +445,9 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     float4 eg[4];
     uint16_t vraw[NB][16];
     bf16x8_t wh[2][4], wl[2][4];
+    HiLo sb[2][NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = split8(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
@@ -474,21 +477,31 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
           }
       }
       __builtin_amdgcn_sched_barrier(0);
-      HiLo sb[NB];
+      // the split of the next step's state slice is interleaved with this step's MFMAs (one MFMA
+      // issues together with about two VALU instructions in its 16 cycles)
+      if (s < 3) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) sb[nb] = split8(St[nb][2 * s], St[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[nb].hi, KS[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[nb].hi, QS[nb][mi]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = split8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+      }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[nb].lo, KS[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[s & 1][nb].hi, QS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[s & 1][nb].lo, KS[nb][mi]);
+      if (s < 3) {
+#pragma unroll
+        for (int i = 0; i < 12 * NB; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // three VALU
+        }
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - e^{G} (.) KS
