@@ -53,6 +53,59 @@ constexpr int PITCH128 = 136;
 constexpr int PITCH64 = 72;
 
 // ---------------------------------------------------------------------------------------------
+// W = L^-1 diag(beta) for a unit lower triangular 64 x 64 L, by forward substitution on the four
+// wavefronts of a workgroup.  Wavefront w owns columns 16 w .. 16 w + 15; the four lanes of a quad share
+// one column and split each row's dot product by l mod 4: lane part p keeps x_l for l = 16 m + 4 e + p
+// in xs[4 m + e], and column j of L is stored at solve_slot(j), which makes those columns contiguous.
+// A row costs ceil(i / 16) float4 reads and 4 ceil(i / 16) FMAs per lane plus a two-step quad
+// reduction.  L must hold zeros on and above the diagonal of every diagonal 16 x 16 block it touches.
+__device__ __forceinline__ int solve_slot(int j) { return 16 * (j & 3) + 4 * (j >> 4) + ((j >> 2) & 3); }
+
+__device__ __forceinline__ void solve_store_w(const float (*L)[68], const float* beta, int wave, int lane,
+                                              uint16_t* Wh, uint16_t* Wl) {
+  const int col = 16 * wave + (lane >> 2), part = lane & 3;
+  const float bcol = beta[col];
+  float xs[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) xs[t] = 0.f;
+  // the L values of row i + 2 are requested while row i is reduced: they do not depend on x
+  float4 ahead[2][4];
+#pragma unroll
+  for (int i = 1; i < 3; ++i) ahead[i & 1][0] = *reinterpret_cast<const float4*>(&L[i][16 * part]);
+#pragma unroll
+  for (int i = 0; i < CHUNK; ++i) {
+    float4 row[4];
+#pragma unroll
+    for (int m = 0; 16 * m < i; ++m) row[m] = ahead[i & 1][m];
+    if (i + 2 < CHUNK) {
+#pragma unroll
+      for (int m = 0; 16 * m < i + 2; ++m)
+        ahead[i & 1][m] = *reinterpret_cast<const float4*>(&L[i + 2][16 * part + 4 * m]);
+    }
+    float acc = 0.f, acc2 = 0.f;
+#pragma unroll
+    for (int m = 0; 16 * m < i; ++m) {
+      acc = fmaf(row[m].x, xs[4 * m + 0], acc);
+      acc2 = fmaf(row[m].y, xs[4 * m + 1], acc2);
+      acc = fmaf(row[m].z, xs[4 * m + 2], acc);
+      acc2 = fmaf(row[m].w, xs[4 * m + 3], acc2);
+    }
+    acc += acc2;
+    acc += dpp_mov<0xB1>(acc);    // quad_perm [1,0,3,2]
+    acc += dpp_mov<0x4E>(acc);    // quad_perm [2,3,0,1]
+    const float xi = (i == col ? bcol : 0.f) - acc;
+    if (part == (i & 3)) xs[4 * (i >> 4) + ((i & 15) >> 2)] = xi;
+  }
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    const int l = 16 * (t >> 2) + 4 * (t & 3) + part;
+    const bf16_t hi = from_float<bf16_t>(xs[t]);
+    Wh[l * 64 + col] = hi.bits;
+    Wl[l * 64 + col] = from_float<bf16_t>(xs[t] - to_float(hi)).bits;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Asynchronous global -> LDS tile copies (global_load_lds_dwordx4: no registers, no LDS store
 // instructions).  Lane i of a wavefront writes its 16 bytes at (wave-uniform LDS base) + 16 i, so
 // a padded tile is filled as linear memory in 1 KiB pieces; a lane whose slot falls into a row's

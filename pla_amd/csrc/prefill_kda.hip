@@ -60,10 +60,6 @@ struct __align__(16) KdaPrepShared {
 };
 static_assert(sizeof(float[CHUNK][68]) <= sizeof(uint16_t[CHUNK][PITCH128]), "L must fit into Qn's storage");
 
-// Column j of L is stored at slot 16 (j % 4) + 4 (j / 16) + (j / 4) % 4, which makes the columns
-// l = 16 m + 4 e + p (e = 0..3) of one lane part p contiguous for the quad-split forward substitution.
-__device__ __forceinline__ int solve_slot(int j) { return 16 * (j & 3) + 4 * (j >> 4) + ((j >> 2) & 3); }
-
 // Eight decayed elements of a bf16 row: x[c] * exp(sign * (G[c] - R[c])) for the lane's two
 // channel quads of contraction step s.
 __device__ __forceinline__ void decayed8(const uint16_t* xrow, const float* grow, const float* rrow, float sign,
@@ -261,60 +257,8 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #ifdef PLA_PROF
   tk[4] = clock64();
 #endif
-  // ---- phase 4: W = L^-1 diag(beta) by forward substitution ------------------------------------
-  // Wavefront w owns columns 16 w .. 16 w + 15; the four lanes of a quad share one column and split
-  // each row's dot product by l mod 4 (lane part p keeps x_l for l = 16 m + 4 e + p in xs[4 m + e],
-  // and L is stored with those columns contiguous), so a row costs ceil(i / 16) float4 reads and
-  // 4 ceil(i / 16) FMAs per lane plus a two-step quad reduction.
-  {
-    const int col = 16 * wave + (lane >> 2), part = lane & 3;
-    const float bcol = sh.B[col];
-    float xs[16];
-#pragma unroll
-    for (int t = 0; t < 16; ++t) xs[t] = 0.f;
-    // the L values of row i + 2 are requested while row i is reduced: they do not depend on x
-    float4 ahead[2][4];
-#pragma unroll
-    for (int i = 1; i < 3; ++i) ahead[i & 1][0] = *reinterpret_cast<const float4*>(&sh.L[i][16 * part]);
-#pragma unroll
-    for (int i = 0; i < CHUNK; ++i) {
-      float4 row[4];
-#pragma unroll
-      for (int m = 0; 16 * m < i; ++m) row[m] = ahead[i & 1][m];
-      if (i + 2 < CHUNK) {
-#pragma unroll
-        for (int m = 0; 16 * m < i + 2; ++m)
-          ahead[i & 1][m] = *reinterpret_cast<const float4*>(&sh.L[i + 2][16 * part + 4 * m]);
-      }
-      float acc = 0.f, acc2 = 0.f;
-#pragma unroll
-      for (int m = 0; 16 * m < i; ++m) {
-        acc = fmaf(row[m].x, xs[4 * m + 0], acc);
-        acc2 = fmaf(row[m].y, xs[4 * m + 1], acc2);
-        acc = fmaf(row[m].z, xs[4 * m + 2], acc);
-        acc2 = fmaf(row[m].w, xs[4 * m + 3], acc2);
-      }
-      acc += acc2;
-      acc += dpp_mov<0xB1>(acc);    // quad_perm [1,0,3,2]
-      acc += dpp_mov<0x4E>(acc);    // quad_perm [2,3,0,1]
-      const float xi = (i == col ? bcol : 0.f) - acc;
-      if (part == (i & 3)) xs[4 * (i >> 4) + ((i & 15) >> 2)] = xi;
-    }
-    uint16_t* const Wh = p.Whi + tile * 4096 + col;
-    uint16_t* const Wl = p.Wlo + tile * 4096 + col;
-#pragma unroll
-    for (int t = 0; t < 16; ++t) {
-      const int l = 16 * (t >> 2) + 4 * (t & 3) + part;
-      const bf16_t hi = from_float<bf16_t>(xs[t]);
-      Wh[l * 64] = hi.bits;
-      Wl[l * 64] = from_float<bf16_t>(xs[t] - to_float(hi)).bits;
-    }
-  }
-#ifdef PLA_PROF
-  tk[5] = clock64();
-  if (blockIdx.x == 100 && blockIdx.y == 3 && lane == 0)
-    printf("prep wave %d: p1 %lld cumsum %lld p2 %lld p3 %lld p4 %lld\n", wave, tk[1] - tk[0], tk[2] - tk[1], tk[3] - tk[2], tk[4] - tk[3], tk[5] - tk[4]);
-#endif
+  // ---- phase 4: W = L^-1 diag(beta), forward substitution on all four wavefronts ----------------
+  solve_store_w(sh.L, sh.B, wave, lane, p.Whi + tile * 4096, p.Wlo + tile * 4096);
 }
 
 // ---------------------------------------------------------------------------------------------
