@@ -21,8 +21,9 @@
 //   kda_prep_solve_kernel   one workgroup per (chunk, head): q/k L2 norm (rounded to bf16), lower-bound
 //                           gate, cumulative decay, decayed operand tiles, M / P on MFMA, FP32 forward
 //                           substitution, W (hi/lo)
-//   kda_chunk_seq_kernel    one workgroup per (sequence, head), 8 wavefronts x 16 V columns, same
-//                           register-chained MFMA pipeline as the GDN kernel
+//   kda_chunk_seq_kernel    one workgroup per (sequence, head) or segment sweep, four wavefronts x 32 V
+//                           columns, same register-chained MFMA pipeline and asynchronous LDS tile
+//                           copies as the GDN kernel
 
 #include "prefill_common.h"
 
@@ -262,24 +263,30 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 }
 
 // ---------------------------------------------------------------------------------------------
-struct __align__(16) KdaSeqTiles {
-  uint16_t Khi[CHUNK][PITCH128];
-  uint16_t Klo[CHUNK][PITCH128];
-  uint16_t Q[CHUNK][PITCH128];
-  uint16_t V[CHUNK][PITCH128];        // doubles as the output tile: wave w only touches columns [16w, 16w+16)
-  uint16_t KtH[128][PITCH64];
-  uint16_t KtL[128][PITCH64];
-  uint16_t Whi[CHUNK][PITCH64];
-  uint16_t Wlo[CHUNK][PITCH64];
-  uint16_t P[CHUNK][PITCH64];
-  float eGl[128];
-};
-
-__global__ __launch_bounds__(512) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
+// Sequential kernel: one workgroup per (sequence, head) or per segment sweep, four wavefronts (one per
+// SIMD), each owning two 16-column blocks of V that share every A operand.  S^T stays in MFMA
+// accumulator layout (an accumulator tile pair is already a valid B operand of the next product); the
+// A operands come from LDS tiles filled by asynchronous global -> LDS copies.  Every tile is single
+// buffered (149 KB of LDS) and there are two barriers per chunk; a tile's next version is requested at
+// the barrier after its last use and has half a chunk of compute time to land:
+//
+//   barrier A   K e^G (hi, lo), scale Q e^G, V, W (hi, lo) of chunk c landed
+//               flush O(c-1); issue (K e^{G_last-G})^T (hi, lo), P, e^{G_last} of chunk c
+//               KS = (K e^G) S^T (three split passes), QS = (scale Q e^G) S^T, X = V - KS, U = W X
+//   barrier B   the tiles issued at A landed; issue the first group for chunk c+1
+//               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U,  O = QS + P U -> O tile
+//
+// Every wait is for all outstanding copies: what is in flight at a barrier is what the next half needs.
+__global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
+  constexpr int NB = 2, WAVES = 4;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
+  using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int vcol = 16 * wave + r16;
+  const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
 
   // What this workgroup sweeps: a whole sequence, or one segment of it in one of three roles.
   int n, h, c_begin, c_end;
@@ -332,185 +339,307 @@ __global__ __launch_bounds__(512) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int seq_start = p.cu_seqlens[n] + chunk_in_seq * CHUNK;
   const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
 
-  __shared__ KdaSeqTiles T;
+  const int n_chunks = c_end - c_begin;
 
-  f32x4_t St[8];
-  {
+  // distinct LDS objects, 16-byte aligned, filled in 1 KiB pieces
+  __shared__ __align__(16) uint16_t tKh[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tKl[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tKtH[128 * PITCH64];
+  __shared__ __align__(16) uint16_t tKtL[128 * PITCH64];
+  __shared__ __align__(16) uint16_t tWh[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tWl[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  __shared__ __align__(16) float tE[128];            // e^{G_last} of the chunk
+
+  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
+  f32x4_t St[NB][8];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
     if (init != nullptr) {
-      const float* src = init + (int64_t)vcol * 128 + 4 * kb;
+      const float* src = init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
         const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
-        St[mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
       }
     } else {
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) St[mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
+  if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
+    for (int i = tid; i < CHUNK * PITCH128 / 2; i += 256) reinterpret_cast<uint32_t*>(tV)[i] = 0u;
   }
 
+  const int64_t tile0 = (int64_t)c_begin * p.H + h;                       // chunk tiles are [chunk, H, ...]
+  const char* const kh_b = reinterpret_cast<const char*>(p.Khi) + tile0 * 16384;
+  const char* const kl_b = reinterpret_cast<const char*>(p.Klo) + tile0 * 16384;
+  const char* const qh_b = reinterpret_cast<const char*>(p.Qh) + tile0 * 16384;
+  const char* const th_b = reinterpret_cast<const char*>(p.KtH) + tile0 * 16384;
+  const char* const tl_b = reinterpret_cast<const char*>(p.KtL) + tile0 * 16384;
+  const char* const wh_b = reinterpret_cast<const char*>(p.Whi) + tile0 * 8192;
+  const char* const wl_b = reinterpret_cast<const char*>(p.Wlo) + tile0 * 8192;
+  const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
+  const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
+  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
+  const int64_t big_step = (int64_t)p.H * 16384, small_step = (int64_t)p.H * 8192, e_step = (int64_t)p.H * 512;
+
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+  CopyWide plan_k, plan_v;
+  CopyNarrow plan_w;
+  CopyKt plan_kt;
+  plan_k.plan(256, CHUNK - 1, wave, lane);
+  plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
+  plan_w.plan(128, CHUNK - 1, wave, lane);
+  plan_kt.plan(128, 127, wave, lane);
+  auto issue_first = [&](int c) {                    // K e^G (hi, lo), scale Q e^G, V, W (hi, lo)
+    plan_k.issue(tKh, kh_b + c * big_step, wave);
+    plan_k.issue(tKl, kl_b + c * big_step, wave);
+    plan_k.issue(tQ, qh_b + c * big_step, wave);
+    if (!zero_v) {
+      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+      const int len = chunk_len(c);
+      if (len == CHUNK) {
+        plan_v.issue(tV, vs, wave);
+      } else {                                       // rows past the sequence re-read its last row
+        CopyWide tail_v;
+        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
+        tail_v.issue(tV, vs, wave);
+      }
+    }
+    plan_w.issue(tWh, wh_b + c * small_step, wave);
+    plan_w.issue(tWl, wl_b + c * small_step, wave);
+  };
+  auto issue_second = [&](int c) {                   // (K e^{G_last-G})^T (hi, lo), P, e^{G_last}
+    plan_kt.issue(tKtH, th_b + c * big_step, wave);
+    plan_kt.issue(tKtL, tl_b + c * big_step, wave);
+    plan_w.issue(tP, pp_b + c * small_step, wave);
+    if (wave == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
+  };
+  // coalesced write of a finished output tile
   const int krow = tid >> 4, kcv = tid & 15;
-  const int srow = tid >> 3, scv = tid & 7;
-  const int64_t tile_stride = (int64_t)p.H * 8192, small_stride = (int64_t)p.H * 4096;
-  int64_t big = ((int64_t)c_begin * p.H + h) * 8192;            // offset of this chunk's 64x128 / 128x64 tiles
-  int64_t small = ((int64_t)c_begin * p.H + h) * 4096;          // offset of the 64x64 tiles
-  const uint16_t* vptr = reinterpret_cast<const uint16_t*>(p.v) + (int64_t)(seq_start + krow) * p.stride_v + h * 128 + 8 * kcv;
-  uint16_t* optr = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
-  const int64_t o_half = (int64_t)32 * p.H * 128;
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
-
-  uint4 pkh0, pkh1, pkl0, pkl1, pq0, pq1, pv0, pv1, pth0, pth1, ptl0, ptl1, pwh, pwl, ppp;
-  float pe = 0.f;
-  auto prefetch = [&](int len) {
-    const int lo = krow * 128 + 8 * kcv, hi2 = lo + 32 * 128;
-    pkh0 = *reinterpret_cast<const uint4*>(p.Khi + big + lo);
-    pkh1 = *reinterpret_cast<const uint4*>(p.Khi + big + hi2);
-    pkl0 = *reinterpret_cast<const uint4*>(p.Klo + big + lo);
-    pkl1 = *reinterpret_cast<const uint4*>(p.Klo + big + hi2);
-    pq0 = *reinterpret_cast<const uint4*>(p.Qh + big + lo);
-    pq1 = *reinterpret_cast<const uint4*>(p.Qh + big + hi2);
-    pth0 = *reinterpret_cast<const uint4*>(p.KtH + big + 8 * tid);
-    pth1 = *reinterpret_cast<const uint4*>(p.KtH + big + 4096 + 8 * tid);
-    ptl0 = *reinterpret_cast<const uint4*>(p.KtL + big + 8 * tid);
-    ptl1 = *reinterpret_cast<const uint4*>(p.KtL + big + 4096 + 8 * tid);
-    pwh = *reinterpret_cast<const uint4*>(p.Whi + small + 8 * tid);
-    pwl = *reinterpret_cast<const uint4*>(p.Wlo + small + 8 * tid);
-    ppp = *reinterpret_cast<const uint4*>(p.P + small + 8 * tid);
-    if (tid < 128) pe = p.eGlast[(small >> 5) + tid];            // tile index * 128
-    const bool ok0 = krow < len, ok1 = krow + 32 < len;
-    const int64_t back0 = ok0 ? 0 : -(int64_t)krow, back1 = ok1 ? 32 : -(int64_t)krow;
-    pv0 = *reinterpret_cast<const uint4*>(vptr + back0 * p.stride_v);
-    pv1 = *reinterpret_cast<const uint4*>(vptr + back1 * p.stride_v);
-    if (!ok0 || zero_v) pv0 = zero4;
-    if (!ok1 || zero_v) pv1 = zero4;
-    big += tile_stride; small += small_stride; vptr += CHUNK * p.stride_v;
-  };
-  auto flush_output = [&](int len) {
+  uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
+  auto flush_output = [&](int c) {
     if (!write_o) return;
-    if (krow < len) *reinterpret_cast<uint4*>(optr) = *reinterpret_cast<const uint4*>(&T.V[krow][8 * kcv]);
-    if (krow + 32 < len) *reinterpret_cast<uint4*>(optr + o_half) = *reinterpret_cast<const uint4*>(&T.V[krow + 32][8 * kcv]);
-    optr += (int64_t)CHUNK * p.H * 128;
+    const int len = chunk_len(c);
+    uint16_t* dst = o_b + (int64_t)c * CHUNK * p.H * 128;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (krow + 16 * i < len)
+        *reinterpret_cast<uint4*>(dst + (int64_t)16 * i * p.H * 128) =
+            *reinterpret_cast<const uint4*>(&tO[(krow + 16 * i) * PITCH128 + 8 * kcv]);
   };
 
-  const int n_chunks = c_end - c_begin;
-  prefetch(min(CHUNK, seq_len));
-  int prev_len = 0;
-  for (int ci = 0; ci < n_chunks; ++ci) {
-    const int len = min(CHUNK, seq_len - ci * CHUNK);
-    __syncthreads();
-    if (ci > 0) flush_output(prev_len);          // reads exactly the vectors this thread overwrites next
-    *reinterpret_cast<uint4*>(&T.Khi[krow][8 * kcv]) = pkh0;
-    *reinterpret_cast<uint4*>(&T.Khi[krow + 32][8 * kcv]) = pkh1;
-    *reinterpret_cast<uint4*>(&T.Klo[krow][8 * kcv]) = pkl0;
-    *reinterpret_cast<uint4*>(&T.Klo[krow + 32][8 * kcv]) = pkl1;
-    *reinterpret_cast<uint4*>(&T.Q[krow][8 * kcv]) = pq0;
-    *reinterpret_cast<uint4*>(&T.Q[krow + 32][8 * kcv]) = pq1;
-    *reinterpret_cast<uint4*>(&T.V[krow][8 * kcv]) = pv0;
-    *reinterpret_cast<uint4*>(&T.V[krow + 32][8 * kcv]) = pv1;
-    *reinterpret_cast<uint4*>(&T.KtH[srow][8 * scv]) = pth0;
-    *reinterpret_cast<uint4*>(&T.KtH[64 + srow][8 * scv]) = pth1;
-    *reinterpret_cast<uint4*>(&T.KtL[srow][8 * scv]) = ptl0;
-    *reinterpret_cast<uint4*>(&T.KtL[64 + srow][8 * scv]) = ptl1;
-    *reinterpret_cast<uint4*>(&T.Whi[srow][8 * scv]) = pwh;
-    *reinterpret_cast<uint4*>(&T.Wlo[srow][8 * scv]) = pwl;
-    *reinterpret_cast<uint4*>(&T.P[srow][8 * scv]) = ppp;
-    if (tid < 128) T.eGl[tid] = pe;
-    __syncthreads();
-    if (ci + 1 < n_chunks) prefetch(min(CHUNK, seq_len - (ci + 1) * CHUNK));
+  issue_first(0);
 
-    // KS = (K e^{G}) S^T (three split passes) and QS = (scale Q e^{G}) S^T
-    f32x4_t KS[4], QS[4];
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const bool more = ci + 1 < n_chunks;
+
+    // barrier A
+    wait_vmcnt<0>();
+    __syncthreads();
+    bf16x8_t kh[2][4], kl[2][4], qa[2][4];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) { KS[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[mi] = KS[mi]; }
+    for (int mi = 0; mi < 4; ++mi) {
+      kh[0][mi] = operand_from(&tKh[(16 * mi + r16) * PITCH128], 0, kb);
+      kl[0][mi] = operand_from(&tKl[(16 * mi + r16) * PITCH128], 0, kb);
+      qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (ci > 0) flush_output(ci - 1);
+    issue_second(ci);
+
+    f32x4_t KS[NB][4], QS[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
+    uint16_t vraw[NB][16];
+    bf16x8_t wh[2][4], wl[2][4];
+    HiLo sb[2][NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = split8(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const HiLo sb = split8(St[2 * s], St[2 * s + 1]);
+      if (s < 3) {
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t kh = operand_from(&T.Khi[16 * mi + r16][0], s, kb);
-        const bf16x8_t kl = operand_from(&T.Klo[16 * mi + r16][0], s, kb);
-        const bf16x8_t qa = operand_from(&T.Q[16 * mi + r16][0], s, kb);
-        KS[mi] = mfma16(kh, sb.hi, KS[mi]);
-        QS[mi] = mfma16(qa, sb.hi, QS[mi]);
-        KS[mi] = mfma16(kl, sb.hi, KS[mi]);
-        KS[mi] = mfma16(kh, sb.lo, KS[mi]);
+        for (int mi = 0; mi < 4; ++mi) {
+          kh[(s + 1) & 1][mi] = operand_from(&tKh[(16 * mi + r16) * PITCH128], s + 1, kb);
+          kl[(s + 1) & 1][mi] = operand_from(&tKl[(16 * mi + r16) * PITCH128], s + 1, kb);
+          qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
+        }
+      } else {
+        // the last step's MFMAs cover the reads for X and for U = W X
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+          }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            wh[s2][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s2, kb);
+            wl[s2][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s2, kb);
+          }
       }
-    }
-
-    f32x4_t X[4];
+      __builtin_amdgcn_sched_barrier(0);
+      // the split of the next step's state slice is interleaved with this step's MFMAs
+      if (s < 3) {
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      const uint16_t* vr = &T.V[16 * mi + 4 * kb][vcol];
-      X[mi][0] = to_float(bf16_t{vr[0]}) - KS[mi][0];
-      X[mi][1] = to_float(bf16_t{vr[PITCH128]}) - KS[mi][1];
-      X[mi][2] = to_float(bf16_t{vr[2 * PITCH128]}) - KS[mi][2];
-      X[mi][3] = to_float(bf16_t{vr[3 * PITCH128]}) - KS[mi][3];
-    }
-
-    f32x4_t U[4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) U[mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const HiLo xb = split8(X[2 * s], X[2 * s + 1]);
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        const bf16x8_t wh = operand_from(&T.Whi[16 * mi + r16][0], s, kb);
-        const bf16x8_t wl = operand_from(&T.Wlo[16 * mi + r16][0], s, kb);
-        U[mi] = mfma16(wh, xb.hi, U[mi]);
-        U[mi] = mfma16(wl, xb.hi, U[mi]);
-        U[mi] = mfma16(wh, xb.lo, U[mi]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = split8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
       }
-    }
-
-    // S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U
 #pragma unroll
-    for (int mc = 0; mc < 8; ++mc) {
-      const float4 e = *reinterpret_cast<const float4*>(&T.eGl[16 * mc + 4 * kb]);
-      St[mc] = f32x4_t{St[mc][0] * e.x, St[mc][1] * e.y, St[mc][2] * e.z, St[mc][3] * e.w};
-    }
+      for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const HiLo ub = split8(U[2 * s], U[2 * s + 1]);
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kh[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) {
-        const bf16x8_t th = operand_from(&T.KtH[16 * mc + r16][0], s, kb);
-        const bf16x8_t tl = operand_from(&T.KtL[16 * mc + r16][0], s, kb);
-        St[mc] = mfma16(th, ub.hi, St[mc]);
-        St[mc] = mfma16(tl, ub.hi, St[mc]);
-        St[mc] = mfma16(th, ub.lo, St[mc]);
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[s & 1][nb].hi, QS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kl[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kh[s & 1][mi], sb[s & 1][nb].lo, KS[nb][mi]);
+      if (s < 3) {
+#pragma unroll
+        for (int i = 0; i < 16 * NB; ++i) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);   // two VALU
+        }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-
-    // O = QS + P U
-    f32x4_t O[4];
+    // X = V - KS
+    f32x4_t X[NB][4];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) O[mi] = QS[mi];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      const bf16x8_t ub = round8(U[2 * s], U[2 * s + 1]);
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi)
-        O[mi] = mfma16(operand_from(&T.P[16 * mi + r16][0], s, kb), ub, O[mi]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) X[nb][mi][r] = to_float(bf16_t{vraw[nb][4 * mi + r]}) - KS[nb][mi][r];
+    // U = W X
+    f32x4_t U[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      HiLo xb[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = split8(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].hi, U[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wl[s][mi], xb[nb].hi, U[nb][mi]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
+    }
+
+    // barrier B
+    wait_vmcnt<0>();
+    __syncthreads();
+    bf16x8_t th[8], tl[8];
+#pragma unroll
+    for (int mc = 0; mc < 8; ++mc) {
+      th[mc] = operand_from(&tKtH[(16 * mc + r16) * PITCH64], 0, kb);
+      tl[mc] = operand_from(&tKtL[(16 * mc + r16) * PITCH64], 0, kb);
+    }
+    float4 eg[8];
+#pragma unroll
+    for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) issue_first(ci + 1);
+    // S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        St[nb][mc] = f32x4_t{St[nb][mc][0] * eg[mc].x, St[nb][mc][1] * eg[mc].y, St[nb][mc][2] * eg[mc].z,
+                             St[nb][mc][3] * eg[mc].w};
+    bf16x8_t pa[2][4];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      if (s == 1) {
+        // second contraction step: its operands and those of the output product are requested together
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) {
+          th[mc] = operand_from(&tKtH[(16 * mc + r16) * PITCH64], 1, kb);
+          tl[mc] = operand_from(&tKtL[(16 * mc + r16) * PITCH64], 1, kb);
+        }
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      HiLo ub[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) ub[nb] = split8(U[nb][2 * s], U[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(th[mc], ub[nb].hi, St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(tl[mc], ub[nb].hi, St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(th[mc], ub[nb].lo, St[nb][mc]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // O = QS + P U -> O tile
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      bf16x8_t ur[NB];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) ur[nb] = round8(U[nb][2 * s], U[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(pa[s][mi], ur[nb], QS[nb][mi]);
     }
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      uint16_t* orow = &T.V[16 * mi + 4 * kb][vcol];
-      orow[0] = from_float<bf16_t>(O[mi][0]).bits;
-      orow[PITCH128] = from_float<bf16_t>(O[mi][1]).bits;
-      orow[2 * PITCH128] = from_float<bf16_t>(O[mi][2]).bits;
-      orow[3 * PITCH128] = from_float<bf16_t>(O[mi][3]).bits;
-    }
-    prev_len = len;
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+        orow[0] = from_float<bf16_t>(QS[nb][mi][0]).bits;
+        orow[PITCH128] = from_float<bf16_t>(QS[nb][mi][1]).bits;
+        orow[2 * PITCH128] = from_float<bf16_t>(QS[nb][mi][2]).bits;
+        orow[3 * PITCH128] = from_float<bf16_t>(QS[nb][mi][3]).bits;
+      }
   }
   __syncthreads();
-  flush_output(prev_len);
+  flush_output(n_chunks - 1);
 
   if (fin != nullptr) {
-    float* dst = fin + (int64_t)vcol * 128 + 4 * kb;
 #pragma unroll
-    for (int mc = 0; mc < 8; ++mc)
-      *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[mc].x, St[mc].y, St[mc].z, St[mc].w);
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
   }
 }
 
@@ -608,7 +737,7 @@ extern "C" int pla_kda_prefill_launch(
   hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, s, p);
   if (L.seg_chunks == 0) {
     p.pass = 0;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)N * H), dim3(512), 0, s, p);
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)N * H), dim3(256), 0, s, p);
   } else {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
@@ -623,10 +752,10 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.max_segments = L.max_segments;
     hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
     p.pass = 1;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H * 2), dim3(512), 0, s, p);
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H * 2), dim3(256), 0, s, p);
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H), dim3(256), 0, s, p.seg, H, ht, ht_indices, ht_slot_stride);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(512), 0, s, p);
+    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
