@@ -94,23 +94,38 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #endif
   // ---- phase 1: normalised q / k, per-channel log-decay, beta ---------------------------------
   {
-    uint32_t qw[16], kw[16];
+    // q, k: thread handles eight channels of rows tid / 16 + 16 u (a row is one 16-lane DPP row, so its
+    // sum of squares is a row reduction); all eight 16-byte loads are in flight at once
+    const int nrow = tid >> 4, nc0 = 8 * (tid & 15);
+    uint4 qv[4], kv[4];
 #pragma unroll
-    for (int x = 0; x < 16; ++x) {
-      const int j = 16 * wave + x;
+    for (int u = 0; u < 4; ++u) {
+      const int j = nrow + 16 * u;
       const int64_t t = t0 + (j < len ? j : 0);
-      qw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128 + 2 * lane);
-      kw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + 2 * lane);
+      qv[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128 + nc0);
+      kv[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + nc0);
     }
 #pragma unroll
-    for (int x = 0; x < 16; ++x) {
-      const int j = 16 * wave + x;
-      float q0 = lo16<bf16_t>(qw[x]), q1 = hi16<bf16_t>(qw[x]), k0 = lo16<bf16_t>(kw[x]), k1 = hi16<bf16_t>(kw[x]);
-      const float qi = rsqrtf(wave64_allreduce(q0 * q0 + q1 * q1) + 1e-6f);
-      const float ki = rsqrtf(wave64_allreduce(k0 * k0 + k1 * k1) + 1e-6f);
+    for (int u = 0; u < 4; ++u) {
+      const int j = nrow + 16 * u;
+      const uint32_t qw[4] = {qv[u].x, qv[u].y, qv[u].z, qv[u].w}, kw[4] = {kv[u].x, kv[u].y, kv[u].z, kv[u].w};
+      float qs = 0.f, ks = 0.f;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float q0 = lo16<bf16_t>(qw[e]), q1 = hi16<bf16_t>(qw[e]), k0 = lo16<bf16_t>(kw[e]), k1 = hi16<bf16_t>(kw[e]);
+        qs += q0 * q0 + q1 * q1;
+        ks += k0 * k0 + k1 * k1;
+      }
+      const float qi = rsqrtf(row16_allreduce(qs) + 1e-6f), ki = rsqrtf(row16_allreduce(ks) + 1e-6f);
       const bool ok = j < len;
-      *reinterpret_cast<uint32_t*>(&sh.Qn[j][2 * lane]) = ok ? pack2<bf16_t>(q0 * qi, q1 * qi) : 0u;
-      *reinterpret_cast<uint32_t*>(&sh.Kn[j][2 * lane]) = ok ? pack2<bf16_t>(k0 * ki, k1 * ki) : 0u;
+      uint32_t qo[4], ko[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        qo[e] = ok ? pack2<bf16_t>(lo16<bf16_t>(qw[e]) * qi, hi16<bf16_t>(qw[e]) * qi) : 0u;
+        ko[e] = ok ? pack2<bf16_t>(lo16<bf16_t>(kw[e]) * ki, hi16<bf16_t>(kw[e]) * ki) : 0u;
+      }
+      *reinterpret_cast<uint4*>(&sh.Qn[j][nc0]) = make_uint4(qo[0], qo[1], qo[2], qo[3]);
+      *reinterpret_cast<uint4*>(&sh.Kn[j][nc0]) = make_uint4(ko[0], ko[1], ko[2], ko[3]);
     }
     // gate: thread handles eight channels of rows tid / 16 + 16 u; all four 16-byte loads are in flight at once
     const float eA = expf(p.A_log[h]);
@@ -699,8 +714,9 @@ extern "C" int pla_kda_prefill_launch(
   PLA_REQUIRE(act_dtype == PLA_BF16, "KDA prefill takes bf16 activations (the MFMA operands are bf16)");
   PLA_REQUIRE(q && k && v && g && beta && A_log && dt_bias && o && cu_seqlens && workspace, "null tensor pointer");
   PLA_REQUIRE(lower_bound <= 0.f && lower_bound >= -5.f, "lower_bound must lie in [-5, 0], got %g", (double)lower_bound);
-  PLA_REQUIRE(((uintptr_t)q % 4 == 0) && ((uintptr_t)k % 4 == 0) && stride_q % 2 == 0 && stride_k % 2 == 0,
-              "q/k rows require 4-byte alignment");
+  PLA_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)k % 16 == 0) && ((uintptr_t)g % 16 == 0) && stride_q % 8 == 0 &&
+                  stride_k % 8 == 0 && stride_g % 8 == 0,
+              "q/k/g rows require 16-byte alignment");
   PLA_REQUIRE(((uintptr_t)v % 16 == 0) && stride_v % 8 == 0, "v rows require 16-byte alignment");
   PLA_REQUIRE(((uintptr_t)o % 16 == 0), "out requires 16-byte alignment");
   const KdaWorkspaceLayout L = kda_layout(T, N, H);
