@@ -219,6 +219,67 @@ struct SegmentTable {
   int max_segments;
 };
 
+// What one workgroup of a sequential kernel sweeps: a whole sequence (pass 0) or one segment in one of
+// the roles above (pass 1: blockIdx = (segment, head, from-identity flag); pass 2: (segment, head)).
+struct SweepRole {
+  int n, head, c_begin, c_end;
+  const float* init;      // [V, K] tile the state starts from (nullptr: zero)
+  float* fin;             // [V, K] tile that receives the state at the end (nullptr: none)
+  bool zero_v, write_o, active;
+};
+__device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, const int32_t* seq_chunk_off,
+                                                  const SegmentTable& seg, const float* h0, const int32_t* h0_indices,
+                                                  int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
+                                                  int64_t ht_slot_stride) {
+  SweepRole r{};
+  r.write_o = true;
+  auto state_in = [&](int n, int head) -> const float* {
+    const int slot = (h0 != nullptr) ? (h0_indices ? h0_indices[n] : n) : -1;
+    return slot >= 0 ? h0 + (int64_t)slot * h0_slot_stride + (int64_t)head * 16384 : nullptr;
+  };
+  auto state_out = [&](int n, int head) -> float* {
+    const int slot = (ht != nullptr) ? (ht_indices ? ht_indices[n] : n) : -1;
+    return slot >= 0 ? ht + (int64_t)slot * ht_slot_stride + (int64_t)head * 16384 : nullptr;
+  };
+  if (pass == 0) {
+    r.n = blockIdx.x / heads;
+    r.head = blockIdx.x - r.n * heads;
+    r.c_begin = seq_chunk_off[r.n];
+    r.c_end = seq_chunk_off[r.n + 1];
+    if (r.c_begin >= r.c_end) return r;              // empty sequence: state untouched, no output
+    r.init = state_in(r.n, r.head);
+    r.fin = state_out(r.n, r.head);
+    r.active = true;
+    return r;
+  }
+  const int item = pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+  const bool from_identity = pass == 1 && (blockIdx.x & 1);
+  const int s = item / heads;
+  r.head = item - s * heads;
+  if (s >= seg.seq_seg_off[N]) return r;
+  r.n = seg.seg_seq[s];
+  const bool first = s == seg.seq_seg_off[r.n], last = s + 1 == seg.seq_seg_off[r.n + 1];
+  r.c_begin = seg.seg_c0[s];
+  r.c_end = r.c_begin + seg.seg_nc[s];
+  const int64_t tile = ((int64_t)s * heads + r.head) * 16384;
+  if (pass == 1) {
+    if (first) {
+      if (from_identity) return r;
+      r.init = state_in(r.n, r.head);
+      r.fin = last ? state_out(r.n, r.head) : seg.B + tile;     // B of a first segment: the state entering the second
+    } else {
+      r.write_o = false;
+      if (from_identity) { r.init = seg.identity; r.zero_v = true; r.fin = seg.M + tile; }
+      else r.fin = seg.B + tile;
+    }
+  } else {
+    if (first) return r;
+    r.init = seg.S + tile;                            // the final state came out of the combine step
+  }
+  r.active = true;
+  return r;
+}
+
 // Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map_kernel.
 static __global__ void segment_map_kernel(const int32_t* seq_chunk_off, int N, SegmentTable t) {
   if (threadIdx.x == 0) {

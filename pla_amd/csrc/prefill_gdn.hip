@@ -53,6 +53,8 @@ struct GdnPrefillParams {
   float* gcum; float* beta;
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
+  SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
+  int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments
   int H, HV, NC_max;
 };
 
@@ -306,18 +308,19 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
   using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
-  const int n = blockIdx.x / p.HV;
-  const int hv = blockIdx.x - n * p.HV;
+  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride);
+  if (!role.active) return;
+  const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
+  const bool zero_v = role.zero_v, write_o = role.write_o;
   const int h = hv / (p.HV / p.H);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
   const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the others: +16 each)
-  const int c_begin = p.seq_chunk_off[n], c_end = p.seq_chunk_off[n + 1];
-  if (c_begin >= c_end) return;
-  const int seq_start = p.cu_seqlens[n];
-  const int seq_len = p.cu_seqlens[n + 1] - seq_start;
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
   const int n_chunks = c_end - c_begin;
 
   // distinct LDS objects: the compiler tracks outstanding direct-to-LDS loads per object
@@ -335,11 +338,10 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
   f32x4_t St[NB][8];
   {
-    const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
-      if (slot >= 0) {
-        const float* src = p.h0 + (int64_t)slot * p.h0_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
+      if (role.init != nullptr) {
+        const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
         for (int mc = 0; mc < 8; ++mc) {
           const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
@@ -349,6 +351,10 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 #pragma unroll
         for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       }
+  }
+
+  if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
+    for (int i = tid; i < CHUNK * PITCH128 / 2; i += 256 * 2 / NB) reinterpret_cast<uint32_t*>(tV)[i] = 0u;
   }
 
   const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
@@ -379,14 +385,16 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     if (len == CHUNK) {
       plan_kq.issue(tK, ks, wave);
       plan_kq.issue(tQ, qs, wave);
-      plan_v.issue(tV, vs, wave);
+      if (!zero_v) plan_v.issue(tV, vs, wave);
     } else {
       CopyWide tail_kq, tail_v;
       tail_kq.plan((uint32_t)tok_pitch_b, len - 1, wave, lane);
-      tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
       tail_kq.issue(tK, ks, wave);
       tail_kq.issue(tQ, qs, wave);
-      tail_v.issue(tV, vs, wave);
+      if (!zero_v) {
+        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
+        tail_v.issue(tV, vs, wave);
+      }
     }
   };
   auto issue_w = [&](int c) {
@@ -403,6 +411,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   const int krow = tid >> 4, kcv = tid & 15;
   uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
   auto flush_output = [&](int c) {
+    if (!write_o) return;
     const int len = chunk_len(c);
     uint16_t* dst = o_b + (int64_t)c * CHUNK * p.HV * 128;
 #pragma unroll
@@ -628,23 +637,21 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   __syncthreads();
   flush_output(n_chunks - 1);
 
-  if (p.ht != nullptr) {
-    const int slot = p.ht_indices ? p.ht_indices[n] : n;
-    if (slot >= 0) {
+  if (role.fin != nullptr) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        float* dst = p.ht + (int64_t)slot * p.ht_slot_stride + ((int64_t)hv * 128 + vcol + 16 * nb) * 128 + 4 * kb;
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc)
-          *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
-      }
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
     }
   }
 }
 
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P, total;
-  int NC_max;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P;
+  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity, total;
+  int NC_max, seg_chunks, max_segments;
 };
 static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   GdnWorkspaceLayout L;
@@ -664,6 +671,17 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   L.Whi = take((size_t)L.NC_max * HV * 4096 * 2);
   L.Wlo = take((size_t)L.NC_max * HV * 4096 * 2);
   L.P = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.seg_chunks = pick_segment_chunks(T, N, HV);
+  L.max_segments = max_segments(T, N, L.seg_chunks);
+  if (L.seg_chunks > 0) {
+    L.seq_seg_off = take((size_t)(N + 1) * 4);
+    L.seg_seq = take((size_t)L.max_segments * 4);
+    L.seg_c0 = take((size_t)L.max_segments * 4);
+    L.seg_nc = take((size_t)L.max_segments * 4);
+    const size_t states = (size_t)L.max_segments * HV * 16384 * 4;
+    L.segM = take(states); L.segB = take(states); L.segS = take(states);
+    L.identity = take(16384 * 4);
+  }
   L.total = off;
   return L;
 }
@@ -736,6 +754,27 @@ extern "C" int pla_gdn_prefill_launch(
     hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   }
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
-  hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
+  if (L.seg_chunks == 0) {
+    p.pass = 0;
+    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
+  } else {
+    // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
+    p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
+    p.seg.seg_seq = reinterpret_cast<int32_t*>(ws + L.seg_seq);
+    p.seg.seg_c0 = reinterpret_cast<int32_t*>(ws + L.seg_c0);
+    p.seg.seg_nc = reinterpret_cast<int32_t*>(ws + L.seg_nc);
+    p.seg.M = reinterpret_cast<float*>(ws + L.segM);
+    p.seg.B = reinterpret_cast<float*>(ws + L.segB);
+    p.seg.S = reinterpret_cast<float*>(ws + L.segS);
+    p.seg.identity = reinterpret_cast<float*>(ws + L.identity);
+    p.seg.seg_chunks = L.seg_chunks;
+    p.seg.max_segments = L.max_segments;
+    hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
+    p.pass = 1;
+    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV * 2), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV), dim3(256), 0, s, p.seg, HV, ht, ht_indices, ht_slot_stride);
+    p.pass = 2;
+    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+  }
   return check_launch("gdn prefill launch");
 }

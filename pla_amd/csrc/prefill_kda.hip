@@ -303,53 +303,13 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int r16 = lane & 15, kb = lane >> 4;
   const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
 
-  // What this workgroup sweeps: a whole sequence, or one segment of it in one of three roles.
-  int n, h, c_begin, c_end;
-  const float* init = nullptr;        // [V, K] tile the state starts from (nullptr: zero)
-  float* fin = nullptr;               // [V, K] tile that receives the state at the end (nullptr: none)
-  bool zero_v = false, write_o = true;
-  if (p.pass == 0) {
-    n = blockIdx.x / p.H;
-    h = blockIdx.x - n * p.H;
-    c_begin = p.seq_chunk_off[n];
-    c_end = p.seq_chunk_off[n + 1];
-    if (c_begin >= c_end) return;
-    const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
-    if (slot >= 0) init = p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)h * 16384;
-    const int oslot = (p.ht != nullptr) ? (p.ht_indices ? p.ht_indices[n] : n) : -1;
-    if (oslot >= 0) fin = p.ht + (int64_t)oslot * p.ht_slot_stride + (int64_t)h * 16384;
-  } else {
-    const int item = p.pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
-    const int from_identity = p.pass == 1 ? (int)(blockIdx.x & 1) : 0;
-    const int seg = item / p.H;
-    h = item - seg * p.H;
-    if (seg >= p.seg.seq_seg_off[p.N]) return;
-    n = p.seg.seg_seq[seg];
-    const bool first = seg == p.seg.seq_seg_off[n], last = seg + 1 == p.seg.seq_seg_off[n + 1];
-    c_begin = p.seg.seg_c0[seg];
-    c_end = c_begin + p.seg.seg_nc[seg];
-    const int64_t tile = ((int64_t)seg * p.H + h) * 16384;
-    if (p.pass == 1) {
-      if (first) {
-        if (from_identity) return;
-        const int slot = (p.h0 != nullptr) ? (p.h0_indices ? p.h0_indices[n] : n) : -1;
-        if (slot >= 0) init = p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)h * 16384;
-        if (!last) {
-          fin = p.seg.B + tile;                       // the state that enters the second segment
-        } else {
-          const int oslot = (p.ht != nullptr) ? (p.ht_indices ? p.ht_indices[n] : n) : -1;
-          if (oslot >= 0) fin = p.ht + (int64_t)oslot * p.ht_slot_stride + (int64_t)h * 16384;
-        }
-      } else {
-        write_o = false;
-        if (from_identity) { init = p.seg.identity; zero_v = true; fin = p.seg.M + tile; }
-        else fin = p.seg.B + tile;
-      }
-    } else {
-      if (first) return;
-      init = p.seg.S + tile;                          // the final state came out of the combine step
-    }
-  }
+  const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride);
+  if (!role.active) return;
+  const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
+  const float* const init = role.init;
+  float* const fin = role.fin;
+  const bool zero_v = role.zero_v, write_o = role.write_o;
   const int chunk_in_seq = c_begin - p.seq_chunk_off[n];
   const int seq_start = p.cu_seqlens[n] + chunk_in_seq * CHUNK;
   const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);

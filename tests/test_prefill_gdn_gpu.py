@@ -137,3 +137,18 @@ def test_config3_gdn_prefill_32k_varlen():
     lengths = ragged_lengths(8, 512, 8192, seed=303)
     w = gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=64, seed=303)
     _check(w, fast=True)
+
+
+@pytest.mark.parametrize("lengths,tail_pad,H,HV", [([2500, 0, 1111, 40], 5, 1, 2), ([4096], 0, 2, 2), ([1030, 2049], 0, 1, 4)])
+def test_gdn_prefill_split_sequences_match_oracle(lengths, tail_pad, H, HV):
+    """Calls with few (sequence, head) chains and long sequences are split into 16-chunk segments that
+    are swept concurrently (zero-state and identity sweeps, a combine step, a second sweep): ragged
+    lengths, an empty sequence, a sequence shorter than one segment, indexed pool, against the oracle."""
+    from pla_amd import _lib
+    from pla_amd.workloads import gdn_prefill_packed
+    T, N = sum(lengths) + tail_pad, len(lengths)
+    size = _lib.load().pla_gdn_prefill_workspace_bytes
+    unsplit_per_head = size(T, N, 65 * H, 65 * HV) / (65 * HV)      # more than 64 chains are never split
+    assert size(T, N, H, HV) > 1.1 * HV * unsplit_per_head           # so this call carries the segment buffers
+    w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=N + 3, seed=99 + T, tail_pad=tail_pad)
+    _check(w, fast=True)
