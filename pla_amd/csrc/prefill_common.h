@@ -305,63 +305,57 @@ static __global__ void segment_map_kernel(const int32_t* seq_chunk_off, int N, S
   }
 }
 
-// One workgroup of 256 threads per (sequence, head): walks the sequence's segments, stores the state
-// entering each later segment and the final state.  Thread (tv, tk) owns the 8 x 8 block of S at rows
-// 8 tv, columns 8 tk; S lives in LDS between steps, M and B are streamed from global memory.
+// Eight workgroups of 256 threads per (sequence, head), each owning 16 rows of the state (rows transform
+// independently): walks the sequence's segments, stores the state entering each later segment and the
+// final state.  Thread (row, tk) owns columns 8 tk .. 8 tk + 7 of its row; the row slice of S lives in
+// LDS between steps, M and B are streamed from global memory.
+constexpr int COMBINE_SPLIT = 8;
 static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads, float* ht,
                                                                      const int32_t* ht_indices, int64_t ht_slot_stride) {
-  const int n = blockIdx.x / heads, h = blockIdx.x - n * heads;
+  const int part = blockIdx.x % COMBINE_SPLIT;
+  const int chain = blockIdx.x / COMBINE_SPLIT;
+  const int n = chain / heads, h = chain - n * heads;
   const int first = t.seq_seg_off[n], end = t.seq_seg_off[n + 1];
   if (end - first < 2) return;                 // a single segment wrote its final state itself
-  __shared__ float S[128][129];
-  const int tv = threadIdx.x >> 4, tk = threadIdx.x & 15;
-  float acc[8][8];
+  __shared__ float S[16][132];
+  const int row = threadIdx.x >> 4, tk = threadIdx.x & 15;
+  const int64_t at = (int64_t)(16 * part + row) * 128 + 8 * tk;      // this thread's place in a [128, 128] tile
+  float acc[8];
   {
-    const float* src = t.B + ((int64_t)first * heads + h) * 16384;
-#pragma unroll
-    for (int r = 0; r < 8; ++r)
-#pragma unroll
-      for (int c = 0; c < 8; ++c) acc[r][c] = src[(8 * tv + r) * 128 + 8 * tk + c];
+    const float* src = t.B + ((int64_t)first * heads + h) * 16384 + at;
+    const float4 b0 = *reinterpret_cast<const float4*>(src), b1 = *reinterpret_cast<const float4*>(src + 4);
+    acc[0] = b0.x; acc[1] = b0.y; acc[2] = b0.z; acc[3] = b0.w; acc[4] = b1.x; acc[5] = b1.y; acc[6] = b1.z; acc[7] = b1.w;
   }
   for (int seg = first + 1; seg < end; ++seg) {
     const int64_t tile = ((int64_t)seg * heads + h) * 16384;
-    float* sin = t.S + tile;
-#pragma unroll
-    for (int r = 0; r < 8; ++r) {
-#pragma unroll
-      for (int c = 0; c < 8; ++c) S[8 * tv + r][8 * tk + c] = acc[r][c];
-      *reinterpret_cast<float4*>(sin + (8 * tv + r) * 128 + 8 * tk) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
-      *reinterpret_cast<float4*>(sin + (8 * tv + r) * 128 + 8 * tk + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
-    }
+    *reinterpret_cast<float4*>(&S[row][8 * tk]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4*>(&S[row][8 * tk + 4]) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    *reinterpret_cast<float4*>(t.S + tile + at) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4*>(t.S + tile + at + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
     __syncthreads();
-    const float* Mt = t.M + tile;
-    const float* Bt = t.B + tile;
-#pragma unroll
-    for (int r = 0; r < 8; ++r)
-#pragma unroll
-      for (int c = 0; c < 8; ++c) acc[r][c] = Bt[(8 * tv + r) * 128 + 8 * tk + c];
+    const float* Mt = t.M + tile + 8 * tk;
+    {
+      const float4 b0 = *reinterpret_cast<const float4*>(t.B + tile + at);
+      const float4 b1 = *reinterpret_cast<const float4*>(t.B + tile + at + 4);
+      acc[0] = b0.x; acc[1] = b0.y; acc[2] = b0.z; acc[3] = b0.w; acc[4] = b1.x; acc[5] = b1.y; acc[6] = b1.z; acc[7] = b1.w;
+    }
+#pragma unroll 8
     for (int j = 0; j < 128; ++j) {
-      const float4 m0 = *reinterpret_cast<const float4*>(Mt + j * 128 + 8 * tk);
-      const float4 m1 = *reinterpret_cast<const float4*>(Mt + j * 128 + 8 * tk + 4);
-      const float mrow[8] = {m0.x, m0.y, m0.z, m0.w, m1.x, m1.y, m1.z, m1.w};
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        const float sv = S[8 * tv + r][j];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) acc[r][c] = fmaf(sv, mrow[c], acc[r][c]);
-      }
+      const float4 m0 = *reinterpret_cast<const float4*>(Mt + j * 128);
+      const float4 m1 = *reinterpret_cast<const float4*>(Mt + j * 128 + 4);
+      const float sv = S[row][j];
+      acc[0] = fmaf(sv, m0.x, acc[0]); acc[1] = fmaf(sv, m0.y, acc[1]); acc[2] = fmaf(sv, m0.z, acc[2]);
+      acc[3] = fmaf(sv, m0.w, acc[3]); acc[4] = fmaf(sv, m1.x, acc[4]); acc[5] = fmaf(sv, m1.y, acc[5]);
+      acc[6] = fmaf(sv, m1.z, acc[6]); acc[7] = fmaf(sv, m1.w, acc[7]);
     }
     __syncthreads();
   }
   if (ht != nullptr) {
     const int slot = ht_indices ? ht_indices[n] : n;
     if (slot >= 0) {
-      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384;
-#pragma unroll
-      for (int r = 0; r < 8; ++r) {
-        *reinterpret_cast<float4*>(dst + (8 * tv + r) * 128 + 8 * tk) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
-        *reinterpret_cast<float4*>(dst + (8 * tv + r) * 128 + 8 * tk + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
-      }
+      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384 + at;
+      *reinterpret_cast<float4*>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
     }
   }
 }

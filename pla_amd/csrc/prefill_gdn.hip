@@ -772,7 +772,7 @@ extern "C" int pla_gdn_prefill_launch(
     hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
     p.pass = 1;
     hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV * 2), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV), dim3(256), 0, s, p.seg, HV, ht, ht_indices, ht_slot_stride);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht, ht_indices, ht_slot_stride);
     p.pass = 2;
     hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
   }

@@ -729,7 +729,7 @@ extern "C" int pla_kda_prefill_launch(
     hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
     p.pass = 1;
     hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H * 2), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H), dim3(256), 0, s, p.seg, H, ht, ht_indices, ht_slot_stride);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht, ht_indices, ht_slot_stride);
     p.pass = 2;
     hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
   }
