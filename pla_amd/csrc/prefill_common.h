@@ -219,8 +219,62 @@ struct SegmentTable {
   int max_segments;
 };
 
+// ---------------------------------------------------------------------------------------------
+// Stages: with enough chains to fill the chip the per-chunk preparation (which every CU works on) and
+// the sequential sweep (one workgroup per chain, most of a CU idle) are pipelined.  Each sequence is cut
+// into `stages` consecutive parts; stage s of the sweep needs only the preparation of stage s, so the
+// preparation of stage s + 1 runs on a second stream underneath the sweep of stage s.  The state is
+// carried from stage to stage through one [V, K] tile per chain.
+struct StageTable {
+  int32_t* order;         // [chunks] global chunk ids, all of stage 0 first, then stage 1, ...
+  int32_t* stage_begin;   // [stages + 1] offsets into `order`
+  int32_t* seq_stage_lo;  // [N, stages + 1] first chunk (local to the sequence) of each stage
+  float* carry;           // [N, heads, V, K]
+  int stages;             // 0: not staged
+};
+constexpr int MAX_STAGES = 4;
+
+// Single workgroup of 256 threads, after chunk_map_kernel.  Thread (stage, sequence) pairs count their
+// chunks, a serial prefix over the stages x N counts places them, then every pair writes its own ids.
+static __global__ void stage_map_kernel(const int32_t* seq_chunk_off, int N, int NC_max, StageTable t) {
+  extern __shared__ int32_t pair_begin[];              // [stages * N + 1]
+  const int S = t.stages;
+  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+    const int nc = seq_chunk_off[n + 1] - seq_chunk_off[n];
+    for (int s = 0; s <= S; ++s) t.seq_stage_lo[n * (S + 1) + s] = (int)((int64_t)nc * s / S);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int k = 0;
+    for (int s = 0; s < S; ++s) {
+      t.stage_begin[s] = k;
+      for (int n = 0; n < N; ++n) {
+        pair_begin[s * N + n] = k;
+        k += t.seq_stage_lo[n * (S + 1) + s + 1] - t.seq_stage_lo[n * (S + 1) + s];
+      }
+    }
+    pair_begin[S * N] = k;
+    t.stage_begin[S] = k;
+  }
+  __syncthreads();
+  for (int pair = threadIdx.x >> 3; pair < S * N; pair += blockDim.x >> 3) {      // eight threads per pair
+    const int s = pair / N, n = pair - s * N;
+    const int lo = t.seq_stage_lo[n * (S + 1) + s], hi = t.seq_stage_lo[n * (S + 1) + s + 1];
+    const int base = pair_begin[pair];
+    for (int cc = lo + (threadIdx.x & 7); cc < hi; cc += 8)
+      if (base + cc - lo < NC_max) t.order[base + cc - lo] = seq_chunk_off[n] + cc;
+  }
+}
+// Chunk handled by workgroup `index` of a per-chunk kernel: all chunks in order, or those of one stage.
+__device__ __forceinline__ int staged_chunk(const StageTable& t, int stage, int index, int total_chunks) {
+  if (t.stages == 0) return index < total_chunks ? index : -1;
+  const int begin = t.stage_begin[stage], end = t.stage_begin[stage + 1];
+  return begin + index < end ? t.order[begin + index] : -1;
+}
+
 // What one workgroup of a sequential kernel sweeps: a whole sequence (pass 0) or one segment in one of
-// the roles above (pass 1: blockIdx = (segment, head, from-identity flag); pass 2: (segment, head)).
+// the roles above (pass 1: blockIdx = (segment, head, from-identity flag); pass 2: (segment, head)), or one
+// stage of a sequence (pass 3: blockIdx = (sequence, head)).
 struct SweepRole {
   int n, head, c_begin, c_end;
   const float* init;      // [V, K] tile the state starts from (nullptr: zero)
@@ -228,7 +282,8 @@ struct SweepRole {
   bool zero_v, write_o, active;
 };
 __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, const int32_t* seq_chunk_off,
-                                                  const SegmentTable& seg, const float* h0, const int32_t* h0_indices,
+                                                  const SegmentTable& seg, const StageTable& stg, int stage,
+                                                  const float* h0, const int32_t* h0_indices,
                                                   int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
                                                   int64_t ht_slot_stride) {
   SweepRole r{};
@@ -249,6 +304,19 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     if (r.c_begin >= r.c_end) return r;              // empty sequence: state untouched, no output
     r.init = state_in(r.n, r.head);
     r.fin = state_out(r.n, r.head);
+    r.active = true;
+    return r;
+  }
+  if (pass == 3) {                                   // one stage of every sequence; may hold no chunk at all
+    r.n = blockIdx.x / heads;
+    r.head = blockIdx.x - r.n * heads;
+    if (seq_chunk_off[r.n] >= seq_chunk_off[r.n + 1]) return r;
+    const int32_t* lo = stg.seq_stage_lo + r.n * (stg.stages + 1);
+    r.c_begin = seq_chunk_off[r.n] + lo[stage];
+    r.c_end = seq_chunk_off[r.n] + lo[stage + 1];
+    float* carry = stg.carry + ((int64_t)r.n * heads + r.head) * 16384;
+    r.init = stage == 0 ? state_in(r.n, r.head) : carry;
+    r.fin = stage == stg.stages - 1 ? state_out(r.n, r.head) : carry;
     r.active = true;
     return r;
   }

@@ -54,7 +54,9 @@ struct GdnPrefillParams {
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
   SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
-  int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments
+  StageTable stg;        // pipelined preparation and sweep (stg.stages > 0)
+  int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments; 3: one stage
+  int stage;             // stage handled by this launch (per-chunk kernels and pass 3)
   int H, HV, NC_max;
 };
 
@@ -64,8 +66,8 @@ struct GdnPrefillParams {
 // the transposed K tile; blockIdx.y == H: gate, beta and the chunk-local cumulative log-decay.
 template <typename act_t>
 __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
-  const int cb = blockIdx.x;
-  if (cb >= p.seq_chunk_off[p.N]) return;
+  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x, p.seq_chunk_off[p.N]);
+  if (cb < 0) return;
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -169,9 +171,9 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
 // ---------------------------------------------------------------------------------------------
 // One wavefront per (chunk, value head).
 __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillParams p) {
-  const int cb = blockIdx.x / p.HV;
-  const int hv = blockIdx.x - cb * p.HV;
-  if (cb >= p.seq_chunk_off[p.N]) return;
+  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / p.HV, p.seq_chunk_off[p.N]);
+  const int hv = blockIdx.x % p.HV;
+  if (cb < 0) return;
   const int h = hv / (p.HV / p.H);
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
@@ -308,7 +310,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
   using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
-  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.h0, p.h0_indices, p.h0_slot_stride,
+  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
@@ -421,9 +423,11 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
             *reinterpret_cast<const uint4*>(&tO[(krow + FLUSH_ROWS * i) * PITCH128 + 8 * kcv]);
   };
 
-  issue_gates(0);
-  issue_kqv(0);
-  issue_w(0);
+  if (n_chunks > 0) {                                // a stage of a short sequence may hold no chunk
+    issue_gates(0);
+    issue_kqv(0);
+    issue_w(0);
+  }
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
@@ -635,7 +639,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       }
   }
   __syncthreads();
-  flush_output(n_chunks - 1);
+  if (n_chunks > 0) flush_output(n_chunks - 1);
 
   if (role.fin != nullptr) {
 #pragma unroll
@@ -650,8 +654,9 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P;
-  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity, total;
-  int NC_max, seg_chunks, max_segments;
+  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
+  size_t order, stage_begin, seq_stage_lo, carry, total;
+  int NC_max, seg_chunks, max_segments, stages;
 };
 static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   GdnWorkspaceLayout L;
@@ -682,8 +687,39 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
     L.segM = take(states); L.segB = take(states); L.segS = take(states);
     L.identity = take(16384 * 4);
   }
+  // enough chains and enough chunks per chain: pipeline the preparation with the sweep in stages
+  L.stages = (L.seg_chunks == 0 && (int64_t)N * HV >= 128 && T / CHUNK >= 16 * N) ? MAX_STAGES : 0;
+  if (L.stages > 0) {
+    L.order = take((size_t)L.NC_max * 4);
+    L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);
+    L.seq_stage_lo = take((size_t)N * (MAX_STAGES + 1) * 4);
+    L.carry = take((size_t)N * HV * 16384 * 4);
+  }
   L.total = off;
   return L;
+}
+
+// One side stream (default priority, non-blocking) and its events per device, created on first use and
+// kept for the life of the process.  Calls are expected from one host thread at a time per device.
+struct SideStream {
+  hipStream_t stream;
+  hipEvent_t fork;
+  hipEvent_t ready[MAX_STAGES];
+};
+static SideStream* side_stream() {
+  static SideStream table[16];
+  static bool made[16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  if (!made[dev]) {
+    SideStream& t = table[dev];
+    if (hipStreamCreateWithFlags(&t.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
+    if (hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
+    for (int i = 0; i < MAX_STAGES; ++i)
+      if (hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) != hipSuccess) return nullptr;
+    made[dev] = true;
+  }
+  return &table[dev];
 }
 
 }  // namespace pla
@@ -748,11 +784,38 @@ extern "C" int pla_gdn_prefill_launch(
   hipLaunchKernelGGL(chunk_map_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, N, L.NC_max, p.seq_chunk_off,
                      p.chunk_seq, p.chunk_tok, p.chunk_len);
   hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, HV);
-  if (act_dtype == PLA_BF16) {
-    hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
-  } else {
-    hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
+  if (L.stages > 0) {
+    // The caller's stream sweeps stage after stage; a side stream prepares the next stages underneath.
+    SideStream* side = side_stream();
+    PLA_REQUIRE(side != nullptr, "could not create the side stream for the staged prefill");
+    p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
+    p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
+    p.stg.seq_stage_lo = reinterpret_cast<int32_t*>(ws + L.seq_stage_lo);
+    p.stg.carry = reinterpret_cast<float*>(ws + L.carry);
+    p.stg.stages = L.stages;
+    p.pass = 3;
+    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * N + 1) * 4, s, p.seq_chunk_off, N,
+                       L.NC_max, p.stg);
+    for (int st = 0; st < L.stages; ++st) {
+      p.stage = st;
+      hipStream_t ps = st == 0 ? s : side->stream;            // stage 0 is prepared on the caller's stream, alone
+      hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
+      hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
+      if (st == 0) {
+        hipEventRecord(side->fork, s);
+        hipStreamWaitEvent(side->stream, side->fork, 0);
+      } else {
+        hipEventRecord(side->ready[st], side->stream);
+      }
+    }
+    for (int st = 0; st < L.stages; ++st) {
+      p.stage = st;
+      if (st > 0) hipStreamWaitEvent(s, side->ready[st], 0);
+      hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
+    }
+    return check_launch("gdn prefill launch");
   }
+  hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
   hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
   if (L.seg_chunks == 0) {
     p.pass = 0;

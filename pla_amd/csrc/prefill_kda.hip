@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int r16 = lane & 15, kb = lane >> 4;
   const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
 
-  const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.h0, p.h0_indices, p.h0_slot_stride,
+  const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, StageTable{}, 0, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;

@@ -152,3 +152,38 @@ def test_gdn_prefill_split_sequences_match_oracle(lengths, tail_pad, H, HV):
     assert size(T, N, H, HV) > 1.1 * HV * unsplit_per_head           # so this call carries the segment buffers
     w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=N + 3, seed=99 + T, tail_pad=tail_pad)
     _check(w, fast=True)
+
+
+def test_gdn_prefill_staged_pipeline_matches_oracle_and_unstaged_bits():
+    """With at least 128 chains and 16 chunks per sequence on average the preparation and the sweep
+    are pipelined in stages on two streams.  Ragged lengths with an empty sequence and sequences
+    shorter than the number of stages (empty stages), against the oracle; and the same tokens run
+    sequence by sequence (too few chains to be staged) give bit-identical o and states."""
+    from pla_amd.workloads import gdn_prefill_packed
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    lengths = [3000, 0, 70, 1500, 64, 2100, 1, 1500]
+    H, HV = 4, 16
+    w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=777, tail_pad=7)
+    pool0 = w["initial_state"].clone()
+    _check(w, fast=True)
+    # rerun staged on a fresh pool, keep o and pool
+    w["initial_state"].copy_(pool0)
+    _, _, o_staged, _, _ = _run_workload(w)
+    pool_staged = w["initial_state"].clone()
+    # one call per sequence: 16 chains each, never staged; the long ones are split into segments, so
+    # only the short sequences (a single segment) are compared bit for bit
+    w["initial_state"].copy_(pool0)
+    offs = w["_meta"]["offsets"]
+    idx = w["initial_state_indices"]
+    for n, length in enumerate(lengths):
+        if length == 0 or length >= 2048:
+            continue
+        lo, hi = offs[n], offs[n + 1]
+        cu = torch.tensor([0, hi - lo], dtype=torch.int32, device="cuda")
+        r = gdn_prefill_packed_qkv_fwd(w["packed_qkv"][lo:hi], w["raw_gate_a"][lo:hi], w["raw_beta_b"][lo:hi],
+                                       w["A_log"], w["dt_bias"], cu, num_qk_heads=H, num_v_heads=HV, scale=w["scale"],
+                                       initial_state=w["initial_state"], initial_state_indices=idx[n:n + 1])
+        torch.cuda.synchronize()
+        assert torch.equal(r[2][0], o_staged[0, lo:hi]), n
+        slot = int(idx[n])
+        assert torch.equal(w["initial_state"][slot], pool_staged[slot]), n
