@@ -187,3 +187,35 @@ def test_gdn_prefill_staged_pipeline_matches_oracle_and_unstaged_bits():
         assert torch.equal(r[2][0], o_staged[0, lo:hi]), n
         slot = int(idx[n])
         assert torch.equal(w["initial_state"][slot], pool_staged[slot]), n
+
+
+def test_gdn_prefill_staged_pipeline_in_a_graph():
+    """The staged call forks to a side stream and joins again, so it can be captured: three replays with
+    eager work and synchronisation in between reproduce the eager result bit for bit."""
+    from pla_amd.workloads import gdn_prefill_packed
+    lengths = [1500, 2100, 900, 1500, 1300, 1100, 700, 1200]
+    w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 2, seed=31)
+    pool0 = w["initial_state"].clone()
+    _, _, o_eager, _, _ = _run_workload(w, output_final_state=False)
+    torch.cuda.synchronize()
+    pool_eager = w["initial_state"].clone()
+    w["initial_state"].copy_(pool0)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        _run_workload(w, output_final_state=False)            # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    w["initial_state"].copy_(pool0)
+    with torch.cuda.graph(graph, stream=stream):
+        _, _, o_graph, _, _ = _run_workload(w, output_final_state=False)
+    for replay in range(3):
+        w["initial_state"].copy_(pool0)
+        o_graph.zero_()
+        scratch = torch.randn(1 << 20, device="cuda").sum().item()     # eager work and a sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert scratch == scratch
+        assert torch.equal(o_graph, o_eager), replay
+        assert torch.equal(w["initial_state"], pool_eager), replay
