@@ -182,13 +182,14 @@ static __global__ void chunk_map_kernel(const int32_t* cu_seqlens, int N, int NC
     seq_chunk_off[N] = acc;
   }
   __syncthreads();
-  for (int n = threadIdx.x; n < N; n += blockDim.x) {
+  // one wavefront per sequence, its lanes stride over the chunks
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
+  for (int n = wave; n < N; n += waves) {
     const int start = cu_seqlens[n];
     const int len = max(cu_seqlens[n + 1] - start, 0);
     const int c0 = seq_chunk_off[n];
     const int nc = (len + CHUNK - 1) / CHUNK;
-    for (int c = 0; c < nc; ++c) {
-      if (c0 + c >= NC_max) break;
+    for (int c = lane; c < nc && c0 + c < NC_max; c += 64) {
       chunk_seq[c0 + c] = n;
       chunk_tok[c0 + c] = start + c * CHUNK;
       chunk_len[c0 + c] = min(CHUNK, len - c * CHUNK);
@@ -228,41 +229,42 @@ struct SegmentTable {
 struct StageTable {
   int32_t* order;         // [chunks] global chunk ids, all of stage 0 first, then stage 1, ...
   int32_t* stage_begin;   // [stages + 1] offsets into `order`
-  int32_t* seq_stage_lo;  // [N, stages + 1] first chunk (local to the sequence) of each stage
-  float* carry;           // [N, heads, V, K]
+  float* carry;           // [N, heads, V, K] (whole sequences; segments carry in their own tiles)
   int stages;             // 0: not staged
 };
 constexpr int MAX_STAGES = 4;
+// Chunks [lo, hi) of an item of `nc` chunks that belong to stage s of S.
+__device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((int64_t)nc * s / S); }
 
-// Single workgroup of 256 threads, after chunk_map_kernel.  Thread (stage, sequence) pairs count their
-// chunks, a serial prefix over the stages x N counts places them, then every pair writes its own ids.
-static __global__ void stage_map_kernel(const int32_t* seq_chunk_off, int N, int NC_max, StageTable t) {
-  extern __shared__ int32_t pair_begin[];              // [stages * N + 1]
+// Single workgroup of 256 threads.  The items are sequences (`counts` null: item i holds chunks
+// starts[i] .. starts[i + 1]) or segments (chunks starts[i] .. starts[i] + counts[i]); `n_items` is read
+// on the device.  (Stage, item) pairs count their chunks, a serial prefix places them, then every pair
+// writes its own chunk ids.
+static __global__ void stage_map_kernel(const int32_t* starts, const int32_t* counts, const int32_t* n_items_ptr,
+                                        int n_items_max, int NC_max, StageTable t) {
+  extern __shared__ int32_t pair_begin[];              // [stages * n_items_max + 1]
   const int S = t.stages;
-  for (int n = threadIdx.x; n < N; n += blockDim.x) {
-    const int nc = seq_chunk_off[n + 1] - seq_chunk_off[n];
-    for (int s = 0; s <= S; ++s) t.seq_stage_lo[n * (S + 1) + s] = (int)((int64_t)nc * s / S);
-  }
-  __syncthreads();
+  const int n_items = n_items_ptr ? min(*n_items_ptr, n_items_max) : n_items_max;
+  auto count_of = [&](int i) { return counts ? counts[i] : starts[i + 1] - starts[i]; };
   if (threadIdx.x == 0) {
     int k = 0;
     for (int s = 0; s < S; ++s) {
       t.stage_begin[s] = k;
-      for (int n = 0; n < N; ++n) {
-        pair_begin[s * N + n] = k;
-        k += t.seq_stage_lo[n * (S + 1) + s + 1] - t.seq_stage_lo[n * (S + 1) + s];
+      for (int i = 0; i < n_items; ++i) {
+        const int nc = count_of(i);
+        pair_begin[s * n_items + i] = k;
+        k += stage_cut(nc, s + 1, S) - stage_cut(nc, s, S);
       }
     }
-    pair_begin[S * N] = k;
     t.stage_begin[S] = k;
   }
   __syncthreads();
-  for (int pair = threadIdx.x >> 3; pair < S * N; pair += blockDim.x >> 3) {      // eight threads per pair
-    const int s = pair / N, n = pair - s * N;
-    const int lo = t.seq_stage_lo[n * (S + 1) + s], hi = t.seq_stage_lo[n * (S + 1) + s + 1];
+  for (int pair = threadIdx.x >> 3; pair < S * n_items; pair += blockDim.x >> 3) {      // eight threads per pair
+    const int s = pair / n_items, i = pair - s * n_items;
+    const int nc = count_of(i), lo = stage_cut(nc, s, S), hi = stage_cut(nc, s + 1, S);
     const int base = pair_begin[pair];
     for (int cc = lo + (threadIdx.x & 7); cc < hi; cc += 8)
-      if (base + cc - lo < NC_max) t.order[base + cc - lo] = seq_chunk_off[n] + cc;
+      if (base + cc - lo < NC_max) t.order[base + cc - lo] = starts[i] + cc;
   }
 }
 // Chunk handled by workgroup `index` of a per-chunk kernel: all chunks in order, or those of one stage.
@@ -272,9 +274,10 @@ __device__ __forceinline__ int staged_chunk(const StageTable& t, int stage, int 
   return begin + index < end ? t.order[begin + index] : -1;
 }
 
-// What one workgroup of a sequential kernel sweeps: a whole sequence (pass 0) or one segment in one of
-// the roles above (pass 1: blockIdx = (segment, head, from-identity flag); pass 2: (segment, head)), or one
-// stage of a sequence (pass 3: blockIdx = (sequence, head)).
+// What one workgroup of a sequential kernel sweeps: a whole sequence (pass 0, blockIdx = (sequence,
+// head)) or one segment in one of the roles above (pass 1: blockIdx = (segment, head, from-identity
+// flag); pass 2: (segment, head)); with stages (passes 0 and 1) only the part of it that belongs to
+// `stage`, which may hold no chunk at all, the state being carried from stage to stage in a tile.
 struct SweepRole {
   int n, head, c_begin, c_end;
   const float* init;      // [V, K] tile the state starts from (nullptr: zero)
@@ -296,6 +299,7 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     const int slot = (ht != nullptr) ? (ht_indices ? ht_indices[n] : n) : -1;
     return slot >= 0 ? ht + (int64_t)slot * ht_slot_stride + (int64_t)head * 16384 : nullptr;
   };
+  float* carry = nullptr;
   if (pass == 0) {
     r.n = blockIdx.x / heads;
     r.head = blockIdx.x - r.n * heads;
@@ -304,45 +308,41 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     if (r.c_begin >= r.c_end) return r;              // empty sequence: state untouched, no output
     r.init = state_in(r.n, r.head);
     r.fin = state_out(r.n, r.head);
-    r.active = true;
-    return r;
-  }
-  if (pass == 3) {                                   // one stage of every sequence; may hold no chunk at all
-    r.n = blockIdx.x / heads;
-    r.head = blockIdx.x - r.n * heads;
-    if (seq_chunk_off[r.n] >= seq_chunk_off[r.n + 1]) return r;
-    const int32_t* lo = stg.seq_stage_lo + r.n * (stg.stages + 1);
-    r.c_begin = seq_chunk_off[r.n] + lo[stage];
-    r.c_end = seq_chunk_off[r.n] + lo[stage + 1];
-    float* carry = stg.carry + ((int64_t)r.n * heads + r.head) * 16384;
-    r.init = stage == 0 ? state_in(r.n, r.head) : carry;
-    r.fin = stage == stg.stages - 1 ? state_out(r.n, r.head) : carry;
-    r.active = true;
-    return r;
-  }
-  const int item = pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
-  const bool from_identity = pass == 1 && (blockIdx.x & 1);
-  const int s = item / heads;
-  r.head = item - s * heads;
-  if (s >= seg.seq_seg_off[N]) return r;
-  r.n = seg.seg_seq[s];
-  const bool first = s == seg.seq_seg_off[r.n], last = s + 1 == seg.seq_seg_off[r.n + 1];
-  r.c_begin = seg.seg_c0[s];
-  r.c_end = r.c_begin + seg.seg_nc[s];
-  const int64_t tile = ((int64_t)s * heads + r.head) * 16384;
-  if (pass == 1) {
-    if (first) {
-      if (from_identity) return r;
-      r.init = state_in(r.n, r.head);
-      r.fin = last ? state_out(r.n, r.head) : seg.B + tile;     // B of a first segment: the state entering the second
-    } else {
-      r.write_o = false;
-      if (from_identity) { r.init = seg.identity; r.zero_v = true; r.fin = seg.M + tile; }
-      else r.fin = seg.B + tile;
-    }
+    if (stg.stages > 0) carry = stg.carry + ((int64_t)r.n * heads + r.head) * 16384;
   } else {
-    if (first) return r;
-    r.init = seg.S + tile;                            // the final state came out of the combine step
+    const int item = pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
+    const bool from_identity = pass == 1 && (blockIdx.x & 1);
+    const int s = item / heads;
+    r.head = item - s * heads;
+    if (s >= seg.seq_seg_off[N]) return r;
+    r.n = seg.seg_seq[s];
+    const bool first = s == seg.seq_seg_off[r.n], last = s + 1 == seg.seq_seg_off[r.n + 1];
+    r.c_begin = seg.seg_c0[s];
+    r.c_end = r.c_begin + seg.seg_nc[s];
+    const int64_t tile = ((int64_t)s * heads + r.head) * 16384;
+    if (pass == 1) {
+      if (first) {
+        if (from_identity) return r;
+        r.init = state_in(r.n, r.head);
+        r.fin = last ? state_out(r.n, r.head) : seg.B + tile;   // B of a first segment: the state entering the second
+        carry = seg.B + tile;
+      } else {
+        r.write_o = false;
+        if (from_identity) { r.init = seg.identity; r.zero_v = true; r.fin = seg.M + tile; }
+        else r.fin = seg.B + tile;
+        carry = r.fin;
+      }
+    } else {
+      if (first) return r;
+      r.init = seg.S + tile;                          // the final state came out of the combine step
+    }
+  }
+  if (carry != nullptr && stg.stages > 0) {
+    const int nc = r.c_end - r.c_begin, c0 = r.c_begin;
+    r.c_begin = c0 + stage_cut(nc, stage, stg.stages);
+    r.c_end = c0 + stage_cut(nc, stage + 1, stg.stages);
+    if (stage > 0) r.init = carry;
+    if (stage < stg.stages - 1) r.fin = carry;
   }
   r.active = true;
   return r;
@@ -449,5 +449,74 @@ static __global__ void zero_tail_kernel(uint16_t* o, const int32_t* cu_seqlens, 
 }
 
 inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// One side stream (default priority, non-blocking) and its events per device, created on first use and
+// kept for the life of the process.  Calls are expected from one host thread at a time per device.
+struct SideStream {
+  hipStream_t stream;
+  hipEvent_t fork;
+  hipEvent_t ready[MAX_STAGES];
+};
+static inline SideStream* side_stream() {
+  static SideStream table[16];
+  static bool made[16] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  if (!made[dev]) {
+    SideStream& t = table[dev];
+    if (hipStreamCreateWithFlags(&t.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
+    if (hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
+    for (int i = 0; i < MAX_STAGES; ++i)
+      if (hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) != hipSuccess) return nullptr;
+    made[dev] = true;
+  }
+  return &table[dev];
+}
+
+// Number of stages for a call of whole sequences: enough chains to fill the chip and 16 chunks per
+// sequence on average.  (Segmented calls already keep every CU busy with sweeps; and staging only pays
+// where a preparation workgroup fits into a CU next to a sweep workgroup, which holds for GDN - 115 KB
+// + 18 or 33 KB of LDS - and not for KDA - 149 KB + 69 KB -, where it was measured to double the sweep
+// times.)
+inline int pick_stages(int T, int N, int heads, int seg_chunks) {
+  if (seg_chunks > 0) return 0;
+  return ((int64_t)N * heads >= 128 && T / CHUNK >= 16 * N) ? MAX_STAGES : 0;
+}
+
+// Launch order of a prefill call, shared by both paths.  `prepare(stream)` launches the per-chunk
+// kernels of stage *stage_field, `sweep(grid)` the sequential kernel for (*pass_field, *stage_field).
+// Stage 0 is prepared on the caller's stream, alone; the side stream prepares the other stages
+// underneath the sweeps and is joined before the last sweep starts.
+template <typename Prepare, typename Sweep>
+inline bool launch_pipeline(hipStream_t s, int stages, bool segmented, unsigned grid_whole, unsigned grid_segments,
+                            int* pass_field, int* stage_field, Prepare prepare, Sweep sweep) {
+  *pass_field = segmented ? 1 : 0;
+  const unsigned grid = segmented ? 2 * grid_segments : grid_whole;
+  if (stages == 0) {
+    *stage_field = 0;
+    prepare(s);
+    sweep(grid);
+    return true;
+  }
+  SideStream* side = side_stream();
+  if (side == nullptr) return false;
+  bool ok = true;
+  for (int st = 0; st < stages; ++st) {
+    *stage_field = st;
+    prepare(st == 0 ? s : side->stream);
+    if (st == 0) {
+      ok = ok && hipEventRecord(side->fork, s) == hipSuccess;
+      ok = ok && hipStreamWaitEvent(side->stream, side->fork, 0) == hipSuccess;
+    } else {
+      ok = ok && hipEventRecord(side->ready[st], side->stream) == hipSuccess;
+    }
+  }
+  for (int st = 0; st < stages; ++st) {
+    *stage_field = st;
+    if (st > 0) ok = ok && hipStreamWaitEvent(s, side->ready[st], 0) == hipSuccess;
+    sweep(grid);
+  }
+  return ok;
+}
 
 }  // namespace pla

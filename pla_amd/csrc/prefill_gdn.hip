@@ -55,7 +55,7 @@ struct GdnPrefillParams {
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
   SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
   StageTable stg;        // pipelined preparation and sweep (stg.stages > 0)
-  int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments; 3: one stage
+  int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments
   int stage;             // stage handled by this launch (per-chunk kernels and pass 3)
   int H, HV, NC_max;
 };
@@ -655,7 +655,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
-  size_t order, stage_begin, seq_stage_lo, carry, total;
+  size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
 };
 static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
@@ -687,39 +687,15 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
     L.segM = take(states); L.segB = take(states); L.segS = take(states);
     L.identity = take(16384 * 4);
   }
-  // enough chains and enough chunks per chain: pipeline the preparation with the sweep in stages
-  L.stages = (L.seg_chunks == 0 && (int64_t)N * HV >= 128 && T / CHUNK >= 16 * N) ? MAX_STAGES : 0;
+  // pipeline the preparation with the sweeps in stages where that pays
+  L.stages = pick_stages(T, N, HV, L.seg_chunks);
   if (L.stages > 0) {
     L.order = take((size_t)L.NC_max * 4);
     L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);
-    L.seq_stage_lo = take((size_t)N * (MAX_STAGES + 1) * 4);
-    L.carry = take((size_t)N * HV * 16384 * 4);
+    L.carry = L.seg_chunks > 0 ? 0 : take((size_t)N * HV * 16384 * 4);
   }
   L.total = off;
   return L;
-}
-
-// One side stream (default priority, non-blocking) and its events per device, created on first use and
-// kept for the life of the process.  Calls are expected from one host thread at a time per device.
-struct SideStream {
-  hipStream_t stream;
-  hipEvent_t fork;
-  hipEvent_t ready[MAX_STAGES];
-};
-static SideStream* side_stream() {
-  static SideStream table[16];
-  static bool made[16] = {};
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-  if (!made[dev]) {
-    SideStream& t = table[dev];
-    if (hipStreamCreateWithFlags(&t.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
-    if (hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
-    for (int i = 0; i < MAX_STAGES; ++i)
-      if (hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) != hipSuccess) return nullptr;
-    made[dev] = true;
-  }
-  return &table[dev];
 }
 
 }  // namespace pla
@@ -784,43 +760,8 @@ extern "C" int pla_gdn_prefill_launch(
   hipLaunchKernelGGL(chunk_map_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, N, L.NC_max, p.seq_chunk_off,
                      p.chunk_seq, p.chunk_tok, p.chunk_len);
   hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, HV);
-  if (L.stages > 0) {
-    // The caller's stream sweeps stage after stage; a side stream prepares the next stages underneath.
-    SideStream* side = side_stream();
-    PLA_REQUIRE(side != nullptr, "could not create the side stream for the staged prefill");
-    p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
-    p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
-    p.stg.seq_stage_lo = reinterpret_cast<int32_t*>(ws + L.seq_stage_lo);
-    p.stg.carry = reinterpret_cast<float*>(ws + L.carry);
-    p.stg.stages = L.stages;
-    p.pass = 3;
-    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * N + 1) * 4, s, p.seq_chunk_off, N,
-                       L.NC_max, p.stg);
-    for (int st = 0; st < L.stages; ++st) {
-      p.stage = st;
-      hipStream_t ps = st == 0 ? s : side->stream;            // stage 0 is prepared on the caller's stream, alone
-      hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
-      hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
-      if (st == 0) {
-        hipEventRecord(side->fork, s);
-        hipStreamWaitEvent(side->stream, side->fork, 0);
-      } else {
-        hipEventRecord(side->ready[st], side->stream);
-      }
-    }
-    for (int st = 0; st < L.stages; ++st) {
-      p.stage = st;
-      if (st > 0) hipStreamWaitEvent(s, side->ready[st], 0);
-      hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
-    }
-    return check_launch("gdn prefill launch");
-  }
-  hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, s, p);
-  hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, s, p);
-  if (L.seg_chunks == 0) {
-    p.pass = 0;
-    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)N * HV), dim3(256), 0, s, p);
-  } else {
+  const bool segmented = L.seg_chunks > 0;
+  if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
     p.seg.seg_seq = reinterpret_cast<int32_t*>(ws + L.seg_seq);
@@ -833,9 +774,28 @@ extern "C" int pla_gdn_prefill_launch(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
     hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
-    p.pass = 1;
-    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV * 2), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht, ht_indices, ht_slot_stride);
+  }
+  if (L.stages > 0) {
+    p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
+    p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
+    p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
+    p.stg.stages = L.stages;
+    const int items = segmented ? L.max_segments : N;
+    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * items + 1) * 4, s,
+                       segmented ? p.seg.seg_c0 : p.seq_chunk_off, segmented ? p.seg.seg_nc : nullptr,
+                       segmented ? p.seg.seq_seg_off + N : nullptr, items, L.NC_max, p.stg);
+  }
+  const bool ok = launch_pipeline(
+      s, L.stages, segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
+      [&](hipStream_t ps) {
+        hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
+        hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
+      },
+      [&](unsigned grid) { hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3(grid), dim3(256), 0, s, p); });
+  PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
+  if (segmented) {
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
+                       ht_indices, ht_slot_stride);
     p.pass = 2;
     hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
   }

@@ -44,7 +44,9 @@ struct KdaPrefillParams {
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;       // [chunk, H, 64, 64]
   float* eGlast;                                   // [chunk, H, 128]: e^{G_last}
   SegmentTable seg;                                // split long sequences (seg.seg_chunks > 0)
+  StageTable stg;                                  // pipelined preparation and sweep (stg.stages > 0)
   int pass;                                        // 0: whole sequences; 1, 2: the two sweeps over segments
+  int stage;                                       // stage handled by this launch (prep kernel, passes 0 and 1)
   int H, NC_max;
 };
 
@@ -79,9 +81,9 @@ __device__ __forceinline__ void decayed8(const uint16_t* xrow, const float* grow
 }
 
 __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillParams p) {
-  const int cb = blockIdx.x;
+  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x, p.seq_chunk_off[p.N]);
   const int h = blockIdx.y;
-  if (cb >= p.seq_chunk_off[p.N]) return;
+  if (cb < 0) return;
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -303,7 +305,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int r16 = lane & 15, kb = lane >> 4;
   const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
 
-  const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, StageTable{}, 0, p.h0, p.h0_indices, p.h0_slot_stride,
+  const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
@@ -407,7 +409,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
             *reinterpret_cast<const uint4*>(&tO[(krow + 16 * i) * PITCH128 + 8 * kcv]);
   };
 
-  issue_first(0);
+  if (n_chunks > 0) issue_first(0);                  // a stage of a short sequence may hold no chunk
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const bool more = ci + 1 < n_chunks;
@@ -605,7 +607,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
       }
   }
   __syncthreads();
-  flush_output(n_chunks - 1);
+  if (n_chunks > 0) flush_output(n_chunks - 1);
 
   if (fin != nullptr) {
 #pragma unroll
@@ -620,8 +622,9 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 
 struct KdaWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Khi, Klo, Qh, KtH, KtL, Whi, Wlo, P, eGlast;
-  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity, total;
-  int NC_max, seg_chunks, max_segments;
+  size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
+  size_t order, stage_begin, carry, total;
+  int NC_max, seg_chunks, max_segments, stages;
 };
 static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   KdaWorkspaceLayout L;
@@ -646,6 +649,13 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
     const size_t states = (size_t)L.max_segments * H * 16384 * 4;
     L.segM = take(states); L.segB = take(states); L.segS = take(states);
     L.identity = take(16384 * 4);
+  }
+  // pipeline the preparation with the sweeps in stages where that pays
+  L.stages = 0;                                      // see pick_stages: the KDA kernels do not fit a CU together
+  if (L.stages > 0) {
+    L.order = take((size_t)L.NC_max * 4);
+    L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);
+    L.carry = L.seg_chunks > 0 ? 0 : take((size_t)N * H * 16384 * 4);
   }
   L.total = off;
   return L;
@@ -710,11 +720,8 @@ extern "C" int pla_kda_prefill_launch(
   hipLaunchKernelGGL(chunk_map_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, N, L.NC_max, p.seq_chunk_off,
                      p.chunk_seq, p.chunk_tok, p.chunk_len);
   hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, H);
-  hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, s, p);
-  if (L.seg_chunks == 0) {
-    p.pass = 0;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)N * H), dim3(256), 0, s, p);
-  } else {
+  const bool segmented = L.seg_chunks > 0;
+  if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
     p.seg.seg_seq = reinterpret_cast<int32_t*>(ws + L.seg_seq);
@@ -727,9 +734,25 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
     hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
-    p.pass = 1;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H * 2), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht, ht_indices, ht_slot_stride);
+  }
+  if (L.stages > 0) {
+    p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
+    p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
+    p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
+    p.stg.stages = L.stages;
+    const int items = segmented ? L.max_segments : N;
+    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * items + 1) * 4, s,
+                       segmented ? p.seg.seg_c0 : p.seq_chunk_off, segmented ? p.seg.seg_nc : nullptr,
+                       segmented ? p.seg.seq_seg_off + N : nullptr, items, L.NC_max, p.stg);
+  }
+  const bool ok = launch_pipeline(
+      s, L.stages, segmented, (unsigned)N * H, (unsigned)L.max_segments * H, &p.pass, &p.stage,
+      [&](hipStream_t ps) { hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, ps, p); },
+      [&](unsigned grid) { hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3(grid), dim3(256), 0, s, p); });
+  PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
+  if (segmented) {
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
+                       ht_indices, ht_slot_stride);
     p.pass = 2;
     hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
   }
