@@ -193,6 +193,23 @@ def bench_small_decode(device, steps=200):
                                       v["cu_seqlens"], scale=v["scale"]))
     out["config2_kda_verify_t4_b64_us"] = round(us, 2)
     out["config2_verify_state_read_GBps"] = round(64 * 32 * 65536 / us / 1e3, 1)
+    # accepted-prefix commit of the same window: per-slot records, num_accepted ~ U{0..4}
+    from pla_amd.decode.kda_replayssm_sglang import fold_accepted_prefix
+    B, T, HV, slots = 64, 4, 32, 1024
+    idx = v["indices"].long()
+    rawk = torch.zeros(slots, HV, T, 128, dtype=torch.bfloat16, device=device)
+    rawv = torch.zeros_like(rawk)
+    gk = torch.zeros(slots, HV, T, 128, dtype=torch.float32, device=device)
+    beta = torch.zeros(slots, HV, T, dtype=torch.float32, device=device)
+    rawk[idx] = v["k"][0].view(B, T, HV, 128).transpose(1, 2)
+    rawv[idx] = v["v"][0].view(B, T, HV, 128).transpose(1, 2)
+    gk[idx] = v["log_decay"].view(B, T, HV, 128).transpose(1, 2)
+    beta[idx] = v["beta"].view(B, T, HV).transpose(1, 2)
+    us = timed(lambda: fold_accepted_prefix(v["state"][None], rawv[None], rawk[None], gk[None], beta[None],
+                                            v["indices"], v["num_accepted"], null_block_id=-1))
+    touched = int((v["num_accepted"] > 0).sum().item())
+    out["config2_kda_commit_b64_us"] = round(us, 2)
+    out["config2_commit_state_GBps"] = round(touched * 32 * 2 * 65536 / us / 1e3, 1)     # tiles read and written
     return out
 
 
