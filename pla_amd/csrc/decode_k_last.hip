@@ -201,7 +201,13 @@ __device__ __forceinline__ float gate_decay(float a, float dt, float eA, float p
   return __expf(-eA * sp);
 }
 
-template <typename act_t, bool IS_KDA, bool MTP, int RPW>
+// READONCE (verify of up to four draft tokens that writes no state, no snapshots and follows no tree):
+// the recurrence is unrolled algebraically instead of being stepped through the state,
+//     o_t = S_0 w_t + sum_{j <= t} c_{j,t} v_j,   w_t = A_1 ... A_t q_t,   A_j = D_j (I - beta_j k_j k_j^T),
+// where w_t and the coefficients c_{j,t} = beta_j k_j^T (A_{j+1} ... A_t q_t) need only K-vectors (ten
+// dot products for four tokens).  The state tile is then used once: four dot products per row and no
+// update (the read-once verify of src/decode/kda_replayssm/kda_mtp_verify.cu:630-652).
+template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false>
 __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   constexpr int R = RPW / 2;
   const int lane = threadIdx.x & 63;
@@ -299,6 +305,14 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   };
 
   TokenIn cur = fetch(0);
+  // read-once verify: every token is requested ahead of the state tile, so that the K-vector algebra runs
+  // while the tile is in flight (memory returns in issue order)
+  TokenIn ahead[3] = {cur, cur, cur};
+  if constexpr (READONCE) {
+#pragma unroll
+    for (int t = 1; t < 4; ++t)
+      if (t < T) ahead[t - 1] = fetch(t);
+  }
   float s[R][4];
   if (have_state) {
     load_state<R>(h_tile, lane_off, s);
@@ -314,6 +328,101 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   float dt_scalar = 0.f;
   if constexpr (IS_KDA) decode_k4<act_t>(dt_raw_k4, dt_wide || log_decay, dt);
   else dt_scalar = decode_scalar_act<act_t>(dt_raw, dt_wide || log_decay);
+
+  if constexpr (READONCE) {
+    const TokenIn tok[4] = {cur, ahead[0], ahead[1], ahead[2]};        // absent tokens repeat token 0, never stored
+    float qv[4][4], kv[4][4], dec[4][4], beta[4], vv[4][R];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const TokenIn& in = tok[t];
+      const float q4[4] = {lo16<act_t>(in.qw.x), hi16<act_t>(in.qw.x), lo16<act_t>(in.qw.y), hi16<act_t>(in.qw.y)};
+      const float k4[4] = {lo16<act_t>(in.kw.x), hi16<act_t>(in.kw.x), lo16<act_t>(in.kw.y), hi16<act_t>(in.kw.y)};
+      float qn = p.scale, kn = 1.f;
+      if (p.use_qk_l2norm) {
+        float qs = 0.f, ks = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { qs = fmaf(q4[e], q4[e], qs); ks = fmaf(k4[e], k4[e], ks); }
+        qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
+        kn = fast_rsqrt(row32_allreduce(ks) + 1e-6f);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { qv[t][e] = q4[e] * qn; kv[t][e] = k4[e] * kn; }
+      if constexpr (IS_KDA) {
+        float av[4];
+        decode_k4<act_t>(in.a4, log_decay, av);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          dec[t][e] = gate_decay(av[e], dt[e], eA, p.gate_p0, p.softplus_threshold, p.gate_mode);
+      } else {
+        const float d1 = gate_decay(decode_scalar_act<act_t>(in.a1, log_decay), dt_scalar, eA, p.gate_p0,
+                                    p.softplus_threshold, p.gate_mode);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dec[t][e] = d1;
+      }
+      const float b_in = decode_scalar_act<act_t>(in.b1, beta_wide);
+      beta[t] = beta_wide ? b_in : fast_sigmoid(b_in);
+      row_scalars<act_t, RPW>(in.vw, half, vv[t]);
+    }
+    // effective queries w_t and bias coefficients c_{j,t}
+    float qeff[4][4], coef[4][4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      float w[4] = {qv[t][0], qv[t][1], qv[t][2], qv[t][3]};
+#pragma unroll
+      for (int j = 3; j >= 0; --j) {
+        if (j > t) { coef[j][t] = 0.f; continue; }
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dot = fmaf(kv[j][e], w[e], dot);
+        const float cf = beta[j] * row32_allreduce(dot);
+        coef[j][t] = cf;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf, kv[j][e], w[e]);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) qeff[t][e] = w[e];
+    }
+    // The lane's partial sums of S_0 w_t for its R rows.  They are reduced over the 32 lanes of a state
+    // row in two steps: a lane swap between the two DPP rows of a half (one swap and one add per pair
+    // of values: the even DPP row ends up with tokens 0 and 1, the odd one with tokens 2 and 3), then
+    // four DPP adds inside the 16 lanes.
+    const bool odd_row = (lane >> 4) & 1;
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      float keep[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        float a = 0.f, b = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a = fmaf(s[j][e], qeff[tt][e], a);
+          b = fmaf(s[j][e], qeff[tt + 2][e], b);
+        }
+        asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+        keep[j] = row16_allreduce(a + b);
+      }
+      float cs[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cs[j] = odd_row ? coef[j][tt + 2] : coef[j][tt];
+      uint32_t wout[R];
+#pragma unroll
+      for (int j = 0; j < R; ++j) {
+        float o = keep[j];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) o = fmaf(cs[jj], vv[jj][j], o);
+        const LanePair both = swap_halves(o);      // even state row from lanes 0-31, odd one from lanes 32-63
+        wout[j] = pack2<act_t>(both.lo, both.hi);
+      }
+      const int t_mine = tt + (odd_row ? 2 : 0);
+      if ((lane & 47) == 0 && t_mine < T) {         // lanes 0 and 16 write two tokens each
+        act_t* dst = o_base + (int64_t)t_mine * p.HV * 128;
+#pragma unroll
+        for (int i = 0; i < RPW / 8; ++i)
+          reinterpret_cast<uint4*>(dst)[i] = make_uint4(wout[4 * i], wout[4 * i + 1], wout[4 * i + 2], wout[4 * i + 3]);
+      }
+    }
+    return;
+  }
 
   const int steps = MTP ? T : 1;
   for (int t = 0; t < steps; ++t) {
@@ -543,6 +652,20 @@ template <typename act_t, bool IS_KDA, bool MTP>
 static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
   const dim3 block(256);
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
+  if constexpr (MTP) {
+    // a verify that leaves no trace in memory but o: the state is read once and used once
+    const bool read_once = p.disable_state_update && p.T_max <= 4 && p.cache == nullptr && p.cache_indices == nullptr &&
+                           p.parents == nullptr && p.stride_h0_indices_seq == 0;
+    if (read_once) {
+      switch (rpw) {
+        case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true>), dim3(tiles, 1), block, 0, stream, p); break;
+        case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 16, true>), dim3(tiles, 2), block, 0, stream, p); break;
+        case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 8, true>),  dim3(tiles, 4), block, 0, stream, p); break;
+        default: return fail("rows_per_wave must be 0, 8, 16 or 32, got %d", rpw);
+      }
+      return check_launch("k_last_kernel launch");
+    }
+  }
   switch (rpw) {
     case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 32>), dim3(tiles, 1), block, 0, stream, p); break;
     case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 16>), dim3(tiles, 2), block, 0, stream, p); break;
