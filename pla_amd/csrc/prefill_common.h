@@ -2,6 +2,8 @@
 // splitting, operand access for v_mfma_f32_16x16x32_bf16 and the device-side chunk table.
 #pragma once
 
+#include <mutex>
+
 #include "common.h"
 
 namespace pla {
@@ -451,7 +453,8 @@ static __global__ void zero_tail_kernel(uint16_t* o, const int32_t* cu_seqlens, 
 inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 // One side stream (default priority, non-blocking) and its events per device, created on first use and
-// kept for the life of the process.  Calls are expected from one host thread at a time per device.
+// kept for the life of the process (creation is serialised; the calls themselves are expected from one
+// host thread at a time per device, as the events are shared).
 struct SideStream {
   hipStream_t stream;
   hipEvent_t fork;
@@ -460,8 +463,10 @@ struct SideStream {
 static inline SideStream* side_stream() {
   static SideStream table[16];
   static bool made[16] = {};
+  static std::mutex guard;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(guard);
   if (!made[dev]) {
     SideStream& t = table[dev];
     if (hipStreamCreateWithFlags(&t.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
