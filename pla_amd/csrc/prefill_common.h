@@ -49,6 +49,20 @@ __device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s,
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
+// The same operand from the TRANSPOSE of a row-major 128-wide bf16 tile (row pitch PITCH128): lane
+// (r = lane%16, kb) takes rows [32s+4kb, +4) and [32s+16+4kb, +4) of column 16 m + r.  ds_read_b64_tr_b16
+// transposes inside each group of 16 lanes: lane t of the group addresses four consecutive columns
+// 16 m + 4 (t%4) .. +3 of row base + t/4, and lane i receives column 16 m + i of rows base .. base + 3.
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ bf16x8_t operand_transposed(const uint16_t* tile, int s, int m, int kb, int r) {
+  const uint16_t* at = tile + (32 * s + 4 * kb + (r >> 2)) * 136 + 16 * m + 4 * (r & 3);
+  const i16x4_t p0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)at);
+  const i16x4_t p1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(at + 16 * 136));
+  typedef short i16x8_t __attribute__((ext_vector_type(8)));
+  const i16x8_t u = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+
 // LDS tile pitches (bf16 elements): rows stay 16-byte aligned and consecutive rows start 4 (128-wide)
 // or 36 (64-wide) banks apart, which keeps the 8-byte operand reads of a wavefront conflict free.
 constexpr int PITCH128 = 136;

@@ -19,7 +19,7 @@
 // Kernels:
 //   chunk_map_kernel         chunk table from cu_seqlens (device side, graph-capturable)
 //   gdn_prep_kernel          gate, beta, chunk-local cumsum and per-chunk decay-factor tiles, q/k L2
-//                            norm (rounded to bf16), K^T tiles
+//                            norm (rounded to bf16)
 //   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
 //                            forward substitution in LDS, W (hi/lo) and P to the workspace
 //   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), four wavefronts each owning a
@@ -49,7 +49,7 @@ struct GdnPrefillParams {
   void* o;                                            // [T, HV, 128] dense
   // workspace
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
-  uint16_t* qn; uint16_t* kn; uint16_t* knT;
+  uint16_t* qn; uint16_t* kn;
   float* gcum; float* beta;
   uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
@@ -71,8 +71,7 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  __shared__ union {
-    uint16_t tile[CHUNK][130];        // normalised k of one head, for the transposed copy
+  __shared__ struct {
     float g[CHUNK][129];              // per-token log-decay of up to 128 value heads
   } sh;
 
@@ -144,27 +143,11 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
       const float qi = rsqrtf(qs + 1e-6f), ki = rsqrtf(ks + 1e-6f);
       q0 *= qi; q1 *= qi; k0 *= ki; k1 *= ki;
     }
-    uint32_t ko = 0;
     if (j < len) {
-      ko = pack2<bf16_t>(k0, k1);
       const int64_t t = t0 + j;
       *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2<bf16_t>(q0, q1);
-      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = ko;
+      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2<bf16_t>(k0, k1);
     }
-    *reinterpret_cast<uint32_t*>(&sh.tile[j][2 * lane]) = ko;       // zero rows beyond the chunk
-  }
-  __syncthreads();
-  // K^T tile [128][64]: thread (c, half) gathers 32 tokens of column c
-  {
-    const int c = threadIdx.x >> 1, half = threadIdx.x & 1;
-    uint16_t* dst = p.knT + (((int64_t)cb * p.H + h) * 128 + c) * CHUNK + 32 * half;
-    uint32_t w[16];
-#pragma unroll
-    for (int jj = 0; jj < 16; ++jj)
-      w[jj] = (uint32_t)sh.tile[32 * half + 2 * jj][c] | ((uint32_t)sh.tile[32 * half + 2 * jj + 1][c] << 16);
-#pragma unroll
-    for (int x = 0; x < 4; ++x)
-      reinterpret_cast<uint4*>(dst)[x] = make_uint4(w[4 * x], w[4 * x + 1], w[4 * x + 2], w[4 * x + 3]);
   }
 }
 
@@ -293,13 +276,15 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
 // wavefront reads every A tile once per chunk, so fewer, wider wavefronts halve the LDS traffic,
 // which is what bounds this kernel).  S^T stays in MFMA
 // accumulator layout (an accumulator tile pair is already a valid B operand of the next product),
-// A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  Every tile
-// is single buffered and there are two barriers per chunk; a tile's next version is requested at the
-// barrier after its last use and has half a chunk of compute time to land:
+// A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  There are two
+// barriers per chunk; a tile's next version is requested at the barrier after its last use and has
+// half a chunk of compute time to land.  The K tile is used in both halves (as K for K S^T, and
+// transposed by ds_read_b64_tr_b16 for the state update), so it alone is double buffered by chunk
+// parity; no K^T copy exists in memory:
 //
-//   barrier A   K, Q, V, W, decay factors of chunk c landed   flush O(c-1); issue K^T(c), P(c), factors of c+1
+//   barrier A   K, Q, V, W, decay factors of chunk c landed   flush O(c-1); issue P(c), factors of c+1
 //               KS = K S^T, QS = Q S^T, X = V - e^G (.) KS, U = W X
-//   barrier B   K^T, P of chunk c landed                      issue K, Q, V, W of chunk c+1
+//   barrier B   P of chunk c landed                           issue K, Q, V, W of chunk c+1
 //               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U),  O = scale e^G (.) QS + P U -> O tile
 //
 // Every wait is for all outstanding copies (s_waitcnt vmcnt(0)): whatever is in flight at a barrier is
@@ -309,7 +294,6 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   constexpr int WAVES = 8 / NB;                            // NB 16-column blocks of V per wavefront
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
-  using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride);
   if (!role.active) return;
@@ -326,11 +310,10 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   const int n_chunks = c_end - c_begin;
 
   // distinct LDS objects: the compiler tracks outstanding direct-to-LDS loads per object
-  __shared__ __align__(16) uint16_t tK[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];      // by chunk parity: the state update reads it last
   __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tKt[128 * PITCH64];
   __shared__ __align__(16) uint16_t tWh[CHUNK * PITCH64];
   __shared__ __align__(16) uint16_t tWl[CHUNK * PITCH64];
   __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
@@ -363,7 +346,6 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-  const char* const kt_b = reinterpret_cast<const char*>(p.knT) + ((int64_t)c_begin * p.H + h) * 16384;
   const char* const wh_b = reinterpret_cast<const char*>(p.Whi) + ((int64_t)c_begin * p.HV + hv) * 8192;
   const char* const wl_b = reinterpret_cast<const char*>(p.Wlo) + ((int64_t)c_begin * p.HV + hv) * 8192;
   const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
@@ -374,24 +356,22 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   // that keep rows past the sequence end inside it.
   CopyWide plan_kq, plan_v;
   CopyNarrow plan_w;
-  CopyKt plan_kt;
   plan_kq.plan((uint32_t)tok_pitch_b, CHUNK - 1, wave, lane);
   plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
   plan_w.plan(128, CHUNK - 1, wave, lane);
-  plan_kt.plan(128, 127, wave, lane);
   auto issue_kqv = [&](int c) {
     const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
     const char* qs = qn_b + (int64_t)c * CHUNK * tok_pitch_b;
     const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
     const int len = chunk_len(c);
     if (len == CHUNK) {
-      plan_kq.issue(tK, ks, wave);
+      plan_kq.issue(tK[c & 1], ks, wave);
       plan_kq.issue(tQ, qs, wave);
       if (!zero_v) plan_v.issue(tV, vs, wave);
     } else {
       CopyWide tail_kq, tail_v;
       tail_kq.plan((uint32_t)tok_pitch_b, len - 1, wave, lane);
-      tail_kq.issue(tK, ks, wave);
+      tail_kq.issue(tK[c & 1], ks, wave);
       tail_kq.issue(tQ, qs, wave);
       if (!zero_v) {
         tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
@@ -403,7 +383,6 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     plan_w.issue(tWh, wh_b + (int64_t)c * p.HV * 8192, wave);
     plan_w.issue(tWl, wl_b + (int64_t)c * p.HV * 8192, wave);
   };
-  auto issue_kt = [&](int c) { plan_kt.issue(tKt, kt_b + (int64_t)c * p.H * 16384, wave); };
   auto issue_p = [&](int c) { plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave); };
   auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
     if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
@@ -441,12 +420,11 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     bf16x8_t ka[2][4], qa[2][4];
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
-      ka[0][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], 0, kb);
+      ka[0][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], 0, kb);
       qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (ci > 0) flush_output(ci - 1);
-    issue_kt(ci);
     issue_p(ci);
     if (more) issue_gates(ci + 1);
 
@@ -466,7 +444,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       if (s < 3) {
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          ka[(s + 1) & 1][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], s + 1, kb);
+          ka[(s + 1) & 1][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], s + 1, kb);
           qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
         }
       } else {
@@ -553,14 +531,14 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
     }
 
-    // barrier B: K^T and P of this chunk have landed; K, Q, V, W are free for the next chunk
+    // barrier B: P of this chunk has landed; Q, V, W and the other K tile are free for the next chunk
     wait_vmcnt<0>();
     __syncthreads();
     bf16x8_t kt[2][8];
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_from(&tKt[(16 * mc + r16) * PITCH64], s, kb);
+      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tK[par], s, mc, kb, r16);
     float4 dg[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -653,7 +631,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 }
 
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, knT, gcum, beta, gtile, Whi, Wlo, P;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, Whi, Wlo, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -669,7 +647,6 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   L.chunk_len = take((size_t)L.NC_max * 4);
   L.qn = take((size_t)T * H * 128 * 2);
   L.kn = take((size_t)T * H * 128 * 2);
-  L.knT = take((size_t)L.NC_max * H * 128 * CHUNK * 2);
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
   L.gtile = take((size_t)L.NC_max * HV * 256 * 4);
@@ -747,7 +724,6 @@ extern "C" int pla_gdn_prefill_launch(
   p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
   p.qn = reinterpret_cast<uint16_t*>(ws + L.qn);
   p.kn = reinterpret_cast<uint16_t*>(ws + L.kn);
-  p.knT = reinterpret_cast<uint16_t*>(ws + L.knT);
   p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
   p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
   p.gtile = reinterpret_cast<float*>(ws + L.gtile);
