@@ -125,6 +125,41 @@ int pla_kda_fold_launch(
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
 
 /*
+ * Fused KDA decode step (one token per request): width-4 causal conv1d update + SiLU on the packed
+ * q|k|v projection, q/k L2 norm, per-channel gate, delta-rule update of the indexed k-last FP32
+ * state pool, optional gated RMSNorm of the output.  Replaces launch_kda_decode_mega
+ * (src/decode/k-last/k_last_mega_abi.h:57-71; kernel
+ * src/decode/k-last/fused_kda_decode_mega_kernel.cuh:138-729) argument for argument, with the
+ * dtype enum replaced by PLA_BF16 / PLA_F16 and the stream passed as void*.
+ *
+ *   x_q, x_k, x_v   the three H*128-wide segments of a row of x [B, 3*H*128] (act dtype), row pitch x_row
+ *   w_*_t           [4, H*128] float32 width-major conv weights per segment; bias_* [H*128] or NULL
+ *   cs_q/k/v        the segments of conv_state [slots, 3*H*128, 3] in the SD layout: channel stride 1,
+ *                   tap stride 3*H*128, slot pitch conv_slot (elements); shifted in place
+ *   g [B,H,128], beta [B,H] (row pitch beta_row) raw gate / beta logits (act dtype);
+ *   a_log [H], dt_bias [H*128] float32:  decay = exp(-exp(a_log) softplus(g + dt_bias)), or
+ *                   exp(lower_bound sigmoid(exp(a_log) (g + dt_bias))) when use_lower_bound
+ *   state [slots,H,128,128] float32 with slot pitch state_slot; state_indices [B] int32; a negative
+ *                   slot writes zeros to the request's output row and touches neither pool
+ *   out [B,H,128] act dtype, dense.  apply_onorm: out = o rsqrt(mean(o^2) + norm_eps) o_norm_weight
+ *                   sigmoid(g_out), g_out [B,H,128] act dtype with row pitch onorm_row, weight [128] float32
+ *   H must equal HV.  v is rounded to the activation dtype after SiLU (as the reference kernel does);
+ *   q and k stay FP32.
+ */
+int pla_kda_decode_mega_launch(
+    int act_dtype, int apply_onorm, int use_lower_bound,
+    const float* a_log, const void* g, const float* dt_bias,
+    const void* x_q, const void* x_k, const void* x_v, const void* beta,
+    const float* w_q_t, const float* w_k_t, const float* w_v_t,
+    const float* bias_q, const float* bias_k, const float* bias_v,
+    void* cs_q, void* cs_k, void* cs_v,
+    const void* g_out, const float* o_norm_weight, float norm_eps,
+    float* state, const int32_t* state_indices, void* out,
+    float scale, float lower_bound, int B, int H, int HV,
+    int64_t x_row, int64_t beta_row, int64_t onorm_row,
+    int64_t conv_slot, int64_t state_slot, void* stream);
+
+/*
  * Workspace size in bytes (256-byte aligned buffer) needed by pla_gdn_prefill_launch for T physical
  * tokens in N sequences.  Chunk metadata is sized for the worst case T/64 + N chunks so that no
  * host copy of cu_seqlens is needed.

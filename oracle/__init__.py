@@ -15,7 +15,10 @@ prefix/commit consistency).  No function here is "parity unpinned".
 """
 
 from .gates import softplus_gate, lower_bound_gate, l2norm, sigmoid_beta  # noqa: F401
-from .decode import k_last_reference, fold_reference, recurrent_step  # noqa: F401
+from .decode import (  # noqa: F401
+    k_last_reference, fold_reference, recurrent_step,
+    causal_conv1d_update_reference, kda_decode_mega_reference,
+)
 from .prefill import (  # noqa: F401
     gdn_prefill_reference,
     kda_prefill_reference,

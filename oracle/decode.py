@@ -162,3 +162,82 @@ def fold_reference(state, rawk, rawv, g, beta, slot_indices, accept_lens, *,
             h = h + u[:, :, None] * kk[:, None, :]
         state[slot] = h.to(state.dtype)
     return state
+
+
+def causal_conv1d_update_reference(x, conv_state, weight, bias, slots):
+    """Width-4 causal conv1d update + SiLU for one new sample per request.
+
+    ``x [B, C]``, ``conv_state [slots, C, 3]`` (oldest tap first; updated copy returned),
+    ``weight [4, C]`` width-major float32, ``bias [C]`` or None, ``slots`` a list of ints
+    (negative: the request is skipped).  Returns ``(y [B, C] float32, conv_state_new)``.
+    Follows scripts/decode/kda_fusion/compare_kda_decode_fusion.py:243-255: the window is the
+    three stored taps followed by the new sample; the stored taps shift by one and the new sample
+    (unrounded copy of ``x``) becomes the newest tap.
+    """
+    conv = conv_state.clone()
+    y = torch.zeros(x.shape, dtype=torch.float32)
+    w = weight.float()
+    for n, slot in enumerate(slots):
+        if slot < 0:
+            continue
+        window = torch.cat([conv[slot].float(), x[n].float()[:, None]], dim=1)      # [C, 4]
+        acc = (window * w.t()).sum(-1)
+        if bias is not None:
+            acc = acc + bias.float()
+        y[n] = acc * torch.sigmoid(acc)
+        conv[slot, :, 0] = conv_state[slot, :, 1]
+        conv[slot, :, 1] = conv_state[slot, :, 2]
+        conv[slot, :, 2] = x[n]
+    return y, conv
+
+
+def kda_decode_mega_reference(x, weight, bias, conv_state, raw_g, raw_beta, a_log, dt_bias, state_indices,
+                              state, *, lower_bound=None, output_gate=None, norm_weight=None, norm_eps=1e-5,
+                              round_v=True):
+    """Reference for ``fused_kda_decode_mega_forward`` (one decode token per request).
+
+    Follows the reference's own step-by-step float32 golden
+    scripts/decode/kda_fusion/compare_kda_decode_fusion.py:209-282 (conv + SiLU, q/k L2 norm with
+    eps 1e-6 inside the root, q scaled by 128^-0.5, softplus or lower-bound per-channel decay,
+    sigmoid beta, k-last recurrence, RMSNorm * weight * sigmoid(gate)), and the pad rule of
+    scripts/decode/kda_fusion/test_pad_slot.py:37-53 (slot < 0: zero output, no pool write).
+    ``round_v``: the activated v is rounded to the activation dtype before the recurrence, as the
+    reference kernel does (src/decode/k-last/fused_kda_decode_mega_kernel.cuh:384, :463); the
+    float32 golden of the script does not round.
+
+    ``x [B,3*H*128]``, ``weight [3,4,H*128]``, ``bias [3*H*128]`` or None,
+    ``conv_state [slots,3*H*128,3]``, ``raw_g [1,B,H,128]``, ``raw_beta [1,B,H]``, ``a_log [H]``,
+    ``dt_bias [H*128]``, ``state [slots,H,128,128]`` float32, ``output_gate [B,H,128]``.
+    Returns ``(out [1,B,H,128] in x.dtype, state_new, conv_state_new)``.
+    """
+    B = x.shape[0]
+    D = 128
+    H = x.shape[1] // (3 * D)
+    dim = H * D
+    slots = [int(s) for s in state_indices.tolist()]
+    w_flat = weight.float().permute(1, 0, 2).reshape(4, 3 * dim)                   # [4, 3*dim] width-major
+    mixed, conv_new = causal_conv1d_update_reference(x, conv_state, w_flat, bias, slots)
+    state_new = state.clone()
+    out = torch.zeros(1, B, H, D, dtype=x.dtype)
+    dt = dt_bias.float().reshape(H, D)
+    for n, slot in enumerate(slots):
+        if slot < 0:
+            continue
+        q = l2norm(mixed[n, :dim].reshape(H, D)) * (float(D) ** -0.5)
+        k = l2norm(mixed[n, dim:2 * dim].reshape(H, D))
+        v = mixed[n, 2 * dim:].reshape(H, D)
+        if round_v:
+            v = v.to(x.dtype).float()
+        g = raw_g[0, n].float()
+        if lower_bound is not None:
+            log_decay = lower_bound_gate(g, dt, a_log, lower_bound, per_channel=True)
+        else:
+            log_decay = softplus_gate(g, dt, a_log, per_channel=True)
+        beta = sigmoid_beta(raw_beta[0, n])
+        S, o = recurrent_step(state_new[slot].float(), q, k, v, log_decay, beta)
+        state_new[slot] = S
+        if output_gate is not None:
+            gate = torch.sigmoid(output_gate.reshape(B, H, D)[n].float())
+            o = o * torch.rsqrt(o.square().mean(-1, keepdim=True) + norm_eps) * norm_weight.float()[None, :] * gate
+        out[0, n] = o.to(x.dtype)
+    return out, state_new, conv_new

@@ -33,6 +33,12 @@ SIGNATURES = {
         _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
         _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_kda_decode_mega_launch": [
+        _c_int, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_p, _c_f, _c_p, _c_p, _c_p,
+        _c_f, _c_f, _c_int, _c_int, _c_int,
+        _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_p],
     "pla_gdn_prefill_launch": [
         _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64,
         _c_p, _c_p, _c_i64, _c_i64,

@@ -177,3 +177,55 @@ def kda_prefill(T=65536, H=32, seed=0, device="cuda", dtype=torch.bfloat16, lowe
         cu_seqlens=to(torch.tensor([0, T], dtype=torch.int32)), raw_cu_seqlens=(0, T),
         _meta=dict(T=T, H=H),
     )
+
+
+def kda_decode_mega(B, H, seed=0, device="cuda", dtype=torch.bfloat16, pad_rows=(), bias=False, slots=None):
+    """Fused KDA decode step (conv + gate + recurrence + norm), one token per request.
+
+    Layouts follow the reference's own input builder for this op
+    (scripts/decode/kda_fusion/compare_kda_decode_fusion.py:124-186, :288-312): rows of ``x``,
+    ``raw_beta`` and ``output_gate`` are views into wider storage, the conv window and the FP32
+    state of a slot share one page of a paged cache (conv in the SD layout: channel stride 1, tap
+    stride 3*H*128), slot ids count down from ``B`` so that none equals its row.  ``pad_rows``
+    get slot -1.  Returns call arguments (device tensors) under their argument names plus
+    ``_cache`` (the page storage, uint8).
+    """
+    device = torch.device(device)
+    g = _gen(seed)
+    dim = H * D
+    slots = slots or B + 2
+    W = 4
+    eb = torch.empty((), dtype=dtype).element_size()
+
+    def rand(*shape, scale=1.0):
+        return torch.randn(*shape, generator=g) * scale
+
+    x_store = rand(B, 3 * dim + 24).to(dtype).to(device)
+    beta_store = rand(1, B, H + 1).to(dtype).to(device)
+    gate_store = rand(B, dim + 8).to(dtype).to(device)
+    conv_elems = 3 * dim * (W - 1)
+    page_bytes = conv_elems * eb + H * D * D * 4
+    cache = torch.zeros(slots * page_bytes, dtype=torch.uint8, device=device)
+    conv = torch.as_strided(cache.view(dtype), (slots, 3 * dim, W - 1), (page_bytes // eb, 1, 3 * dim))
+    state = torch.as_strided(cache.view(torch.float32), (slots, H, D, D), (page_bytes // 4, D * D, D, 1),
+                             storage_offset=conv_elems * eb // 4)
+    conv.copy_(rand(slots, W - 1, 3 * dim, scale=0.1).to(dtype).transpose(1, 2))
+    state.copy_(rand(slots, H, D, D, scale=0.01))
+    idx = torch.arange(B, 0, -1, dtype=torch.int32)
+    for r in pad_rows:
+        idx[r] = -1
+    return {
+        "x": x_store[:, :3 * dim],
+        "weight": rand(3, W, dim, scale=0.1).to(device),
+        "bias": rand(3 * dim, scale=0.1).to(device) if bias else None,
+        "conv_state": conv,
+        "raw_g": rand(1, B, H, D).to(dtype).to(device),
+        "raw_beta": beta_store[:, :, :H],
+        "a_log": rand(H, scale=0.5).to(device),
+        "dt_bias": rand(dim, scale=0.1).to(device),
+        "state_indices": idx.to(device),
+        "state": state,
+        "output_gate": gate_store[:, :dim].view(B, H, D),
+        "norm_weight": rand(D).to(device),
+        "_cache": cache,
+    }
