@@ -213,6 +213,40 @@ def bench_small_decode(device, steps=200):
     return out
 
 
+def bench_decode_mega(device, steps=100, B=256, H=12, sets=16):
+    """Fused KDA decode step (conv + gate + recurrence + gated RMSNorm), B=256 requests x 12 heads
+    (the per-rank head count of the reference's Kimi K3 TP8 fixture).  Consecutive steps use
+    disjoint slot sets so that no state tile is served from a cache."""
+    import torch
+    from pla_amd.decode.kda import fused_kda_decode_mega_forward as mega
+    from pla_amd.workloads import kda_decode_mega
+    w = kda_decode_mega(B, H, seed=404, device=device, slots=sets * B + 2)
+    base = w["state_indices"].clone()
+    idx = [(base + i * B).contiguous() for i in range(sets)]
+    out = torch.empty(1, B, H, 128, dtype=torch.bfloat16, device=device)
+
+    def step(i):
+        mega(x=w["x"], weight=w["weight"], bias=None, conv_state=w["conv_state"], raw_g=w["raw_g"],
+             raw_beta=w["raw_beta"], a_log=w["a_log"], dt_bias=w["dt_bias"], state_indices=idx[i % sets],
+             state=w["state"], out=out, lower_bound=-5.0, output_gate=w["output_gate"],
+             norm_weight=w["norm_weight"], norm_eps=1e-5)
+
+    for i in range(sets):
+        step(i)
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for i in range(steps):
+        step(i)
+    e.record()
+    torch.cuda.synchronize()
+    us = s.elapsed_time(e) / steps * 1e3
+    state_bytes = B * H * 131072
+    return {"workload": "fused KDA decode step, B=%d, H=%d, bf16 activations, lower-bound gate, gated RMSNorm" % (B, H),
+            "us_per_step": round(us, 2), "state_GBps": round(state_bytes / us / 1e3, 1),
+            "frac_of_hbm_peak": round(state_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
+
+
 def cpu_baseline_decode(w, sample_requests=32, reps=5):
     """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
     sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
@@ -290,6 +324,8 @@ def main():
     torch.cuda.empty_cache()
     if not args.decode_only:
         result["other_decode"] = bench_small_decode(device)
+        result["decode_mega"] = bench_decode_mega(device)
+        torch.cuda.empty_cache()
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
         torch.cuda.empty_cache()
         result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)

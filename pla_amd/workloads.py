@@ -209,8 +209,15 @@ def kda_decode_mega(B, H, seed=0, device="cuda", dtype=torch.bfloat16, pad_rows=
     conv = torch.as_strided(cache.view(dtype), (slots, 3 * dim, W - 1), (page_bytes // eb, 1, 3 * dim))
     state = torch.as_strided(cache.view(torch.float32), (slots, H, D, D), (page_bytes // 4, D * D, D, 1),
                              storage_offset=conv_elems * eb // 4)
-    conv.copy_(rand(slots, W - 1, 3 * dim, scale=0.1).to(dtype).transpose(1, 2))
-    state.copy_(rand(slots, H, D, D, scale=0.01))
+    if device.type == "cuda":                      # the pools can be several GB: draw them on the device
+        dg = torch.Generator(device=device).manual_seed(seed + 1)
+        conv.copy_((torch.randn(slots, W - 1, 3 * dim, generator=dg, device=device) * 0.1).to(dtype).transpose(1, 2))
+        for s0 in range(0, slots, 256):
+            n = min(256, slots - s0)
+            state[s0:s0 + n].copy_(torch.randn(n, H, D, D, generator=dg, device=device) * 0.01)
+    else:
+        conv.copy_(rand(slots, W - 1, 3 * dim, scale=0.1).to(dtype).transpose(1, 2))
+        state.copy_(rand(slots, H, D, D, scale=0.01))
     idx = torch.arange(B, 0, -1, dtype=torch.int32)
     for r in pad_rows:
         idx[r] = -1
