@@ -127,3 +127,49 @@ def sanity_k_last(q, k, v, a, b, A_log, dt_bias, state, indices, cu, is_kda, cac
             for t in range(1, length):
                 if row[t] >= t:
                     _fail(op, "a parent step must precede its token")
+
+
+def sanity_kda_decode_mega(x, weight, bias, conv_state, state_indices, state, lower_bound, output_gate,
+                           norm_weight, norm_eps):
+    """Diagnostic checks of the fused KDA decode step
+    (src/decode/k-last/kda_decode_sanity.h:44-109): slot pitch alignment, finite negative
+    ``lower_bound``, finite ``norm_eps``; value checks (skipped during capture): active slots inside
+    both pools, no two requests on one non-zero slot, finite selected inputs and pool rows."""
+    import math
+    op = "fused_kda_decode"
+    if state_indices.dim() != 1:
+        _fail(op, "state_indices must be a vector")
+    if state.storage_offset() % 4 != 0 or state.stride(0) % 4 != 0:
+        _fail(op, "state slots must be 16-byte aligned for float4 access")
+    if lower_bound is not None and not (math.isfinite(lower_bound) and lower_bound < 0.0):
+        _fail(op, "lower_bound must be a finite negative float32 value")
+    if output_gate is not None and not (math.isfinite(norm_eps) and norm_eps >= 0.0):
+        _fail(op, "norm_eps must be a finite non-negative float32 value")
+    if _capturing():
+        return
+    seen = set()
+    active = False
+    for n, slot in enumerate(state_indices.tolist()):
+        if slot < 0:
+            continue
+        if slot >= state.size(0) or slot >= conv_state.size(0):
+            _fail(op, f"state index {slot} exceeds recurrent/conv pool capacity")
+        if slot != 0:
+            if slot in seen:
+                _fail(op, f"requests must not concurrently update the same state slot: {slot}")
+            seen.add(slot)
+        else:
+            continue
+        active = True
+        for name, t in (("selected x", x[n]), ("selected state", state[slot]),
+                        ("selected conv_state", conv_state[slot])):
+            if not bool(torch.isfinite(t).all()):
+                _fail(op, f"{name} must be finite")
+        if output_gate is not None:
+            gate = output_gate[n] if output_gate.dim() == 3 else output_gate[0, n]
+            if not bool(torch.isfinite(gate).all()):
+                _fail(op, "selected output_gate must be finite")
+    if active:
+        for name, t in (("weight", weight), ("bias", bias), ("norm_weight", norm_weight)):
+            if t is not None and not bool(torch.isfinite(t).all()):
+                _fail(op, f"{name} must be finite")

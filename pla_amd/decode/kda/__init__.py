@@ -167,6 +167,11 @@ def fused_kda_decode_mega_forward(x, weight, bias=None, conv_state=None, raw_g=N
         _require(bias.is_cuda and bias.dtype == torch.float32, "bias must be a CUDA float32 tensor")
         _require(bias.is_contiguous() and bias.numel() == 3 * dim, "bias must be contiguous with 3 * H * 128 elements")
 
+    if os.environ.get("PLA_SANITY_CHECK", "0") == "1":           # read on every call, like src/sanity_check.h
+        from ..._sanity import sanity_kda_decode_mega
+        sanity_kda_decode_mega(x, weight, bias, conv_state, state_indices, state, lower_bound, output_gate,
+                               norm_weight, norm_eps)
+
     eb = x.element_size()
     xp, wp, cp = x.data_ptr(), weight.data_ptr(), conv_state.data_ptr()
     seg_b, wseg_b, cseg_b = dim * eb, dim * W * 4, dim * conv_state.stride(1) * eb

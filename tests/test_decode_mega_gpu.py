@@ -175,3 +175,27 @@ def test_mega_in_a_graph_matches_eager():
         torch.cuda.synchronize()
         assert torch.equal(out, eager[i])
     assert torch.equal(w["_cache"], eager_cache)
+
+
+def test_mega_sanity_mode_rejects_aliased_slots_and_bad_values(monkeypatch):
+    monkeypatch.setenv("PLA_SANITY_CHECK", "1")
+    w = kda_decode_mega(4, 4, seed=5)
+    _run(w, -5.0, True)                                                               # a clean call passes
+    snapshot = w["_cache"].clone()
+    bad = dict(w)
+    bad["state_indices"] = torch.tensor([2, 1, 2, -1], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match=r"PLA_SANITY_CHECK \[fused_kda_decode\]: requests must not concurrently"):
+        _run(bad, -5.0, True)
+    bad["state_indices"] = torch.tensor([2, 1, 99, -1], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="exceeds recurrent/conv pool capacity"):
+        _run(bad, -5.0, True)
+    with pytest.raises(RuntimeError, match="lower_bound must be a finite negative"):
+        _run(w, 1.0, True)
+    bad = dict(w)
+    bad["x"] = w["x"].clone()
+    bad["x"][1, 5] = float("nan")
+    with pytest.raises(RuntimeError, match="selected x must be finite"):
+        _run(bad, -5.0, True)
+    bad["state_indices"] = torch.tensor([4, -1, 2, 1], dtype=torch.int32, device="cuda")   # the poisoned row is a pad
+    _run(bad, -5.0, True)
+    assert not torch.equal(w["_cache"], snapshot)
