@@ -82,6 +82,38 @@ def bench_decode(steps, warmup, device):
         value_gbps=bytes_state * steps / wall / 1e9, workload=w)
 
 
+def bench_decode_bf16_pool(w, steps, device):
+    """The headline workload with the pool stored in bf16 (FP32 recurrence, tiles widened on load and
+    rounded on store): half the state bytes per step."""
+    import torch
+    from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
+    B, HV, slots, pad = 256, 32, 4096, 0.05
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    sets, n_active = build_decode_sets(w, slots // B, slots, B, pad, 11, device)
+    pool32 = call["initial_state_source"]
+    pool16 = torch.empty(pool32.shape, dtype=torch.bfloat16, device=device)
+    for s0 in range(0, slots, 256):
+        pool16[s0:s0 + 256].copy_(pool32[s0:s0 + 256])
+    call["initial_state_source"] = pool16
+
+    def step(i):
+        call["initial_state_indices"] = sets[i % len(sets)]
+        packed(**call)
+
+    for i in range(16):
+        step(i)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(steps):
+        step(i)
+    end.record()
+    torch.cuda.synchronize()
+    us = start.elapsed_time(end) / steps * 1e3
+    nbytes = n_active * HV * 65536
+    return {"config1_bf16_pool_us": round(us, 2), "config1_bf16_pool_state_GBps": round(nbytes / us / 1e3, 1)}
+
+
 PREFILL_SEED = 348      # ragged_lengths(8, 512, 8192, 348) sums to 32 810 tokens
 GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64, K = V = 128, HV = 32, H = 16
 KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
@@ -320,10 +352,12 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_decode(d["workload"])
+    bf16_pool = None if args.decode_only else bench_decode_bf16_pool(d["workload"], args.steps, device)
     del d
     torch.cuda.empty_cache()
     if not args.decode_only:
         result["other_decode"] = bench_small_decode(device)
+        result["other_decode"].update(bf16_pool)
         result["decode_mega"] = bench_decode_mega(device)
         torch.cuda.empty_cache()
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)

@@ -42,7 +42,7 @@ const char* pla_version(void);
 const char* pla_last_error(void);
 
 /*
- * Packed one-token decode over an indexed FP32 k-last state pool.
+ * Packed one-token decode over an indexed k-last state pool.
  * Replaces k_last_packed_launcher_t
  * (src/decode/k-last/fused_sigmoid_gating_cuda_k_last_packed.cpp:53-80) and the
  * kernel fused_sigmoid_gating_delta_kernel_packed
@@ -53,7 +53,9 @@ const char* pla_last_error(void);
  *   b          [tokens, HV], pitch stride_b
  *   A_log      [HV] of alog_dtype;  dt_bias [HV] or [HV*128] act dtype
  *   o          [tokens, HV, 128] act dtype, dense
- *   h0         state pool, slot pitch h0_slot_stride floats, slot = [HV,128(V),128(K)]
+ *   h0         state pool of state_dtype (PLA_F32, or PLA_BF16: widened on load, the FP32 result
+ *              rounded to nearest even on store), slot pitch h0_slot_stride elements,
+ *              slot = [HV,128(V),128(K)]
  *   cu_seqlens [B+1] int32 or NULL (then request n owns token n)
  *   h0_indices [B] int32; invalid slot (<0 when is_sglang, <=0 otherwise) => zeros in o,
  *              no state access;  a request of length 0 touches nothing.
@@ -62,7 +64,7 @@ const char* pla_last_error(void);
 int pla_k_last_packed_launch(
     const void* A_log, int alog_dtype, const void* a, const void* dt_bias,
     float softplus_beta, float softplus_threshold,
-    const void* mixed_qkv, const void* b, void* o, float* h0,
+    const void* mixed_qkv, const void* b, void* o, void* h0, int state_dtype,
     const int32_t* cu_seqlens, const int32_t* h0_indices,
     float scale, int T_max,
     int64_t stride_a, int64_t stride_qkv, int64_t stride_b, int64_t h0_slot_stride,
@@ -81,7 +83,8 @@ int pla_k_last_packed_launch(
  *   a: gate input (see gate_mode); with PLA_GATE_LOG_DECAY it is float32
  *   b: raw beta logits (act dtype), or float32 activated beta when beta_is_activated
  *   dt_bias: float32 when dt_bias_is_f32 else act dtype
- *   cache: SGLang intermediate-state buffer [rows, cache_steps, HV,128,128] float32 or NULL;
+ *   h0, cache: of state_dtype (PLA_F32 or PLA_BF16; snapshots are rounded like the pool)
+ *   cache: SGLang intermediate-state buffer [rows, cache_steps, HV,128,128] or NULL;
  *          step t of request n is written to cache[cache_indices[n]*cache_steps + t]
  *          when is_sglang and cache_indices[n] >= 0
  *   parents: int64 [B, >=T] eagle-tree parent steps (needs cache), or NULL
@@ -94,7 +97,7 @@ int pla_k_last_launch(
     const void* A_log, int alog_dtype, const void* a, const void* dt_bias, int dt_bias_is_f32,
     float softplus_beta_or_lower_bound, float softplus_threshold, int gate_mode,
     const void* q, const void* k, const void* v, const void* b, int beta_is_activated,
-    void* o, float* h0, const int32_t* cu_seqlens, float* cache,
+    void* o, void* h0, int state_dtype, const int32_t* cu_seqlens, void* cache,
     const int32_t* h0_indices, const int32_t* cache_indices, int cache_steps,
     const int64_t* parents, int64_t stride_parent_seq, int64_t stride_parent_token,
     float scale, int T_max,

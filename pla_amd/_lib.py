@@ -18,13 +18,13 @@ _c_int, _c_i64, _c_f, _c_p = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctype
 # name -> argtypes, in the order of include/pla_gfx950.h
 SIGNATURES = {
     "pla_k_last_packed_launch": [
-        _c_p, _c_int, _c_p, _c_p, _c_f, _c_f, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_int, _c_p, _c_p, _c_f, _c_f, _c_p, _c_p, _c_p, _c_p, _c_int, _c_p, _c_p,
         _c_f, _c_int, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
     "pla_k_last_launch": [
         _c_p, _c_int, _c_p, _c_p, _c_int, _c_f, _c_f, _c_int,
         _c_p, _c_p, _c_p, _c_p, _c_int,
-        _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_int,
+        _c_p, _c_p, _c_int, _c_p, _c_p, _c_p, _c_p, _c_int,
         _c_p, _c_i64, _c_i64, _c_f, _c_int,
         _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,

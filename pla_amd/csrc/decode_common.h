@@ -108,17 +108,21 @@ typedef float v4f_t __attribute__((ext_vector_type(4)));
 constexpr int kLoadPolicy = 2;        // nt
 constexpr int kStorePolicy = 2 | 16;  // nt | sc1
 
+// state_t is float or bf16_t (pools stored in bf16: the recurrence still runs in FP32, tiles are
+// widened on load and rounded to nearest even on store).
+template <typename state_t>
 struct Tile {
   __amdgpu_buffer_rsrc_t rsrc;
-  __device__ __forceinline__ explicit Tile(float* tile_base)
-      : rsrc(__builtin_amdgcn_make_buffer_rsrc(tile_base, 0, 65536, 0x00020000)) {}
+  __device__ __forceinline__ explicit Tile(state_t* tile_base)
+      : rsrc(__builtin_amdgcn_make_buffer_rsrc(tile_base, 0, 16384 * sizeof(state_t), 0x00020000)) {}
 };
+typedef int v2i_t __attribute__((ext_vector_type(2)));
 
 // `lane_off` is the lane's byte offset of (rowbase + half, channel 4c) inside the
 // tile; consecutive j are two rows (1 KiB) apart, so each instruction of the
 // wave moves 1 KiB of contiguous memory.
 template <int R>
-__device__ __forceinline__ void load_state(const Tile& t, int lane_off, float (&s)[R][4]) {
+__device__ __forceinline__ void load_state(const Tile<float>& t, int lane_off, float (&s)[R][4]) {
 #pragma unroll
   for (int j = 0; j < R; ++j) {
     // Whole-vector bit cast: a bit cast applied to a single vector component reads component 0.
@@ -128,11 +132,32 @@ __device__ __forceinline__ void load_state(const Tile& t, int lane_off, float (&
   }
 }
 template <int R>
-__device__ __forceinline__ void store_state(const Tile& t, int lane_off, const float (&s)[R][4]) {
+__device__ __forceinline__ void store_state(const Tile<float>& t, int lane_off, const float (&s)[R][4]) {
 #pragma unroll
   for (int j = 0; j < R; ++j) {
     const v4f_t v = {s[j][0], s[j][1], s[j][2], s[j][3]};
     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i_t, v), t.rsrc, lane_off + j * 1024, 0, kStorePolicy);
+  }
+}
+
+// bf16 pools: `lane_off` stays the FP32 byte offset; a bf16 tile is half as large, so an instruction
+// of the wave moves two adjacent rows = 512 bytes.
+template <int R>
+__device__ __forceinline__ void load_state(const Tile<bf16_t>& t, int lane_off, float (&s)[R][4]) {
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const v2i_t v = __builtin_bit_cast(
+        v2i_t, __builtin_amdgcn_raw_buffer_load_b64(t.rsrc, (lane_off >> 1) + j * 512, 0, kLoadPolicy));
+    s[j][0] = lo16<bf16_t>((uint32_t)v.x); s[j][1] = hi16<bf16_t>((uint32_t)v.x);
+    s[j][2] = lo16<bf16_t>((uint32_t)v.y); s[j][3] = hi16<bf16_t>((uint32_t)v.y);
+  }
+}
+template <int R>
+__device__ __forceinline__ void store_state(const Tile<bf16_t>& t, int lane_off, const float (&s)[R][4]) {
+#pragma unroll
+  for (int j = 0; j < R; ++j) {
+    const v2i_t v = {(int)pack2<bf16_t>(s[j][0], s[j][1]), (int)pack2<bf16_t>(s[j][2], s[j][3])};
+    __builtin_amdgcn_raw_buffer_store_b64(v, t.rsrc, (lane_off >> 1) + j * 512, 0, kStorePolicy);
   }
 }
 

@@ -27,7 +27,7 @@ struct KLastParams {
   float gate_p0;            // softplus_beta or lower_bound
   float softplus_threshold; int gate_mode;
   const void* q; const void* k; const void* v; const void* b; int beta_is_activated;
-  void* o; float* h0; const int32_t* cu_seqlens; float* cache;
+  void* o; void* h0; const int32_t* cu_seqlens; void* cache;   // pools of state_t
   const int32_t* h0_indices; const int32_t* cache_indices; int cache_steps;
   const int64_t* parents; int64_t stride_parent_seq, stride_parent_token;
   float scale; int T_max;
@@ -43,8 +43,10 @@ struct KLastParams {
 // where w_t and the coefficients c_{j,t} = beta_j k_j^T (A_{j+1} ... A_t q_t) need only K-vectors (ten
 // dot products for four tokens).  The state tile is then used once: four dot products per row and no
 // update (the read-once verify of src/decode/kda_replayssm/kda_mtp_verify.cu:630-652).
-template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false>
+template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false, typename state_t = float>
 __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
+  state_t* const pool = reinterpret_cast<state_t*>(p.h0);
+  state_t* const snapshots = reinterpret_cast<state_t*>(p.cache);
   constexpr int R = RPW / 2;
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   const bool have_state = p.h0 != nullptr && h0_idx >= 0;
   const int64_t tile_off = (int64_t)i_hv * 16384;                 // tile of this head inside a slot
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;      // bytes inside the tile
-  const Tile h_tile(have_state ? p.h0 + (int64_t)h0_idx * p.h0_slot_stride + tile_off : nullptr);
+  const Tile<state_t> h_tile(have_state ? pool + (int64_t)h0_idx * p.h0_slot_stride + tile_off : nullptr);
 
   int cidx = -1;
   if (MTP && p.cache != nullptr && p.cache_indices != nullptr) cidx = p.cache_indices[i_n];
@@ -302,7 +304,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         const int64_t parent = p.parents[(int64_t)i_n * p.stride_parent_seq + (int64_t)t * p.stride_parent_token];
         if (parent >= 0 && parent < t && parent != t - 1) {
           __threadfence();   // the snapshot was written by these same lanes at step `parent`
-          const Tile parent_tile(p.cache + ((int64_t)cidx * p.cache_steps + parent) * p.HV * 16384 + tile_off);
+          const Tile<state_t> parent_tile(snapshots + ((int64_t)cidx * p.cache_steps + parent) * p.HV * 16384 + tile_off);
           load_state<R>(parent_tile, lane_off, s);
         }
       }
@@ -312,15 +314,15 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     delta_rows<R, IS_KDA, true>(s, dec, dec_scalar, kv, qv, vv, beta, outv);
 
     if constexpr (MTP) {
-      float* snap = nullptr;
+      state_t* snap = nullptr;
       if (p.is_sglang) {
         if (p.cache != nullptr && cidx >= 0)
-          snap = p.cache + ((int64_t)cidx * p.cache_steps + t) * p.HV * 16384 + tile_off;
+          snap = snapshots + ((int64_t)cidx * p.cache_steps + t) * p.HV * 16384 + tile_off;
       } else if (p.stride_h0_indices_seq > 0 && p.h0_indices != nullptr && p.h0 != nullptr) {
         const int step_slot = p.h0_indices[(int64_t)i_n * p.stride_h0_indices_seq + t];
-        if (step_slot > 0) snap = p.h0 + (int64_t)step_slot * p.h0_slot_stride + tile_off;
+        if (step_slot > 0) snap = pool + (int64_t)step_slot * p.h0_slot_stride + tile_off;
       }
-      if (snap != nullptr) store_state<R>(Tile(snap), lane_off, s);
+      if (snap != nullptr) store_state<R>(Tile<state_t>(snap), lane_off, s);
     }
     store_row_scalars<act_t, RPW>(o_base + (int64_t)t * p.HV * 128, lane, outv);
     cur = nxt;
@@ -337,13 +339,13 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
 // instruction stream per wave by about a third.
 struct DecodeParams {
   const float* A_log; const void* a; const void* dt_bias; const void* q; const void* k; const void* v;
-  const void* b; void* o; float* h0; const int32_t* cu_seqlens; const int32_t* h0_indices;
+  const void* b; void* o; void* h0; const int32_t* cu_seqlens; const int32_t* h0_indices;
   float softplus_beta, softplus_threshold, scale;
   int64_t stride_a, stride_q, stride_k, stride_v, stride_b, h0_slot_stride;
   int H, HV, use_qk_l2norm, is_sglang;
 };
 
-template <typename act_t, bool IS_KDA, int RPW>
+template <typename act_t, bool IS_KDA, int RPW, typename state_t = float>
 __global__ __launch_bounds__(256) void k_last_decode_kernel(const DecodeParams p) {
   constexpr int R = RPW / 2;
   const int lane = threadIdx.x & 63;
@@ -372,7 +374,7 @@ __global__ __launch_bounds__(256) void k_last_decode_kernel(const DecodeParams p
   }
   const bool have_state = h0_idx >= 0;
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
-  const Tile h_tile(have_state ? p.h0 + (int64_t)h0_idx * p.h0_slot_stride + (int64_t)i_hv * 16384 : nullptr);
+  const Tile<state_t> h_tile(have_state ? reinterpret_cast<state_t*>(p.h0) + (int64_t)h0_idx * p.h0_slot_stride + (int64_t)i_hv * 16384 : nullptr);
   float s[R][4];
   if (have_state) {
     load_state<R>(h_tile, lane_off, s);
@@ -445,7 +447,7 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
   if (slot <= p.null_block_id || n_acc <= 0) return;
   if (n_acc > p.L) n_acc = p.L;
 
-  const Tile h_tile(p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
+  const Tile<float> h_tile(p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
   float s[R][4];
   load_state<R>(h_tile, lane_off, s);
@@ -484,11 +486,11 @@ static int pick_rows_per_wave(int tiles, bool mtp) {
   return 8;
 }
 
-template <typename act_t, bool IS_KDA, bool MTP>
+template <typename act_t, bool IS_KDA, bool MTP, typename state_t>
 static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
   const dim3 block(256);
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
-  if constexpr (MTP) {
+  if constexpr (MTP && sizeof(state_t) == 4) {
     // a verify that leaves no trace in memory but o: the state is read once and used once
     const bool read_once = p.disable_state_update && p.T_max <= 4 && p.cache == nullptr && p.cache_indices == nullptr &&
                            p.parents == nullptr && p.stride_h0_indices_seq == 0;
@@ -503,18 +505,18 @@ static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
     }
   }
   switch (rpw) {
-    case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 32>), dim3(tiles, 1), block, 0, stream, p); break;
-    case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 16>), dim3(tiles, 2), block, 0, stream, p); break;
-    case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 8>),  dim3(tiles, 4), block, 0, stream, p); break;
+    case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 32, false, state_t>), dim3(tiles, 1), block, 0, stream, p); break;
+    case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 16, false, state_t>), dim3(tiles, 2), block, 0, stream, p); break;
+    case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 8, false, state_t>),  dim3(tiles, 4), block, 0, stream, p); break;
     default: return fail("rows_per_wave must be 0, 8, 16 or 32, got %d", rpw);
   }
   return check_launch("k_last_kernel launch");
 }
 
-template <typename act_t>
+template <typename act_t, typename state_t>
 static int launch_flags(const KLastParams& p, bool is_kda, bool mtp, int rpw, hipStream_t stream) {
-  if (is_kda) return mtp ? launch_rpw<act_t, true, true>(p, rpw, stream) : launch_rpw<act_t, true, false>(p, rpw, stream);
-  return mtp ? launch_rpw<act_t, false, true>(p, rpw, stream) : launch_rpw<act_t, false, false>(p, rpw, stream);
+  if (is_kda) return mtp ? launch_rpw<act_t, true, true, state_t>(p, rpw, stream) : launch_rpw<act_t, true, false, state_t>(p, rpw, stream);
+  return mtp ? launch_rpw<act_t, false, true, state_t>(p, rpw, stream) : launch_rpw<act_t, false, false, state_t>(p, rpw, stream);
 }
 
 static int check_common(int B, int H, int HV, int K, int V, int act_dtype, int alog_dtype, int T_max) {
@@ -530,19 +532,20 @@ static int check_common(int B, int H, int HV, int K, int V, int act_dtype, int a
 
 static bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-template <typename act_t, bool IS_KDA>
+template <typename act_t, bool IS_KDA, typename state_t>
 static int launch_decode(const DecodeParams& d, unsigned tiles, int rpw, hipStream_t stream) {
   const dim3 block(256);
   switch (rpw) {
-    case 32: hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 32>), dim3(tiles, 1), block, 0, stream, d); break;
-    case 16: hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 16>), dim3(tiles, 2), block, 0, stream, d); break;
-    case 8:  hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 8>),  dim3(tiles, 4), block, 0, stream, d); break;
+    case 32: hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 32, state_t>), dim3(tiles, 1), block, 0, stream, d); break;
+    case 16: hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 16, state_t>), dim3(tiles, 2), block, 0, stream, d); break;
+    case 8:  hipLaunchKernelGGL((k_last_decode_kernel<act_t, IS_KDA, 8, state_t>),  dim3(tiles, 4), block, 0, stream, d); break;
     default: return fail("rows_per_wave must be 0, 8, 16 or 32, got %d", rpw);
   }
   return check_launch("k_last_decode_kernel launch");
 }
 
-static int run_k_last(const KLastParams& p, bool is_kda, bool mtp, int act_dtype, int rows_per_wave, void* stream) {
+template <typename state_t>
+static int run_k_last_typed(const KLastParams& p, bool is_kda, bool mtp, int act_dtype, int rows_per_wave, void* stream) {
   const int rpw = rows_per_wave > 0 ? rows_per_wave : pick_rows_per_wave(p.B * p.HV, mtp);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool lean = !mtp && p.T_max == 1 && p.alog_dtype == PLA_F32 && p.gate_mode == PLA_GATE_SOFTPLUS &&
@@ -554,11 +557,23 @@ static int run_k_last(const KLastParams& p, bool is_kda, bool mtp, int act_dtype
                    p.H, p.HV, p.use_qk_l2norm, p.is_sglang};
     const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
     if (act_dtype == PLA_BF16)
-      return is_kda ? launch_decode<bf16_t, true>(d, tiles, rpw, s) : launch_decode<bf16_t, false>(d, tiles, rpw, s);
-    return is_kda ? launch_decode<f16_t, true>(d, tiles, rpw, s) : launch_decode<f16_t, false>(d, tiles, rpw, s);
+      return is_kda ? launch_decode<bf16_t, true, state_t>(d, tiles, rpw, s) : launch_decode<bf16_t, false, state_t>(d, tiles, rpw, s);
+    return is_kda ? launch_decode<f16_t, true, state_t>(d, tiles, rpw, s) : launch_decode<f16_t, false, state_t>(d, tiles, rpw, s);
   }
-  if (act_dtype == PLA_BF16) return launch_flags<bf16_t>(p, is_kda, mtp, rpw, s);
-  return launch_flags<f16_t>(p, is_kda, mtp, rpw, s);
+  if (act_dtype == PLA_BF16) return launch_flags<bf16_t, state_t>(p, is_kda, mtp, rpw, s);
+  return launch_flags<f16_t, state_t>(p, is_kda, mtp, rpw, s);
+}
+static int run_k_last(const KLastParams& p, bool is_kda, bool mtp, int act_dtype, int state_dtype, int rows_per_wave,
+                      void* stream) {
+  return state_dtype == PLA_BF16 ? run_k_last_typed<bf16_t>(p, is_kda, mtp, act_dtype, rows_per_wave, stream)
+                                 : run_k_last_typed<float>(p, is_kda, mtp, act_dtype, rows_per_wave, stream);
+}
+// Pool base and slot pitch: four elements (16 bytes FP32, 8 bytes bf16).
+static int check_pool(const void* h0, int state_dtype, int64_t h0_slot_stride, int HV, size_t base_align) {
+  PLA_REQUIRE(state_dtype == PLA_F32 || state_dtype == PLA_BF16, "state dtype must be float32 or bfloat16");
+  PLA_REQUIRE(aligned(h0, base_align) && h0_slot_stride % 4 == 0, "state base and slot pitch require 16-byte alignment");
+  PLA_REQUIRE(h0_slot_stride >= (int64_t)HV * 16384, "state slot pitch must cover HV*V*K");
+  return 0;
 }
 
 }  // namespace pla
@@ -568,7 +583,7 @@ using namespace pla;
 extern "C" int pla_k_last_packed_launch(
     const void* A_log, int alog_dtype, const void* a, const void* dt_bias,
     float softplus_beta, float softplus_threshold,
-    const void* mixed_qkv, const void* b, void* o, float* h0,
+    const void* mixed_qkv, const void* b, void* o, void* h0, int state_dtype,
     const int32_t* cu_seqlens, const int32_t* h0_indices,
     float scale, int T_max,
     int64_t stride_a, int64_t stride_qkv, int64_t stride_b, int64_t h0_slot_stride,
@@ -580,9 +595,8 @@ extern "C" int pla_k_last_packed_launch(
   PLA_REQUIRE(A_log && a && dt_bias && mixed_qkv && b && o, "null tensor pointer");
   PLA_REQUIRE(h0 != nullptr, "initial_state_source is required for k_last_packed");
   PLA_REQUIRE(aligned(mixed_qkv, 16) && stride_qkv % 8 == 0, "mixed_qkv base and token stride require 16-byte alignment");
-  PLA_REQUIRE(aligned(h0, 16) && h0_slot_stride % 4 == 0, "state base and slot pitch require 16-byte alignment");
+  if (check_pool(h0, state_dtype, h0_slot_stride, HV, 16)) return 1;
   PLA_REQUIRE(aligned(o, 16), "out requires 16-byte alignment");
-  PLA_REQUIRE(h0_slot_stride >= (int64_t)HV * 16384, "state slot pitch must cover HV*V*K");
   PLA_REQUIRE(stride_qkv >= (int64_t)(2 * H + HV) * 128, "mixed_qkv token stride must cover its complete row");
   if (is_kda) PLA_REQUIRE(aligned(a, 8) && stride_a % 4 == 0 && aligned(dt_bias, 8), "KDA a/dt_bias require 8-byte alignment");
   KLastParams p{};
@@ -597,14 +611,14 @@ extern "C" int pla_k_last_packed_launch(
   p.stride_a = stride_a; p.stride_q = p.stride_k = p.stride_v = stride_qkv; p.stride_b = stride_b;
   p.h0_slot_stride = h0_slot_stride; p.B = B; p.H = H; p.HV = HV;
   p.use_qk_l2norm = use_qk_l2norm; p.disable_state_update = 0; p.is_sglang = is_sglang;
-  return run_k_last(p, is_kda != 0, false, act_dtype, rows_per_wave, stream);
+  return run_k_last(p, is_kda != 0, false, act_dtype, state_dtype, rows_per_wave, stream);
 }
 
 extern "C" int pla_k_last_launch(
     const void* A_log, int alog_dtype, const void* a, const void* dt_bias, int dt_bias_is_f32,
     float softplus_beta_or_lower_bound, float softplus_threshold, int gate_mode,
     const void* q, const void* k, const void* v, const void* b, int beta_is_activated,
-    void* o, float* h0, const int32_t* cu_seqlens, float* cache,
+    void* o, void* h0, int state_dtype, const int32_t* cu_seqlens, void* cache,
     const int32_t* h0_indices, const int32_t* cache_indices, int cache_steps,
     const int64_t* parents, int64_t stride_parent_seq, int64_t stride_parent_token,
     float scale, int T_max,
@@ -622,9 +636,10 @@ extern "C" int pla_k_last_launch(
   PLA_REQUIRE(aligned(q, 8) && aligned(k, 8) && aligned(v, 16) && stride_q % 4 == 0 && stride_k % 4 == 0 && stride_v % 8 == 0,
               "q/k/v base and token stride require 16-byte alignment");
   PLA_REQUIRE(aligned(o, 16), "out requires 16-byte alignment");
-  if (h0) PLA_REQUIRE(aligned(h0, 16) && h0_slot_stride % 4 == 0 && h0_slot_stride >= (int64_t)HV * 16384,
-                      "state base and slot pitch require 16-byte alignment and must cover HV*V*K");
-  if (cache) PLA_REQUIRE(aligned(cache, 16), "intermediate cache base requires 16-byte vector alignment");
+  PLA_REQUIRE(state_dtype == PLA_F32 || state_dtype == PLA_BF16, "state dtype must be float32 or bfloat16");
+  const size_t pool_align = state_dtype == PLA_F32 ? 16 : 8;
+  if (h0 && check_pool(h0, state_dtype, h0_slot_stride, HV, pool_align)) return 1;
+  if (cache) PLA_REQUIRE(aligned(cache, pool_align), "intermediate cache base requires vector alignment (four elements)");
   if (cache) PLA_REQUIRE(cache_steps > 0, "intermediate cache requires a positive step pitch");
   if (is_kda) {
     const size_t need = gate_mode == PLA_GATE_LOG_DECAY ? 16 : 8;
@@ -648,7 +663,7 @@ extern "C" int pla_k_last_launch(
   p.num_accepted = num_accepted; p.stride_h0_indices_seq = stride_h0_indices_seq; p.is_sglang = is_sglang;
   const bool mtp = T_max > 1 || disable_state_update || cache != nullptr || cache_indices != nullptr ||
                    parents != nullptr || stride_h0_indices_seq > 0;
-  return run_k_last(p, is_kda != 0, mtp, act_dtype, rows_per_wave, stream);
+  return run_k_last(p, is_kda != 0, mtp, act_dtype, state_dtype, rows_per_wave, stream);
 }
 
 extern "C" int pla_kda_fold_launch(

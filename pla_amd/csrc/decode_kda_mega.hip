@@ -74,7 +74,7 @@ __global__ __launch_bounds__(256) void kda_decode_mega_kernel(const MegaParams p
   // state tile first: everything below overlaps its latency
   const int rowbase = wave * RPW;
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
-  const Tile h_tile(p.state + (int64_t)slot * p.state_slot + (int64_t)i_h * 16384);
+  const Tile<float> h_tile(p.state + (int64_t)slot * p.state_slot + (int64_t)i_h * 16384);
   float s[R][4];
   load_state<R>(h_tile, lane_off, s);
 

@@ -89,8 +89,8 @@ def _packed_impl(mixed_qkv, a, b, A_log, dt_bias, softplus_beta, softplus_thresh
     _check(mixed_qkv.dtype in (torch.bfloat16, torch.float16), "mixed_qkv must be fp16 or bf16")
     _check(a.dtype == mixed_qkv.dtype and b.dtype == mixed_qkv.dtype and dt_bias.dtype == mixed_qkv.dtype
            and out.dtype == mixed_qkv.dtype, "a, b, dt_bias and out must have mixed_qkv's dtype")
-    _check(state.dtype == torch.float32,
-           f"initial_state_source dtype not supported: {state.dtype} (this build streams float32 pools)")
+    _check(state.dtype in (torch.float32, torch.bfloat16),
+           f"k-last state dtype must be float32 or bfloat16, got {state.dtype}")
     _check(mixed_qkv.stride(1) == 1 and state.stride(-1) == 1 and state.stride(-2) == K
            and state.stride(-3) == V * K, "mixed_qkv rows and state slots must be dense")
     _check(out.is_contiguous(), "out must be contiguous")
@@ -110,7 +110,7 @@ def _packed_impl(mixed_qkv, a, b, A_log, dt_bias, softplus_beta, softplus_thresh
         "pla_k_last_packed_launch",
         A_log.data_ptr(), _lib.dtype_code(A_log.dtype), a.data_ptr(), dt_bias.data_ptr(),
         float(softplus_beta), float(softplus_threshold),
-        mixed_qkv.data_ptr(), b.data_ptr(), out.data_ptr(), state.data_ptr(),
+        mixed_qkv.data_ptr(), b.data_ptr(), out.data_ptr(), state.data_ptr(), _lib.dtype_code(state.dtype),
         _lib.ptr(cu_seqlens), _lib.ptr(initial_state_indices),
         scale_val, 1,
         a.stride(a.dim() - 2), mixed_qkv.stride(0), b.stride(b.dim() - 2), state.stride(0),
@@ -227,7 +227,6 @@ def _k_last_impl(A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, 
            f"k-last state dtype must be float32 or bfloat16, got {state_dtype}")
     _check(cache is None or cache.dtype == state_dtype,
            "initial_state_source and intermediate_states_buffer must have the same dtype")
-    _check(state_dtype == torch.float32, "this build streams float32 state pools only")
 
     B = cu_seqlens.size(0) - 1 if cu_seqlens is not None else k.size(0)
     target_verify = (cache is not None or intermediate_state_indices is not None
@@ -297,7 +296,7 @@ def _k_last_impl(A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, 
         A_log.data_ptr(), _lib.dtype_code(A_log.dtype), a.data_ptr(), dt_bias.data_ptr(),
         int(dt_bias.dtype == torch.float32), p0, float(softplus_threshold), gate_mode,
         q.data_ptr(), k.data_ptr(), v.data_ptr(), b.data_ptr(), 0,
-        o.data_ptr(), _lib.ptr(state), _lib.ptr(cu_seqlens), _lib.ptr(cache),
+        o.data_ptr(), _lib.ptr(state), _lib.dtype_code(state_dtype), _lib.ptr(cu_seqlens), _lib.ptr(cache),
         _lib.ptr(idx), _lib.ptr(intermediate_state_indices), int(cache_steps_eff),
         _lib.ptr(parents), sps, spt, scale_val, int(T_max),
         stride_a, _token_stride(q), _token_stride(k), _token_stride(v), b.stride(b.dim() - 2),

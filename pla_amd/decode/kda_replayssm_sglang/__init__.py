@@ -106,7 +106,7 @@ def kda_mtp_verify(q, k, v, g, beta, recurrent_state, ssm_state_indices, cu_seql
         "pla_k_last_launch",
         None, _lib.F32, g.data_ptr(), None, 0, 0.0, 20.0, _lib.GATE_LOG_DECAY,
         q.data_ptr(), k.data_ptr(), v.data_ptr(), beta.data_ptr(), 1,
-        out.data_ptr(), recurrent_state.data_ptr(), cu_seqlens.data_ptr(), None,
+        out.data_ptr(), recurrent_state.data_ptr(), _lib.F32, cu_seqlens.data_ptr(), None,
         ssm_state_indices.data_ptr(), None, 0, None, 0, 0,
         float(scale) if scale is not None else K ** -0.5, int(max_tokens),
         HV * 128, q.stride(1), k.stride(1), v.stride(1), HV, recurrent_state.stride(0),

@@ -11,7 +11,7 @@ def rel_l2(got, want):
 
 
 def make_k_last_case(is_kda, mode, *, H=4, HV=8, B=3, T=None, seed=2026, padded=True,
-                     act_dtype=torch.bfloat16, device="cuda"):
+                     act_dtype=torch.bfloat16, device="cuda", state_dtype=torch.float32):
     """Small decode / MTP case in the style of the reference's k-last tests
     (tests/test_k_last_state_dtype.py:55-105): slot pool with a padded pitch and guard
     floats, non-trivial slot ids including an SGLang pad, a sentinel-filled cache."""
@@ -28,12 +28,12 @@ def make_k_last_case(is_kda, mode, *, H=4, HV=8, B=3, T=None, seed=2026, padded=
         return torch.randn(*shape, generator=g).to(dtype).to(device)
 
     slots = max(7, B + 2)
-    backing = (torch.randn(slots, HV * D * D + 256, generator=g) * 0.1).to(device)
+    backing = (torch.randn(slots, HV * D * D + 256, generator=g) * 0.1).to(state_dtype).to(device)
     state = backing[:, : HV * D * D].view(slots, HV, D, D)
     state_ids = [3, 0, -1] if padded and B == 3 else list(range(B))
     cache_ids = [2, 0, 1] if padded and B == 3 else list(reversed(range(B)))
     cache = None if mode == "decode" else torch.full(
-        (max(4, B + 1), T + 3, HV, D, D), -7.0, dtype=torch.float32, device=device)
+        (max(4, B + 1), T + 3, HV, D, D), -7.0, dtype=state_dtype, device=device)
     parents = None
     if mode == "tree":
         parents = torch.tensor([[max(0, t - 2) for t in range(T)]] * B, dtype=torch.int32, device=device)

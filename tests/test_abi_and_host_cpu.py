@@ -58,10 +58,10 @@ def test_native_entry_points_reject_bad_arguments_without_a_gpu():
     """Argument checks run before any launch, so they are testable on a CPU-only host."""
     from pla_amd import _lib
     lib = _lib.load()
-    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, None, None,
+    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, _lib.F32, None, None,
                                       0.1, 1, 0, 0, 0, 0, 4, 2, 4, 64, 64, 1, 1, 0, _lib.BF16, 0, None)
     assert rc != 0 and b"K == V == 128" in lib.pla_last_error()
-    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, None, None,
+    rc = lib.pla_k_last_packed_launch(None, 0, None, None, 1.0, 20.0, None, None, None, None, _lib.F32, None, None,
                                       0.1, 1, 0, 0, 0, 0, 4, 3, 4, 128, 128, 1, 1, 0, _lib.BF16, 0, None)
     assert rc != 0 and b"multiple of H" in lib.pla_last_error()
     rc = lib.pla_kda_prefill_launch(None, None, None, None, None, 0, 0, 0, 0, 0, None, None, -7.0, 1.0,

@@ -90,6 +90,62 @@ def test_k_last_modes(is_kda, mode, H, HV, act_dtype):
     _check_case("k_last", args, backing, lengths, state_ids, cache_ids, tile=tile, graph=mode == "graph")
 
 
+@pytest.mark.parametrize("is_kda", [False, True])
+@pytest.mark.parametrize("mode", ["decode", "packed", "verify", "writeback", "tree", "ragged", "graph", "tunable"])
+@pytest.mark.parametrize("H,HV", [(4, 8), (6, 18)])
+@pytest.mark.parametrize("act_dtype", [torch.bfloat16, torch.float16])
+def test_k_last_modes_bf16_state_pool(is_kda, mode, H, HV, act_dtype):
+    """bf16 pools and snapshot caches: FP32 recurrence, tiles widened on load and rounded on store; a
+    tree branch reloads the rounded snapshot (tests/test_k_last_state_dtype.py:108-196)."""
+    case_mode = "verify" if mode in ("graph", "tunable") else ("decode" if mode == "packed" else mode)
+    args, backing, lengths, state_ids, cache_ids = make_k_last_case(
+        is_kda, case_mode, H=H, HV=HV, act_dtype=act_dtype, state_dtype=torch.bfloat16)
+    tile = dict(bv=64, wn=8, sn=4, hv_per_cta=1) if mode == "tunable" else None
+    _check_case("packed" if mode == "packed" else "k_last", args, backing, lengths, state_ids, cache_ids,
+                tile=tile, graph=mode == "graph")
+    assert args["initial_state_source"].dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("state_dtype,cache_dtype,message", [
+    (torch.float16, torch.float16, "state dtype must be"),
+    (torch.float32, torch.bfloat16, "must have the same dtype"),
+    (torch.bfloat16, torch.float32, "must have the same dtype")])
+def test_rejects_state_dtype_combinations(state_dtype, cache_dtype, message):
+    forward = _ops()[0]
+    args, backing, _, _, _ = make_k_last_case(False, "verify", state_dtype=state_dtype)
+    args["intermediate_states_buffer"] = args["intermediate_states_buffer"].to(cache_dtype)
+    before = backing.clone()
+    with pytest.raises(RuntimeError, match=message):
+        forward(**args)
+    torch.cuda.synchronize()
+    assert torch.equal(backing.view(torch.int16 if state_dtype != torch.float32 else torch.int32),
+                       before.view(torch.int16 if state_dtype != torch.float32 else torch.int32))
+
+
+def test_bf16_pool_b64_kda_packed_decode_at_scale():
+    """B=64 x 32 heads over a 128-slot bf16 pool with a padded pitch, 5 % padded requests."""
+    from pla_amd.workloads import gdn_decode_packed
+    from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
+    w = gdn_decode_packed(64, H=32, HV=32, pool_slots=128, pad_frac=0.05, seed=77, is_kda=True, pitch_pad=64)
+    pool32 = w["initial_state_source"]
+    backing = torch.zeros(128, 32 * 128 * 128 + 64, dtype=torch.bfloat16, device="cuda")
+    pool = backing[:, :32 * 128 * 128].view(128, 32, 128, 128)
+    pool.copy_(pool32)
+    w["initial_state_source"] = pool
+    before = backing.clone()
+    exp_out, exp_states = oracle_packed_workload(w)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    out = packed(**call)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu().float().reshape(exp_out.shape), exp_out.float(), atol=2e-2, rtol=2e-2)
+    for slot, want in exp_states.items():
+        assert want.dtype == torch.bfloat16
+        torch.testing.assert_close(pool[slot].cpu(), want, **STATE_TOL)
+    untouched = [s for s in range(128) if s not in exp_states]
+    assert torch.equal(backing[untouched].view(torch.int16), before[untouched].view(torch.int16))
+    assert torch.equal(backing[:, -64:].view(torch.int16), before[:, -64:].view(torch.int16))
+
+
 @pytest.mark.parametrize("kernel", ["k_last", "packed"])
 @pytest.mark.parametrize("H,HV", [(3, 3), (5, 5), (3, 6), (12, 24), (4, 12), (1, 1), (16, 32), (32, 32), (64, 64)])
 @pytest.mark.parametrize("is_kda", [False, True])
