@@ -18,6 +18,7 @@
 // above T_max) make the request a no-op instead of trapping the device.
 
 #include "decode_common.h"
+#include "mfma_bf16.h"
 
 namespace pla {
 
@@ -41,8 +42,12 @@ struct KLastParams {
 // the recurrence is unrolled algebraically instead of being stepped through the state,
 //     o_t = S_0 w_t + sum_{j <= t} c_{j,t} v_j,   w_t = A_1 ... A_t q_t,   A_j = D_j (I - beta_j k_j k_j^T),
 // where w_t and the coefficients c_{j,t} = beta_j k_j^T (A_{j+1} ... A_t q_t) need only K-vectors (ten
-// dot products for four tokens).  The state tile is then used once: four dot products per row and no
-// update (the read-once verify of src/decode/kda_replayssm/kda_mtp_verify.cu:630-652).
+// dot products for four tokens; wavefront t of the workgroup works out token t and publishes w_t and
+// c_{.,t} in LDS).  The state tile is then used once, as the A operand of S_0 [w_0 .. w_3] on
+// v_mfma_f32_16x16x32_bf16: FP32 rows and effective queries are split into bf16 hi + lo parts (three
+// products keep 16 mantissa bits), so there are no cross-lane reductions over the tile at all (the
+// read-once verify of src/decode/kda_replayssm/kda_mtp_verify.cu:630-652).  One workgroup covers a
+// whole tile: RPW is 32 and wavefront w owns rows 32 w .. 32 w + 31 as two 16-row MFMA tiles.
 template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false, typename state_t = float>
 __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   state_t* const pool = reinterpret_cast<state_t*>(p.h0);
@@ -126,7 +131,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     uint32_t vw[R];
   };
   auto fetch = [&](int t) {
-    TokenIn in;
+    TokenIn in{};
     const int64_t tok = (int64_t)bos + t;
     in.qw = *reinterpret_cast<const uint2*>(qp + tok * p.stride_q);
     in.kw = *reinterpret_cast<const uint2*>(kp + tok * p.stride_k);
@@ -138,7 +143,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       in.a1 = fetch_scalar(p.a, log_decay, tok * p.stride_a + i_hv);
     }
     in.b1 = fetch_scalar(p.b, beta_wide, tok * p.stride_b + i_hv);
-    load_row_words<RPW>(vp + tok * p.stride_v, in.vw);
+    if constexpr (!READONCE) load_row_words<RPW>(vp + tok * p.stride_v, in.vw);
     return in;
   };
 
@@ -152,7 +157,31 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       if (t < T) ahead[t - 1] = fetch(t);
   }
   float s[R][4];
-  if (have_state) {
+  // read-once verify: the tile in MFMA A-operand layout, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
+  const int r16 = lane & 15, kb = lane >> 4;
+  f32x4_t sa[2][4][2];
+  uint2 vq[2][4];
+  if constexpr (READONCE) {
+    static_assert(!READONCE || (RPW == 32 && sizeof(state_t) == 4), "the read-once verify covers a whole FP32 tile per workgroup");
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+          sa[m][ks][hf] = have_state ? __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                           h_tile.rsrc, at + 16 * hf, 0, kLoadPolicy))
+                                     : f32x4_t{0.f, 0.f, 0.f, 0.f};
+      }
+    // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one)
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
+                                                   ((int64_t)bos + min(t, T - 1)) * p.stride_v);
+  } else if (have_state) {
     load_state<R>(h_tile, lane_off, s);
   } else {
 #pragma unroll
@@ -169,22 +198,22 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
 
   if constexpr (READONCE) {
     const TokenIn tok[4] = {cur, ahead[0], ahead[1], ahead[2]};        // absent tokens repeat token 0, never stored
-    float qv[4][4], kv[4][4], dec[4][4], beta[4], vv[4][R];
+    __shared__ __align__(16) float sW[4][128];     // effective queries w_t
+    __shared__ __align__(16) float sC[4][4];       // sC[t][j] = c_{j,t}
+    float kv[4][4], dec[4][4], beta[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const TokenIn& in = tok[t];
-      const float q4[4] = {lo16<act_t>(in.qw.x), hi16<act_t>(in.qw.x), lo16<act_t>(in.qw.y), hi16<act_t>(in.qw.y)};
       const float k4[4] = {lo16<act_t>(in.kw.x), hi16<act_t>(in.kw.x), lo16<act_t>(in.kw.y), hi16<act_t>(in.kw.y)};
-      float qn = p.scale, kn = 1.f;
+      float kn = 1.f;
       if (p.use_qk_l2norm) {
-        float qs = 0.f, ks = 0.f;
+        float ks = 0.f;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { qs = fmaf(q4[e], q4[e], qs); ks = fmaf(k4[e], k4[e], ks); }
-        qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
+        for (int e = 0; e < 4; ++e) ks = fmaf(k4[e], k4[e], ks);
         kn = fast_rsqrt(row32_allreduce(ks) + 1e-6f);
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) { qv[t][e] = q4[e] * qn; kv[t][e] = k4[e] * kn; }
+      for (int e = 0; e < 4; ++e) kv[t][e] = k4[e] * kn;
       if constexpr (IS_KDA) {
         float av[4];
         decode_k4<act_t>(in.a4, log_decay, av);
@@ -199,65 +228,71 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       }
       const float b_in = decode_scalar_act<act_t>(in.b1, beta_wide);
       beta[t] = beta_wide ? b_in : fast_sigmoid(b_in);
-      row_scalars<act_t, RPW>(in.vw, half, vv[t]);
     }
-    // effective queries w_t and bias coefficients c_{j,t}
-    float qeff[4][4], coef[4][4];
+    // wavefront t: effective query w_t and bias coefficients c_{j,t} of token t
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      float w[4] = {qv[t][0], qv[t][1], qv[t][2], qv[t][3]};
+      if (wave != t) continue;
+      const TokenIn& in = tok[t];
+      const float q4[4] = {lo16<act_t>(in.qw.x), hi16<act_t>(in.qw.x), lo16<act_t>(in.qw.y), hi16<act_t>(in.qw.y)};
+      float qn = p.scale;
+      if (p.use_qk_l2norm) {
+        float qs = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) qs = fmaf(q4[e], q4[e], qs);
+        qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
+      }
+      float w[4] = {q4[0] * qn, q4[1] * qn, q4[2] * qn, q4[3] * qn};
+      float cf[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 3; j >= 0; --j) {
-        if (j > t) { coef[j][t] = 0.f; continue; }
+        if (j > t) continue;
         float dot = 0.f;
 #pragma unroll
         for (int e = 0; e < 4; ++e) dot = fmaf(kv[j][e], w[e], dot);
-        const float cf = beta[j] * row32_allreduce(dot);
-        coef[j][t] = cf;
+        cf[j] = beta[j] * row32_allreduce(dot);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf, kv[j][e], w[e]);
+        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf[j], kv[j][e], w[e]);
       }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) qeff[t][e] = w[e];
+      if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
+      if (lane == 0) *reinterpret_cast<float4*>(&sC[t][0]) = make_float4(cf[0], cf[1], cf[2], cf[3]);
     }
-    // The lane's partial sums of S_0 w_t for its R rows.  They are reduced over the 32 lanes of a state
-    // row in two steps: a lane swap between the two DPP rows of a half (one swap and one add per pair
-    // of values: the even DPP row ends up with tokens 0 and 1, the odd one with tokens 2 and 3), then
-    // four DPP adds inside the 16 lanes.
-    const bool odd_row = (lane >> 4) & 1;
+    __syncthreads();
+    // B operands: column r16 of [w_0 .. w_3 0 .. 0], contraction elements 32 ks + 8 kb .. + 7
+    const int tcol = min(r16, 3);
+    const float keep = r16 < 4 ? 1.f : 0.f;
+    HiLo wb[4];
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      float keep[R];
+    for (int ks = 0; ks < 4; ++ks) {
+      const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb]);
+      const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb + 4]);
+      wb[ks] = split8(f32x4_t{w0.x * keep, w0.y * keep, w0.z * keep, w0.w * keep},
+                      f32x4_t{w1.x * keep, w1.y * keep, w1.z * keep, w1.w * keep});
+    }
+    const float4 cmine = *reinterpret_cast<const float4*>(&sC[tcol][0]);
+    const float cs[4] = {cmine.x, cmine.y, cmine.z, cmine.w};
 #pragma unroll
-      for (int j = 0; j < R; ++j) {
-        float a = 0.f, b = 0.f;
+    for (int m = 0; m < 2; ++m) {
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          a = fmaf(s[j][e], qeff[tt][e], a);
-          b = fmaf(s[j][e], qeff[tt + 2][e], b);
-        }
-        asm("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
-        keep[j] = row16_allreduce(a + b);
+      for (int ks = 0; ks < 4; ++ks) {
+        const HiLo a = split8(sa[m][ks][0], sa[m][ks][1]);
+        acc = mfma16(a.hi, wb[ks].hi, acc);
+        acc = mfma16(a.lo, wb[ks].hi, acc);
+        acc = mfma16(a.hi, wb[ks].lo, acc);
       }
-      float cs[4];
+      // lane (r16 = token, kb): rows 16 m + 4 kb .. + 3 of S_0 w_token; add the bias terms
+      float o[4] = {acc[0], acc[1], acc[2], acc[3]};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) cs[j] = odd_row ? coef[j][tt + 2] : coef[j][tt];
-      uint32_t wout[R];
-#pragma unroll
-      for (int j = 0; j < R; ++j) {
-        float o = keep[j];
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) o = fmaf(cs[jj], vv[jj][j], o);
-        const LanePair both = swap_halves(o);      // even state row from lanes 0-31, odd one from lanes 32-63
-        wout[j] = pack2<act_t>(both.lo, both.hi);
+      for (int j = 0; j < 4; ++j) {
+        o[0] = fmaf(cs[j], lo16<act_t>(vq[m][j].x), o[0]);
+        o[1] = fmaf(cs[j], hi16<act_t>(vq[m][j].x), o[1]);
+        o[2] = fmaf(cs[j], lo16<act_t>(vq[m][j].y), o[2]);
+        o[3] = fmaf(cs[j], hi16<act_t>(vq[m][j].y), o[3]);
       }
-      const int t_mine = tt + (odd_row ? 2 : 0);
-      if ((lane & 47) == 0 && t_mine < T) {         // lanes 0 and 16 write two tokens each
-        act_t* dst = o_base + (int64_t)t_mine * p.HV * 128;
-#pragma unroll
-        for (int i = 0; i < RPW / 8; ++i)
-          reinterpret_cast<uint4*>(dst)[i] = make_uint4(wout[4 * i], wout[4 * i + 1], wout[4 * i + 2], wout[4 * i + 3]);
-      }
+      if (r16 < 4 && r16 < T)
+        *reinterpret_cast<uint2*>(o_base + (int64_t)r16 * p.HV * 128 + 16 * m + 4 * kb) =
+            make_uint2(pack2<act_t>(o[0], o[1]), pack2<act_t>(o[2], o[3]));
     }
     return;
   }
@@ -495,12 +530,7 @@ static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
     const bool read_once = p.disable_state_update && p.T_max <= 4 && p.cache == nullptr && p.cache_indices == nullptr &&
                            p.parents == nullptr && p.stride_h0_indices_seq == 0;
     if (read_once) {
-      switch (rpw) {
-        case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true>), dim3(tiles, 1), block, 0, stream, p); break;
-        case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 16, true>), dim3(tiles, 2), block, 0, stream, p); break;
-        case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 8, true>),  dim3(tiles, 4), block, 0, stream, p); break;
-        default: return fail("rows_per_wave must be 0, 8, 16 or 32, got %d", rpw);
-      }
+      hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true>), dim3(tiles, 1), block, 0, stream, p);
       return check_launch("k_last_kernel launch");
     }
   }

@@ -198,6 +198,60 @@ def test_mtp_lengths(T, mode, lower_bound):
     _check_case("k_last", args, backing, lengths, state_ids, cache_ids)
 
 
+@pytest.mark.parametrize("is_kda,lower_bound", [(False, None), (True, None), (True, -5.0)])
+@pytest.mark.parametrize("T", [1, 2, 3, 4])
+@pytest.mark.parametrize("H,HV", [(4, 8), (6, 6)])
+@pytest.mark.parametrize("act_dtype", [torch.bfloat16, torch.float16])
+def test_read_once_verify(is_kda, lower_bound, T, H, HV, act_dtype):
+    """A verify that writes neither state nor snapshots (up to four draft tokens, [B, T, ...] inputs, no
+    cache) takes the read-once kernel: outputs equal the stepped recurrence, the pool stays bit-identical."""
+    forward = _ops()[0]
+    args, backing, lengths, state_ids, _ = make_k_last_case(is_kda, "verify", H=H, HV=HV, T=T, act_dtype=act_dtype)
+    B = len(lengths)
+    for name in ("q", "k", "v", "a", "b"):
+        args[name] = args[name].reshape(B, T, *args[name].shape[2:]).contiguous()
+    args.update(cu_seqlens=None, intermediate_states_buffer=None, intermediate_state_indices=None,
+                cache_steps_or_num_accept=None, disable_state_update=True)
+    if lower_bound is not None:
+        args["lower_bound"] = lower_bound
+    flat = dict(args)
+    for name in ("q", "k", "v", "a", "b"):
+        flat[name] = args[name].reshape(1, B * T, *args[name].shape[2:])
+    exp_out, _, _ = oracle_k_last(flat, lengths, state_ids, None)
+    before = backing.clone()
+    out = forward(**args)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.reshape(exp_out.shape).cpu().float(), exp_out.float(), **_out_tol(out.dtype))
+    assert torch.equal(backing, before)
+    pad = [n for n, s in enumerate(state_ids) if s < 0]
+    assert pad and all(torch.count_nonzero(out[n]) == 0 for n in pad)
+
+
+def test_read_once_verify_ragged_requests():
+    """Requests of 4, 2, 0, 3 and 1 draft tokens in one launch, a padded request among them."""
+    from pla_amd.decode.kda_replayssm_sglang import kda_mtp_verify
+    from oracle import k_last_reference
+    g = torch.Generator().manual_seed(77)
+    lengths, slots = [4, 2, 0, 3, 1, 4], [5, 0, 3, -1, 2, 6]
+    nt, H, D = sum(lengths), 6, 128
+    rnd = lambda *shape: torch.randn(*shape, generator=g)
+    q, k, v = (rnd(1, nt, H, D).to(torch.bfloat16) for _ in range(3))
+    log_decay = -torch.nn.functional.softplus(rnd(nt, H, D)) * torch.rand(nt, H, D, generator=g)
+    beta = torch.sigmoid(rnd(nt, H))
+    pool = rnd(8, H, D, D) * 0.1
+    cu = torch.tensor([0] + torch.tensor(lengths).cumsum(0).tolist(), dtype=torch.int32)
+    want, _, _ = k_last_reference(q[0], k[0], v[0], None, None, None, None, pool, slots, lengths, is_kda=True,
+                                  disable_state_update=True, log_decay=log_decay, beta_activated=beta)
+    pool_d = pool.cuda()
+    before = pool_d.clone()
+    out = kda_mtp_verify(q.cuda(), k.cuda(), v.cuda(), log_decay.cuda(), beta.cuda(), pool_d,
+                         torch.tensor(slots, dtype=torch.int32, device="cuda"), cu.cuda(), max_tokens=4)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out[0].cpu().float(), want.float(), atol=1e-3, rtol=1.6e-2)
+    assert torch.equal(pool_d, before)
+    assert torch.count_nonzero(out[0, 6:9]) == 0                                      # the padded request's three tokens
+
+
 @pytest.mark.parametrize("layout", ["heads3", "strided_heads3", "flat2", "flat3", "batch4"])
 @pytest.mark.parametrize("mode", ["decode", "tree"])
 def test_kda_gate_layouts(layout, mode):
