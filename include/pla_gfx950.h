@@ -163,6 +163,58 @@ int pla_kda_decode_mega_launch(
     int64_t conv_slot, int64_t state_slot, void* stream);
 
 /*
+ * KDA speculative verify with replay records, ring mode (SGLang ReplaySSM).  Replaces launch_verify
+ * (src/decode/kda_replayssm/kda_mtp_abi.h:316-330; kernel src/decode/kda_replayssm/kda_mtp_verify.cu,
+ * host contract src/decode/kda_replayssm_sglang/kda_mtp_verify_host.cpp:50-243) with the stride structs
+ * flattened and the index tensors passed as (pointer, is_int64).
+ *
+ *   x_q, x_k, x_v, g_in [T,H,128] bf16 (token strides strides[0..3]), beta_in [T,H] bf16 (strides[4])
+ *   w_q, w_k, w_v   [H*128, 4] float32 conv weights, taps oldest first
+ *   cs_q, cs_k, cs_v  conv states [slot, H*128, 3] bf16, read-only; strides[5..13] = (slot, channel, window) x 3
+ *   ic_q, ic_k, ic_v  scratch windows [row, step, H*128, 3] bf16, written: the window after each token;
+ *                   strides[14..25] = (row, step, channel, window) x 3
+ *   a_log [H], dt_bias [H*128] float32: log-decay = lower_bound * sigmoid(exp(a_log) * (g + dt_bias))
+ *   h0              [slots,H,128,128] float32 dense, read once, never written
+ *   ring_rawv, ring_rawk [slots,H,L,128] bf16 (post-conv v and k, k before its L2 norm), ring_g
+ *                   [slots,H,L,128] float32 log-decay, ring_beta [slots,H,L] float32: records of token t of
+ *                   a request go to position t of its slot's rings
+ *   out             [T,H,128] bf16 dense.  onorm_gate != NULL: out = o rsqrt(mean(o^2) + eps) weight
+ *                   sigmoid(gate), gate [T,H,128] bf16 with token stride onorm_gate_stride
+ *   slot_idx, scratch_idx, cu_seqlens: int32 or int64 ([N], [>=N], [N+1]); slot < 0: the request's
+ *                   output rows are zeroed and nothing else is touched
+ *   t_loop          draft tokens per request (1..8); ring_len = L >= t_loop
+ */
+int pla_kda_verify_dspark_launch(
+    const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
+    const float* w_q, const float* w_k, const float* w_v,
+    const void* cs_q, const void* cs_k, const void* cs_v,
+    const float* a_log, const float* dt_bias, const float* h0,
+    void* out, void* ic_q, void* ic_k, void* ic_v,
+    void* ring_rawv, void* ring_rawk, float* ring_g, float* ring_beta,
+    const void* slot_idx, int slot_idx_wide, const void* scratch_idx, int scratch_idx_wide,
+    const void* cu_seqlens, int cu_seqlens_wide,
+    int H, int N, int t_loop, int ring_len, float scale, float lower_bound,
+    const int64_t* strides,
+    const void* onorm_gate, const float* onorm_weight, int64_t onorm_gate_stride, float onorm_eps,
+    void* stream);
+
+/*
+ * Conv-window rollback of the commit: dst[layer, dst_idx[r], :, :] = src[layer, r, step_idx[r], :, :]
+ * for every request r with step_idx[r] >= 0, 0 <= dst_idx[r] < dst_reqs, r < src_reqs and
+ * step_idx[r] < src_steps.  Replaces launch_conv_scatter
+ * (src/decode/kda_replayssm/kda_mtp_abi.h:177-186; kernel src/decode/kda_replayssm/kda_mtp_fold.cu:595-635).
+ * src [layers, src_reqs, src_steps, dim, km1] with strides src_s0..4, dst [layers, dst_reqs, dim, km1]
+ * with strides dst_s0..3 (elements of elem_bytes = 2 or 4); km1 = conv width - 1 (1..4).
+ */
+int pla_conv_window_scatter_launch(
+    int elem_bytes, int km1, const void* src, void* dst,
+    const void* dst_idx, int dst_idx_wide, const void* step_idx, int step_idx_wide,
+    int layers, int dim, int reqs,
+    int64_t src_s0, int64_t src_s1, int64_t src_s2, int64_t src_s3, int64_t src_s4,
+    int64_t dst_s0, int64_t dst_s1, int64_t dst_s2, int64_t dst_s3,
+    int src_reqs, int src_steps, int dst_reqs, void* stream);
+
+/*
  * Workspace size in bytes (256-byte aligned buffer) needed by pla_gdn_prefill_launch for T physical
  * tokens in N sequences.  Chunk metadata is sized for the worst case T/64 + N chunks so that no
  * host copy of cu_seqlens is needed.

@@ -241,3 +241,93 @@ def kda_decode_mega_reference(x, weight, bias, conv_state, raw_g, raw_beta, a_lo
             o = o * torch.rsqrt(o.square().mean(-1, keepdim=True) + norm_eps) * norm_weight.float()[None, :] * gate
         out[0, n] = o.to(x.dtype)
     return out, state_new, conv_new
+
+
+def causal_conv_silu_sequence(x_seq, window, weight):
+    """Width-4 causal conv + SiLU of ``x_seq [T, C]`` seeded by ``window [C, 3]`` (oldest tap first),
+    ``weight [C, 4]`` (taps oldest first).  Returns ``(y [T, C] float64, windows [T, C, 3])`` where
+    ``windows[t]`` is the window after token ``t`` was consumed
+    (scripts/decode/kda_mtp_sglang/private/_reference.py:66-85)."""
+    T, C = x_seq.shape
+    full = torch.cat([window.double().t(), x_seq.double()], dim=0)                  # [3 + T, C]
+    w = weight.double()
+    y = torch.empty(T, C, dtype=torch.float64)
+    wins = torch.empty(T, C, 3, dtype=torch.float64)
+    for t in range(T):
+        acc = (full[t:t + 4] * w.t()).sum(0)
+        y[t] = acc * torch.sigmoid(acc)
+        wins[t] = full[t + 1:t + 4].t()
+    return y, wins
+
+
+def verify_dspark_reference(*, x_q, x_k, x_v, g, beta, w_q, w_k, w_v, cs_q, cs_k, cs_v, A_log, dt_bias,
+                            recurrent_state, ssm_state_indices, intermediate_state_indices, cu_seqlens,
+                            lower_bound, scale, rings, windows, onorm_gate=None, onorm_weight=None, onorm_eps=None):
+    """Reference for ``fused_kda_decode_mtp_dspark`` (ring mode), float64 throughout.
+
+    Restates scripts/decode/kda_mtp_sglang/private/_reference.py:88-177: per request and head, conv +
+    SiLU of the draft tokens from the (read-only) conv state, records of the post-conv k (before its
+    L2 norm) and v, of the log-decay ``lower_bound * sigmoid(exp(A_log) (g + dt_bias))`` and of
+    ``sigmoid(beta)`` at ring position t, the window after every token in the request's scratch row,
+    and the delta-rule recurrence from the (read-only) state with ``q`` scaled after its L2 norm;
+    optional ``o * rsqrt(mean(o^2) + eps) * weight * sigmoid(gate)``.  ``rings`` = (rawv, rawk, g, beta)
+    and ``windows`` = (ic_q, ic_k, ic_v) are copied and returned updated in their own dtypes; slots < 0
+    are skipped (their output rows stay zero).
+
+    Returns ``dict(out [1,T,H,128] float64, ring_rawv, ring_rawk, ring_g, ring_beta, ic_q, ic_k, ic_v)``.
+    """
+    D = 128
+    T, H = x_q.shape[1], x_q.shape[2]
+    out = torch.zeros(1, T, H, D, dtype=torch.float64)
+    rawv, rawk, ring_g, ring_beta = (r.clone() for r in rings)
+    ic = [w.clone() for w in windows]
+    cu = [int(v) for v in cu_seqlens.tolist()]
+    slots = [int(v) for v in ssm_state_indices.tolist()]
+    rows = [int(v) for v in intermediate_state_indices.tolist()]
+    xs = [x_q[0].double(), x_k[0].double(), x_v[0].double()]
+    ws = [w_q, w_k, w_v]
+    css = [cs_q, cs_k, cs_v]
+    graw, braw = g[0].double(), beta[0].double()
+    dt = dt_bias.double().reshape(H, D)
+    for n, slot in enumerate(slots):
+        if slot < 0:
+            continue
+        bos, eos = cu[n], cu[n + 1]
+        nt = eos - bos
+        for h in range(H):
+            sl = slice(h * D, (h + 1) * D)
+            conv = []
+            for i in range(3):
+                y, wins = causal_conv_silu_sequence(xs[i][bos:eos, h], css[i][slot, sl], ws[i][sl])
+                conv.append(y)
+                ic[i][rows[n], :nt, sl] = wins.to(ic[i].dtype)
+            q_c, k_c, v_c = conv
+            rawk[slot, h, :nt] = k_c.to(rawk.dtype)
+            rawv[slot, h, :nt] = v_c.to(rawv.dtype)
+            q_n = q_c / torch.sqrt((q_c * q_c).sum(-1, keepdim=True) + 1e-6) * scale
+            k_n = k_c / torch.sqrt((k_c * k_c).sum(-1, keepdim=True) + 1e-6)
+            b = torch.sigmoid(braw[bos:eos, h])
+            ring_beta[slot, h, :nt] = b.to(ring_beta.dtype)
+            gk = lower_bound * torch.sigmoid(A_log[h].double().exp() * (graw[bos:eos, h] + dt[h]))
+            ring_g[slot, h, :nt] = gk.to(ring_g.dtype)
+            S = recurrent_state[slot, h].double()[None]
+            for t in range(nt):
+                S, o = recurrent_step(S, q_n[t][None], k_n[t][None], v_c[t][None], gk[t][None], b[t][None])
+                out[0, bos + t, h] = o[0]
+    if onorm_gate is not None:
+        gate = torch.sigmoid(onorm_gate[0].double())
+        rms = torch.rsqrt((out[0] * out[0]).mean(-1, keepdim=True) + onorm_eps)
+        out = (out[0] * rms * onorm_weight.double()[None, None, :] * gate)[None]
+    return dict(out=out, ring_rawv=rawv, ring_rawk=rawk, ring_g=ring_g, ring_beta=ring_beta,
+                ic_q=ic[0], ic_k=ic[1], ic_v=ic[2])
+
+
+def conv_window_scatter_reference(dst, src, dst_idx, step_idx):
+    """``dst[layer, dst_idx[r]] = src[layer, r, step_idx[r]]`` for requests with a non-negative step and an
+    in-range destination (src/decode/kda_replayssm/kda_mtp_fold.cu:602-634).  Returns the updated copy."""
+    out = dst.clone()
+    for r, (d, s) in enumerate(zip(dst_idx.tolist(), step_idx.tolist())):
+        if s < 0 or d < 0 or d >= dst.shape[1] or r >= src.shape[1] or s >= src.shape[2]:
+            continue
+        out[:, d] = src[:, r, s]
+    return out

@@ -1,0 +1,380 @@
+// KDA speculative verify with replay records (SGLang ReplaySSM, ring mode) and the conv-window
+// rollback of the commit, for gfx950.
+//
+// Verify (reference: src/decode/kda_replayssm/kda_mtp_verify.cu:700-1100, contract
+// src/decode/kda_replayssm_sglang/kda_mtp_verify_host.cpp:50-243, Python model
+// scripts/decode/kda_mtp_sglang/private/_reference.py:88-177): for every request the T draft tokens
+// run through the width-4 causal convolution + SiLU (seeded from the request's conv state, which
+// is read-only here), the lower-bound gate and the delta-rule recurrence starting from the
+// request's FP32 state, which is read once and never written.  Side effects besides the output:
+// the conv window after every token goes to the request's scratch row, and the per-token records
+// (post-conv k and v in bf16, log-decay and beta in FP32) go to the slot's rings, from which the
+// commit later replays the accepted prefix.
+//
+// One workgroup of four wavefronts per (request, head).  The state tile is requested first, in
+// MFMA A-operand layout.  Threads 0-127 then run the convolution of one q and one k channel
+// through all tokens, threads 128-255 that of one v channel plus the channel's gate; everything
+// the recurrence needs meets in LDS.  The recurrence itself is not stepped: with
+//     o_t = S_0 w_t + sum_{j <= t} c_{j,t} v_j,  w_t = A_1 .. A_t q_t,  A_j = D_j (I - beta_j k_j k_j^T)
+// wavefront w works out w_t and c_{.,t} for tokens t = w, w + 4 from K-vectors alone, and the tile
+// is used once as the A operand of S_0 [w_0 .. w_{T-1}] on v_mfma_f32_16x16x32_bf16 (FP32 data split
+// into bf16 hi + lo, three products).  Up to eight draft tokens.
+//
+// Conv-window scatter (reference: conv_scatter_kernel, src/decode/kda_replayssm/kda_mtp_fold.cu:595-635):
+// dst[layer, dst_idx[r], :, :] = src[layer, r, step_idx[r], :, :] for every request r with a
+// non-negative step and an in-range destination.
+
+#include "decode_common.h"
+#include "mfma_bf16.h"
+
+namespace pla {
+
+struct ReplayVerifyParams {
+  const uint16_t* x_q; const uint16_t* x_k; const uint16_t* x_v; const uint16_t* g; const uint16_t* beta;
+  const float* w_q; const float* w_k; const float* w_v;
+  const uint16_t* cs_q; const uint16_t* cs_k; const uint16_t* cs_v;
+  const float* a_log; const float* dt_bias; float* h0;
+  uint16_t* out; uint16_t* ic_q; uint16_t* ic_k; uint16_t* ic_v;
+  uint16_t* ring_rawv; uint16_t* ring_rawk; float* ring_g; float* ring_beta;
+  const void* slot_idx; const void* scratch_idx; const void* cu;
+  int slot_wide, scratch_wide, cu_wide;
+  int H, N, T, L;
+  float scale, lower_bound;
+  int64_t sx_q, sx_k, sx_v, sg, sbeta;
+  int64_t cs[3][3];        // q, k, v conv state: slot, channel, window strides
+  int64_t ic[3][4];        // q, k, v scratch windows: row, step, channel, window strides
+  const uint16_t* onorm_gate; const float* onorm_weight; int64_t onorm_gate_stride; float onorm_eps;
+};
+
+__device__ __forceinline__ int64_t index_at(const void* p, int wide, int64_t i) {
+  return wide ? reinterpret_cast<const int64_t*>(p)[i] : (int64_t) reinterpret_cast<const int32_t*>(p)[i];
+}
+__device__ __forceinline__ float bf(uint16_t x) { return to_float(bf16_t{x}); }
+__device__ __forceinline__ uint16_t to_bf(float x) { return from_float<bf16_t>(x).bits; }
+
+// Convolution of one channel over the draft tokens.  `taps` holds the window (oldest first) and is
+// advanced; returns silu(conv).  Same operation order as the reference (:815-818).
+__device__ __forceinline__ float conv_step(float (&taps)[3], float x, const float4 w) {
+  float acc = x * w.w;
+  acc = fmaf(taps[0], w.x, acc);
+  acc = fmaf(taps[1], w.y, acc);
+  acc = fmaf(taps[2], w.z, acc);
+  taps[0] = taps[1]; taps[1] = taps[2]; taps[2] = x;
+  return acc * fast_sigmoid(acc);
+}
+
+template <int TMAX, bool ONORM>
+__global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVerifyParams p) {
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, c = lane & 31;
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int n = blockIdx.x / p.H, h = blockIdx.x - n * p.H;
+  const int64_t slot = index_at(p.slot_idx, p.slot_wide, n);
+  const int64_t bos = index_at(p.cu, p.cu_wide, n);
+  const int n_tok = (int)min((int64_t)p.T, index_at(p.cu, p.cu_wide, n + 1) - bos);
+  if (bos < 0 || n_tok <= 0) return;
+  const int rowbase = 32 * wave;
+
+  if (slot < 0) {                                   // padded request: zero output rows, nothing else
+    for (int i = tid; i < n_tok * 128; i += 256)
+      p.out[((bos + i / 128) * p.H + h) * 128 + (i & 127)] = 0;
+    return;
+  }
+  const int64_t srow = index_at(p.scratch_idx, p.scratch_wide, n);
+
+  // state tile first, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
+  const Tile<float> h_tile(p.h0 + (slot * p.H + h) * 16384);
+  f32x4_t sa[2][4][2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+        sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
+            h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
+
+  __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128], sW[TMAX][128];
+  __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
+  __shared__ float sBeta[TMAX], sNorm[2][2][TMAX], sSq[4][TMAX];
+
+  const int64_t ring_row = (slot * p.H + h) * p.L;   // first record of this (slot, head)
+  if (tid < 128) {
+    const int64_t ch = (int64_t)h * 128 + tid;
+    const float4 wq = reinterpret_cast<const float4*>(p.w_q)[ch];
+    const float4 wk = reinterpret_cast<const float4*>(p.w_k)[ch];
+    float cq[3], ck[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) {
+      cq[j] = bf(p.cs_q[slot * p.cs[0][0] + ch * p.cs[0][1] + j * p.cs[0][2]]);
+      ck[j] = bf(p.cs_k[slot * p.cs[1][0] + ch * p.cs[1][1] + j * p.cs[1][2]]);
+    }
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+      if (t >= n_tok) break;
+      const float xq = bf(p.x_q[(bos + t) * p.sx_q + ch]);
+      const float xk = bf(p.x_k[(bos + t) * p.sx_k + ch]);
+      const float q = conv_step(cq, xq, wq);
+      const float k = conv_step(ck, xk, wk);
+      sQ[t][tid] = q;
+      sK[t][tid] = k;
+      p.ring_rawk[(ring_row + t) * 128 + tid] = to_bf(k);
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        p.ic_q[srow * p.ic[0][0] + t * p.ic[0][1] + ch * p.ic[0][2] + j * p.ic[0][3]] = to_bf(cq[j]);
+        p.ic_k[srow * p.ic[1][0] + t * p.ic[1][1] + ch * p.ic[1][2] + j * p.ic[1][3]] = to_bf(ck[j]);
+      }
+      const float q2 = wave64_allreduce(q * q), k2 = wave64_allreduce(k * k);
+      if (lane == 0) { sNorm[0][wave][t] = q2; sNorm[1][wave][t] = k2; }
+    }
+  } else {
+    const int i = tid - 128;
+    const int64_t ch = (int64_t)h * 128 + i;
+    const float4 wv = reinterpret_cast<const float4*>(p.w_v)[ch];
+    const float eA = __expf(p.a_log[h]);
+    const float bias = p.dt_bias[ch];
+    float cv[3];
+#pragma unroll
+    for (int j = 0; j < 3; ++j) cv[j] = bf(p.cs_v[slot * p.cs[2][0] + ch * p.cs[2][1] + j * p.cs[2][2]]);
+#pragma unroll
+    for (int t = 0; t < TMAX; ++t) {
+      if (t >= n_tok) break;
+      const float xv = bf(p.x_v[(bos + t) * p.sx_v + ch]);
+      const float v = conv_step(cv, xv, wv);
+      sV[t][i] = v;
+      p.ring_rawv[(ring_row + t) * 128 + i] = to_bf(v);
+#pragma unroll
+      for (int j = 0; j < 3; ++j)
+        p.ic_v[srow * p.ic[2][0] + t * p.ic[2][1] + ch * p.ic[2][2] + j * p.ic[2][3]] = to_bf(cv[j]);
+      const float gk = p.lower_bound * fast_sigmoid(eA * (bf(p.g[(bos + t) * p.sg + ch]) + bias));
+      p.ring_g[(ring_row + t) * 128 + i] = gk;
+      sD[t][i] = __expf(gk);
+      if (i == 0) {
+        const float b = fast_sigmoid(bf(p.beta[(bos + t) * p.sbeta + h]));
+        sBeta[t] = b;
+        p.ring_beta[ring_row + t] = b;
+      }
+    }
+  }
+  __syncthreads();
+
+  // K-vector algebra: wavefront w handles tokens w and w + 4
+  {
+    float kv[TMAX][4], dec[TMAX][4], beta[TMAX];
+#pragma unroll
+    for (int j = 0; j < TMAX; ++j) {
+      const int jj = min(j, n_tok - 1);
+      const float kn = fast_rsqrt(sNorm[1][0][jj] + sNorm[1][1][jj] + 1e-6f);
+      const float4 k4 = *reinterpret_cast<const float4*>(&sK[jj][4 * c]);
+      const float4 d4 = *reinterpret_cast<const float4*>(&sD[jj][4 * c]);
+      kv[j][0] = k4.x * kn; kv[j][1] = k4.y * kn; kv[j][2] = k4.z * kn; kv[j][3] = k4.w * kn;
+      dec[j][0] = d4.x; dec[j][1] = d4.y; dec[j][2] = d4.z; dec[j][3] = d4.w;
+      beta[j] = sBeta[jj];
+    }
+#pragma unroll
+    for (int tt = 0; tt < TMAX / 4; ++tt) {
+      const int t = wave + 4 * tt;
+      if (t >= n_tok) break;
+      const float qn = fast_rsqrt(sNorm[0][0][t] + sNorm[0][1][t] + 1e-6f) * p.scale;
+      const float4 q4 = *reinterpret_cast<const float4*>(&sQ[t][4 * c]);
+      float w[4] = {q4.x * qn, q4.y * qn, q4.z * qn, q4.w * qn};
+      float cf[TMAX];
+#pragma unroll
+      for (int j = TMAX - 1; j >= 0; --j) {
+        cf[j] = 0.f;
+        if (j > t) continue;
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dot = fmaf(kv[j][e], w[e], dot);
+        cf[j] = beta[j] * row32_allreduce(dot);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf[j], kv[j][e], w[e]);
+      }
+      if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
+      if (lane == 0) {
+#pragma unroll
+        for (int j = 0; j < TMAX; ++j) sC[t][j] = cf[j];
+      }
+    }
+  }
+  __syncthreads();
+
+  // B operands: column r16 of [w_0 .. w_{T-1} 0 .. 0]
+  const int tcol = min(r16, n_tok - 1);
+  const bool mine = r16 < n_tok;
+  const float keep = mine ? 1.f : 0.f;
+  HiLo wb[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb]);
+    const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb + 4]);
+    wb[ks] = split8(f32x4_t{w0.x * keep, w0.y * keep, w0.z * keep, w0.w * keep},
+                    f32x4_t{w1.x * keep, w1.y * keep, w1.z * keep, w1.w * keep});
+  }
+  float cs[TMAX];
+#pragma unroll
+  for (int j = 0; j < TMAX; ++j) cs[j] = sC[tcol][j];
+
+  float o[2][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int m = 0; m < 2; ++m) {
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const HiLo a = split8(sa[m][ks][0], sa[m][ks][1]);
+      acc = mfma16(a.hi, wb[ks].hi, acc);
+      acc = mfma16(a.lo, wb[ks].hi, acc);
+      acc = mfma16(a.hi, wb[ks].lo, acc);
+    }
+    // lane (r16 = token, kb): rows 32 w + 16 m + 4 kb .. + 3 of S_0 w_token, plus the bias terms
+    o[m][0] = acc[0]; o[m][1] = acc[1]; o[m][2] = acc[2]; o[m][3] = acc[3];
+#pragma unroll
+    for (int j = 0; j < TMAX; ++j) {
+      if (j >= n_tok) break;
+      const float4 v4 = *reinterpret_cast<const float4*>(&sV[j][rowbase + 16 * m + 4 * kb]);
+      o[m][0] = fmaf(cs[j], v4.x, o[m][0]);
+      o[m][1] = fmaf(cs[j], v4.y, o[m][1]);
+      o[m][2] = fmaf(cs[j], v4.z, o[m][2]);
+      o[m][3] = fmaf(cs[j], v4.w, o[m][3]);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) ss = fmaf(o[m][r], o[m][r], ss);
+  }
+
+  float rstd = 1.f;
+  if constexpr (ONORM) {
+    // sum of squares of the token's 128 outputs: over the four 16-lane rows of the wavefront, then over
+    // the four wavefronts through LDS
+    const LanePair rows = swap_rows16(ss);
+    const LanePair halves = swap_halves(rows.lo + rows.hi);
+    if (lane < TMAX) sSq[wave][lane] = halves.lo + halves.hi;
+    __syncthreads();
+    const float total = sSq[0][tcol] + sSq[1][tcol] + sSq[2][tcol] + sSq[3][tcol];
+    rstd = fast_rsqrt(total * (1.0f / 128.0f) + p.onorm_eps);
+  }
+  if (mine) {
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const int row = rowbase + 16 * m + 4 * kb;
+      float val[4] = {o[m][0], o[m][1], o[m][2], o[m][3]};
+      if constexpr (ONORM) {
+        const uint2 gw = *reinterpret_cast<const uint2*>(p.onorm_gate + (bos + r16) * p.onorm_gate_stride + h * 128 + row);
+        const float4 w4 = *reinterpret_cast<const float4*>(p.onorm_weight + row);
+        val[0] *= rstd * w4.x * fast_sigmoid(lo16<bf16_t>(gw.x));
+        val[1] *= rstd * w4.y * fast_sigmoid(hi16<bf16_t>(gw.x));
+        val[2] *= rstd * w4.z * fast_sigmoid(lo16<bf16_t>(gw.y));
+        val[3] *= rstd * w4.w * fast_sigmoid(hi16<bf16_t>(gw.y));
+      }
+      *reinterpret_cast<uint2*>(p.out + ((bos + r16) * p.H + h) * 128 + row) =
+          make_uint2(pack2<bf16_t>(val[0], val[1]), pack2<bf16_t>(val[2], val[3]));
+    }
+  }
+}
+
+// One thread per channel: copies the window of the selected step into the destination slot.
+template <typename T>
+__global__ __launch_bounds__(256) void conv_window_scatter_kernel(
+    const T* src, T* dst, const void* dst_idx, int dst_wide, const void* step_idx, int step_wide,
+    int dim, int km1, int64_t s_layer, int64_t s_req, int64_t s_step, int64_t s_dim, int64_t s_win,
+    int64_t d_layer, int64_t d_req, int64_t d_dim, int64_t d_win, int src_reqs, int src_steps, int dst_reqs) {
+  const int r = blockIdx.x;
+  const int64_t layer = blockIdx.y;
+  const int64_t step = index_at(step_idx, step_wide, r);
+  const int64_t d_i = index_at(dst_idx, dst_wide, r);
+  if (step < 0 || d_i < 0 || d_i >= dst_reqs || r >= src_reqs || step >= src_steps) return;
+  const int d = blockIdx.z * 256 + threadIdx.x;
+  if (d >= dim) return;
+  const T* sp = src + layer * s_layer + (int64_t)r * s_req + step * s_step + (int64_t)d * s_dim;
+  T* dp = dst + layer * d_layer + d_i * d_req + (int64_t)d * d_dim;
+  for (int w = 0; w < km1; ++w) dp[w * d_win] = sp[w * s_win];
+}
+
+static bool aligned_at(const void* ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
+
+}  // namespace pla
+
+extern "C" int pla_kda_verify_dspark_launch(
+    const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
+    const float* w_q, const float* w_k, const float* w_v,
+    const void* cs_q, const void* cs_k, const void* cs_v,
+    const float* a_log, const float* dt_bias, const float* h0,
+    void* out, void* ic_q, void* ic_k, void* ic_v,
+    void* ring_rawv, void* ring_rawk, float* ring_g, float* ring_beta,
+    const void* slot_idx, int slot_idx_wide, const void* scratch_idx, int scratch_idx_wide,
+    const void* cu_seqlens, int cu_seqlens_wide,
+    int H, int N, int t_loop, int ring_len, float scale, float lower_bound,
+    const int64_t* strides,
+    const void* onorm_gate, const float* onorm_weight, int64_t onorm_gate_stride, float onorm_eps,
+    void* stream) {
+  using namespace pla;
+  PLA_REQUIRE(x_q && x_k && x_v && g_in && beta_in && w_q && w_k && w_v && cs_q && cs_k && cs_v && a_log && dt_bias && h0 &&
+              out && ic_q && ic_k && ic_v && ring_rawv && ring_rawk && ring_g && ring_beta && slot_idx && scratch_idx &&
+              cu_seqlens && strides, "null tensor pointer");
+  PLA_REQUIRE(H > 0 && N > 0 && t_loop > 0, "verify requires H > 0, N > 0 and at least one token per request");
+  PLA_REQUIRE(t_loop <= 8, "the gfx950 verify handles up to 8 draft tokens per request, got %d", t_loop);
+  PLA_REQUIRE(ring_len >= t_loop, "ring shorter than the draft window");
+  PLA_REQUIRE((int64_t)N * H <= 0x7fffffffLL, "N * H exceeds the grid limit");
+  PLA_REQUIRE(aligned_at(h0, 16) && aligned_at(w_q, 16) && aligned_at(w_k, 16) && aligned_at(w_v, 16) && aligned_at(out, 8),
+              "state, conv weights and out require vector alignment");
+  const bool onorm = onorm_gate != nullptr;
+  PLA_REQUIRE(!onorm || (onorm_weight != nullptr && aligned_at(onorm_weight, 16) && aligned_at(onorm_gate, 8) &&
+                         onorm_gate_stride % 4 == 0 && onorm_eps >= 0.f),
+              "fused output norm requires an aligned gate (token stride a multiple of 4), a weight and eps >= 0");
+  for (int i = 0; i < 26; ++i) PLA_REQUIRE(strides[i] > 0, "stride %d must be positive", i);
+  ReplayVerifyParams p;
+  p.x_q = (const uint16_t*)x_q; p.x_k = (const uint16_t*)x_k; p.x_v = (const uint16_t*)x_v;
+  p.g = (const uint16_t*)g_in; p.beta = (const uint16_t*)beta_in;
+  p.w_q = w_q; p.w_k = w_k; p.w_v = w_v;
+  p.cs_q = (const uint16_t*)cs_q; p.cs_k = (const uint16_t*)cs_k; p.cs_v = (const uint16_t*)cs_v;
+  p.a_log = a_log; p.dt_bias = dt_bias; p.h0 = const_cast<float*>(h0);
+  p.out = (uint16_t*)out; p.ic_q = (uint16_t*)ic_q; p.ic_k = (uint16_t*)ic_k; p.ic_v = (uint16_t*)ic_v;
+  p.ring_rawv = (uint16_t*)ring_rawv; p.ring_rawk = (uint16_t*)ring_rawk; p.ring_g = ring_g; p.ring_beta = ring_beta;
+  p.slot_idx = slot_idx; p.scratch_idx = scratch_idx; p.cu = cu_seqlens;
+  p.slot_wide = slot_idx_wide; p.scratch_wide = scratch_idx_wide; p.cu_wide = cu_seqlens_wide;
+  p.H = H; p.N = N; p.T = t_loop; p.L = ring_len; p.scale = scale; p.lower_bound = lower_bound;
+  p.sx_q = strides[0]; p.sx_k = strides[1]; p.sx_v = strides[2]; p.sg = strides[3]; p.sbeta = strides[4];
+  for (int t = 0; t < 3; ++t)
+    for (int j = 0; j < 3; ++j) p.cs[t][j] = strides[5 + 3 * t + j];
+  for (int t = 0; t < 3; ++t)
+    for (int j = 0; j < 4; ++j) p.ic[t][j] = strides[14 + 4 * t + j];
+  p.onorm_gate = (const uint16_t*)onorm_gate; p.onorm_weight = onorm_weight;
+  p.onorm_gate_stride = onorm_gate_stride; p.onorm_eps = onorm_eps;
+  const dim3 grid((unsigned)N * (unsigned)H), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (t_loop <= 4) {
+    if (onorm) kda_verify_dspark_kernel<4, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<4, false><<<grid, block, 0, s>>>(p);
+  } else {
+    if (onorm) kda_verify_dspark_kernel<8, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<8, false><<<grid, block, 0, s>>>(p);
+  }
+  return check_launch("kda_verify_dspark_kernel");
+}
+
+extern "C" int pla_conv_window_scatter_launch(
+    int elem_bytes, int km1, const void* src, void* dst,
+    const void* dst_idx, int dst_idx_wide, const void* step_idx, int step_idx_wide,
+    int layers, int dim, int reqs,
+    int64_t src_s0, int64_t src_s1, int64_t src_s2, int64_t src_s3, int64_t src_s4,
+    int64_t dst_s0, int64_t dst_s1, int64_t dst_s2, int64_t dst_s3,
+    int src_reqs, int src_steps, int dst_reqs, void* stream) {
+  using namespace pla;
+  PLA_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "conv scatter: element size must be 2 or 4 bytes, got %d", elem_bytes);
+  PLA_REQUIRE(km1 >= 1 && km1 <= 4, "conv scatter: unsupported conv window %d", km1);
+  if (reqs == 0) return 0;
+  PLA_REQUIRE(src && dst && dst_idx && step_idx, "null tensor pointer");
+  PLA_REQUIRE(layers > 0 && dim > 0 && reqs > 0 && layers <= 65535, "conv scatter: layers, dim and reqs must be positive");
+  const dim3 grid((unsigned)reqs, (unsigned)layers, (unsigned)((dim + 255) / 256)), block(256);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (elem_bytes == 2)
+    conv_window_scatter_kernel<uint16_t><<<grid, block, 0, s>>>(
+        (const uint16_t*)src, (uint16_t*)dst, dst_idx, dst_idx_wide, step_idx, step_idx_wide, dim, km1,
+        src_s0, src_s1, src_s2, src_s3, src_s4, dst_s0, dst_s1, dst_s2, dst_s3, src_reqs, src_steps, dst_reqs);
+  else
+    conv_window_scatter_kernel<uint32_t><<<grid, block, 0, s>>>(
+        (const uint32_t*)src, (uint32_t*)dst, dst_idx, dst_idx_wide, step_idx, step_idx_wide, dim, km1,
+        src_s0, src_s1, src_s2, src_s3, src_s4, dst_s0, dst_s1, dst_s2, dst_s3, src_reqs, src_steps, dst_reqs);
+  return check_launch("conv_window_scatter_kernel");
+}

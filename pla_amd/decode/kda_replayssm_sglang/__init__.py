@@ -1,20 +1,30 @@
-"""Accepted-prefix commit of KDA speculative decoding (``pla.decode.kda_replayssm_sglang``).
+"""KDA speculative decoding with replay records (``pla.decode.kda_replayssm_sglang``).
 
-Covers the recurrence half of the reference's
-``commit_kda_replayssm_after_verify`` (pla/decode/kda_replayssm_sglang/__init__.py:162-215):
-for every layer, each request's accepted prefix of recorded tokens (raw k, raw v, per-channel
-log-decay, beta) is replayed into the FP32 checkpoint ``temporal`` in place.  A request whose
-slot is ``<= null_block_id`` or whose accepted length is ``<= 0`` leaves its checkpoint
-bit-identical (src/decode/kda_replayssm/kda_mtp_fold.cu:306).  The convolution-window
-rollback and the ring writers of the verify kernel belong to the conv front end and are not
-part of this package.
+``fused_kda_decode_mtp_dspark`` (reference pla/decode/kda_replayssm_sglang/__init__.py:74-159): verify of the
+draft tokens in ring mode.  Conv front end, gate and recurrence in one launch; the persistent
+recurrent and conv states are read-only, the per-token records go to the four rings and the conv
+window after every token to the scratch rows.
+
+``commit_kda_replayssm_after_verify`` (same file :162-211): for every layer, each request's accepted
+prefix of recorded tokens (raw k, raw v, per-channel log-decay, beta) is replayed into the FP32
+checkpoint ``temporal`` in place, and the conv state is rolled back to the window of the last
+accepted step.  A request whose slot is ``<= null_block_id`` or whose accepted length is ``<= 0``
+leaves its checkpoint bit-identical (src/decode/kda_replayssm/kda_mtp_fold.cu:306).  Track
+snapshots (``mamba_track_indices``) roll back conv windows only; recurrent track snapshots are
+rejected rather than silently skipped.
 """
+
+import ctypes
+import os
 
 import torch
 
 from ... import _lib
 
-__all__ = ["fold_accepted_prefix", "commit_kda_replayssm_after_verify", "kda_mtp_verify"]
+__all__ = ["fused_kda_decode_mtp_dspark", "commit_kda_replayssm_after_verify", "conv_window_scatter",
+           "fold_accepted_prefix", "kda_mtp_verify"]
+
+_BYPASS = os.environ.get("PLA_BYPASS_EXEC", "0") == "1"   # read once, like src/bypass_exec.h:44-50
 
 
 def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, accept_lens,
@@ -56,18 +66,201 @@ def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, ac
                   beta.stride(1), B, H, HV, L, int(null_block_id), act, stream)
 
 
+def _index(t):
+    if t.dim() != 1 or t.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("indices must be int32/int64 vectors")
+    t = t.contiguous()
+    return t, int(t.dtype == torch.int64)
+
+
+def conv_window_scatter(dst, src, dst_idx, step_idx):
+    """``dst[layer, dst_idx[r]] = src[layer, r, step_idx[r]]`` for every request ``r`` with a non-negative
+    step and destination (reference binding src/decode/kda_replayssm_sglang/kda_mtp_fold_host.cpp:152-224).
+    dst [layers, slots, dim, width-1] (or its ``width_dim`` transpose view), src [layers, rows, steps, dim,
+    width-1], bf16 or float32; out-of-range requests are skipped."""
+    if _BYPASS:
+        return
+    if dst.dim() != 4 or src.dim() != 5:
+        raise RuntimeError("ranks: dst 4, src 5")
+    if not (dst.is_cuda and src.device == dst.device and dst.dtype == src.dtype):
+        raise RuntimeError("conv source and destination must have the same CUDA device and dtype")
+    if not (src.size(0) == dst.size(0) and src.size(3) == dst.size(2) and src.size(4) == dst.size(3)):
+        raise RuntimeError("conv source/destination shape mismatch")
+    if not (dst.is_contiguous() or dst.transpose(-1, -2).is_contiguous()):
+        raise RuntimeError("conv destination must be contiguous in dim_width or width_dim layout")
+    if dst_idx.numel() != step_idx.numel() or dst_idx.device != dst.device or step_idx.device != dst.device:
+        raise RuntimeError("invalid conv scatter indices")
+    di, di_wide = _index(dst_idx)
+    st, st_wide = _index(step_idx)
+    if dst.dtype not in (torch.bfloat16, torch.float32):
+        raise RuntimeError(f"conv scatter: unsupported dtype {dst.dtype}")
+    km1 = dst.size(3)
+    if not 1 <= km1 <= 4:
+        raise RuntimeError(f"conv scatter: unsupported conv window {km1}")
+    if st.numel() == 0:
+        return
+    with torch.cuda.device(dst.device):
+        _lib.call("pla_conv_window_scatter_launch", dst.element_size(), km1, src.data_ptr(), dst.data_ptr(),
+                  di.data_ptr(), di_wide, st.data_ptr(), st_wide, dst.size(0), dst.size(2), st.numel(),
+                  *src.stride(), *dst.stride(), src.size(1), src.size(2), dst.size(1),
+                  _lib.current_stream(dst.device))
+
+
 def commit_kda_replayssm_after_verify(*, spec_state, state_batch_indices, accept_lens,
                                       last_correct_step_indices=None, mamba_track_indices=None,
                                       mamba_steps_to_track=None, null_block_id=-1,
                                       conv_state_layout="dim_width"):
     """Keyword-only entry with the reference's name: folds every layer's accepted window into
-    ``spec_state.temporal``.  Only the recurrent state is committed here; boundary / track
-    snapshots and the conv-window rollback are rejected rather than silently skipped."""
-    if mamba_track_indices is not None or mamba_steps_to_track is not None:
-        raise NotImplementedError("track snapshots are not part of the gfx950 commit path")
+    ``spec_state.temporal`` and rolls the conv states back to the window of the last accepted step.
+    ``spec_state`` carries ``temporal``, ``replayssm_rawv/rawk/g/beta`` and, for the rollback, the lists
+    ``conv`` ([layers, slots, dim, width-1] each) and ``intermediate_conv_window``
+    ([layers, rows, steps, dim, width-1] each); ``conv_state_layout="width_dim"`` takes the transposed
+    pools.  Track snapshots apply to the conv windows only."""
+    assert conv_state_layout in ("dim_width", "width_dim")
     fold_accepted_prefix(spec_state.temporal, spec_state.replayssm_rawv, spec_state.replayssm_rawk,
                          spec_state.replayssm_g, spec_state.replayssm_beta,
                          state_batch_indices, accept_lens, null_block_id)
+    conv = getattr(spec_state, "conv", None)
+    windows = getattr(spec_state, "intermediate_conv_window", None)
+    if conv is None or windows is None:
+        if mamba_track_indices is not None or mamba_steps_to_track is not None:
+            raise NotImplementedError("track snapshots need the conv pools of spec_state")
+        return
+    if last_correct_step_indices is None:
+        raise ValueError("the conv rollback needs last_correct_step_indices")
+    assert len(conv) == len(windows)
+    for conv_states, interm_conv in zip(conv, windows):
+        if conv_state_layout == "width_dim":
+            conv_states = conv_states.transpose(-1, -2)
+            interm_conv = interm_conv.transpose(-1, -2)
+        conv_window_scatter(conv_states, interm_conv, state_batch_indices, last_correct_step_indices)
+        if mamba_track_indices is not None and mamba_steps_to_track is not None:
+            conv_window_scatter(conv_states, interm_conv, mamba_track_indices, mamba_steps_to_track)
+
+
+def fused_kda_decode_mtp_dspark(*, x_q, x_k, x_v, w_q, w_k, w_v, cs_q, cs_k, cs_v, g, beta, A_log, dt_bias,
+                                recurrent_state, intermediate_ssm=None, intermediate_state_indices,
+                                intermediate_conv_q, intermediate_conv_k, intermediate_conv_v,
+                                ssm_state_indices, cu_seqlens, lower_bound, scale=None,
+                                replayssm_rawv=None, replayssm_rawk=None, replayssm_g=None, replayssm_beta=None,
+                                onorm_gate=None, onorm_weight=None, onorm_eps=None, out=None):
+    """KDA verify of the draft tokens in ring mode (all four ``replayssm_*`` rings are required;
+    ``intermediate_ssm`` snapshots are not written).  Returns ``out`` [1, T, H, 128].
+
+    Shapes and layouts as the reference binding checks them
+    (src/decode/kda_replayssm_sglang/kda_mtp_verify_host.cpp:108-222): q/k/v/g bf16 [1, T, H, 128] with an
+    optional token stride, beta bf16 [1, T, H]; conv weights float32 [H*128, 4]; conv states bf16
+    [slots, H*128, 3] and windows bf16 [rows, steps, H*128, 3] with any positive strides; state float32
+    [slots, H, 128, 128], rings [slots, H, L, 128] (bf16 rawv / rawk, float32 g) and [slots, H, L] (float32
+    beta), ``out`` bf16, all contiguous; index tensors int32 or int64.  ``T`` must be ``N`` times the draft
+    window, which is limited to 8 tokens here.
+    """
+    rings = (replayssm_rawv, replayssm_rawk, replayssm_g, replayssm_beta)
+    if any(r is None for r in rings):
+        raise ValueError("pla.decode.kda_mtp_sglang.fused_kda_decode_mtp_dspark implements CACHE_RING only; "
+                         "pass all four replayssm_* rings.")
+    onorm_args = (onorm_gate, onorm_weight, onorm_eps)
+    apply_onorm = all(v is not None for v in onorm_args)
+    if any(v is not None for v in onorm_args) and not apply_onorm:
+        raise ValueError("fused output norm requires onorm_gate, onorm_weight, and onorm_eps")
+    if scale is None:
+        scale = 128 ** -0.5
+    if out is None:
+        out = torch.empty_like(x_v, memory_format=torch.contiguous_format)
+    if _BYPASS:
+        return out
+
+    def need(cond, msg):
+        if not cond:
+            raise RuntimeError(msg)
+
+    D, W = 128, 4
+    need(x_q.dim() == 4 and x_q.size(0) == 1, "x_q must be [1, T, H, 128]")
+    need(x_q.is_cuda, "verify requires CUDA tensors")
+    T, H = x_q.size(1), x_q.size(2)
+    need(x_q.size(3) == D, "specialised for head_dim 128")
+    N = cu_seqlens.numel() - 1
+    need(N > 0 and T > 0 and H > 0 and T % N == 0, "dense 1 + num_spec tokens per request")
+    t_loop = T // N
+    need(replayssm_rawv.dim() == 4, "rawv ring must be [slot, H, L, 128]")
+    L, slots = replayssm_rawv.size(2), replayssm_rawv.size(0)
+    need(L >= t_loop, "ring shorter than the draft window")
+    need(recurrent_state.dtype == torch.float32, "recurrent state must be fp32")
+    need(x_q.dtype == torch.bfloat16, "inputs must be bf16")
+    need(tuple(recurrent_state.shape) == (slots, H, D, D), "state must be [slot, H, 128, 128]")
+    everything = [x_k, x_v, g, beta, w_q, w_k, w_v, cs_q, cs_k, cs_v, A_log, dt_bias, recurrent_state, out,
+                  intermediate_conv_q, intermediate_conv_k, intermediate_conv_v, *rings, ssm_state_indices,
+                  intermediate_state_indices, cu_seqlens]
+    need(all(t.device == x_q.device for t in everything), "verify tensors must share one device")
+    need(all(tuple(t.shape) == (slots, H, L, D) for t in rings[:3]), "invalid verify ring shape")
+    need(tuple(replayssm_beta.shape) == (slots, H, L) and replayssm_rawv.dtype == torch.bfloat16
+         and replayssm_rawk.dtype == torch.bfloat16 and replayssm_g.dtype == torch.float32
+         and replayssm_beta.dtype == torch.float32, "invalid verify ring dtype/shape")
+    w_q, w_k, w_v = w_q.contiguous(), w_k.contiguous(), w_v.contiguous()
+    need(all(tuple(t.shape) == (H * D, W) and t.dtype == torch.float32 for t in (w_q, w_k, w_v)),
+         "conv weights must be contiguous fp32 [H*128, 4]")
+    A_log, dt_bias = A_log.contiguous(), dt_bias.contiguous()
+    need(A_log.numel() == H and dt_bias.numel() == H * D and A_log.dtype == torch.float32
+         and dt_bias.dtype == torch.float32, "invalid gate weights")
+    need(recurrent_state.storage_offset() % 4 == 0, "recurrent state must be 16-byte aligned for float4 loads")
+    need(ssm_state_indices.numel() == N and intermediate_state_indices.numel() >= N, "verify index count mismatch")
+
+    def input_stride(x):
+        need(x.shape == x_q.shape and x.dtype == torch.bfloat16, "Q/K/V and g must be bf16 [1, T, H, 128]")
+        need(x.stride(3) == 1 and x.stride(2) == D and x.stride(1) >= H * D,
+             "Q/K/V and g must have contiguous head/channel dimensions")
+        return [x.stride(1)]
+
+    def conv_strides(x):
+        need(x.dim() == 3 and x.size(0) == slots and x.size(1) == H * D and x.size(2) == W - 1
+             and x.dtype == torch.bfloat16, "conv states must be bf16 [slot, H*128, 3]")
+        need(all(st > 0 for st in x.stride()), "conv state strides must be positive")
+        return list(x.stride())
+
+    def window_strides(x):
+        need(x.dim() == 4 and x.size(1) >= t_loop and x.size(2) == H * D and x.size(3) == W - 1
+             and x.dtype == torch.bfloat16, "conv windows must be bf16 [scratch, step, H*128, 3]")
+        need(all(st > 0 for st in x.stride()), "conv window strides must be positive")
+        return list(x.stride())
+
+    need(beta.dim() == 3 and beta.size(0) == 1 and beta.size(1) == T and beta.size(2) == H
+         and beta.dtype == torch.bfloat16 and beta.stride(2) == 1 and beta.stride(1) >= H,
+         "beta must be bf16 [1, T, H] with contiguous heads")
+    need(out.shape == x_q.shape and out.is_contiguous() and out.dtype == torch.bfloat16
+         and recurrent_state.is_contiguous() and all(r.is_contiguous() for r in rings),
+         "output, recurrent state and rings must be contiguous")
+    strides = (input_stride(x_q) + input_stride(x_k) + input_stride(x_v) + input_stride(g) + [beta.stride(1)]
+               + conv_strides(cs_q) + conv_strides(cs_k) + conv_strides(cs_v)
+               + window_strides(intermediate_conv_q) + window_strides(intermediate_conv_k)
+               + window_strides(intermediate_conv_v))
+    gate_stride = 0
+    if apply_onorm:
+        need(onorm_gate.device == x_q.device and onorm_weight.device == x_q.device,
+             "output-norm tensors must share the verify device")
+        need(onorm_gate.shape == x_q.shape and onorm_gate.dtype == torch.bfloat16 and onorm_gate.stride(3) == 1
+             and onorm_gate.stride(2) == D and onorm_gate.stride(1) >= H * D,
+             "output-norm gate must be bf16 [1, T, H, 128] with contiguous head/channel dimensions")
+        need(onorm_weight.dim() == 1 and onorm_weight.size(0) == D and onorm_weight.is_contiguous()
+             and onorm_weight.dtype == torch.float32, "output-norm weight must be contiguous fp32 [128]")
+        need(onorm_eps == onorm_eps and abs(onorm_eps) != float("inf") and onorm_eps >= 0.0,
+             "output-norm eps must be finite and non-negative")
+        gate_stride = onorm_gate.stride(1)
+    si, si_wide = _index(ssm_state_indices)
+    sc, sc_wide = _index(intermediate_state_indices)
+    cu, cu_wide = _index(cu_seqlens)
+    c_strides = (ctypes.c_int64 * 26)(*strides)
+    with torch.cuda.device(x_q.device):
+        _lib.call(
+            "pla_kda_verify_dspark_launch", x_q.data_ptr(), x_k.data_ptr(), x_v.data_ptr(), g.data_ptr(),
+            beta.data_ptr(), w_q.data_ptr(), w_k.data_ptr(), w_v.data_ptr(), cs_q.data_ptr(), cs_k.data_ptr(),
+            cs_v.data_ptr(), A_log.data_ptr(), dt_bias.data_ptr(), recurrent_state.data_ptr(), out.data_ptr(),
+            intermediate_conv_q.data_ptr(), intermediate_conv_k.data_ptr(), intermediate_conv_v.data_ptr(),
+            replayssm_rawv.data_ptr(), replayssm_rawk.data_ptr(), replayssm_g.data_ptr(), replayssm_beta.data_ptr(),
+            si.data_ptr(), si_wide, sc.data_ptr(), sc_wide, cu.data_ptr(), cu_wide,
+            H, N, t_loop, L, float(scale), float(lower_bound), ctypes.cast(c_strides, ctypes.c_void_p),
+            _lib.ptr(onorm_gate) if apply_onorm else None, _lib.ptr(onorm_weight) if apply_onorm else None,
+            gate_stride, float(onorm_eps) if apply_onorm else 0.0, _lib.current_stream(x_q.device))
+    return out
 
 
 def kda_mtp_verify(q, k, v, g, beta, recurrent_state, ssm_state_indices, cu_seqlens, scale=None,

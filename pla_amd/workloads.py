@@ -236,3 +236,65 @@ def kda_decode_mega(B, H, seed=0, device="cuda", dtype=torch.bfloat16, pad_rows=
         "norm_weight": rand(D).to(device),
         "_cache": cache,
     }
+
+
+def kda_replay_verify(N, H, num_draft, seed=0, device="cuda", ring_len=16, slots=None, lower_bound=-8.0,
+                      onorm=True, pad_rows=(), strided=True, index_dtype=torch.int32):
+    """KDA speculative verify with replay records (ring mode): ``N`` requests of ``num_draft`` tokens.
+
+    Shapes and distributions follow the reference's input builder
+    (scripts/decode/kda_mtp_sglang/private/_common.py:84-166).  With ``strided`` the q/k/v inputs are the
+    three segments of one mixed row, the conv states the transposed segments of a [slots, 3, 3*H*128]
+    pool and the scratch windows segments of one [rows, steps, 3*H*128, 3] buffer, as SGLang passes them.
+    Slot ids are a seeded permutation, scratch rows a different one; ``pad_rows`` get slot -1.
+    Returns the keyword arguments of ``fused_kda_decode_mtp_dspark``.
+    """
+    device = torch.device(device)
+    g = _gen(seed)
+    dim, T, W = H * D, N * num_draft, 4
+    slots = slots or N + 2
+
+    def bf16(*shape, scale=1.0):
+        return (torch.randn(*shape, generator=g) * scale).to(torch.bfloat16)
+
+    if strided:
+        mixed = bf16(1, T, 3 * dim + 64, scale=0.5).to(device)
+        x_q, x_k, x_v = (mixed[:, :, i * dim:(i + 1) * dim].view(1, T, H, D) for i in range(3))
+        pool = bf16(slots, W - 1, 3 * dim, scale=0.3).to(device)
+        cs_q, cs_k, cs_v = (pool[:, :, i * dim:(i + 1) * dim].transpose(-1, -2) for i in range(3))
+        ic = torch.zeros(N + 1, num_draft + 1, 3 * dim, W - 1, dtype=torch.bfloat16, device=device)
+        ic_q, ic_k, ic_v = (ic[:, :, i * dim:(i + 1) * dim] for i in range(3))
+        gate_store = bf16(1, T, dim + 32, scale=0.5).to(device)
+        onorm_gate = gate_store[:, :, :dim].view(1, T, H, D)
+    else:
+        x_q, x_k, x_v = (bf16(1, T, H, D, scale=0.5).to(device) for _ in range(3))
+        cs_q, cs_k, cs_v = (bf16(slots, dim, W - 1, scale=0.3).to(device) for _ in range(3))
+        ic_q, ic_k, ic_v = (torch.zeros(N + 1, num_draft, dim, W - 1, dtype=torch.bfloat16, device=device)
+                            for _ in range(3))
+        onorm_gate = bf16(1, T, H, D, scale=0.5).to(device)
+    conv_w = (torch.randn(3 * dim, W, generator=g) * 0.3).to(device)
+    idx = torch.randperm(slots, generator=g)[:N].to(index_dtype)
+    for r in pad_rows:
+        idx[r] = -1
+    out = dict(
+        x_q=x_q, x_k=x_k, x_v=x_v, w_q=conv_w[:dim], w_k=conv_w[dim:2 * dim], w_v=conv_w[2 * dim:],
+        cs_q=cs_q, cs_k=cs_k, cs_v=cs_v,
+        g=bf16(1, T, H, D, scale=0.5).to(device), beta=bf16(1, T, H).to(device),
+        A_log=(torch.rand(H, generator=g) * 0.5 + 0.5).to(device),
+        dt_bias=(torch.randn(dim, generator=g) * 0.1).to(device),
+        recurrent_state=(torch.randn(slots, H, D, D, generator=g) * 0.1).to(device),
+        intermediate_ssm=None,
+        intermediate_state_indices=torch.randperm(N + 1, generator=g)[:N].to(index_dtype).to(device),
+        intermediate_conv_q=ic_q, intermediate_conv_k=ic_k, intermediate_conv_v=ic_v,
+        ssm_state_indices=idx.to(device),
+        cu_seqlens=torch.arange(0, T + 1, num_draft, dtype=index_dtype).to(device),
+        lower_bound=lower_bound, scale=D ** -0.5,
+        replayssm_rawv=torch.full((slots, H, ring_len, D), 3.0, dtype=torch.bfloat16, device=device),
+        replayssm_rawk=torch.full((slots, H, ring_len, D), 3.0, dtype=torch.bfloat16, device=device),
+        replayssm_g=torch.full((slots, H, ring_len, D), 3.0, dtype=torch.float32, device=device),
+        replayssm_beta=torch.full((slots, H, ring_len), 3.0, dtype=torch.float32, device=device),
+    )
+    if onorm:
+        out.update(onorm_gate=onorm_gate, onorm_weight=(torch.rand(D, generator=g) * 0.5 + 0.75).to(device),
+                   onorm_eps=1e-6)
+    return out
