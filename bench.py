@@ -279,6 +279,57 @@ def bench_decode_mega(device, steps=100, B=256, H=12, sets=16):
             "frac_of_hbm_peak": round(state_bytes / us / 1e3 / HBM_PEAK_GBPS, 4)}
 
 
+def bench_replay_verify(device, steps=100, N=64, H=32, T=4):
+    """Config 2 through the production contract: conv front end + gate + verify of 4 draft tokens with replay
+    records and scratch windows in one launch, then the commit (fold of the accepted prefix + conv rollback)."""
+    import types
+    import torch
+    from pla_amd.decode.kda_replayssm_sglang import fused_kda_decode_mtp_dspark, commit_kda_replayssm_after_verify
+    from pla_amd.workloads import kda_replay_verify
+    w = kda_replay_verify(N, H, T, seed=505, device=device, slots=1024, ring_len=8, onorm=True, strided=False)
+    w["intermediate_state_indices"] = torch.arange(N, dtype=torch.int32, device=device)
+    out = torch.empty(1, N * T, H, 128, dtype=torch.bfloat16, device=device)
+
+    def timed(fn):
+        # replayed from a graph: the Python facade (argument checks) costs more than these kernels
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(10):
+            graph.replay()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / steps * 1e3
+
+    us_verify = timed(lambda: fused_kda_decode_mtp_dspark(out=out, **w))
+    g = torch.Generator().manual_seed(6)
+    accept = torch.randint(0, T + 1, (N,), generator=g).to(torch.int32).to(device)
+    spec = types.SimpleNamespace(
+        temporal=w["recurrent_state"][None], replayssm_rawv=w["replayssm_rawv"][None],
+        replayssm_rawk=w["replayssm_rawk"][None], replayssm_g=w["replayssm_g"][None],
+        replayssm_beta=w["replayssm_beta"][None],
+        conv=[w["cs_q"][None], w["cs_k"][None], w["cs_v"][None]],
+        intermediate_conv_window=[w["intermediate_conv_q"][None], w["intermediate_conv_k"][None],
+                                  w["intermediate_conv_v"][None]])
+    last = accept.long() - 1
+    us_commit = timed(lambda: commit_kda_replayssm_after_verify(
+        spec_state=spec, state_batch_indices=w["ssm_state_indices"], accept_lens=accept,
+        last_correct_step_indices=last))
+    return {"workload": "KDA verify with replay records + commit, B=%d, H=%d, %d draft tokens, gated RMSNorm" % (N, H, T),
+            "verify_us": round(us_verify, 2), "verify_state_read_GBps": round(N * H * 65536 / us_verify / 1e3, 1),
+            "commit_us": round(us_commit, 2)}
+
+
 def cpu_baseline_decode(w, sample_requests=32, reps=5):
     """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
     sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
@@ -359,6 +410,7 @@ def main():
         result["other_decode"] = bench_small_decode(device)
         result["other_decode"].update(bf16_pool)
         result["decode_mega"] = bench_decode_mega(device)
+        result["replay_verify"] = bench_replay_verify(device)
         torch.cuda.empty_cache()
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
         torch.cuda.empty_cache()

@@ -83,7 +83,37 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   }
   const int64_t srow = index_at(p.scratch_idx, p.scratch_wide, n);
 
-  // state tile first, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
+  __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128], sW[TMAX][128];
+  __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
+  __shared__ float sBeta[TMAX], sNorm[2][2][TMAX], sSq[4][TMAX];
+
+  // Small inputs first, the state tile after them: memory returns in issue order, so the convolution
+  // starts as soon as its inputs are there while the 64 KiB tile is still in flight.  Wavefronts 0-1
+  // (threads 0-127) own one q and one k channel each, wavefronts 2-3 one v channel and its gate.
+  const bool qk_side = tid < 128;
+  const int i128 = tid & 127;
+  const int64_t ch = (int64_t)h * 128 + i128;
+  const float4 cwa = reinterpret_cast<const float4*>(qk_side ? p.w_q : p.w_v)[ch];
+  const float4 cwb = reinterpret_cast<const float4*>(p.w_k)[ch];
+  const uint16_t* const cs_a = qk_side ? p.cs_q : p.cs_v;
+  const int ia = qk_side ? 0 : 2;
+  uint16_t ta[3], tb[3], xa[TMAX], xb[TMAX], xc[TMAX];
+#pragma unroll
+  for (int j = 0; j < 3; ++j) {
+    ta[j] = cs_a[slot * p.cs[ia][0] + ch * p.cs[ia][1] + j * p.cs[ia][2]];
+    tb[j] = p.cs_k[slot * p.cs[1][0] + ch * p.cs[1][1] + j * p.cs[1][2]];
+  }
+#pragma unroll
+  for (int t = 0; t < TMAX; ++t) {                   // absent tokens repeat the last one
+    const int64_t tok = bos + min(t, n_tok - 1);
+    xa[t] = qk_side ? p.x_q[tok * p.sx_q + ch] : p.x_v[tok * p.sx_v + ch];
+    xb[t] = qk_side ? p.x_k[tok * p.sx_k + ch] : p.g[tok * p.sg + ch];
+    xc[t] = p.beta[tok * p.sbeta + h];
+  }
+  const float eA = __expf(p.a_log[h]);
+  const float bias = p.dt_bias[ch];
+
+  // state tile, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
   const Tile<float> h_tile(p.h0 + (slot * p.H + h) * 16384);
   f32x4_t sa[2][4][2];
 #pragma unroll
@@ -95,28 +125,14 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
         sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
             h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
 
-  __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128], sW[TMAX][128];
-  __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
-  __shared__ float sBeta[TMAX], sNorm[2][2][TMAX], sSq[4][TMAX];
-
   const int64_t ring_row = (slot * p.H + h) * p.L;   // first record of this (slot, head)
-  if (tid < 128) {
-    const int64_t ch = (int64_t)h * 128 + tid;
-    const float4 wq = reinterpret_cast<const float4*>(p.w_q)[ch];
-    const float4 wk = reinterpret_cast<const float4*>(p.w_k)[ch];
-    float cq[3], ck[3];
-#pragma unroll
-    for (int j = 0; j < 3; ++j) {
-      cq[j] = bf(p.cs_q[slot * p.cs[0][0] + ch * p.cs[0][1] + j * p.cs[0][2]]);
-      ck[j] = bf(p.cs_k[slot * p.cs[1][0] + ch * p.cs[1][1] + j * p.cs[1][2]]);
-    }
+  if (qk_side) {
+    float cq[3] = {bf(ta[0]), bf(ta[1]), bf(ta[2])}, ck[3] = {bf(tb[0]), bf(tb[1]), bf(tb[2])};
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
       if (t >= n_tok) break;
-      const float xq = bf(p.x_q[(bos + t) * p.sx_q + ch]);
-      const float xk = bf(p.x_k[(bos + t) * p.sx_k + ch]);
-      const float q = conv_step(cq, xq, wq);
-      const float k = conv_step(ck, xk, wk);
+      const float q = conv_step(cq, bf(xa[t]), cwa);
+      const float k = conv_step(ck, bf(xb[t]), cwb);
       sQ[t][tid] = q;
       sK[t][tid] = k;
       p.ring_rawk[(ring_row + t) * 128 + tid] = to_bf(k);
@@ -129,29 +145,21 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       if (lane == 0) { sNorm[0][wave][t] = q2; sNorm[1][wave][t] = k2; }
     }
   } else {
-    const int i = tid - 128;
-    const int64_t ch = (int64_t)h * 128 + i;
-    const float4 wv = reinterpret_cast<const float4*>(p.w_v)[ch];
-    const float eA = __expf(p.a_log[h]);
-    const float bias = p.dt_bias[ch];
-    float cv[3];
-#pragma unroll
-    for (int j = 0; j < 3; ++j) cv[j] = bf(p.cs_v[slot * p.cs[2][0] + ch * p.cs[2][1] + j * p.cs[2][2]]);
+    float cv[3] = {bf(ta[0]), bf(ta[1]), bf(ta[2])};
 #pragma unroll
     for (int t = 0; t < TMAX; ++t) {
       if (t >= n_tok) break;
-      const float xv = bf(p.x_v[(bos + t) * p.sx_v + ch]);
-      const float v = conv_step(cv, xv, wv);
-      sV[t][i] = v;
-      p.ring_rawv[(ring_row + t) * 128 + i] = to_bf(v);
+      const float v = conv_step(cv, bf(xa[t]), cwa);
+      sV[t][i128] = v;
+      p.ring_rawv[(ring_row + t) * 128 + i128] = to_bf(v);
 #pragma unroll
       for (int j = 0; j < 3; ++j)
         p.ic_v[srow * p.ic[2][0] + t * p.ic[2][1] + ch * p.ic[2][2] + j * p.ic[2][3]] = to_bf(cv[j]);
-      const float gk = p.lower_bound * fast_sigmoid(eA * (bf(p.g[(bos + t) * p.sg + ch]) + bias));
-      p.ring_g[(ring_row + t) * 128 + i] = gk;
-      sD[t][i] = __expf(gk);
-      if (i == 0) {
-        const float b = fast_sigmoid(bf(p.beta[(bos + t) * p.sbeta + h]));
+      const float gk = p.lower_bound * fast_sigmoid(eA * (bf(xb[t]) + bias));
+      p.ring_g[(ring_row + t) * 128 + i128] = gk;
+      sD[t][i128] = __expf(gk);
+      if (i128 == 0) {
+        const float b = fast_sigmoid(bf(xc[t]));
         sBeta[t] = b;
         p.ring_beta[ring_row + t] = b;
       }
