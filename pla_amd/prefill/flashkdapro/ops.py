@@ -16,6 +16,7 @@ from typing import Optional, Tuple
 import torch
 
 from ... import _lib
+from .. import _sanity
 
 CHUNK_SIZE = 64
 DK = 128
@@ -96,6 +97,7 @@ def flashkda_fwd(
     if A_log.numel() != H:
         raise ValueError("A_log must be [H]")
 
+    _sanity.offsets(cu_seqlens, T, raw_cu_seqlens, reference=q)
     if cu_seqlens is None:
         cu32 = torch.tensor([0, T], dtype=torch.int32, device=q.device)
     else:

@@ -22,6 +22,7 @@ from typing import Optional, Sequence, Tuple, Union
 import torch
 
 from ... import _lib
+from .. import _sanity
 
 CHUNK_SIZE = 64
 DK = 128
@@ -94,6 +95,8 @@ def chunk_gated_delta_rule_fwd(
     if scale is None:
         scale = q.size(-1) ** -0.5
 
+    _sanity.offsets(cu_seqlens, num_tokens,
+                    raw_cu_seqlens.tolist() if isinstance(raw_cu_seqlens, torch.Tensor) else raw_cu_seqlens, reference=q)
     if cu_seqlens is None:
         cu_seqlens = torch.tensor([0, num_tokens], dtype=torch.int32, device=q.device)
     cu32 = cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()

@@ -98,3 +98,28 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libpla_gfx950.so")
     with pytest.raises(RuntimeError, match="there is no fallback path"):
         _lib.load()
+
+
+def test_prefill_sanity_mode_checks_offsets(monkeypatch):
+    """PLA_SANITY_CHECK=1: offsets are validated before they are narrowed to int32 (reference helper
+    pla/prefill/_sanity.py:46-110); violations raise AssertionError with the reference's prefix."""
+    import torch
+    from pla_amd.prefill import _sanity
+    cu = torch.tensor([0, 5, 5, 9], dtype=torch.int64)
+    monkeypatch.delenv("PLA_SANITY_CHECK", raising=False)
+    _sanity.offsets(torch.tensor([3, 1]), 2)                                         # off: nothing is checked
+    monkeypatch.setenv("PLA_SANITY_CHECK", "1")
+    _sanity.offsets(cu, 9, (0, 5, 5, 9))
+    _sanity.offsets(None, 7, (0, 7))
+    for bad_cu, cap, raw, msg in (
+            (torch.tensor([1, 5]), 9, None, "start at zero"),
+            (torch.tensor([0, 5, 4]), 9, None, "monotonic"),
+            (torch.tensor([0, 5, 10]), 9, None, "within token capacity"),
+            (torch.tensor([0, 2 ** 31], dtype=torch.int64), 2 ** 31 + 5, None, "token capacity must fit int32"),
+            (cu, 9, (0, 5, 6, 9), "raw_cu_seqlens must equal device cu_seqlens"),
+            (cu, 9, (0, 5, 9), "batch\\+1 entries"),
+            (cu.float(), 9, None, "int32 or int64"),
+            (cu.reshape(2, 2), 9, None, r"\[batch\+1\]"),
+            (None, 7, (0, 6), r"must be \[0,T\]")):
+        with pytest.raises(AssertionError, match=r"PLA_SANITY_CHECK \[prefill\]: .*" + msg):
+            _sanity.offsets(bad_cu, cap, raw)
