@@ -514,10 +514,13 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
 // gfx950 tuning table: rows of the 128-row tile owned by one wavefront, chosen
 // from the number of (request, value-head) tiles so that small batches still
 // spread over all 256 CUs while large batches keep 64 state VGPRs in flight.
+// Measured on MI355X (packed GDN decode, HV = 32, us per step at 8 / 16 / 32 rows per wavefront):
+//   32 tiles 3.9 / 4.6 / 6.0    128 tiles 5.2 / 5.6 / 6.9     256 tiles 8.2 / 7.8 / 9.2
+//   512 tiles 15.8 / 15.4 / 14.8    2048 tiles 53.5 / 53.5 / 50.9    8192 tiles 207.6 / 205.8 / 190.3
 static int pick_rows_per_wave(int tiles, bool mtp) {
   (void)mtp;
-  if (tiles >= 2048) return 32;
-  if (tiles >= 512) return 16;
+  if (tiles >= 512) return 32;
+  if (tiles >= 192) return 16;
   return 8;
 }
 
