@@ -117,6 +117,10 @@ def bench_decode_bf16_pool(w, steps, device):
 PREFILL_SEED = 348      # ragged_lengths(8, 512, 8192, 348) sums to 32 810 tokens
 GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64, K = V = 128, HV = 32, H = 16
 KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
+# HBM bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00), summed over the kernels of
+# one call (profiles/gdn_prefill_kernels_32k.txt, profiles/kda_prefill_kernels_64k.txt)
+GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 3290000000
+KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 17100000000
 
 
 def bench_prefill(steps, warmup, device):
@@ -147,7 +151,8 @@ def bench_prefill(steps, warmup, device):
     tflops = GDN_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     return dict(tokens=T, lengths=lengths, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=None,
+                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=GDN_PREFILL_TRAFFIC_BYTES_PER_CALL,
+                              hbm_GBps=round(GDN_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
                               flop_per_token=GDN_FLOP_PER_TOKEN,
                               note="algorithmic flops (dense, no hi/lo passes) over the whole call: "
                                    "chunk map + prep + gram/solve + sequential kernels"))
@@ -179,7 +184,8 @@ def bench_prefill_kda(steps, device):
     tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     return dict(tokens=T, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
-                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=None,
+                              frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=KDA_PREFILL_TRAFFIC_BYTES_PER_CALL,
+                              hbm_GBps=round(KDA_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
                               flop_per_token=KDA_FLOP_PER_TOKEN))
 
 
@@ -368,6 +374,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--decode-only", action="store_true", help="skip the secondary decode / prefill measurements")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the two prefill workloads (for rocprofv3 --pmc byte counters) and print their objects")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a 1 GiB device copy (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -381,6 +389,14 @@ def main():
         sys.exit(2)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.prefill_only:
+        result = {"prefill": bench_prefill(max(args.steps // 10, 5), 3, device)}
+        torch.cuda.empty_cache()
+        result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+        if args.copy_calibration:
+            result["copy_calibration"] = copy_calibration(device)
+        print(json.dumps(result))
+        return
     d = bench_decode(args.steps, args.warmup, device)
     result = {
         "metric": "gdn_packed_decode_state_hbm_GBps@B=256",
