@@ -173,3 +173,52 @@ def sanity_kda_decode_mega(x, weight, bias, conv_state, state_indices, state, lo
         for name, t in (("weight", weight), ("bias", bias), ("norm_weight", norm_weight)):
             if t is not None and not bool(torch.isfinite(t).all()):
                 _fail(op, f"{name} must be finite")
+
+
+def sanity_verify_dspark(x_q, x_k, x_v, w_q, w_k, w_v, cs_q, cs_k, cs_v, h0, ic_q, slot_idx, scratch_idx, cu_seqlens,
+                         N, T, t_loop, slots, scale, lower_bound, onorm_weight, onorm_eps):
+    """Diagnostic checks of the KDA verify with replay records
+    (src/decode/kda_replayssm_sglang/sanity_checks.h:90-160): finite float32 scalars; value checks
+    (skipped during capture): dense offsets of ``t_loop`` tokens per request, active slots and scratch
+    rows in range, no two requests writing one slot's rings or one scratch row, finite selected inputs."""
+    import math
+    op = "kda_verify_dspark"
+    if not math.isfinite(scale):
+        _fail(op, "scale must be representable as a finite float32 value")
+    if not (math.isfinite(lower_bound) and lower_bound < 0.0):
+        _fail(op, "lower_bound must be a finite negative float32 value")
+    if onorm_eps is not None and not (math.isfinite(onorm_eps) and onorm_eps >= 0.0):
+        _fail(op, "onorm_eps must be a finite non-negative float32 value")
+    if _capturing():
+        return
+    offsets = cu_seqlens.tolist()
+    if offsets[0] != 0 or offsets[-1] != T:
+        _fail(op, "cu_seqlens must cover exactly the packed tokens")
+    ring_writers, window_writers = set(), set()
+    active = False
+    for n, (slot, row) in enumerate(zip(slot_idx.tolist(), scratch_idx.tolist()[:N])):
+        if offsets[n + 1] - offsets[n] != t_loop:
+            _fail(op, f"every request must own exactly {t_loop} tokens (request {n})")
+        if slot < 0:
+            continue
+        if slot >= slots:
+            _fail(op, f"state/ring slot is out of bounds at request {n}")
+        if not 0 <= row < ic_q.size(0):
+            _fail(op, f"scratch row is out of bounds at request {n}")
+        if slot in ring_writers:
+            _fail(op, f"two requests write the rings of slot {slot}")
+        if row in window_writers:
+            _fail(op, f"two requests write scratch row {row}")
+        ring_writers.add(slot)
+        window_writers.add(row)
+        active = True
+        for name, t in (("selected h0", h0[slot]), ("selected cs_q", cs_q[slot]), ("selected cs_k", cs_k[slot]),
+                        ("selected cs_v", cs_v[slot]), ("selected x_q", x_q[:, offsets[n]:offsets[n + 1]]),
+                        ("selected x_k", x_k[:, offsets[n]:offsets[n + 1]]),
+                        ("selected x_v", x_v[:, offsets[n]:offsets[n + 1]])):
+            if not bool(torch.isfinite(t).all()):
+                _fail(op, f"{name} must be finite")
+    if active:
+        for name, t in (("w_q", w_q), ("w_k", w_k), ("w_v", w_v), ("onorm_weight", onorm_weight)):
+            if t is not None and not bool(torch.isfinite(t).all()):
+                _fail(op, f"{name} must be finite")

@@ -248,6 +248,11 @@ def fused_kda_decode_mtp_dspark(*, x_q, x_k, x_v, w_q, w_k, w_v, cs_q, cs_k, cs_
     si, si_wide = _index(ssm_state_indices)
     sc, sc_wide = _index(intermediate_state_indices)
     cu, cu_wide = _index(cu_seqlens)
+    if os.environ.get("PLA_SANITY_CHECK", "0") == "1":            # read on every call, like src/sanity_check.h
+        from ..._sanity import sanity_verify_dspark
+        sanity_verify_dspark(x_q, x_k, x_v, w_q, w_k, w_v, cs_q, cs_k, cs_v, recurrent_state, intermediate_conv_q,
+                             si, sc, cu, N, T, t_loop, slots, float(scale), float(lower_bound),
+                             onorm_weight if apply_onorm else None, onorm_eps if apply_onorm else None)
     c_strides = (ctypes.c_int64 * 26)(*strides)
     with torch.cuda.device(x_q.device):
         _lib.call(

@@ -155,3 +155,37 @@ def test_verify_then_commit_round_trip():
     for k in ("x_q", "x_k", "x_v", "g"):
         w[k].copy_((torch.randn(w[k].shape, generator=g) * 0.5).to(torch.bfloat16))
     _check(w)
+
+
+def test_verify_sanity_mode(monkeypatch):
+    monkeypatch.setenv("PLA_SANITY_CHECK", "1")
+    w = kda_replay_verify(4, 4, 3, seed=12, pad_rows=(1,))
+    _check(w)                                                                        # a clean call passes
+    rings_before = w["replayssm_g"].clone()
+    bad = dict(w)
+    bad["ssm_state_indices"] = torch.tensor([2, -1, 2, 0], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match=r"PLA_SANITY_CHECK \[kda_verify_dspark\]: two requests write the rings"):
+        fused_kda_decode_mtp_dspark(**bad)
+    bad = dict(w)
+    bad["ssm_state_indices"] = torch.tensor([2, -1, 77, 0], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="slot is out of bounds"):
+        fused_kda_decode_mtp_dspark(**bad)
+    bad = dict(w)
+    bad["cu_seqlens"] = torch.tensor([0, 3, 5, 9, 12], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="must own exactly 3 tokens"):
+        fused_kda_decode_mtp_dspark(**bad)
+    bad = dict(w)
+    bad["lower_bound"] = 0.5
+    with pytest.raises(RuntimeError, match="lower_bound must be a finite negative"):
+        fused_kda_decode_mtp_dspark(**bad)
+    bad = dict(w)
+    bad["x_k"] = w["x_k"].clone()
+    bad["x_k"][0, 7, 1, 3] = float("inf")
+    with pytest.raises(RuntimeError, match="selected x_k must be finite"):
+        fused_kda_decode_mtp_dspark(**bad)
+    bad["x_k"][0, 7, 1, 3] = 0.0
+    bad["x_k"][0, 4, 1, 3] = float("nan")                                              # token of the padded request
+    fused_kda_decode_mtp_dspark(**bad)
+    torch.cuda.synchronize()
+    unused = [s for s in range(w["replayssm_g"].shape[0]) if s not in w["ssm_state_indices"].tolist()]
+    assert torch.equal(w["replayssm_g"][unused], rings_before[unused])
