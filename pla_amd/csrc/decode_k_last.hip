@@ -18,7 +18,7 @@
 // above T_max) make the request a no-op instead of trapping the device.
 
 #include "decode_common.h"
-#include "mfma_bf16.h"
+#include "readonce_verify.h"
 
 namespace pla {
 
@@ -39,15 +39,11 @@ struct KLastParams {
 };
 
 // READONCE (verify of up to four draft tokens that writes no state, no snapshots and follows no tree):
-// the recurrence is unrolled algebraically instead of being stepped through the state,
-//     o_t = S_0 w_t + sum_{j <= t} c_{j,t} v_j,   w_t = A_1 ... A_t q_t,   A_j = D_j (I - beta_j k_j k_j^T),
-// where w_t and the coefficients c_{j,t} = beta_j k_j^T (A_{j+1} ... A_t q_t) need only K-vectors (ten
-// dot products for four tokens; wavefront t of the workgroup works out token t and publishes w_t and
-// c_{.,t} in LDS).  The state tile is then used once, as the A operand of S_0 [w_0 .. w_3] on
-// v_mfma_f32_16x16x32_bf16: FP32 rows and effective queries are split into bf16 hi + lo parts (three
-// products keep 16 mantissa bits), so there are no cross-lane reductions over the tile at all (the
-// read-once verify of src/decode/kda_replayssm/kda_mtp_verify.cu:630-652).  One workgroup covers a
-// whole tile: RPW is 32 and wavefront w owns rows 32 w .. 32 w + 31 as two 16-row MFMA tiles.
+// the recurrence is unrolled algebraically instead of being stepped through the state (readonce_verify.h):
+// wavefront t of the workgroup works out the effective query w_t and the coefficients c_{.,t} of token t
+// from K-vectors and publishes them in LDS; the state tile is then used once, as the MFMA A operand of
+// S_0 [w_0 .. w_3].  One workgroup covers a whole tile: RPW is 32 and wavefront w owns rows
+// 32 w .. 32 w + 31 as two 16-row MFMA tiles.
 template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false, typename state_t = float>
 __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   state_t* const pool = reinterpret_cast<state_t*>(p.h0);
@@ -243,17 +239,8 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
       }
       float w[4] = {q4[0] * qn, q4[1] * qn, q4[2] * qn, q4[3] * qn};
-      float cf[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 3; j >= 0; --j) {
-        if (j > t) continue;
-        float dot = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dot = fmaf(kv[j][e], w[e], dot);
-        cf[j] = beta[j] * row32_allreduce(dot);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf[j], kv[j][e], w[e]);
-      }
+      float cf[4];
+      effective_query<4>(t, w, kv, dec, beta, cf);
       if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
       if (lane == 0) *reinterpret_cast<float4*>(&sC[t][0]) = make_float4(cf[0], cf[1], cf[2], cf[3]);
     }
@@ -262,25 +249,12 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     const int tcol = min(r16, 3);
     const float keep = r16 < 4 ? 1.f : 0.f;
     HiLo wb[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb]);
-      const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb + 4]);
-      wb[ks] = split8(f32x4_t{w0.x * keep, w0.y * keep, w0.z * keep, w0.w * keep},
-                      f32x4_t{w1.x * keep, w1.y * keep, w1.z * keep, w1.w * keep});
-    }
+    query_operands(sW, tcol, keep, kb, wb);
     const float4 cmine = *reinterpret_cast<const float4*>(&sC[tcol][0]);
     const float cs[4] = {cmine.x, cmine.y, cmine.z, cmine.w};
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const HiLo a = split8(sa[m][ks][0], sa[m][ks][1]);
-        acc = mfma16(a.hi, wb[ks].hi, acc);
-        acc = mfma16(a.lo, wb[ks].hi, acc);
-        acc = mfma16(a.hi, wb[ks].lo, acc);
-      }
+      const f32x4_t acc = rows_times_queries(sa[m], wb);
       // lane (r16 = token, kb): rows 16 m + 4 kb .. + 3 of S_0 w_token; add the bias terms
       float o[4] = {acc[0], acc[1], acc[2], acc[3]};
 #pragma unroll

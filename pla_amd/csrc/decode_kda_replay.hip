@@ -25,7 +25,7 @@
 // non-negative step and an in-range destination.
 
 #include "decode_common.h"
-#include "mfma_bf16.h"
+#include "readonce_verify.h"
 
 namespace pla {
 
@@ -188,17 +188,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       const float4 q4 = *reinterpret_cast<const float4*>(&sQ[t][4 * c]);
       float w[4] = {q4.x * qn, q4.y * qn, q4.z * qn, q4.w * qn};
       float cf[TMAX];
-#pragma unroll
-      for (int j = TMAX - 1; j >= 0; --j) {
-        cf[j] = 0.f;
-        if (j > t) continue;
-        float dot = 0.f;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) dot = fmaf(kv[j][e], w[e], dot);
-        cf[j] = beta[j] * row32_allreduce(dot);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = dec[j][e] * fmaf(-cf[j], kv[j][e], w[e]);
-      }
+      effective_query<TMAX>(t, w, kv, dec, beta, cf);
       if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
       if (lane == 0) {
 #pragma unroll
@@ -213,13 +203,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   const bool mine = r16 < n_tok;
   const float keep = mine ? 1.f : 0.f;
   HiLo wb[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb]);
-    const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 8 * kb + 4]);
-    wb[ks] = split8(f32x4_t{w0.x * keep, w0.y * keep, w0.z * keep, w0.w * keep},
-                    f32x4_t{w1.x * keep, w1.y * keep, w1.z * keep, w1.w * keep});
-  }
+  query_operands(sW, tcol, keep, kb, wb);
   float cs[TMAX];
 #pragma unroll
   for (int j = 0; j < TMAX; ++j) cs[j] = sC[tcol][j];
@@ -228,14 +212,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   float ss = 0.f;
 #pragma unroll
   for (int m = 0; m < 2; ++m) {
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const HiLo a = split8(sa[m][ks][0], sa[m][ks][1]);
-      acc = mfma16(a.hi, wb[ks].hi, acc);
-      acc = mfma16(a.lo, wb[ks].hi, acc);
-      acc = mfma16(a.hi, wb[ks].lo, acc);
-    }
+    const f32x4_t acc = rows_times_queries(sa[m], wb);
     // lane (r16 = token, kb): rows 32 w + 16 m + 4 kb .. + 3 of S_0 w_token, plus the bias terms
     o[m][0] = acc[0]; o[m][1] = acc[1]; o[m][2] = acc[2]; o[m][3] = acc[3];
 #pragma unroll
