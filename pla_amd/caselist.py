@@ -1,0 +1,271 @@
+"""Replay of OperatorsForge caselists on the gfx950 kernels.
+
+A caselist line names one operator shape, e.g.::
+
+    [GDN]:[D][8]gdn_attn:seqlen_q:1,head_dim_qk:128,...,num_heads_qk:16,num_heads_v:32,...,batch_size:8,dtype:bf16.
+    [KDA]:[P][6,1798]kda_attn:head_dim_qk:128,...,gate_lower_bound:-5.0,batch_size:6,dtype:bf16,cu_seqlens_q:[0,1090,...].
+
+(the format of the reference's ``caselist/decode/*.list`` and ``caselist/prefill/*.list``, which its
+``tests/test_op_forge.py`` replays).  ``parse_case`` turns a line into a dict, ``replay_case`` runs the
+shape on synthetic inputs through the operator that serves it here and times it:
+
+==========================  =====================================================================
+GDN decode, 1 token         ``fused_sigmoid_gating_delta_rule_forward_k_last_packed``
+GDN decode, T tokens        ``fused_sigmoid_gating_delta_rule_forward_k_last`` (verify, state read-only)
+KDA decode, 1 token         ``fused_kda_decode_mega_forward`` (conv + gate + recurrence + norm)
+KDA decode, T tokens        ``fused_kda_decode_mtp_dspark`` (verify with replay records, T <= 8)
+GDN / KDA prefill           ``gdn_prefill_packed_qkv_fwd`` / ``flashkda_fwd``
+==========================  =====================================================================
+
+Shapes outside head_dim 128 and other operator families (``mamba2_ssm``) are reported as skipped.
+Decode shapes are timed as graph replays over rotating slot sets (the host-side argument checks cost
+more than the small kernels, and a fixed slot set would be served from the last-level cache).
+
+Command line: ``python -m pla_amd.caselist FILE [--limit N] [--csv OUT]``.
+"""
+
+import argparse
+import ast
+import csv
+import re
+import sys
+
+import torch
+
+_LINE = re.compile(r"^\[(?P<family>\w+)\]:\[(?P<phase>[DP])\]\[(?P<tag>[^\]]*)\](?P<op>\w+):(?P<body>.*?)\.?$")
+_MEGA_HEADS = (4, 6, 8, 12, 16, 24, 48, 64, 96)
+
+
+def parse_case(line):
+    """One caselist line -> dict (``family``, ``phase``, ``op`` and the line's own keys with integers,
+    floats and the ``cu_seqlens_q`` list converted); ``None`` for blank and comment lines."""
+    line = line.strip()
+    if not line or line.startswith("#"):
+        return None
+    m = _LINE.match(line)
+    if m is None:
+        raise ValueError(f"not a caselist line: {line[:80]!r}")
+    case = dict(family=m["family"], phase=m["phase"], op=m["op"], tag=m["tag"])
+    body = m["body"]
+    lists = {}
+    for key, value in re.findall(r"(\w+):(\[[^\]]*\])", body):
+        lists[key] = list(ast.literal_eval(value))
+    body = re.sub(r"\w+:\[[^\]]*\],?", "", body)
+    for item in filter(None, body.split(",")):
+        key, _, value = item.partition(":")
+        try:
+            case[key] = int(value)
+        except ValueError:
+            try:
+                case[key] = float(value)
+            except ValueError:
+                case[key] = value
+    case.update(lists)
+    return case
+
+
+def read_caselist(path, limit=None):
+    cases = []
+    with open(path) as fh:
+        for line in fh:
+            case = parse_case(line)
+            if case is not None:
+                cases.append(case)
+                if limit is not None and len(cases) >= limit:
+                    break
+    return cases
+
+
+def unsupported_reason(case):
+    """Why a case cannot be replayed here, or ``None``."""
+    if case["op"] not in ("gdn_attn", "kda_attn"):
+        return f"operator family {case['op']} is not part of this library"
+    if case.get("head_dim_qk") != 128 or case.get("head_dim_v") != 128:
+        return "head_dim must be 128"
+    if case.get("dtype") not in ("bf16", "fp16"):
+        return f"dtype {case.get('dtype')}"
+    H, HV = case["num_heads_qk"], case["num_heads_v"]
+    if HV % H:
+        return "num_heads_v must be a multiple of num_heads_qk"
+    if case["phase"] == "D" and case["op"] == "kda_attn":
+        if case.get("seqlen_q", 1) == 1 and H not in _MEGA_HEADS:
+            return f"the fused KDA decode step supports H in {_MEGA_HEADS}"
+        if case.get("seqlen_q", 1) > 8:
+            return "the KDA verify handles up to 8 draft tokens"
+    if case["phase"] == "P" and case.get("dtype") != "bf16":
+        return "prefill takes bf16 activations"
+    return None
+
+
+def _graph_time_us(fns, reps):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for fn in fns:
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for fn in fns:
+            fn()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        graph.replay()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / reps / len(fns) * 1e3
+
+
+def _eager_time_us(fn, reps):
+    for _ in range(2):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(reps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / reps * 1e3
+
+
+def build_case(case, device="cuda", seed=0, sets=None):
+    """Synthetic inputs for a case: returns ``(fns, info)`` where every ``fn()`` runs the operator once
+    (several closures = rotating slot sets) and ``info`` holds the algorithmic bytes / tokens of one run
+    plus the tensors a checker needs (``info["workload"]``)."""
+    from . import workloads
+    from .decode import (fused_sigmoid_gating_delta_rule_forward_k_last as k_last,
+                         fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed)
+    from .decode.kda import fused_kda_decode_mega_forward as mega
+    from .decode.kda_replayssm_sglang import fused_kda_decode_mtp_dspark as verify_dspark
+    from .prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from .prefill.flashkdapro import flashkda_fwd
+    dtype = torch.bfloat16 if case["dtype"] == "bf16" else torch.float16
+    H, HV = case["num_heads_qk"], case["num_heads_v"]
+    B = case["batch_size"]
+    kda = case["op"] == "kda_attn"
+    lb = case.get("gate_lower_bound")
+    if case["phase"] == "D":
+        T = case.get("seqlen_q", 1)
+        if sets is None:
+            sets = max(1, min(8, (1 << 31) // max(1, B * HV * 65536 * 2)))     # at most 4 GiB of state per case
+        if not kda and T == 1:
+            w = workloads.gdn_decode_packed(B, H=H, HV=HV, pool_slots=B * sets, seed=seed, device=device, dtype=dtype)
+            call = {k: v for k, v in w.items() if not k.startswith("_")}
+            g = torch.Generator().manual_seed(seed + 1)
+            idx = [torch.randperm(B * sets, generator=g)[:B].to(torch.int32).to(device) for _ in range(sets)]
+            idx[0] = call["initial_state_indices"]
+            fns = [lambda i=i: packed(**dict(call, initial_state_indices=i)) for i in idx]
+            return fns, dict(kind="gdn_decode", state_bytes=B * HV * 131072, workload=w)
+        if not kda:
+            g = torch.Generator().manual_seed(seed)
+            rnd = lambda *s: torch.randn(*s, generator=g)
+            pool = (rnd(B + 1, HV, 128, 128) * 0.1).to(device)
+            args = dict(
+                A_log=rnd(HV).to(device), a=rnd(B, T, HV).to(dtype).to(device), dt_bias=rnd(HV).to(dtype).to(device),
+                softplus_beta=1.0, softplus_threshold=20.0,
+                q=rnd(B, T, H, 128).to(dtype).to(device), k=rnd(B, T, H, 128).to(dtype).to(device),
+                v=rnd(B, T, HV, 128).to(dtype).to(device), b=rnd(B, T, HV).to(dtype).to(device),
+                initial_state_source=pool,
+                initial_state_indices=torch.randperm(B + 1, generator=g)[:B].to(torch.int32).to(device),
+                scale=128 ** -0.5, use_qk_l2norm_in_kernel=True, cu_seqlens=None, is_kda=False,
+                disable_state_update=True, intermediate_states_buffer=None, intermediate_state_indices=None,
+                cache_steps_or_num_accept=None, retrieve_parent_token=None)
+            out = torch.empty(B, T, HV, 128, dtype=dtype, device=device)
+            return [lambda: k_last(**args, out=out)], dict(kind="gdn_verify", state_bytes=B * HV * 65536,
+                                                           workload=args, out=out)
+        if T == 1:
+            w = workloads.kda_decode_mega(B, H, seed=seed, device=device, dtype=dtype, slots=B * sets + 2)
+            out = torch.empty(1, B, H, 128, dtype=dtype, device=device)
+            base = w["state_indices"]
+            call = dict(x=w["x"], weight=w["weight"], bias=None, conv_state=w["conv_state"], raw_g=w["raw_g"],
+                        raw_beta=w["raw_beta"], a_log=w["a_log"], dt_bias=w["dt_bias"], state=w["state"], out=out,
+                        lower_bound=lb, output_gate=w["output_gate"], norm_weight=w["norm_weight"], norm_eps=1e-5)
+            idx = [(base + i * B).contiguous() for i in range(sets)]
+            fns = [lambda i=i: mega(**call, state_indices=i) for i in idx]
+            return fns, dict(kind="kda_decode", state_bytes=B * H * 131072, workload=w, out=out)
+        if dtype != torch.bfloat16:
+            raise ValueError("the KDA verify takes bf16 activations")
+        w = workloads.kda_replay_verify(B, H, T, seed=seed, device=device, ring_len=max(8, T), slots=B + 2,
+                                        lower_bound=-5.0 if lb is None else lb, onorm=True, strided=True)
+        out = torch.empty(1, B * T, H, 128, dtype=dtype, device=device)
+        return [lambda: verify_dspark(out=out, **w)], dict(kind="kda_verify", state_bytes=B * H * 65536,
+                                                           workload=w, out=out)
+    lengths = [b - a for a, b in zip(case["cu_seqlens_q"], case["cu_seqlens_q"][1:])]
+    tokens = sum(lengths)
+    if not kda:
+        w = workloads.gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=max(8, len(lengths) + 3), seed=seed,
+                                         device=device, dtype=dtype)
+        call = {k: v for k, v in w.items() if not k.startswith("_")}
+        packed_qkv = call.pop("packed_qkv")
+        a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+        fn = lambda: gdn_prefill_packed_qkv_fwd(packed_qkv, a, b, A, dt, cu, output_final_state=False, **call)
+        return [fn], dict(kind="gdn_prefill", tokens=tokens, workload=w)
+    g = torch.Generator().manual_seed(seed)
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    N = len(lengths)
+    w = dict(q=rnd(tokens, H, 128).to(dtype).to(device), k=rnd(tokens, H, 128).to(dtype).to(device),
+             v=rnd(tokens, H, 128).to(dtype).to(device), g=rnd(tokens, H, 128).to(dtype).to(device),
+             beta=rnd(tokens, H).to(dtype).to(device), A_log=(rnd(H) * 0.5).to(device),
+             dt_bias=(rnd(H, 128) * 0.1).to(device),
+             out=torch.empty(tokens, H, 128, dtype=dtype, device=device), scale=128 ** -0.5,
+             lower_bound=-5.0 if lb is None else lb, initial_state=(rnd(N, H, 128, 128) * 0.1).to(device),
+             final_state=torch.empty(N, H, 128, 128, dtype=torch.float32, device=device),
+             cu_seqlens=torch.tensor(case["cu_seqlens_q"], dtype=torch.int32, device=device))
+    fn = lambda: flashkda_fwd(w["q"], w["k"], w["v"], w["g"], w["beta"], w["A_log"], w["dt_bias"], w["out"],
+                              scale=w["scale"], lower_bound=w["lower_bound"], initial_state=w["initial_state"],
+                              final_state=w["final_state"], cu_seqlens=w["cu_seqlens"])
+    return [fn], dict(kind="kda_prefill", tokens=tokens, workload=w)
+
+
+def replay_case(case, device="cuda", reps=20, seed=0):
+    """Runs and times one case.  Returns a result row (dict)."""
+    row = dict(family=case["family"], phase=case["phase"], batch=case.get("batch_size"),
+               heads=f"{case.get('num_heads_qk')}/{case.get('num_heads_v')}", seqlen_q=case.get("seqlen_q"))
+    reason = unsupported_reason(case)
+    if reason is not None:
+        row.update(status="skipped", reason=reason)
+        return row
+    fns, info = build_case(case, device=device, seed=seed)
+    if case["phase"] == "D":
+        us = _graph_time_us(fns, reps)
+        row.update(status="ok", kind=info["kind"], us=round(us, 2),
+                   state_GBps=round(info["state_bytes"] / us / 1e3, 1))
+    else:
+        us = _eager_time_us(fns[0], max(3, reps // 4))
+        row.update(status="ok", kind=info["kind"], us=round(us, 1), tokens=info["tokens"],
+                   tokens_per_s=round(info["tokens"] / us * 1e6))
+    return row
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("caselist")
+    ap.add_argument("--limit", type=int, default=None)
+    ap.add_argument("--csv", default=None)
+    ap.add_argument("--reps", type=int, default=20)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        print("a GPU is required to replay a caselist", file=sys.stderr)
+        return 2
+    rows = []
+    for case in read_caselist(args.caselist, args.limit):
+        row = replay_case(case, reps=args.reps)
+        rows.append(row)
+        print(row, flush=True)
+        torch.cuda.empty_cache()
+    if args.csv:
+        keys = sorted({k for r in rows for k in r})
+        with open(args.csv, "w", newline="") as fh:
+            writer = csv.DictWriter(fh, fieldnames=keys)
+            writer.writeheader()
+            writer.writerows(rows)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
