@@ -155,20 +155,28 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   float s[R][4];
   // read-once verify: the tile in MFMA A-operand layout, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
   const int r16 = lane & 15, kb = lane >> 4;
+  constexpr bool POOL_BF16 = sizeof(state_t) == 2;      // a bf16 tile is an MFMA operand as it is
   f32x4_t sa[2][4][2];
+  bf16x8_t sb16[2][4];
   uint2 vq[2][4];
   if constexpr (READONCE) {
-    static_assert(!READONCE || (RPW == 32 && sizeof(state_t) == 4), "the read-once verify covers a whole FP32 tile per workgroup");
+    static_assert(!READONCE || RPW == 32, "the read-once verify covers a whole tile per workgroup");
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4;
+        const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * (int)sizeof(state_t);
+        if constexpr (POOL_BF16) {
+          const v4i_t zero = {0, 0, 0, 0};
+          sb16[m][ks] = __builtin_bit_cast(bf16x8_t, have_state ? __builtin_bit_cast(v4i_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                                                      h_tile.rsrc, at, 0, kLoadPolicy)) : zero);
+        } else {
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-          sa[m][ks][hf] = have_state ? __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                           h_tile.rsrc, at + 16 * hf, 0, kLoadPolicy))
-                                     : f32x4_t{0.f, 0.f, 0.f, 0.f};
+          for (int hf = 0; hf < 2; ++hf)
+            sa[m][ks][hf] = have_state ? __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                             h_tile.rsrc, at + 16 * hf, 0, kLoadPolicy))
+                                       : f32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
       }
     // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one)
 #pragma unroll
@@ -254,7 +262,16 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     const float cs[4] = {cmine.x, cmine.y, cmine.z, cmine.w};
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
-      const f32x4_t acc = rows_times_queries(sa[m], wb);
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (POOL_BF16) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          acc = mfma16(sb16[m][ks], wb[ks].hi, acc);
+          acc = mfma16(sb16[m][ks], wb[ks].lo, acc);
+        }
+      } else {
+        acc = rows_times_queries(sa[m], wb);
+      }
       // lane (r16 = token, kb): rows 16 m + 4 kb .. + 3 of S_0 w_token; add the bias terms
       float o[4] = {acc[0], acc[1], acc[2], acc[3]};
 #pragma unroll
@@ -502,12 +519,12 @@ template <typename act_t, bool IS_KDA, bool MTP, typename state_t>
 static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
   const dim3 block(256);
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
-  if constexpr (MTP && sizeof(state_t) == 4) {
+  if constexpr (MTP) {
     // a verify that leaves no trace in memory but o: the state is read once and used once
     const bool read_once = p.disable_state_update && p.T_max <= 4 && p.cache == nullptr && p.cache_indices == nullptr &&
                            p.parents == nullptr && p.stride_h0_indices_seq == 0;
     if (read_once) {
-      hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true>), dim3(tiles, 1), block, 0, stream, p);
+      hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true, state_t>), dim3(tiles, 1), block, 0, stream, p);
       return check_launch("k_last_kernel launch");
     }
   }

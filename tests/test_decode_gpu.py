@@ -201,12 +201,14 @@ def test_mtp_lengths(T, mode, lower_bound):
 @pytest.mark.parametrize("is_kda,lower_bound", [(False, None), (True, None), (True, -5.0)])
 @pytest.mark.parametrize("T", [1, 2, 3, 4])
 @pytest.mark.parametrize("H,HV", [(4, 8), (6, 6)])
-@pytest.mark.parametrize("act_dtype", [torch.bfloat16, torch.float16])
-def test_read_once_verify(is_kda, lower_bound, T, H, HV, act_dtype):
+@pytest.mark.parametrize("act_dtype,state_dtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+                                                   (torch.bfloat16, torch.bfloat16)])
+def test_read_once_verify(is_kda, lower_bound, T, H, HV, act_dtype, state_dtype):
     """A verify that writes neither state nor snapshots (up to four draft tokens, [B, T, ...] inputs, no
     cache) takes the read-once kernel: outputs equal the stepped recurrence, the pool stays bit-identical."""
     forward = _ops()[0]
-    args, backing, lengths, state_ids, _ = make_k_last_case(is_kda, "verify", H=H, HV=HV, T=T, act_dtype=act_dtype)
+    args, backing, lengths, state_ids, _ = make_k_last_case(is_kda, "verify", H=H, HV=HV, T=T, act_dtype=act_dtype,
+                                                            state_dtype=state_dtype)
     B = len(lengths)
     for name in ("q", "k", "v", "a", "b"):
         args[name] = args[name].reshape(B, T, *args[name].shape[2:]).contiguous()
