@@ -199,6 +199,27 @@ int pla_kda_verify_dspark_launch(
     void* stream);
 
 /*
+ * The same verify over paged checkpoints with request-row records (vLLM ReplaySSM).  Replaces
+ * launch_verify_native (src/decode/kda_replayssm/kda_mtp_abi.h:127-137; binding
+ * src/decode/kda_replayssm_vllm/kda_replayssm_vllm.cpp:121-235).  Differences from the ring-mode entry:
+ * records rawv / rawk / gate [R,H,Q,128], beta [R,H,Q] and windows ic_* [R,Q,.,3] are indexed by the
+ * request row; the checkpoint pool has a slot pitch (state_slot_stride elements, slots entries); a slot
+ * <= null_block_id (-1 or 0) is padding (zero output rows, nothing else written); a request whose query
+ * interval is empty, longer than Q, not inside [0, tokens] or whose slot is >= slots is skipped entirely;
+ * no fused output norm.  Q <= 8 here.
+ */
+int pla_kda_replay_verify_native_launch(
+    const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
+    const float* w_q, const float* w_k, const float* w_v,
+    const void* cs_q, const void* cs_k, const void* cs_v,
+    const float* a_log, const float* dt_bias, const float* h0,
+    void* out, void* ic_q, void* ic_k, void* ic_v,
+    void* rawv, void* rawk, float* gate, float* beta,
+    const void* slot_idx, int slot_idx_wide, const void* cu_seqlens, int cu_seqlens_wide,
+    int H, int N, int Q, float scale, float lower_bound, const int64_t* strides,
+    int64_t state_slot_stride, int slots, int tokens, int null_block_id, void* stream);
+
+/*
  * Conv-window rollback of the commit: dst[layer, dst_idx[r], :, :] = src[layer, r, step_idx[r], :, :]
  * for every request r with step_idx[r] >= 0, 0 <= dst_idx[r] < dst_reqs, r < src_reqs and
  * step_idx[r] < src_steps.  Replaces launch_conv_scatter

@@ -44,6 +44,11 @@ struct ReplayVerifyParams {
   int64_t cs[3][3];        // q, k, v conv state: slot, channel, window strides
   int64_t ic[3][4];        // q, k, v scratch windows: row, step, channel, window strides
   const uint16_t* onorm_gate; const float* onorm_weight; int64_t onorm_gate_stride; float onorm_eps;
+  // Paged (vLLM) mode: records and scratch windows are indexed by the request row instead of the slot,
+  // the checkpoint pool has a slot pitch, slots <= null_block_id are padding and malformed query
+  // intervals are skipped (src/decode/kda_replayssm/kda_mtp_verify.cu:721-741).
+  int native, null_block_id, slots, tokens;
+  int64_t state_slot;
 };
 
 __device__ __forceinline__ int64_t index_at(const void* p, int wide, int64_t i) {
@@ -70,9 +75,15 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   const int half = lane >> 5, c = lane & 31;
   const int r16 = lane & 15, kb = lane >> 4;
   const int n = blockIdx.x / p.H, h = blockIdx.x - n * p.H;
-  const int64_t slot = index_at(p.slot_idx, p.slot_wide, n);
+  int64_t slot = index_at(p.slot_idx, p.slot_wide, n);
   const int64_t bos = index_at(p.cu, p.cu_wide, n);
-  const int n_tok = (int)min((int64_t)p.T, index_at(p.cu, p.cu_wide, n + 1) - bos);
+  const int64_t eos = index_at(p.cu, p.cu_wide, n + 1);
+  if (p.native) {
+    if (index_at(p.cu, p.cu_wide, 0) != 0 || bos < 0 || eos <= bos || eos > p.tokens || eos - bos > p.T || slot >= p.slots)
+      return;
+    if (slot <= p.null_block_id) slot = -1;
+  }
+  const int n_tok = (int)min((int64_t)p.T, eos - bos);
   if (bos < 0 || n_tok <= 0) return;
   const int rowbase = 32 * wave;
 
@@ -81,7 +92,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       p.out[((bos + i / 128) * p.H + h) * 128 + (i & 127)] = 0;
     return;
   }
-  const int64_t srow = index_at(p.scratch_idx, p.scratch_wide, n);
+  const int64_t srow = p.native ? n : index_at(p.scratch_idx, p.scratch_wide, n);
 
   __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128], sW[TMAX][128];
   __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
@@ -114,7 +125,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   const float bias = p.dt_bias[ch];
 
   // state tile, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
-  const Tile<float> h_tile(p.h0 + (slot * p.H + h) * 16384);
+  const Tile<float> h_tile(p.h0 + slot * p.state_slot + (int64_t)h * 16384);
   f32x4_t sa[2][4][2];
 #pragma unroll
   for (int m = 0; m < 2; ++m)
@@ -125,7 +136,7 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
         sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
             h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
 
-  const int64_t ring_row = (slot * p.H + h) * p.L;   // first record of this (slot, head)
+  const int64_t ring_row = ((p.native ? n : slot) * p.H + h) * p.L;   // first record of this (slot or request, head)
   if (qk_side) {
     float cq[3] = {bf(ta[0]), bf(ta[1]), bf(ta[2])}, ck[3] = {bf(tb[0]), bf(tb[1]), bf(tb[2])};
 #pragma unroll
@@ -280,6 +291,38 @@ static bool aligned_at(const void* ptr, size_t a) { return (reinterpret_cast<uin
 
 }  // namespace pla
 
+namespace pla {
+// Shared by the ring-mode and the paged entry points.
+static int launch_replay_verify(ReplayVerifyParams& p, const int64_t* strides, int t_loop, hipStream_t s) {
+  PLA_REQUIRE(p.H > 0 && p.N > 0 && t_loop > 0, "verify requires H > 0, N > 0 and at least one token per request");
+  PLA_REQUIRE(t_loop <= 8, "the gfx950 verify handles up to 8 draft tokens per request, got %d", t_loop);
+  PLA_REQUIRE(p.L >= t_loop, "record rings shorter than the draft window");
+  PLA_REQUIRE((int64_t)p.N * p.H <= 0x7fffffffLL, "N * H exceeds the grid limit");
+  PLA_REQUIRE(aligned_at(p.h0, 16) && p.state_slot % 4 == 0 && aligned_at(p.w_q, 16) && aligned_at(p.w_k, 16) &&
+              aligned_at(p.w_v, 16) && aligned_at(p.out, 8), "state, conv weights and out require vector alignment");
+  const bool onorm = p.onorm_gate != nullptr;
+  PLA_REQUIRE(!onorm || (p.onorm_weight != nullptr && aligned_at(p.onorm_weight, 16) && aligned_at(p.onorm_gate, 8) &&
+                         p.onorm_gate_stride % 4 == 0 && p.onorm_eps >= 0.f),
+              "fused output norm requires an aligned gate (token stride a multiple of 4), a weight and eps >= 0");
+  for (int i = 0; i < 26; ++i) PLA_REQUIRE(strides[i] > 0, "stride %d must be positive", i);
+  p.T = t_loop;
+  p.sx_q = strides[0]; p.sx_k = strides[1]; p.sx_v = strides[2]; p.sg = strides[3]; p.sbeta = strides[4];
+  for (int t = 0; t < 3; ++t)
+    for (int j = 0; j < 3; ++j) p.cs[t][j] = strides[5 + 3 * t + j];
+  for (int t = 0; t < 3; ++t)
+    for (int j = 0; j < 4; ++j) p.ic[t][j] = strides[14 + 4 * t + j];
+  const dim3 grid((unsigned)p.N * (unsigned)p.H), block(256);
+  if (t_loop <= 4) {
+    if (onorm) kda_verify_dspark_kernel<4, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<4, false><<<grid, block, 0, s>>>(p);
+  } else {
+    if (onorm) kda_verify_dspark_kernel<8, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<8, false><<<grid, block, 0, s>>>(p);
+  }
+  return check_launch("kda_verify_dspark_kernel");
+}
+}  // namespace pla
+
 extern "C" int pla_kda_verify_dspark_launch(
     const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
     const float* w_q, const float* w_k, const float* w_v,
@@ -297,18 +340,7 @@ extern "C" int pla_kda_verify_dspark_launch(
   PLA_REQUIRE(x_q && x_k && x_v && g_in && beta_in && w_q && w_k && w_v && cs_q && cs_k && cs_v && a_log && dt_bias && h0 &&
               out && ic_q && ic_k && ic_v && ring_rawv && ring_rawk && ring_g && ring_beta && slot_idx && scratch_idx &&
               cu_seqlens && strides, "null tensor pointer");
-  PLA_REQUIRE(H > 0 && N > 0 && t_loop > 0, "verify requires H > 0, N > 0 and at least one token per request");
-  PLA_REQUIRE(t_loop <= 8, "the gfx950 verify handles up to 8 draft tokens per request, got %d", t_loop);
-  PLA_REQUIRE(ring_len >= t_loop, "ring shorter than the draft window");
-  PLA_REQUIRE((int64_t)N * H <= 0x7fffffffLL, "N * H exceeds the grid limit");
-  PLA_REQUIRE(aligned_at(h0, 16) && aligned_at(w_q, 16) && aligned_at(w_k, 16) && aligned_at(w_v, 16) && aligned_at(out, 8),
-              "state, conv weights and out require vector alignment");
-  const bool onorm = onorm_gate != nullptr;
-  PLA_REQUIRE(!onorm || (onorm_weight != nullptr && aligned_at(onorm_weight, 16) && aligned_at(onorm_gate, 8) &&
-                         onorm_gate_stride % 4 == 0 && onorm_eps >= 0.f),
-              "fused output norm requires an aligned gate (token stride a multiple of 4), a weight and eps >= 0");
-  for (int i = 0; i < 26; ++i) PLA_REQUIRE(strides[i] > 0, "stride %d must be positive", i);
-  ReplayVerifyParams p;
+  ReplayVerifyParams p{};
   p.x_q = (const uint16_t*)x_q; p.x_k = (const uint16_t*)x_k; p.x_v = (const uint16_t*)x_v;
   p.g = (const uint16_t*)g_in; p.beta = (const uint16_t*)beta_in;
   p.w_q = w_q; p.w_k = w_k; p.w_v = w_v;
@@ -318,24 +350,45 @@ extern "C" int pla_kda_verify_dspark_launch(
   p.ring_rawv = (uint16_t*)ring_rawv; p.ring_rawk = (uint16_t*)ring_rawk; p.ring_g = ring_g; p.ring_beta = ring_beta;
   p.slot_idx = slot_idx; p.scratch_idx = scratch_idx; p.cu = cu_seqlens;
   p.slot_wide = slot_idx_wide; p.scratch_wide = scratch_idx_wide; p.cu_wide = cu_seqlens_wide;
-  p.H = H; p.N = N; p.T = t_loop; p.L = ring_len; p.scale = scale; p.lower_bound = lower_bound;
-  p.sx_q = strides[0]; p.sx_k = strides[1]; p.sx_v = strides[2]; p.sg = strides[3]; p.sbeta = strides[4];
-  for (int t = 0; t < 3; ++t)
-    for (int j = 0; j < 3; ++j) p.cs[t][j] = strides[5 + 3 * t + j];
-  for (int t = 0; t < 3; ++t)
-    for (int j = 0; j < 4; ++j) p.ic[t][j] = strides[14 + 4 * t + j];
+  p.H = H; p.N = N; p.L = ring_len; p.scale = scale; p.lower_bound = lower_bound;
   p.onorm_gate = (const uint16_t*)onorm_gate; p.onorm_weight = onorm_weight;
   p.onorm_gate_stride = onorm_gate_stride; p.onorm_eps = onorm_eps;
-  const dim3 grid((unsigned)N * (unsigned)H), block(256);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (t_loop <= 4) {
-    if (onorm) kda_verify_dspark_kernel<4, true><<<grid, block, 0, s>>>(p);
-    else kda_verify_dspark_kernel<4, false><<<grid, block, 0, s>>>(p);
-  } else {
-    if (onorm) kda_verify_dspark_kernel<8, true><<<grid, block, 0, s>>>(p);
-    else kda_verify_dspark_kernel<8, false><<<grid, block, 0, s>>>(p);
-  }
-  return check_launch("kda_verify_dspark_kernel");
+  p.native = 0; p.null_block_id = -1; p.slots = 0; p.tokens = 0; p.state_slot = (int64_t)H * 16384;
+  return launch_replay_verify(p, strides, t_loop, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int pla_kda_replay_verify_native_launch(
+    const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
+    const float* w_q, const float* w_k, const float* w_v,
+    const void* cs_q, const void* cs_k, const void* cs_v,
+    const float* a_log, const float* dt_bias, const float* h0,
+    void* out, void* ic_q, void* ic_k, void* ic_v,
+    void* rawv, void* rawk, float* gate, float* beta,
+    const void* slot_idx, int slot_idx_wide, const void* cu_seqlens, int cu_seqlens_wide,
+    int H, int N, int Q, float scale, float lower_bound, const int64_t* strides,
+    int64_t state_slot_stride, int slots, int tokens, int null_block_id, void* stream) {
+  using namespace pla;
+  PLA_REQUIRE(x_q && x_k && x_v && g_in && beta_in && w_q && w_k && w_v && cs_q && cs_k && cs_v && a_log && dt_bias && h0 &&
+              out && ic_q && ic_k && ic_v && rawv && rawk && gate && beta && slot_idx && cu_seqlens && strides,
+              "null tensor pointer");
+  PLA_REQUIRE(null_block_id == -1 || null_block_id == 0, "null_block_id must be -1 or 0");
+  PLA_REQUIRE(slots > 0 && tokens >= 0 && state_slot_stride >= (int64_t)H * 16384,
+              "paged state requires slots > 0 and a slot pitch of at least H * 128 * 128");
+  if (N == 0) return 0;
+  ReplayVerifyParams p{};
+  p.x_q = (const uint16_t*)x_q; p.x_k = (const uint16_t*)x_k; p.x_v = (const uint16_t*)x_v;
+  p.g = (const uint16_t*)g_in; p.beta = (const uint16_t*)beta_in;
+  p.w_q = w_q; p.w_k = w_k; p.w_v = w_v;
+  p.cs_q = (const uint16_t*)cs_q; p.cs_k = (const uint16_t*)cs_k; p.cs_v = (const uint16_t*)cs_v;
+  p.a_log = a_log; p.dt_bias = dt_bias; p.h0 = const_cast<float*>(h0);
+  p.out = (uint16_t*)out; p.ic_q = (uint16_t*)ic_q; p.ic_k = (uint16_t*)ic_k; p.ic_v = (uint16_t*)ic_v;
+  p.ring_rawv = (uint16_t*)rawv; p.ring_rawk = (uint16_t*)rawk; p.ring_g = gate; p.ring_beta = beta;
+  p.slot_idx = slot_idx; p.scratch_idx = slot_idx; p.cu = cu_seqlens;
+  p.slot_wide = slot_idx_wide; p.scratch_wide = slot_idx_wide; p.cu_wide = cu_seqlens_wide;
+  p.H = H; p.N = N; p.L = Q; p.scale = scale; p.lower_bound = lower_bound;
+  p.onorm_gate = nullptr; p.onorm_weight = nullptr; p.onorm_gate_stride = 0; p.onorm_eps = 0.f;
+  p.native = 1; p.null_block_id = null_block_id; p.slots = slots; p.tokens = tokens; p.state_slot = state_slot_stride;
+  return launch_replay_verify(p, strides, Q, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int pla_conv_window_scatter_launch(

@@ -1,0 +1,182 @@
+"""Request-row KDA replay for a vLLM-style runner (``pla.decode.kda_replayssm_vllm``).
+
+``kda_replay_verify`` (reference pla/decode/kda_replayssm_vllm/__init__.py:46-76, binding
+src/decode/kda_replayssm_vllm/kda_replayssm_vllm.cpp:121-235): verify of up to ``Q`` draft tokens per
+request against a paged FP32 checkpoint.  The conv history and the checkpoint are read-only; the
+per-token records (post-conv k, v in bf16; log-decay, beta in FP32) and the conv window after every
+token are written to the request's row of ``records``; only real query intervals are written.
+The draft window is limited to 8 tokens here (the reference allows 32).
+"""
+
+import ctypes
+import os
+from dataclasses import dataclass
+from numbers import Integral, Real
+from typing import Optional
+
+import torch
+
+from ... import _lib
+
+__all__ = ["KDAReplayRecords", "kda_replay_verify"]
+
+_BYPASS = os.environ.get("PLA_BYPASS_EXEC", "0") == "1"   # read once, like src/bypass_exec.h:44-50
+D = 128
+
+
+@dataclass(frozen=True)
+class KDAReplayRecords:
+    """Per-request-row records: rawv, rawk [R,H,Q,128] bf16, g [R,H,Q,128] and beta [R,H,Q] float32,
+    conv [R,Q,3*H*128,3] bf16 (the window after each token, q | k | v channels)."""
+    rawv: torch.Tensor
+    rawk: torch.Tensor
+    g: torch.Tensor
+    beta: torch.Tensor
+    conv: torch.Tensor
+
+    @classmethod
+    def allocate(cls, max_num_reqs, num_heads, spec_query_len, device):
+        if max_num_reqs < 0 or num_heads < 1 or not 1 <= spec_query_len <= 32:
+            raise ValueError("records require R >= 0, H > 0 and Q in [1, 32]")
+        shape = (max_num_reqs, num_heads, spec_query_len, D)
+        return cls(torch.empty(shape, dtype=torch.bfloat16, device=device),
+                   torch.empty(shape, dtype=torch.bfloat16, device=device),
+                   torch.empty(shape, dtype=torch.float32, device=device),
+                   torch.empty(shape[:-1], dtype=torch.float32, device=device),
+                   torch.empty((max_num_reqs, spec_query_len, 3 * num_heads * D, 3),
+                               dtype=torch.bfloat16, device=device))
+
+
+def _need(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _index(t, ref):
+    _need(t.device == ref.device and t.dim() == 1 and t.dtype in (torch.int32, torch.int64),
+          "indices must be int32/int64 vectors")
+    t = t.contiguous()
+    return t, int(t.dtype == torch.int64)
+
+
+def _paged_cache(conv, state, layout, H, slots):
+    """Checks of the paged conv / checkpoint pair; returns the conv cache in [slots, channels, history] view
+    (src/decode/kda_replayssm_vllm/kda_replayssm_vllm.cpp:57-82)."""
+    _need(state.is_cuda and H > 0 and slots > 0, "paged state requires a GPU tensor, H > 0, slots > 0")
+    _need(state.dtype == torch.float32 and tuple(state.shape) == (slots, H, D, D) and state.stride(3) == 1
+          and state.stride(2) == D and state.stride(1) == D * D and state.stride(0) >= H * D * D
+          and state.stride(0) % 4 == 0 and state.data_ptr() % 16 == 0,
+          "state must be float4-aligned fp32 [slots,H,128,128] with contiguous pages")
+    _need(layout in ("DS", "SD"), "conv_state_layout must be DS or SD")
+    _need(conv.dim() == 3 and conv.size(0) == slots and conv.dtype == torch.bfloat16 and conv.device == state.device,
+          "conv must be bf16 with three dimensions")
+    ds = conv if layout == "DS" else conv.transpose(1, 2)
+    _need(ds.size(1) == 3 * H * D and ds.size(2) >= 3,
+          "conv must contain 3*H*128 channels and at least three history items")
+    _need((ds.stride(2) == 1 and ds.stride(1) >= ds.size(2)) or (ds.stride(1) == 1 and ds.stride(2) >= ds.size(1)),
+          "conv channel/history dimensions must not overlap")
+    _need(ds.stride(0) >= (ds.size(1) - 1) * ds.stride(1) + (ds.size(2) - 1) * ds.stride(2) + 1,
+          "conv pages must not overlap")
+    return ds
+
+
+def _check_records(records, ref, H, Q, R):
+    _need(1 <= Q <= 32 and R >= 0, "records require Q in [1,32] and R >= 0")
+    for t, dtype, shape in ((records.rawv, torch.bfloat16, (R, H, Q, D)), (records.rawk, torch.bfloat16, (R, H, Q, D)),
+                            (records.g, torch.float32, (R, H, Q, D)), (records.beta, torch.float32, (R, H, Q)),
+                            (records.conv, torch.bfloat16, (R, Q, 3 * H * D, 3))):
+        _need(t.device == ref.device and t.dtype == dtype and tuple(t.shape) == shape and t.is_contiguous(),
+              "invalid replay tensor shape/dtype/contiguity")
+    for t in (records.rawv, records.rawk, records.g, records.beta):
+        _need(t.data_ptr() % 16 == 0, "replay records must be 16-byte aligned")
+
+
+def _span(t):
+    if t.numel() == 0:
+        return t.data_ptr(), t.data_ptr()
+    extent = 1 + sum((t.size(d) - 1) * t.stride(d) for d in range(t.dim()))
+    return t.data_ptr(), t.data_ptr() + extent * t.element_size()
+
+
+def _disjoint(writes, reads):
+    """Conservative byte-span check: written tensors alias neither each other nor anything read."""
+    def overlap(a, b):
+        (a0, a1), (b0, b1) = _span(a), _span(b)
+        return a0 < b1 and b0 < a1
+    for i, w in enumerate(writes):
+        _need(not any(overlap(w, other) for other in writes[:i]), "replay writes must not alias")
+        _need(not any(overlap(w, r) for r in reads), "replay writes must not alias inputs/cache")
+
+
+def kda_replay_verify(*, mixed_qkv, raw_g, raw_beta, conv_weight, conv_state, checkpoint_state, A_log, dt_bias,
+                      lower_bound, records, query_start_loc, state_indices, conv_state_layout,
+                      out: Optional[torch.Tensor] = None, scale=None, null_block_id=0):
+    """Read a paged checkpoint and write only real query intervals and records.
+
+    mixed_qkv [T, 3*H*128], raw_g [T, H*128], raw_beta [T, H]: bf16 projection views (positive token stride,
+    contiguous channels); conv_weight float32 [3*H*128, 4]; conv_state bf16 paged, ``DS`` = [slots, channels,
+    history] or ``SD`` = [slots, history, channels], only its first three history items are read;
+    checkpoint_state float32 [slots, H, 128, 128] with a page pitch; query_start_loc [N+1] and state_indices [N]
+    int32 or int64.  A slot <= null_block_id yields zero output rows; an empty, overlong or out-of-range
+    query interval is skipped.  Returns ``out`` [T, H*128] bf16 (rows outside query intervals are not written).
+    """
+    if not isinstance(lower_bound, Real) or (scale is not None and not isinstance(scale, Real)):
+        raise TypeError("scale and lower_bound must be host numeric scalars")
+    if not isinstance(null_block_id, Integral):
+        raise TypeError("null_block_id must be a host integer")
+    state = checkpoint_state
+    _need(state.dim() == 4 and records.rawv.dim() == 4, "invalid state/records rank")
+    H, slots, Q, R = state.size(1), state.size(0), records.rawv.size(2), records.rawv.size(0)
+    if out is None:
+        out = torch.empty(mixed_qkv.size(0), H * D, dtype=torch.bfloat16, device=mixed_qkv.device)
+    if _BYPASS:
+        return out
+    _need(null_block_id in (-1, 0), "null_block_id must be -1 or 0")
+    cs = _paged_cache(conv_state, state, conv_state_layout, H, slots)
+    _check_records(records, state, H, Q, R)
+    for t in (mixed_qkv, raw_g, raw_beta, conv_weight, A_log, dt_bias, out, query_start_loc, state_indices):
+        _need(t.device == state.device, "replay tensors must share one device")
+    x = mixed_qkv
+    _need(x.dim() == 2 and x.size(1) == 3 * H * D and x.stride(1) == 1 and x.stride(0) >= 3 * H * D
+          and x.dtype == torch.bfloat16, "mixed_qkv must be bf16 [T,3*H*128] with contiguous channels")
+    T = x.size(0)
+    for t, channels in ((raw_g, H * D), (raw_beta, H)):
+        _need(tuple(t.shape) == (T, channels) and t.stride(1) == 1 and t.stride(0) >= channels
+              and t.dtype == torch.bfloat16, "gate/beta must be bf16 projection views")
+    _need(conv_weight.dtype == torch.float32 and tuple(conv_weight.shape) == (3 * H * D, 4) and conv_weight.is_contiguous(),
+          "invalid replay tensor shape/dtype/contiguity")
+    _need(A_log.numel() == H and dt_bias.numel() == H * D and A_log.is_contiguous() and dt_bias.is_contiguous()
+          and A_log.dtype == torch.float32 and dt_bias.dtype == torch.float32, "gate weights must be contiguous fp32")
+    _need(out.dtype == torch.bfloat16 and tuple(out.shape) == (T, H * D) and out.is_contiguous(),
+          "invalid replay tensor shape/dtype/contiguity")
+    scale = D ** -0.5 if scale is None else float(scale)
+    _need(scale == scale and abs(scale) != float("inf") and lower_bound == lower_bound
+          and abs(lower_bound) != float("inf") and lower_bound < 0, "scale/lower_bound must be finite fp32; bound < 0")
+    cu, cu_wide = _index(query_start_loc, state)
+    src, src_wide = _index(state_indices, state)
+    N = src.numel()
+    _need(cu.numel() == N + 1 and N <= R, "query index count exceeds record capacity")
+    _disjoint([out, records.rawv, records.rawk, records.g, records.beta, records.conv],
+              [x, raw_g, raw_beta, conv_weight, conv_state, state, A_log, dt_bias, cu, src])
+    if Q > 8:
+        raise NotImplementedError(f"the gfx950 replay verify handles draft windows of up to 8 tokens, got Q={Q}")
+    if N == 0:
+        return out
+    windows = records.conv
+    strides = ([x.stride(0)] * 3 + [raw_g.stride(0), raw_beta.stride(0)] + list(cs.stride()) * 3
+               + list(windows.stride()) * 3)
+    c_strides = (ctypes.c_int64 * 26)(*strides)
+    cb = H * D * 2                                           # bytes of one q / k / v channel segment
+    xp, cp, wp, wtp = x.data_ptr(), conv_state.data_ptr(), windows.data_ptr(), conv_weight.data_ptr()
+    with torch.cuda.device(state.device):
+        _lib.call(
+            "pla_kda_replay_verify_native_launch", xp, xp + cb, xp + 2 * cb, raw_g.data_ptr(), raw_beta.data_ptr(),
+            wtp, wtp + H * D * 16, wtp + 2 * H * D * 16,
+            cp, cp + cb * cs.stride(1), cp + 2 * cb * cs.stride(1),
+            A_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(), out.data_ptr(),
+            wp, wp + cb * windows.stride(2), wp + 2 * cb * windows.stride(2),
+            records.rawv.data_ptr(), records.rawk.data_ptr(), records.g.data_ptr(), records.beta.data_ptr(),
+            src.data_ptr(), src_wide, cu.data_ptr(), cu_wide, H, N, Q, scale, float(lower_bound),
+            ctypes.cast(c_strides, ctypes.c_void_p), state.stride(0), slots, T, int(null_block_id),
+            _lib.current_stream(state.device))
+    return out

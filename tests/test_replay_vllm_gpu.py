@@ -1,0 +1,176 @@
+"""GPU parity of the request-row (vLLM-style) KDA replay verify against the CPU oracle.
+
+The cases follow the reference's own test of this entry (tests/test_kda_replayssm_vllm.py:45-96, 214-262):
+paged conv / checkpoint caches with a poisoned page layout, projection views with a token stride and a
+storage offset, sentinel-filled records, ragged query lengths including zero, null slots, DS and SD conv
+layouts, int32 and int64 index vectors with a stride.  Tolerances: bf16 output atol = rtol = 2e-2, bf16
+records rtol 8e-3, FP32 records rtol 1e-4; windows, untouched record rows, the persistent pages and the
+input storage bit-exact.
+"""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from oracle import verify_dspark_reference
+from pla_amd.decode.kda_replayssm_vllm import KDAReplayRecords, kda_replay_verify
+
+pytestmark = pytest.mark.gpu
+D = 128
+
+
+def pages(slots, heads, q, layout, gen, padding=256, history=None, conv_offset=0):
+    """Paged cache: every page holds a conv history (DS = [channels, history], SD = [history, channels])
+    followed by the FP32 checkpoint; the rest of the page is poison."""
+    c = 3 * heads * D
+    history = q + 2 if history is None else history
+    conv_shape = (c, history) if layout == "DS" else (history, c)
+    conv_bytes = c * history * 2
+    state_offset = ((conv_offset + conv_bytes + 15) // 16) * 16
+    page_bytes = ((state_offset + heads * D * D * 4 + padding + 15) // 16) * 16
+    raw = torch.full((slots * page_bytes,), 0x5A, dtype=torch.uint8, device="cuda")
+    conv = raw.view(torch.bfloat16).as_strided((slots, *conv_shape), (page_bytes // 2, *torch.empty(conv_shape).stride()),
+                                               conv_offset // 2)
+    state = raw.view(torch.float32).as_strided((slots, heads, D, D), (page_bytes // 4, D * D, D, 1), state_offset // 4)
+    conv.copy_((torch.randn(conv.shape, generator=gen) * 0.2).to(torch.bfloat16))
+    state.copy_(torch.randn(state.shape, generator=gen) * 0.01)
+    return SimpleNamespace(raw=raw, conv=conv, state=state, heads=heads, q=q, layout=layout)
+
+
+def inputs(heads, capacity, gen, offset=2):
+    c = heads * D
+    storage = (torch.randn(offset + capacity + 2, 4 * c + heads + 3, generator=gen) * 0.4).to(torch.bfloat16).cuda()
+    rows = storage[offset:offset + capacity]
+    return dict(mixed_qkv=rows[:, :3 * c], raw_g=rows[:, 3 * c:4 * c], raw_beta=rows[:, 4 * c:4 * c + heads],
+                storage=storage, conv_weight=(torch.randn(3 * c, 4, generator=gen) * 0.2).cuda(),
+                A_log=(torch.randn(heads, generator=gen) * 0.1).cuda(),
+                dt_bias=(torch.randn(c, generator=gen) * 0.2).cuda(), lower_bound=-5.0)
+
+
+def records_filled(rows, heads, q):
+    rec = KDAReplayRecords.allocate(rows, heads, q, "cuda")
+    for name in ("rawv", "rawk", "g", "beta", "conv"):
+        getattr(rec, name).fill_(-7)
+    return rec
+
+
+def vector(values, dtype=torch.int32, strided=False):
+    t = torch.tensor(values, dtype=dtype, device="cuda")
+    if strided:
+        storage = torch.full((len(values) * 2 + 1,), -99, dtype=dtype, device="cuda")
+        storage[1::2] = t
+        t = storage[1::2]
+    return t
+
+
+def oracle(layer, x, offsets, slots, rec, out, null_block_id):
+    """The ring-mode oracle applied per request: records and windows land in the request's row."""
+    h, c = layer.heads, layer.heads * D
+    conv = (layer.conv if layer.layout == "DS" else layer.conv.transpose(-1, -2)).cpu()
+    state = layer.state.cpu()
+    want = {k: getattr(rec, k).cpu().clone() for k in ("rawv", "rawk", "g", "beta", "conv")}
+    want_out = out.cpu().clone().double()
+    xc = {k: v.cpu() for k, v in x.items() if torch.is_tensor(v)}
+    for row, slot in enumerate(slots):
+        begin, end = offsets[row:row + 2]
+        n = end - begin
+        if n == 0:
+            continue
+        if slot <= null_block_id:
+            want_out[begin:end] = 0
+            continue
+        qkv = xc["mixed_qkv"][begin:end].split(c, -1)
+        ws = xc["conv_weight"].split(c)
+        css = conv[slot].split(c)
+        L = want["rawv"].shape[2]
+        rings = tuple(torch.zeros(1, *want[k].shape[1:], dtype=want[k].dtype) for k in ("rawv", "rawk", "g", "beta"))
+        wins = tuple(torch.zeros(1, L, c, 3, dtype=torch.bfloat16) for _ in range(3))
+        ref = verify_dspark_reference(
+            x_q=qkv[0].reshape(1, n, h, D), x_k=qkv[1].reshape(1, n, h, D), x_v=qkv[2].reshape(1, n, h, D),
+            g=xc["raw_g"][begin:end].reshape(1, n, h, D), beta=xc["raw_beta"][begin:end][None],
+            w_q=ws[0], w_k=ws[1], w_v=ws[2], cs_q=css[0][None, :, :3], cs_k=css[1][None, :, :3], cs_v=css[2][None, :, :3],
+            A_log=xc["A_log"], dt_bias=xc["dt_bias"], recurrent_state=state[slot:slot + 1],
+            ssm_state_indices=torch.tensor([0]), intermediate_state_indices=torch.tensor([0]),
+            cu_seqlens=torch.tensor([0, n]), lower_bound=x["lower_bound"], scale=D ** -0.5, rings=rings, windows=wins)
+        want_out[begin:end] = ref["out"].reshape(n, c)
+        for k, name in (("rawv", "ring_rawv"), ("rawk", "ring_rawk"), ("g", "ring_g"), ("beta", "ring_beta")):
+            want[k][row, :, :n] = ref[name][0, :, :n]
+        want["conv"][row, :n] = torch.cat([ref["ic_" + name][0, :n] for name in ("q", "k", "v")], dim=1)
+    return want_out, want
+
+
+@pytest.mark.parametrize("layout", ["DS", "SD"])
+@pytest.mark.parametrize("q,heads", [(1, 1), (3, 2), (5, 4), (8, 2)])
+@pytest.mark.parametrize("index_dtype,null_block_id", [(torch.int32, 0), (torch.int64, -1)])
+def test_replay_verify_paged(layout, q, heads, index_dtype, null_block_id):
+    gen = torch.Generator().manual_seed(41 + q + heads)
+    lengths = [q, max(q - 2, 0), 0, 1, 1]
+    offsets = [0]
+    for n in lengths:
+        offsets.append(offsets[-1] + n)
+    slots = [7, 2, 5, 0, -1]
+    layer = pages(12, heads, q, layout, gen)
+    rec = records_filled(len(slots), heads, q)
+    x = inputs(heads, len(slots) * q + 3, gen)
+    out = torch.full((x["mixed_qkv"].shape[0], heads * D), -11, dtype=torch.bfloat16, device="cuda")
+    want_out, want = oracle(layer, x, offsets, slots, rec, out, null_block_id)
+    before, storage_before = layer.raw.clone(), x["storage"].clone()
+    args = {k: v for k, v in x.items() if k != "storage"}
+    got = kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=rec,
+                            query_start_loc=vector(offsets, index_dtype, True), state_indices=vector(slots, index_dtype, True),
+                            conv_state_layout=layout, out=out, null_block_id=null_block_id)
+    torch.cuda.synchronize()
+    assert got.data_ptr() == out.data_ptr()
+    T = offsets[-1]
+    torch.testing.assert_close(out[:T].cpu().double(), want_out[:T], atol=2e-2, rtol=2e-2)
+    assert bool((out[T:] == -11).all())                                              # rows outside query intervals
+    for name, tol in (("rawv", 8e-3), ("rawk", 8e-3), ("g", 1e-4), ("beta", 1e-4)):
+        torch.testing.assert_close(getattr(rec, name).cpu().float(), want[name].float(), atol=1e-6, rtol=tol)
+        untouched = want[name] == -7
+        assert torch.equal(getattr(rec, name).cpu()[untouched], want[name][untouched])
+    assert torch.equal(rec.conv.cpu(), want["conv"])
+    assert torch.equal(layer.raw, before) and torch.equal(x["storage"], storage_before)
+    for b, n in enumerate(lengths):
+        if slots[b] <= null_block_id or n == 0:
+            assert bool((rec.g[b] == -7).all()) and bool((rec.conv[b] == -7).all())
+    default_out = kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=rec,
+                                    query_start_loc=vector(offsets), state_indices=vector(slots),
+                                    conv_state_layout=layout, null_block_id=null_block_id)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(default_out[:T].cpu().double(), want_out[:T], atol=2e-2, rtol=2e-2)
+
+
+def test_replay_verify_skips_malformed_intervals_and_rejects_bad_arguments():
+    gen = torch.Generator().manual_seed(5)
+    q, heads = 3, 2
+    layer = pages(6, heads, q, "DS", gen)
+    rec = records_filled(4, heads, q)
+    x = inputs(heads, 16, gen)
+    args = {k: v for k, v in x.items() if k != "storage"}
+    out = torch.full((16, heads * D), -11, dtype=torch.bfloat16, device="cuda")
+    # request 1 is longer than Q, request 2 names a slot beyond the pool: both are skipped entirely
+    offsets, slots = [0, 2, 7, 9, 10], [3, 1, 99, 2]
+    kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=rec,
+                      query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS", out=out)
+    torch.cuda.synchronize()
+    assert bool((out[2:9] == -11).all()) and bool((rec.g[1:3] == -7).all())
+    assert not bool((out[0:2] == -11).any()) and not bool((out[9:10] == -11).any())
+    with pytest.raises(RuntimeError, match="null_block_id must be -1 or 0"):
+        kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=rec,
+                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS",
+                          null_block_id=3)
+    with pytest.raises(RuntimeError, match="DS or SD"):
+        kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=rec,
+                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="XX")
+    with pytest.raises(TypeError):
+        kda_replay_verify(**dict(args, lower_bound=torch.tensor(-5.0)), conv_state=layer.conv, checkpoint_state=layer.state,
+                          records=rec, query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS")
+    big = records_filled(8, heads, q)
+    with pytest.raises(RuntimeError, match="must not alias"):
+        kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=big,
+                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS",
+                          out=big.rawv.view(-1)[:16 * heads * D].view(16, heads * D))
+    wide = records_filled(4, heads, 9)
+    with pytest.raises(NotImplementedError, match="up to 8 tokens"):
+        kda_replay_verify(**args, conv_state=pages(6, heads, 9, "DS", gen).conv, checkpoint_state=layer.state, records=wide,
+                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS")
