@@ -119,13 +119,31 @@ int pla_k_last_launch(
  *   rawv  [slots,HV,L,128] act dtype
  *   gk    [slots,HV,L,128] float32 log-decay;  beta [slots,HV,L] float32
  *   slot_idx, accept_lens [B] int32.  slot <= null_block_id or accept_len <= 0 => untouched.
+ *   track_idx, track_step [B] int32 or both NULL: the state after step track_step[n] (0-based) is also
+ *         stored to slot track_idx[n] when that slot is > null_block_id.
  */
 int pla_kda_fold_launch(
     float* h0, const void* rawv, const void* rawk, const float* gk, const float* beta,
     const int32_t* slot_idx, const int32_t* accept_lens,
+    const int32_t* track_idx, const int32_t* track_step,
     int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
     int64_t gk_slot_stride, int64_t beta_slot_stride,
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
+
+/*
+ * The fold of one layer driven by a commit plan over paged checkpoints with request-row records (vLLM
+ * ReplaySSM).  Replaces launch_fold_native (src/decode/kda_replayssm/kda_mtp_abi.h:139-144) for one layer:
+ * request n replays lengths[n] tokens of records row n from state[source[n]] and stores the result to
+ * state[final_indices[n]]; when boundary_lengths[n] > 0 the state after that many tokens also goes to
+ * state[boundary_indices[n]].  Destinations may equal the source slot.  Requests with lengths[n] <= 0 or a
+ * source / final slot outside (null_block_id, slots) are skipped.  Records: rawv, rawk [R,H,Q,128] bf16,
+ * gate [R,H,Q,128], beta [R,H,Q] float32, dense.
+ */
+int pla_kda_fold_native_launch(
+    float* state, int64_t state_slot_stride, const void* rawv, const void* rawk, const float* gate, const float* beta,
+    const int32_t* source, const int32_t* lengths, const int32_t* final_indices,
+    const int32_t* boundary_indices, const int32_t* boundary_lengths,
+    int batch, int heads, int Q, int slots, int null_block_id, void* stream);
 
 /*
  * Fused KDA decode step (one token per request): width-4 causal conv1d update + SiLU on the packed

@@ -454,6 +454,11 @@ struct FoldParams {
   const int32_t* slot_idx; const int32_t* accept_lens;
   int64_t h0_slot_stride, rawv_slot_stride, rawk_slot_stride, gk_slot_stride, beta_slot_stride;
   int B, H, HV, L, null_block_id;
+  // Optional: the folded state goes to final_idx[n] instead of back to the source slot; the state after
+  // step track_step[n] (or after track_step[n] tokens when track_is_len) is also stored to track_idx[n];
+  // records indexed by the request row instead of the slot; slots > 0 bounds every slot id.
+  const int32_t* final_idx; const int32_t* track_idx; const int32_t* track_step;
+  int track_is_len, records_by_request, slots;
 };
 
 template <typename act_t, int RPW>
@@ -470,17 +475,25 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
 
   const int slot = p.slot_idx[i_n];
   int n_acc = p.accept_lens[i_n];
-  if (slot <= p.null_block_id || n_acc <= 0) return;
+  const int final_slot = p.final_idx != nullptr ? p.final_idx[i_n] : slot;
+  const int track_slot = p.track_idx != nullptr ? p.track_idx[i_n] : p.null_block_id;
+  const int track_at = p.track_idx != nullptr ? p.track_step[i_n] - (p.track_is_len ? 1 : 0) : -1;
+  auto usable = [&](int id) { return id > p.null_block_id && (p.slots <= 0 || id < p.slots); };
+  if (!usable(slot) || !usable(final_slot) || n_acc <= 0) return;
   if (n_acc > p.L) n_acc = p.L;
+  const bool tracked = track_at >= 0 && usable(track_slot);
 
+  // Each wavefront reads its rows of the source tile before it writes any of them, so the destinations
+  // may alias the source slot.
   const Tile<float> h_tile(p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
   float s[R][4];
   load_state<R>(h_tile, lane_off, s);
-  const act_t* const kp = reinterpret_cast<const act_t*>(p.rawk) + (int64_t)slot * p.rawk_slot_stride + (int64_t)i_h * p.L * 128;
-  const act_t* const vp = reinterpret_cast<const act_t*>(p.rawv) + (int64_t)slot * p.rawv_slot_stride + (int64_t)i_hv * p.L * 128 + rowbase;
-  const float* const gp = p.gk + (int64_t)slot * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
-  const float* const bp = p.beta + (int64_t)slot * p.beta_slot_stride + (int64_t)i_hv * p.L;
+  const int64_t rec = p.records_by_request ? i_n : slot;
+  const act_t* const kp = reinterpret_cast<const act_t*>(p.rawk) + rec * p.rawk_slot_stride + (int64_t)i_h * p.L * 128;
+  const act_t* const vp = reinterpret_cast<const act_t*>(p.rawv) + rec * p.rawv_slot_stride + (int64_t)i_hv * p.L * 128 + rowbase;
+  const float* const gp = p.gk + rec * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
+  const float* const bp = p.beta + rec * p.beta_slot_stride + (int64_t)i_hv * p.L;
 
   for (int t = 0; t < n_acc; ++t) {
     float kv[4], gv[4], dec[4], vv[R], unused[R];
@@ -496,8 +509,10 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) { kv[e] *= kn; dec[e] = __expf(gv[e]); }
     delta_rows<R, true, false>(s, dec, 1.f, kv, kv, vv, bp[t], unused);
+    if (tracked && t == track_at)
+      store_state<R>(Tile<float>(p.h0 + (int64_t)track_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
   }
-  store_state<R>(h_tile, lane_off, s);
+  store_state<R>(Tile<float>(p.h0 + (int64_t)final_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
 }
 
 // ---- host side ---------------------------------------------------------------
@@ -690,23 +705,16 @@ extern "C" int pla_k_last_launch(
   return run_k_last(p, is_kda != 0, mtp, act_dtype, state_dtype, rows_per_wave, stream);
 }
 
-extern "C" int pla_kda_fold_launch(
-    float* h0, const void* rawv, const void* rawk, const float* gk, const float* beta,
-    const int32_t* slot_idx, const int32_t* accept_lens,
-    int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
-    int64_t gk_slot_stride, int64_t beta_slot_stride,
-    int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream) {
-  PLA_REQUIRE(h0 && rawv && rawk && gk && beta && slot_idx && accept_lens, "null tensor pointer");
-  PLA_REQUIRE(B > 0 && L > 0, "fold requires B > 0 and L > 0");
-  PLA_REQUIRE(H > 0 && HV >= H && HV % H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", H, HV);
+static int launch_fold(const FoldParams& p, int act_dtype, void* stream) {
+  PLA_REQUIRE(p.h0 && p.rawv && p.rawk && p.gk && p.beta && p.slot_idx && p.accept_lens, "null tensor pointer");
+  PLA_REQUIRE(p.B > 0 && p.L > 0, "fold requires B > 0 and L > 0");
+  PLA_REQUIRE(p.H > 0 && p.HV >= p.H && p.HV % p.H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", p.H, p.HV);
   PLA_REQUIRE(act_dtype == PLA_BF16 || act_dtype == PLA_F16, "record dtype must be bf16 or fp16");
-  PLA_REQUIRE(aligned(h0, 16) && h0_slot_stride % 4 == 0 && aligned(gk, 16) && gk_slot_stride % 4 == 0 &&
-              aligned(rawk, 8) && rawk_slot_stride % 4 == 0 && aligned(rawv, 16) && rawv_slot_stride % 8 == 0,
+  PLA_REQUIRE((p.track_idx == nullptr) == (p.track_step == nullptr), "track indices and steps must be given together");
+  PLA_REQUIRE(aligned(p.h0, 16) && p.h0_slot_stride % 4 == 0 && aligned(p.gk, 16) && p.gk_slot_stride % 4 == 0 &&
+              aligned(p.rawk, 8) && p.rawk_slot_stride % 4 == 0 && aligned(p.rawv, 16) && p.rawv_slot_stride % 8 == 0,
               "state and record tensors require 16-byte alignment");
-  FoldParams p{h0, rawv, rawk, gk, beta, slot_idx, accept_lens,
-               h0_slot_stride, rawv_slot_stride, rawk_slot_stride, gk_slot_stride, beta_slot_stride,
-               B, H, HV, L, null_block_id};
-  const unsigned tiles = (unsigned)B * (unsigned)HV;
+  const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const int rpw = pick_rows_per_wave((int)tiles, true);
   const dim3 block(256);
@@ -720,4 +728,32 @@ extern "C" int pla_kda_fold_launch(
     else hipLaunchKernelGGL((kda_fold_kernel<f16_t, 8>), dim3(tiles, 4), block, 0, s, p);
   }
   return check_launch("kda_fold_kernel launch");
+}
+
+extern "C" int pla_kda_fold_launch(
+    float* h0, const void* rawv, const void* rawk, const float* gk, const float* beta,
+    const int32_t* slot_idx, const int32_t* accept_lens,
+    const int32_t* track_idx, const int32_t* track_step,
+    int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
+    int64_t gk_slot_stride, int64_t beta_slot_stride,
+    int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream) {
+  FoldParams p{h0, rawv, rawk, gk, beta, slot_idx, accept_lens,
+               h0_slot_stride, rawv_slot_stride, rawk_slot_stride, gk_slot_stride, beta_slot_stride,
+               B, H, HV, L, null_block_id, nullptr, track_idx, track_step, 0, 0, 0};
+  return launch_fold(p, act_dtype, stream);
+}
+
+extern "C" int pla_kda_fold_native_launch(
+    float* state, int64_t state_slot_stride, const void* rawv, const void* rawk, const float* gate, const float* beta,
+    const int32_t* source, const int32_t* lengths, const int32_t* final_indices,
+    const int32_t* boundary_indices, const int32_t* boundary_lengths,
+    int batch, int heads, int Q, int slots, int null_block_id, void* stream) {
+  PLA_REQUIRE(final_indices && boundary_indices && boundary_lengths, "null plan pointer");
+  PLA_REQUIRE(slots > 0 && (null_block_id == -1 || null_block_id == 0), "paged fold requires slots > 0 and null_block_id -1 or 0");
+  if (batch == 0) return 0;
+  FoldParams p{state, rawv, rawk, gate, beta, source, lengths,
+               state_slot_stride, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128,
+               (int64_t)heads * Q, batch, heads, heads, Q, null_block_id,
+               final_indices, boundary_indices, boundary_lengths, 1, 1, slots};
+  return launch_fold(p, PLA_BF16, stream);
 }

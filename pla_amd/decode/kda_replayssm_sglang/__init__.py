@@ -10,8 +10,8 @@ prefix of recorded tokens (raw k, raw v, per-channel log-decay, beta) is replaye
 checkpoint ``temporal`` in place, and the conv state is rolled back to the window of the last
 accepted step.  A request whose slot is ``<= null_block_id`` or whose accepted length is ``<= 0``
 leaves its checkpoint bit-identical (src/decode/kda_replayssm/kda_mtp_fold.cu:306).  Track
-snapshots (``mamba_track_indices``) roll back conv windows only; recurrent track snapshots are
-rejected rather than silently skipped.
+snapshots (``mamba_track_indices`` / ``mamba_steps_to_track``) store the state after the tracked step
+and the conv window of that step to the tracked slot.
 """
 
 import ctypes
@@ -28,8 +28,11 @@ _BYPASS = os.environ.get("PLA_BYPASS_EXEC", "0") == "1"   # read once, like src/
 
 
 def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, accept_lens,
-                         null_block_id=-1):
+                         null_block_id=-1, track_indices=None, track_steps=None):
     """Replay ``accept_lens[n]`` recorded tokens into ``temporal[:, state_batch_indices[n]]``.
+    With ``track_indices`` / ``track_steps`` (int32 [B]) the state after step ``track_steps[n]`` is also
+    stored to slot ``track_indices[n]`` when that slot is ``> null_block_id``
+    (src/decode/kda_replayssm/kda_mtp_fold.cu:462-478).
 
     temporal [layers, slots, HV, 128, 128] float32; rawv [layers, slots, HV, L, 128] and
     rawk [layers, slots, H, L, 128] in bf16/fp16; gk [layers, slots, HV, L, 128] float32
@@ -55,6 +58,13 @@ def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, ac
     B = state_batch_indices.numel()
     if accept_lens.numel() != B:
         raise RuntimeError("accept_lens must have one entry per request")
+    if (track_indices is None) != (track_steps is None):
+        raise RuntimeError("track indices and steps must be given together")
+    if track_indices is not None:
+        track_indices = track_indices.to(torch.int32).contiguous()
+        track_steps = track_steps.to(torch.int32).contiguous()
+        if track_indices.numel() != B or track_steps.numel() != B:
+            raise RuntimeError("track indices and steps must have one entry per request")
     if not temporal[0, 0].is_contiguous():
         raise RuntimeError("temporal slots must be dense [HV, V, K]")
     stream = _lib.current_stream(temporal.device)
@@ -62,7 +72,7 @@ def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, ac
     for layer in range(layers):
         _lib.call("pla_kda_fold_launch", temporal[layer].data_ptr(), rawv[layer].data_ptr(), rawk[layer].data_ptr(),
                   gk[layer].data_ptr(), beta[layer].data_ptr(), state_batch_indices.data_ptr(),
-                  accept_lens.data_ptr(), temporal.stride(1), rawv.stride(1), rawk.stride(1), gk.stride(1),
+                  accept_lens.data_ptr(), _lib.ptr(track_indices), _lib.ptr(track_steps), temporal.stride(1), rawv.stride(1), rawk.stride(1), gk.stride(1),
                   beta.stride(1), B, H, HV, L, int(null_block_id), act, stream)
 
 
@@ -115,16 +125,17 @@ def commit_kda_replayssm_after_verify(*, spec_state, state_batch_indices, accept
     ``spec_state`` carries ``temporal``, ``replayssm_rawv/rawk/g/beta`` and, for the rollback, the lists
     ``conv`` ([layers, slots, dim, width-1] each) and ``intermediate_conv_window``
     ([layers, rows, steps, dim, width-1] each); ``conv_state_layout="width_dim"`` takes the transposed
-    pools.  Track snapshots apply to the conv windows only."""
+    pools."""
     assert conv_state_layout in ("dim_width", "width_dim")
+    if (mamba_track_indices is None) != (mamba_steps_to_track is None):
+        raise ValueError("mamba_track_indices and mamba_steps_to_track must be given together")
     fold_accepted_prefix(spec_state.temporal, spec_state.replayssm_rawv, spec_state.replayssm_rawk,
                          spec_state.replayssm_g, spec_state.replayssm_beta,
-                         state_batch_indices, accept_lens, null_block_id)
+                         state_batch_indices, accept_lens, null_block_id,
+                         mamba_track_indices, mamba_steps_to_track)
     conv = getattr(spec_state, "conv", None)
     windows = getattr(spec_state, "intermediate_conv_window", None)
     if conv is None or windows is None:
-        if mamba_track_indices is not None or mamba_steps_to_track is not None:
-            raise NotImplementedError("track snapshots need the conv pools of spec_state")
         return
     if last_correct_step_indices is None:
         raise ValueError("the conv rollback needs last_correct_step_indices")

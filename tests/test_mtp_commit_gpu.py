@@ -101,6 +101,34 @@ def test_commit_null_slots_and_clamped_lengths():
     assert torch.equal(temporal, before)                       # every slot <= null_block_id
 
 
+def test_commit_track_snapshots():
+    """Track snapshots: the state after step track_steps[n] also goes to slot track_indices[n]
+    (src/decode/kda_replayssm/kda_mtp_fold.cu:462-478); a tracked slot <= null_block_id is skipped."""
+    from pla_amd.decode.kda_replayssm_sglang import fold_accepted_prefix
+    g = torch.Generator().manual_seed(8)
+    slots, H, HV, L = 8, 2, 4, 4
+    temporal = (torch.randn(1, slots, HV, 128, 128, generator=g) * 0.1).cuda()
+    rawk = torch.randn(1, slots, H, L, 128, generator=g).bfloat16().cuda()
+    rawv = torch.randn(1, slots, HV, L, 128, generator=g).bfloat16().cuda()
+    gk = (-torch.rand(1, slots, HV, L, 128, generator=g)).cuda()
+    beta = torch.rand(1, slots, HV, L, generator=g).cuda()
+    idx = torch.tensor([4, 1, 6], dtype=torch.int32, device="cuda")
+    acc = torch.tensor([4, 3, 2], dtype=torch.int32, device="cuda")
+    track = torch.tensor([5, -1, 7], dtype=torch.int32, device="cuda")
+    steps = torch.tensor([1, 0, 1], dtype=torch.int32, device="cuda")          # snapshot after 2, -, 2 tokens
+    before = temporal.clone()
+    fold_accepted_prefix(temporal, rawv, rawk, gk, beta, idx, acc, null_block_id=-1,
+                         track_indices=track, track_steps=steps)
+    torch.cuda.synchronize()
+    c = lambda t: t[0].cpu()
+    full = fold_reference(c(before), c(rawk), c(rawv), c(gk), c(beta), [4, 1, 6], [4, 3, 2])
+    part = fold_reference(c(before), c(rawk), c(rawv), c(gk), c(beta), [4, 1, 6], [2, 1, 2])
+    for slot in (4, 1, 6):
+        assert rel_l2(temporal[0, slot], full[slot]) <= 1e-4
+    assert rel_l2(temporal[0, 5], part[4]) <= 1e-4 and rel_l2(temporal[0, 7], part[6]) <= 1e-4
+    assert torch.equal(temporal[0, [0, 2, 3]], before[0, [0, 2, 3]])
+
+
 @pytest.mark.parametrize("spec", [False, True])
 def test_fused_recurrent_kda_wrapper(spec):
     from pla_amd.decode.kda import fused_recurrent_kda
