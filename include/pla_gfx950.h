@@ -238,6 +238,22 @@ int pla_kda_replay_verify_native_launch(
     int64_t state_slot_stride, int slots, int tokens, int null_block_id, void* stream);
 
 /*
+ * Device-side commit plan of the request-row replay: plan[c * capacity + b] for c = 0..3 = commit length,
+ * final slot, boundary slot, boundary length of request b (zeroes for inactive, invalid and conflicting
+ * requests).  Replaces launch_commit_plan (src/decode/kda_replayssm_vllm/commit_plan.h:7-14, kernels
+ * commit_plan.cu:19-117).  Index vectors are dense int32 or int64 (is_int64 flags): sampled [sampler_rows],
+ * source [batch], offsets [batch+1], mapping [batch] or NULL, computed [>= sampler rows] and blocks
+ * [block_rows, block_cols] (strides in elements) or both NULL with block_size 0.  candidate and plan:
+ * int32 [4, capacity], distinct buffers.
+ */
+int pla_kda_commit_plan_launch(
+    const void* sampled, int sampled_wide, const void* source, int source_wide, const void* offsets, int offsets_wide,
+    const void* mapping, int mapping_wide, const void* computed, int computed_wide, const void* blocks, int blocks_wide,
+    int batch, int capacity, int sampler_rows, int block_rows, int block_cols, int slots, int Q, int null_block_id,
+    int token_capacity, int64_t block_row_stride, int64_t block_col_stride, int64_t block_size,
+    int32_t* candidate, int32_t* plan, void* stream);
+
+/*
  * Conv-window rollback of the commit: dst[layer, dst_idx[r], :, :] = src[layer, r, step_idx[r], :, :]
  * for every request r with step_idx[r] >= 0, 0 <= dst_idx[r] < dst_reqs, r < src_reqs and
  * step_idx[r] < src_steps.  Replaces launch_conv_scatter

@@ -19,6 +19,7 @@ from .decode import (  # noqa: F401
     k_last_reference, fold_reference, recurrent_step,
     causal_conv1d_update_reference, kda_decode_mega_reference,
     causal_conv_silu_sequence, verify_dspark_reference, conv_window_scatter_reference,
+    replay_commit_plan_reference,
 )
 from .prefill import (  # noqa: F401
     gdn_prefill_reference,

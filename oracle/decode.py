@@ -331,3 +331,78 @@ def conv_window_scatter_reference(dst, src, dst_idx, step_idx):
             continue
         out[:, d] = src[:, r, s]
     return out
+
+
+def replay_commit_plan_reference(num_sampled, state_indices, query_start_loc, *, slots, Q, token_capacity,
+                                 null_block_id=0, request_indices=None, block_table=None, num_computed_tokens=None,
+                                 block_size=None, capacity=None):
+    """Commit plan of the request-row replay as four lists of ``capacity`` integers (commit length, final
+    slot, boundary slot, boundary length).
+
+    Restates src/decode/kda_replayssm_vllm/commit_plan.cu:19-117 (``build_plan`` + ``protect_plan``) and the
+    expected plan of the reference's test oracle tests/test_kda_replayssm_vllm.py:148-178: a request commits
+    ``min(max(sampled, 0), query length)`` tokens if its source slot and query interval are valid; in align
+    mode the final state belongs to the block of token ``p + n - 1`` and, when the window reaches the next
+    block boundary, the state after ``block_size - p % block_size`` tokens to the block of position ``p``;
+    requests whose destinations collide with another live source or another committing request's
+    destinations (or whose source is another's destination) are cancelled on both sides.
+    """
+    N = len(state_indices)
+    capacity = N if capacity is None else capacity
+    valid_slot = lambda s: s > null_block_id and 0 <= s < slots
+    valid_iv = lambda a, b: a >= 0 and b > a and b <= token_capacity and b - a <= Q
+    cand = [[0, 0, 0, 0] for _ in range(capacity)]
+    for b in range(N):
+        row = b if request_indices is None else request_indices[b]
+        src = state_indices[b]
+        begin, end = query_start_loc[b], query_start_loc[b + 1]
+        if not (query_start_loc[0] == 0 and 0 <= row < len(num_sampled) and valid_slot(src) and valid_iv(begin, end)):
+            continue
+        n = min(max(num_sampled[row], 0), end - begin)
+        final, boundary, bc = src, 0, 0
+        if n and block_table is not None:
+            if row >= len(block_table) or num_computed_tokens[row] < 0:
+                n = 0
+            else:
+                p = num_computed_tokens[row]
+                cols = len(block_table[row])
+                f = block_table[row][min((p + n - 1) // block_size, cols - 1)]
+                if not valid_slot(f):
+                    n = 0
+                else:
+                    final = f
+                distance = block_size - p % block_size
+                if n and n >= distance:
+                    col = p // block_size
+                    if col >= cols:
+                        n = 0
+                    else:
+                        dest = block_table[row][col]
+                        if not valid_slot(dest) or (dest == final and distance != n):
+                            n = 0
+                        else:
+                            boundary, bc = dest, distance
+        if n:
+            cand[b] = [n, final, boundary, bc]
+    plan = [list(c) for c in cand]
+    for b in range(N):
+        if not cand[b][0]:
+            continue
+        _, f, d, bc = cand[b]
+        src = state_indices[b]
+        conflict = False
+        for o in range(N):
+            if o == b:
+                continue
+            os_ = state_indices[o]
+            if valid_slot(os_) and valid_iv(query_start_loc[o], query_start_loc[o + 1]):
+                conflict |= f == os_ or (bc > 0 and d == os_)
+            if not cand[o][0]:
+                continue
+            _, of, od, obc = cand[o]
+            conflict |= (f == os_ or f == of or (obc > 0 and f == od)
+                         or (bc > 0 and (d == os_ or d == of or (obc > 0 and d == od)))
+                         or src == of or (obc > 0 and src == od))
+        if conflict:
+            plan[b] = [0, 0, 0, 0]
+    return [[plan[b][c] for b in range(capacity)] for c in range(4)]

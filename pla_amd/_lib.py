@@ -54,6 +54,10 @@ SIGNATURES = {
         _c_p, _c_int, _c_p, _c_int,
         _c_int, _c_int, _c_int, _c_f, _c_f, _c_p,
         _c_i64, _c_int, _c_int, _c_int, _c_p],
+    "pla_kda_commit_plan_launch": [
+        _c_p, _c_int, _c_p, _c_int, _c_p, _c_int, _c_p, _c_int, _c_p, _c_int, _c_p, _c_int,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+        _c_i64, _c_i64, _c_i64, _c_p, _c_p, _c_p],
     "pla_conv_window_scatter_launch": [
         _c_int, _c_int, _c_p, _c_p, _c_p, _c_int, _c_p, _c_int, _c_int, _c_int, _c_int,
         _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,

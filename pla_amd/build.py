@@ -17,7 +17,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpla_gfx950.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["api.hip", "decode_k_last.hip", "decode_kda_mega.hip", "decode_kda_replay.hip", "prefill_gdn.hip", "prefill_kda.hip"]
+SOURCES = ["api.hip", "decode_k_last.hip", "decode_kda_mega.hip", "decode_kda_replay.hip", "commit_plan.hip", "prefill_gdn.hip", "prefill_kda.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wno-inline-asm",

@@ -6,6 +6,11 @@ request against a paged FP32 checkpoint.  The conv history and the checkpoint ar
 per-token records (post-conv k, v in bf16; log-decay, beta in FP32) and the conv window after every
 token are written to the request's row of ``records``; only real query intervals are written.
 The draft window is limited to 8 tokens here (the reference allows 32).
+
+``KDAReplayCommitContext`` (same file :149-232): the commit plan is built on the device from the sampled
+counts (and, in align mode, the block table), so nothing is read back and a commit can be captured in a
+graph; per layer the committed prefix of the records is folded from the source checkpoint into the planned
+final (and boundary) slot and the matching conv windows are copied into those slots' conv history.
 """
 
 import ctypes
@@ -18,7 +23,7 @@ import torch
 
 from ... import _lib
 
-__all__ = ["KDAReplayRecords", "kda_replay_verify"]
+__all__ = ["KDAReplayRecords", "KDAReplayCommitPlan", "KDAReplayCommitContext", "kda_replay_verify"]
 
 _BYPASS = os.environ.get("PLA_BYPASS_EXEC", "0") == "1"   # read once, like src/bypass_exec.h:44-50
 D = 128
@@ -180,3 +185,190 @@ def kda_replay_verify(*, mixed_qkv, raw_g, raw_beta, conv_weight, conv_state, ch
             ctypes.cast(c_strides, ctypes.c_void_p), state.stride(0), slots, T, int(null_block_id),
             _lib.current_stream(state.device))
     return out
+
+
+# ---- commit -----------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class KDAReplayCommitPlan:
+    """Views of the device plan, ``max_num_reqs`` entries each (zeroes for inactive, invalid and
+    conflicting requests)."""
+    commit_lens: torch.Tensor
+    final_state_indices: torch.Tensor
+    boundary_state_indices: torch.Tensor
+    boundary_recovery_lens: torch.Tensor
+
+
+def _page_runs(conv_ds, state):
+    """Writable byte runs of one layer inside a page: (page pitch in bytes, number of pages, run starts of
+    page 0 as absolute addresses, run lengths).  The commit writes the whole checkpoint of a slot and the
+    first three history items of every conv channel."""
+    import numpy as np
+    pitch_s = state.stride(0) * 4
+    starts = [np.array([state.data_ptr()], dtype=np.int64)]
+    lengths = [np.array([state.size(1) * D * D * 4], dtype=np.int64)]
+    channels = conv_ds.size(1)
+    if conv_ds.stride(2) == 1:                       # history contiguous: one 6-byte run per channel
+        starts.append(conv_ds.data_ptr() + np.arange(channels, dtype=np.int64) * conv_ds.stride(1) * 2)
+        lengths.append(np.full(channels, 6, dtype=np.int64))
+    else:                                            # channels contiguous: three runs
+        starts.append(conv_ds.data_ptr() + np.arange(3, dtype=np.int64) * conv_ds.stride(2) * 2)
+        lengths.append(np.full(3, channels * 2, dtype=np.int64))
+    return (pitch_s, conv_ds.stride(0) * 2), state.size(0), np.concatenate(starts), np.concatenate(lengths)
+
+
+def _layers_overlap(a, b):
+    """Whether the writable cache regions of two layers intersect.  Exact when both layers page with one
+    common pitch (their runs are compared modulo the pitch, which may pair pages past either end of a
+    pool: conservative there); otherwise the whole extents are compared."""
+    import numpy as np
+    (pitch_a, conv_pitch_a), pages_a, starts_a, lens_a = a
+    (pitch_b, conv_pitch_b), pages_b, starts_b, lens_b = b
+    if not (pitch_a == conv_pitch_a == pitch_b == conv_pitch_b):
+        lo_a, hi_a = starts_a.min(), (starts_a + lens_a).max() + (pages_a - 1) * max(pitch_a, conv_pitch_a)
+        lo_b, hi_b = starts_b.min(), (starts_b + lens_b).max() + (pages_b - 1) * max(pitch_b, conv_pitch_b)
+        return bool(lo_a < hi_b and lo_b < hi_a)
+    pitch = pitch_a
+    extent_a = (starts_a + lens_a).max() + (pages_a - 1) * pitch
+    extent_b = (starts_b + lens_b).max() + (pages_b - 1) * pitch
+    if not (starts_a.min() < extent_b and starts_b.min() < extent_a):
+        return False
+    origin = min(starts_a.min(), starts_b.min())
+
+    def circle(starts, lens):                        # intervals on [0, pitch), wrapped ones split
+        s = (starts - origin) % pitch
+        e = s + lens
+        wrap = e > pitch
+        return np.concatenate([s, np.zeros(int(wrap.sum()), dtype=np.int64)]), \
+            np.concatenate([np.minimum(e, pitch), (e - pitch)[wrap]])
+    sa, ea = circle(starts_a, lens_a)
+    sb, eb = circle(starts_b, lens_b)
+    order = np.argsort(sb)
+    sb, eb = sb[order], np.maximum.accumulate(eb[order])
+    # an interval of a overlaps some interval of b iff a b-interval starting before its end reaches past its start
+    idx = np.searchsorted(sb, ea, side="left") - 1
+    hit = (idx >= 0) & (eb[np.maximum(idx, 0)] > sa)
+    return bool(hit.any())
+
+
+class KDAReplayCommitContext:
+    """Layer descriptors and reusable device plan buffers of the request-row commit
+    (reference pla/decode/kda_replayssm_vllm/__init__.py:149-232).
+
+    Create outside graph capture and keep the cache and record tensors in place for the lifetime of the
+    context; writable cache regions of different layers must be disjoint.  Commits, reads of the returned
+    plan and replays of graphs captured with this context must be ordered on one stream: the next commit
+    overwrites the plan.  ``layers``: objects with ``kv_cache = (conv, state)`` and ``replay_records``.
+    """
+
+    @classmethod
+    def create(cls, layers, spec_query_len, max_num_reqs, conv_state_layout="SD", null_block_id=0):
+        layers = tuple(layers)
+        if not layers or not 1 <= spec_query_len <= 32 or max_num_reqs < 0:
+            raise ValueError("context requires layers, R >= 0 and Q in [1, 32]")
+        if null_block_id not in (-1, 0):
+            raise ValueError("null_block_id must be -1 or 0")
+        device = layers[0].kv_cache[1].device
+        if device.type != "cuda":
+            raise ValueError("commit context requires GPU tensors")
+        with torch.cuda.device(device):
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("create commit context before graph capture")
+        slots, heads = layers[0].kv_cache[1].shape[:2]
+        views, runs = [], []
+        for index, layer in enumerate(layers):
+            conv, state = layer.kv_cache
+            records = layer.replay_records
+            tensors = (conv, state, records.rawv, records.rawk, records.g, records.beta, records.conv)
+            if any(t.device != device for t in tensors):
+                raise ValueError("all context layers must share one device")
+            ds = _paged_cache(conv, state, conv_state_layout, heads, slots)
+            _check_records(records, state, heads, spec_query_len, max_num_reqs)
+            _disjoint([records.rawv, records.rawk, records.g, records.beta, records.conv], [conv, state])
+            layer_runs = _page_runs(ds, state)
+            for previous, other in enumerate(runs):
+                if _layers_overlap(layer_runs, other):
+                    raise ValueError(f"context layers {previous} and {index} have overlapping writable caches")
+            runs.append(layer_runs)
+            views.append((ds, state, records))
+        self = cls()
+        self._layers, self._views = layers, tuple(views)
+        self._candidate = torch.zeros((4, max_num_reqs), dtype=torch.int32, device=device)
+        self._buffer = torch.zeros_like(self._candidate)
+        self._steps = torch.zeros((2, max_num_reqs), dtype=torch.int32, device=device)
+        self.plan = KDAReplayCommitPlan(*self._buffer.unbind(0))
+        self._heads, self._slots = heads, slots
+        self._q, self._capacity, self._null = spec_query_len, max_num_reqs, null_block_id
+        self._device = device
+        return self
+
+    def commit(self, num_sampled, state_indices, query_start_loc, request_indices=None, block_table=None,
+               num_computed_tokens=None, mamba_block_size=None, *, token_capacity):
+        """Builds the plan on the device (sampled counts clamped to the query length, no bonus token
+        subtracted), then, per layer, folds each request's committed prefix of records from its source
+        checkpoint into the planned slots and copies the matching conv windows.  ``token_capacity`` is the
+        verify projection's ``mixed_qkv.shape[0]``; query intervals beyond it are skipped.  Align mode needs
+        ``block_table``, ``num_computed_tokens`` and ``mamba_block_size >= Q`` together.  Returns the plan."""
+        if not isinstance(token_capacity, Integral):
+            raise TypeError("token_capacity must be a host integer")
+        align = (block_table is not None, num_computed_tokens is not None, mamba_block_size is not None)
+        if any(align) and not all(align):
+            raise ValueError("align requires block_table, computed tokens and block size")
+        if all(align) and not isinstance(mamba_block_size, Integral):
+            raise TypeError("mamba_block_size must be a host integer")
+        if all(align) and mamba_block_size < self._q:
+            raise ValueError("align block_size must be >= spec_query_len")
+        if _BYPASS:
+            return self.plan
+        _need(0 <= token_capacity <= 2 ** 31 - 1, "token_capacity must be between 0 and INT32_MAX")
+        ref = self._buffer
+        sampled, sampled_wide = _index(num_sampled, ref)
+        source, source_wide = _index(state_indices, ref)
+        cu, cu_wide = _index(query_start_loc, ref)
+        N, R = source.numel(), self._capacity
+        _need(N <= R and cu.numel() == N + 1, "commit query count exceeds capacity")
+        mapping = mapping_wide = None
+        if request_indices is not None:
+            mapping, mapping_wide = _index(request_indices, ref)
+            _need(mapping.numel() == N, "mapping must have N rows")
+        else:
+            _need(sampled.numel() >= N, "sampler count must cover query rows")
+        computed = computed_wide = None
+        blocks_wide, block_rows, block_cols, row_stride, col_stride, block_size = 0, 0, 0, 0, 0, 0
+        if all(align):
+            computed, computed_wide = _index(num_computed_tokens, ref)
+            _need(block_table.device == ref.device and block_table.dim() == 2 and block_table.size(1) > 0
+                  and block_table.dtype in (torch.int32, torch.int64) and computed.numel() >= sampled.numel(),
+                  "invalid align table/count/block size")
+            blocks_wide = int(block_table.dtype == torch.int64)
+            block_rows, block_cols = block_table.shape
+            row_stride, col_stride = block_table.stride()
+            block_size = int(mamba_block_size)
+        if source.dtype != torch.int32:
+            source32 = source.to(torch.int32)
+        else:
+            source32 = source
+        stream = _lib.current_stream(self._device)
+        with torch.cuda.device(self._device):
+            _lib.call("pla_kda_commit_plan_launch", sampled.data_ptr(), sampled_wide, source.data_ptr(), source_wide,
+                      cu.data_ptr(), cu_wide, _lib.ptr(mapping), int(mapping_wide or 0), _lib.ptr(computed),
+                      int(computed_wide or 0), _lib.ptr(block_table) if all(align) else None, blocks_wide,
+                      N, R, sampled.numel(), block_rows, block_cols, self._slots, self._q, self._null,
+                      int(token_capacity), row_stride, col_stride, block_size,
+                      self._candidate.data_ptr(), self._buffer.data_ptr(), stream)
+            if N == 0:
+                return self.plan
+            lens, final, boundary, bc = (t[:N] for t in self._buffer.unbind(0))
+            torch.sub(lens, 1, out=self._steps[0, :N])          # window of the last committed token
+            torch.sub(bc, 1, out=self._steps[1, :N])            # -1 (skipped) without a boundary
+            for ds, state, records in self._views:
+                _lib.call("pla_kda_fold_native_launch", state.data_ptr(), state.stride(0), records.rawv.data_ptr(),
+                          records.rawk.data_ptr(), records.g.data_ptr(), records.beta.data_ptr(),
+                          source32.data_ptr(), lens.data_ptr(), final.data_ptr(), boundary.data_ptr(), bc.data_ptr(),
+                          N, self._heads, self._q, self._slots, self._null, stream)
+                win = records.conv
+                for dst_idx, steps in ((boundary, self._steps[1, :N]), (final, self._steps[0, :N])):
+                    _lib.call("pla_conv_window_scatter_launch", 2, 3, win.data_ptr(), ds.data_ptr(),
+                              dst_idx.data_ptr(), 0, steps.data_ptr(), 0, 1, ds.size(1), N,
+                              0, *win.stride(), 0, *ds.stride(), win.size(0), win.size(1), self._slots, stream)
+        return self.plan

@@ -127,3 +127,33 @@ def test_conv_window_scatter_reference_masks():
     assert torch.equal(out[:, 3], src[:, 0, 2])
     keep = [0, 1, 2, 4]
     assert torch.equal(out[:, keep], dst[:, keep])
+
+
+def test_commit_plan_reference_known_answers():
+    """Hand-derived plans (block size 4): positions count tokens already computed."""
+    from oracle import replay_commit_plan_reference as plan
+    # no align: counts are clamped to the query length, null / negative sources and empty queries commit nothing
+    got = plan([3, 9, 2, -1, 1], [7, 2, 0, 5, 4], [0, 3, 5, 5, 6, 7], slots=12, Q=3, token_capacity=7)
+    assert got == [[3, 2, 0, 0, 1], [7, 2, 0, 0, 4], [0, 0, 0, 0, 0], [0, 0, 0, 0, 0]]
+    # align: request 0 at position 2 commits 3 tokens -> tokens 2, 3, 4: boundary after 2 tokens into the block of
+    # position 2 (column 0), final in the block of token 4 (column 1); request 1 at position 4 commits 2 tokens inside
+    # block 1 -> no boundary; request 2 at position 3 commits 1 token = exactly up to the boundary: boundary == final
+    table = [[5, 6, 7], [8, 9, 1], [2, 3, 4]]
+    got = plan([3, 2, 1], [5, 9, 2], [0, 3, 5, 6], slots=12, Q=3, token_capacity=6, block_table=table,
+               num_computed_tokens=[2, 4, 3], block_size=4)
+    assert got == [[3, 2, 1], [6, 9, 2], [5, 0, 2], [2, 0, 1]]
+    # conflicts cancel both sides: request 1's final block is request 0's source
+    got = plan([1, 1], [5, 9], [0, 1, 2], slots=12, Q=2, token_capacity=2, block_table=[[5], [5]],
+               num_computed_tokens=[0, 0], block_size=4)
+    assert got == [[0, 0], [0, 0], [0, 0], [0, 0]]
+    # a live query that commits nothing still protects its source
+    got = plan([0, 1], [5, 9], [0, 1, 2], slots=12, Q=2, token_capacity=2, block_table=[[5], [5]],
+               num_computed_tokens=[0, 0], block_size=4)
+    assert got == [[0, 0], [0, 0], [0, 0], [0, 0]]
+    # mapping, capacity padding, token capacity and a boundary that differs from the final block with equal slots
+    got = plan([2, 1], [3, 4], [0, 2, 3], slots=8, Q=2, token_capacity=3, request_indices=[1, 0], capacity=4)
+    assert got == [[1, 1, 0, 0], [3, 4, 0, 0], [0, 0, 0, 0], [0, 0, 0, 0]]
+    got = plan([2, 2], [3, 4], [0, 2, 4], slots=8, Q=2, token_capacity=3)
+    assert got == [[2, 0], [3, 0], [0, 0], [0, 0]]
+    got = plan([2], [3], [0, 2], slots=8, Q=2, token_capacity=2, block_table=[[6, 6]], num_computed_tokens=[3], block_size=4)
+    assert got == [[0], [0], [0], [0]]                                                # boundary == final, lengths differ

@@ -174,3 +174,181 @@ def test_replay_verify_skips_malformed_intervals_and_rejects_bad_arguments():
     with pytest.raises(NotImplementedError, match="up to 8 tokens"):
         kda_replay_verify(**args, conv_state=pages(6, heads, 9, "DS", gen).conv, checkpoint_state=layer.state, records=wide,
                           query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS")
+
+
+# ---- commit --------------------------------------------------------------------------------------------
+
+from oracle import fold_reference, replay_commit_plan_reference            # noqa: E402
+from pla_amd.decode.kda_replayssm_vllm import KDAReplayCommitContext        # noqa: E402
+from helpers import rel_l2                                                  # noqa: E402
+
+
+def _ds(layer):
+    return layer.conv if layer.layout == "DS" else layer.conv.transpose(-1, -2)
+
+
+def _expected_commit(layer, plan, sources):
+    """Expected pools of one layer from a plan: per request, fold the committed prefix of its records from
+    its source checkpoint into the final (and boundary) slot, copy the matching conv windows."""
+    rec = layer.replay_records
+    state0, conv0 = layer.state.cpu().clone(), _ds(layer).cpu().clone()
+    state, conv = state0.clone(), conv0.clone()
+    rk, rv, g, bt, win = (t.cpu() for t in (rec.rawk, rec.rawv, rec.g, rec.beta, rec.conv))
+    for b, src in enumerate(sources):
+        n, final, boundary, bc = (plan[c][b] for c in range(4))
+        if not n:
+            continue
+        def folded(count):
+            one = fold_reference(state0[src][None], rk[b][None], rv[b][None], g[b][None], bt[b][None], [0], [count],
+                                 compute_dtype=torch.float64)
+            return one[0].float()
+        if bc:
+            state[boundary] = folded(bc)
+            conv[boundary, :, :3] = win[b, bc - 1]
+        state[final] = folded(n)
+        conv[final, :, :3] = win[b, n - 1]
+    return state, conv
+
+
+def _verify_then_commit(layers, x, offsets, slots, q, counts, *, layout, null_block_id=0, mapping=None, align=None,
+                        index_dtype=torch.int32):
+    rows = len(slots)
+    args = {k: v for k, v in x.items() if k != "storage"}
+    T = x["mixed_qkv"].shape[0]
+    for layer in layers:
+        layer.replay_records = records_filled(rows, layer.heads, q)
+        layer.kv_cache = (layer.conv, layer.state)
+        kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=layer.replay_records,
+                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout=layout,
+                          null_block_id=null_block_id)
+    torch.cuda.synchronize()
+    ctx = KDAReplayCommitContext.create(layers, q, rows, layout, null_block_id)
+    kw = {}
+    if align is not None:
+        kw = dict(block_table=torch.tensor(align["table"], dtype=index_dtype, device="cuda"),
+                  num_computed_tokens=vector(align["computed"], index_dtype), mamba_block_size=align["block_size"])
+    want_plan = replay_commit_plan_reference(
+        counts, slots, offsets, slots=layers[0].state.shape[0], Q=q, token_capacity=T, null_block_id=null_block_id,
+        request_indices=mapping, block_table=None if align is None else align["table"],
+        num_computed_tokens=None if align is None else align["computed"],
+        block_size=None if align is None else align["block_size"], capacity=rows)
+    expected = [_expected_commit(layer, want_plan, slots) for layer in layers]
+    plan = ctx.commit(vector(counts, index_dtype, True), vector(slots, index_dtype, True), vector(offsets, index_dtype, True),
+                      request_indices=None if mapping is None else vector(mapping, index_dtype), token_capacity=T, **kw)
+    torch.cuda.synchronize()
+    got_plan = [t.cpu().tolist() for t in (plan.commit_lens, plan.final_state_indices, plan.boundary_state_indices,
+                                           plan.boundary_recovery_lens)]
+    assert got_plan == want_plan
+    for layer, (want_state, want_conv) in zip(layers, expected):
+        state, conv = layer.state.cpu(), _ds(layer).cpu()
+        for s in range(state.shape[0]):
+            if torch.equal(want_state[s], layer._state_before[s]):
+                assert torch.equal(state[s], want_state[s])                         # untouched slots stay bit-identical
+            else:
+                assert rel_l2(state[s], want_state[s]) <= 1e-4
+        assert torch.equal(conv, want_conv)
+    return ctx, want_plan
+
+
+def _snapshot(layers):
+    for layer in layers:
+        layer._state_before = layer.state.cpu().clone()
+
+
+@pytest.mark.parametrize("layout", ["DS", "SD"])
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+def test_replay_commit_in_place(layout, index_dtype):
+    gen = torch.Generator().manual_seed(11)
+    q, heads = 4, 2
+    lengths = [4, 2, 0, 1, 3]
+    offsets = [0]
+    for n in lengths:
+        offsets.append(offsets[-1] + n)
+    slots = [7, 2, 5, 0, 9]
+    layers = [pages(12, heads, q, layout, gen)]
+    x = inputs(heads, offsets[-1] + 3, gen)
+    _snapshot(layers)
+    _, plan = _verify_then_commit(layers, x, offsets, slots, q, [3, 9, 2, 1, -1], layout=layout, index_dtype=index_dtype)
+    assert plan[0] == [3, 2, 0, 0, 0] and plan[1] == [7, 2, 0, 0, 0]                   # slot 0 is the null block
+
+
+def test_replay_commit_align_boundaries_conflicts_and_mapping():
+    gen = torch.Generator().manual_seed(12)
+    q, heads, layout = 3, 2, "SD"
+    offsets, slots = [0, 3, 5, 6, 9], [5, 9, 2, 11]
+    layers = [pages(14, heads, q, layout, gen), pages(14, heads, q, layout, gen)]
+    x = inputs(heads, 12, gen)
+    _snapshot(layers)
+    # request 0: boundary after 2 tokens (block 5 = its own source), final block 6; request 1: inside block 9;
+    # request 2: exactly up to the boundary (boundary == final == 3); request 3 wants block 6 too -> cancelled with request 0
+    align = dict(table=[[5, 6, 7], [8, 9, 1], [3, 3, 4], [6, 6, 6]], computed=[2, 4, 3, 1], block_size=4)
+    _, plan = _verify_then_commit(layers, x, offsets, slots, q, [3, 2, 1, 2], layout=layout, align=align)
+    assert plan == [[0, 2, 1, 0], [0, 9, 3, 0], [0, 0, 3, 0], [0, 0, 1, 0]]
+    # the same without the conflicting request: request 0 commits with a boundary snapshot into its own source block
+    layers = [pages(14, heads, q, layout, gen)]
+    _snapshot(layers)
+    align = dict(table=[[5, 6, 7], [8, 9, 1], [3, 3, 4], [10, 12, 13]], computed=[2, 4, 3, 1], block_size=4)
+    _, plan = _verify_then_commit(layers, x, offsets, slots, q, [3, 2, 1, 2], layout=layout, align=align,
+                                  index_dtype=torch.int64)
+    assert plan == [[3, 2, 1, 2], [6, 9, 3, 10], [5, 0, 3, 0], [2, 0, 1, 0]]
+    # request rows mapped onto sampler rows
+    layers = [pages(14, heads, q, layout, gen)]
+    _snapshot(layers)
+    _, plan = _verify_then_commit(layers, x, offsets, slots, q, [1, 3, 0, 2], layout=layout, mapping=[3, 2, 1, 0])
+    assert plan[0] == [2, 0, 1, 1]
+
+
+def test_replay_commit_context_checks_and_graph_replay():
+    gen = torch.Generator().manual_seed(13)
+    q, heads, layout = 2, 1, "DS"
+    # two layers interleaved in one set of pages: disjoint runs are accepted, overlapping ones rejected
+    first = pages(6, heads, q, layout, gen, padding=3 * heads * D * 4 * 2 + heads * D * D * 4 + 512)
+    span = 3 * heads * D * (q + 2) * 2
+    second_offset = ((span + 15) // 16) * 16 + heads * D * D * 4 + 64
+    c = 3 * heads * D
+    history = q + 2
+    raw = first.raw
+    page_bytes = raw.numel() // 6
+    conv2 = raw.view(torch.bfloat16).as_strided((6, c, history), (page_bytes // 2, history, 1), second_offset // 2)
+    state_off2 = ((second_offset + c * history * 2 + 15) // 16) * 16
+    state2 = raw.view(torch.float32).as_strided((6, heads, D, D), (page_bytes // 4, D * D, D, 1), state_off2 // 4)
+    assert state_off2 + heads * D * D * 4 <= page_bytes
+    second = SimpleNamespace(raw=raw, conv=conv2, state=state2, heads=heads, q=q, layout=layout)
+    conv2.copy_((torch.randn(conv2.shape, generator=gen) * 0.2).to(torch.bfloat16))
+    state2.copy_(torch.randn(state2.shape, generator=gen) * 0.01)
+    layers = [first, second]
+    x = inputs(heads, 8, gen)
+    offsets, slots = [0, 2, 3, 5], [4, 1, 3]
+    _snapshot(layers)
+    ctx, _ = _verify_then_commit(layers, x, offsets, slots, q, [2, 1, 1], layout=layout)
+    overlapping = SimpleNamespace(kv_cache=(first.conv, first.state), replay_records=first.replay_records)
+    with pytest.raises(ValueError, match="layers 0 and 1 have overlapping writable caches"):
+        KDAReplayCommitContext.create([first, overlapping], q, 3, layout, 0)
+    with pytest.raises(ValueError, match="null_block_id must be -1 or 0"):
+        KDAReplayCommitContext.create([first], q, 3, layout, 2)
+    with pytest.raises(ValueError, match="align requires"):
+        ctx.commit(vector([1, 1, 1]), vector(slots), vector(offsets), block_table=torch.zeros(3, 2, dtype=torch.int32, device="cuda"),
+                   token_capacity=8)
+    with pytest.raises(TypeError):
+        ctx.commit(vector([1, 1, 1]), vector(slots), vector(offsets), token_capacity=torch.tensor(8))
+    # graph replay: the plan is built on the device, so the captured commit follows new sampled counts
+    counts = vector([2, 1, 1])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ctx.commit(counts, vector(slots), vector(offsets), token_capacity=8)
+    torch.cuda.current_stream().wait_stream(side)
+    src, off = vector(slots), vector(offsets)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        plan = ctx.commit(counts, src, off, token_capacity=8)
+    for new_counts, want in (([1, 0, 2], [1, 0, 2]), ([0, 5, 1], [0, 1, 1])):
+        counts.copy_(torch.tensor(new_counts, dtype=torch.int32))
+        before = [layer.state.clone() for layer in layers]
+        graph.replay()
+        torch.cuda.synchronize()
+        assert plan.commit_lens.cpu().tolist() == want
+        for layer, old in zip(layers, before):
+            for b, s in enumerate(slots):
+                changed = not torch.equal(layer.state[s], old[s])
+                assert changed == (want[b] > 0)
