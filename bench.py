@@ -292,7 +292,7 @@ def bench_replay_verify(device, steps=100, N=64, H=32, T=4):
     import torch
     from pla_amd.decode.kda_replayssm_sglang import fused_kda_decode_mtp_dspark, commit_kda_replayssm_after_verify
     from pla_amd.workloads import kda_replay_verify
-    w = kda_replay_verify(N, H, T, seed=505, device=device, slots=1024, ring_len=8, onorm=True, strided=False)
+    w = kda_replay_verify(N, H, T, seed=505, device=device, slots=1024, ring_len=max(8, T), onorm=True, strided=False)
     w["intermediate_state_indices"] = torch.arange(N, dtype=torch.int32, device=device)
     out = torch.empty(1, N * T, H, 128, dtype=torch.bfloat16, device=device)
 

@@ -200,7 +200,7 @@ int pla_kda_decode_mega_launch(
  *                   sigmoid(gate), gate [T,H,128] bf16 with token stride onorm_gate_stride
  *   slot_idx, scratch_idx, cu_seqlens: int32 or int64 ([N], [>=N], [N+1]); slot < 0: the request's
  *                   output rows are zeroed and nothing else is touched
- *   t_loop          draft tokens per request (1..8); ring_len = L >= t_loop
+ *   t_loop          draft tokens per request (1..32); ring_len = L >= t_loop
  */
 int pla_kda_verify_dspark_launch(
     const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,
@@ -224,7 +224,7 @@ int pla_kda_verify_dspark_launch(
  * request row; the checkpoint pool has a slot pitch (state_slot_stride elements, slots entries); a slot
  * <= null_block_id (-1 or 0) is padding (zero output rows, nothing else written); a request whose query
  * interval is empty, longer than Q, not inside [0, tokens] or whose slot is >= slots is skipped entirely;
- * no fused output norm.  Q <= 8 here.
+ * no fused output norm.  Q <= 32.
  */
 int pla_kda_replay_verify_native_launch(
     const void* x_q, const void* x_k, const void* x_v, const void* g_in, const void* beta_in,

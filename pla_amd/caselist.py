@@ -13,7 +13,7 @@ shape on synthetic inputs through the operator that serves it here and times it:
 GDN decode, 1 token         ``fused_sigmoid_gating_delta_rule_forward_k_last_packed``
 GDN decode, T tokens        ``fused_sigmoid_gating_delta_rule_forward_k_last`` (verify, state read-only)
 KDA decode, 1 token         ``fused_kda_decode_mega_forward`` (conv + gate + recurrence + norm)
-KDA decode, T tokens        ``fused_kda_decode_mtp_dspark`` (verify with replay records, T <= 8)
+KDA decode, T tokens        ``fused_kda_decode_mtp_dspark`` (verify with replay records, T <= 32)
 GDN / KDA prefill           ``gdn_prefill_packed_qkv_fwd`` / ``flashkda_fwd``
 ==========================  =====================================================================
 
@@ -90,8 +90,8 @@ def unsupported_reason(case):
     if case["phase"] == "D" and case["op"] == "kda_attn":
         if case.get("seqlen_q", 1) == 1 and H not in _MEGA_HEADS:
             return f"the fused KDA decode step supports H in {_MEGA_HEADS}"
-        if case.get("seqlen_q", 1) > 8:
-            return "the KDA verify handles up to 8 draft tokens"
+        if case.get("seqlen_q", 1) > 32:
+            return "the KDA verify handles up to 32 draft tokens"
     if case["phase"] == "P" and case.get("dtype") != "bf16":
         return "prefill takes bf16 activations"
     return None

@@ -18,7 +18,8 @@
 //     o_t = S_0 w_t + sum_{j <= t} c_{j,t} v_j,  w_t = A_1 .. A_t q_t,  A_j = D_j (I - beta_j k_j k_j^T)
 // wavefront w works out w_t and c_{.,t} for tokens t = w, w + 4 from K-vectors alone, and the tile
 // is used once as the A operand of S_0 [w_0 .. w_{T-1}] on v_mfma_f32_16x16x32_bf16 (FP32 data split
-// into bf16 hi + lo, three products).  Up to eight draft tokens.
+// into bf16 hi + lo, three products), sixteen tokens per pass.  Up to 32 draft tokens (the reference's
+// limit); windows of up to eight keep all K-vectors in registers, wider ones re-read them from LDS.
 //
 // Conv-window scatter (reference: conv_scatter_kernel, src/decode/kda_replayssm/kda_mtp_fold.cu:595-635):
 // dst[layer, dst_idx[r], :, :] = src[layer, r, step_idx[r], :, :] for every request r with a
@@ -94,8 +95,11 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   }
   const int64_t srow = p.native ? n : index_at(p.scratch_idx, p.scratch_wide, n);
 
-  __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128], sW[TMAX][128];
+  // sQ[t] holds q_t after the convolution and the effective query w_t after the algebra (only the
+  // wavefront that owns token t touches the row in between).
+  __shared__ __align__(16) float sQ[TMAX][128], sK[TMAX][128], sV[TMAX][128], sD[TMAX][128];
   __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
+  float (*const sW)[128] = sQ;
   __shared__ float sBeta[TMAX], sNorm[2][2][TMAX], sSq[4][TMAX];
 
   // Small inputs first, the state tile after them: memory returns in issue order, so the convolution
@@ -178,8 +182,8 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   }
   __syncthreads();
 
-  // K-vector algebra: wavefront w handles tokens w and w + 4
-  {
+  // K-vector algebra: wavefront w handles tokens w, w + 4, ...
+  if constexpr (TMAX <= 8) {                        // all K-vectors in registers
     float kv[TMAX][4], dec[TMAX][4], beta[TMAX];
 #pragma unroll
     for (int j = 0; j < TMAX; ++j) {
@@ -206,64 +210,104 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
         for (int j = 0; j < TMAX; ++j) sC[t][j] = cf[j];
       }
     }
+  } else {                                          // wide draft windows: K-vectors stay in LDS
+    for (int t = wave; t < n_tok; t += 4) {
+      const float qn = fast_rsqrt(sNorm[0][0][t] + sNorm[0][1][t] + 1e-6f) * p.scale;
+      const float4 q4 = *reinterpret_cast<const float4*>(&sQ[t][4 * c]);
+      float w[4] = {q4.x * qn, q4.y * qn, q4.z * qn, q4.w * qn};
+      if (lane > t && lane < TMAX) sC[t][lane] = 0.f;
+      for (int j = t; j >= 0; --j) {
+        const float kn = fast_rsqrt(sNorm[1][0][j] + sNorm[1][1][j] + 1e-6f);
+        const float4 k4 = *reinterpret_cast<const float4*>(&sK[j][4 * c]);
+        const float4 d4 = *reinterpret_cast<const float4*>(&sD[j][4 * c]);
+        const float kj[4] = {k4.x * kn, k4.y * kn, k4.z * kn, k4.w * kn};
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dot = fmaf(kj[e], w[e], dot);
+        const float cf = sBeta[j] * row32_allreduce(dot);
+        w[0] = d4.x * fmaf(-cf, kj[0], w[0]);
+        w[1] = d4.y * fmaf(-cf, kj[1], w[1]);
+        w[2] = d4.z * fmaf(-cf, kj[2], w[2]);
+        w[3] = d4.w * fmaf(-cf, kj[3], w[3]);
+        if (lane == 0) sC[t][j] = cf;
+      }
+      if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
+    }
   }
   __syncthreads();
 
-  // B operands: column r16 of [w_0 .. w_{T-1} 0 .. 0]
-  const int tcol = min(r16, n_tok - 1);
-  const bool mine = r16 < n_tok;
-  const float keep = mine ? 1.f : 0.f;
-  HiLo wb[4];
-  query_operands(sW, tcol, keep, kb, wb);
-  float cs[TMAX];
+  // Tile pass, sixteen tokens (MFMA columns) at a time: column r16 of [w_0 .. w_{T-1} 0 .. 0]
+  constexpr int NCOL = (TMAX + 15) / 16;
+  float o[NCOL][2][4];
+  float ss[NCOL];
 #pragma unroll
-  for (int j = 0; j < TMAX; ++j) cs[j] = sC[tcol][j];
-
-  float o[2][4];
-  float ss = 0.f;
+  for (int cg = 0; cg < NCOL; ++cg) {
+    const int token = 16 * cg + r16;
+    const int tcol = min(token, n_tok - 1);
+    const float keep = token < n_tok ? 1.f : 0.f;
+    HiLo wb[4];
+    query_operands(sW, tcol, keep, kb, wb);
+    ss[cg] = 0.f;
+    if (16 * cg >= n_tok) continue;                 // uniform: no token in this column group
 #pragma unroll
-  for (int m = 0; m < 2; ++m) {
-    const f32x4_t acc = rows_times_queries(sa[m], wb);
-    // lane (r16 = token, kb): rows 32 w + 16 m + 4 kb .. + 3 of S_0 w_token, plus the bias terms
-    o[m][0] = acc[0]; o[m][1] = acc[1]; o[m][2] = acc[2]; o[m][3] = acc[3];
+    for (int m = 0; m < 2; ++m) {
+      const f32x4_t acc = rows_times_queries(sa[m], wb);
+      // lane (r16 = token, kb): rows 32 w + 16 m + 4 kb .. + 3 of S_0 w_token, plus the bias terms
+      o[cg][m][0] = acc[0]; o[cg][m][1] = acc[1]; o[cg][m][2] = acc[2]; o[cg][m][3] = acc[3];
+    }
+    const int last = min(n_tok, 16 * cg + 16);      // c_{j,t} = 0 for j > t
+#pragma unroll(TMAX <= 8 ? TMAX : 4)
+    for (int jt = 0; jt < (TMAX <= 8 ? TMAX : last); ++jt) {
+      if (TMAX <= 8 && jt >= n_tok) break;
+      const float cj = sC[tcol][jt];
 #pragma unroll
-    for (int j = 0; j < TMAX; ++j) {
-      if (j >= n_tok) break;
-      const float4 v4 = *reinterpret_cast<const float4*>(&sV[j][rowbase + 16 * m + 4 * kb]);
-      o[m][0] = fmaf(cs[j], v4.x, o[m][0]);
-      o[m][1] = fmaf(cs[j], v4.y, o[m][1]);
-      o[m][2] = fmaf(cs[j], v4.z, o[m][2]);
-      o[m][3] = fmaf(cs[j], v4.w, o[m][3]);
+      for (int m = 0; m < 2; ++m) {
+        const float4 v4 = *reinterpret_cast<const float4*>(&sV[jt][rowbase + 16 * m + 4 * kb]);
+        o[cg][m][0] = fmaf(cj, v4.x, o[cg][m][0]);
+        o[cg][m][1] = fmaf(cj, v4.y, o[cg][m][1]);
+        o[cg][m][2] = fmaf(cj, v4.z, o[cg][m][2]);
+        o[cg][m][3] = fmaf(cj, v4.w, o[cg][m][3]);
+      }
     }
 #pragma unroll
-    for (int r = 0; r < 4; ++r) ss = fmaf(o[m][r], o[m][r], ss);
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) ss[cg] = fmaf(o[cg][m][r], o[cg][m][r], ss[cg]);
   }
 
-  float rstd = 1.f;
   if constexpr (ONORM) {
-    // sum of squares of the token's 128 outputs: over the four 16-lane rows of the wavefront, then over
+    // sum of squares of a token's 128 outputs: over the four 16-lane rows of the wavefront, then over
     // the four wavefronts through LDS
-    const LanePair rows = swap_rows16(ss);
-    const LanePair halves = swap_halves(rows.lo + rows.hi);
-    if (lane < TMAX) sSq[wave][lane] = halves.lo + halves.hi;
+#pragma unroll
+    for (int cg = 0; cg < NCOL; ++cg) {
+      const LanePair rows = swap_rows16(ss[cg]);
+      const LanePair halves = swap_halves(rows.lo + rows.hi);
+      if (lane < 16 && 16 * cg + lane < TMAX) sSq[wave][16 * cg + lane] = halves.lo + halves.hi;
+    }
     __syncthreads();
-    const float total = sSq[0][tcol] + sSq[1][tcol] + sSq[2][tcol] + sSq[3][tcol];
-    rstd = fast_rsqrt(total * (1.0f / 128.0f) + p.onorm_eps);
   }
-  if (mine) {
+#pragma unroll
+  for (int cg = 0; cg < NCOL; ++cg) {
+    const int token = 16 * cg + r16;
+    if (token >= n_tok) continue;
+    float rstd = 1.f;
+    if constexpr (ONORM) {
+      const float total = sSq[0][token] + sSq[1][token] + sSq[2][token] + sSq[3][token];
+      rstd = fast_rsqrt(total * (1.0f / 128.0f) + p.onorm_eps);
+    }
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
       const int row = rowbase + 16 * m + 4 * kb;
-      float val[4] = {o[m][0], o[m][1], o[m][2], o[m][3]};
+      float val[4] = {o[cg][m][0], o[cg][m][1], o[cg][m][2], o[cg][m][3]};
       if constexpr (ONORM) {
-        const uint2 gw = *reinterpret_cast<const uint2*>(p.onorm_gate + (bos + r16) * p.onorm_gate_stride + h * 128 + row);
+        const uint2 gw = *reinterpret_cast<const uint2*>(p.onorm_gate + (bos + token) * p.onorm_gate_stride + h * 128 + row);
         const float4 w4 = *reinterpret_cast<const float4*>(p.onorm_weight + row);
         val[0] *= rstd * w4.x * fast_sigmoid(lo16<bf16_t>(gw.x));
         val[1] *= rstd * w4.y * fast_sigmoid(hi16<bf16_t>(gw.x));
         val[2] *= rstd * w4.z * fast_sigmoid(lo16<bf16_t>(gw.y));
         val[3] *= rstd * w4.w * fast_sigmoid(hi16<bf16_t>(gw.y));
       }
-      *reinterpret_cast<uint2*>(p.out + ((bos + r16) * p.H + h) * 128 + row) =
+      *reinterpret_cast<uint2*>(p.out + ((bos + token) * p.H + h) * 128 + row) =
           make_uint2(pack2<bf16_t>(val[0], val[1]), pack2<bf16_t>(val[2], val[3]));
     }
   }
@@ -295,7 +339,7 @@ namespace pla {
 // Shared by the ring-mode and the paged entry points.
 static int launch_replay_verify(ReplayVerifyParams& p, const int64_t* strides, int t_loop, hipStream_t s) {
   PLA_REQUIRE(p.H > 0 && p.N > 0 && t_loop > 0, "verify requires H > 0, N > 0 and at least one token per request");
-  PLA_REQUIRE(t_loop <= 8, "the gfx950 verify handles up to 8 draft tokens per request, got %d", t_loop);
+  PLA_REQUIRE(t_loop <= 32, "the verify handles up to 32 draft tokens per request, got %d", t_loop);
   PLA_REQUIRE(p.L >= t_loop, "record rings shorter than the draft window");
   PLA_REQUIRE((int64_t)p.N * p.H <= 0x7fffffffLL, "N * H exceeds the grid limit");
   PLA_REQUIRE(aligned_at(p.h0, 16) && p.state_slot % 4 == 0 && aligned_at(p.w_q, 16) && aligned_at(p.w_k, 16) &&
@@ -315,9 +359,15 @@ static int launch_replay_verify(ReplayVerifyParams& p, const int64_t* strides, i
   if (t_loop <= 4) {
     if (onorm) kda_verify_dspark_kernel<4, true><<<grid, block, 0, s>>>(p);
     else kda_verify_dspark_kernel<4, false><<<grid, block, 0, s>>>(p);
-  } else {
+  } else if (t_loop <= 8) {
     if (onorm) kda_verify_dspark_kernel<8, true><<<grid, block, 0, s>>>(p);
     else kda_verify_dspark_kernel<8, false><<<grid, block, 0, s>>>(p);
+  } else if (t_loop <= 16) {
+    if (onorm) kda_verify_dspark_kernel<16, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<16, false><<<grid, block, 0, s>>>(p);
+  } else {
+    if (onorm) kda_verify_dspark_kernel<32, true><<<grid, block, 0, s>>>(p);
+    else kda_verify_dspark_kernel<32, false><<<grid, block, 0, s>>>(p);
   }
   return check_launch("kda_verify_dspark_kernel");
 }

@@ -163,8 +163,6 @@ def kda_replay_verify(*, mixed_qkv, raw_g, raw_beta, conv_weight, conv_state, ch
     _need(cu.numel() == N + 1 and N <= R, "query index count exceeds record capacity")
     _disjoint([out, records.rawv, records.rawk, records.g, records.beta, records.conv],
               [x, raw_g, raw_beta, conv_weight, conv_state, state, A_log, dt_bias, cu, src])
-    if Q > 8:
-        raise NotImplementedError(f"the gfx950 replay verify handles draft windows of up to 8 tokens, got Q={Q}")
     if N == 0:
         return out
     windows = records.conv

@@ -238,7 +238,7 @@ def kda_decode_mega(B, H, seed=0, device="cuda", dtype=torch.bfloat16, pad_rows=
     }
 
 
-def kda_replay_verify(N, H, num_draft, seed=0, device="cuda", ring_len=16, slots=None, lower_bound=-8.0,
+def kda_replay_verify(N, H, num_draft, seed=0, device="cuda", ring_len=None, slots=None, lower_bound=-8.0,
                       onorm=True, pad_rows=(), strided=True, index_dtype=torch.int32):
     """KDA speculative verify with replay records (ring mode): ``N`` requests of ``num_draft`` tokens.
 
@@ -252,6 +252,7 @@ def kda_replay_verify(N, H, num_draft, seed=0, device="cuda", ring_len=16, slots
     device = torch.device(device)
     g = _gen(seed)
     dim, T, W = H * D, N * num_draft, 4
+    ring_len = ring_len or max(16, num_draft)
     slots = slots or N + 2
 
     def bf16(*shape, scale=1.0):

@@ -58,7 +58,8 @@ def _check(w):
     return out
 
 
-@pytest.mark.parametrize("N,H,T", [(1, 4, 1), (3, 4, 2), (2, 6, 3), (8, 12, 4), (3, 4, 5), (2, 12, 7), (8, 12, 8), (64, 32, 4)])
+@pytest.mark.parametrize("N,H,T", [(1, 4, 1), (3, 4, 2), (2, 6, 3), (8, 12, 4), (3, 4, 5), (2, 12, 7), (8, 12, 8), (64, 32, 4),
+                                   (3, 4, 9), (2, 6, 13), (4, 4, 16), (3, 4, 17), (2, 6, 25), (4, 4, 32)])
 @pytest.mark.parametrize("onorm", [False, True])
 def test_verify_matches_oracle(N, H, T, onorm):
     _check(kda_replay_verify(N, H, T, seed=10 * N + T, onorm=onorm, strided=True))
@@ -91,8 +92,8 @@ def test_verify_rejects_bad_arguments():
     bad["replayssm_rawv"] = w["replayssm_rawv"][:, :, :2]
     with pytest.raises(RuntimeError, match="ring shorter than the draft window|invalid verify ring shape"):
         fused_kda_decode_mtp_dspark(**bad)
-    wide = kda_replay_verify(1, 4, 9, seed=1)
-    with pytest.raises(RuntimeError, match="up to 8 draft tokens"):
+    wide = kda_replay_verify(1, 4, 33, seed=1)
+    with pytest.raises(RuntimeError, match="up to 32 draft tokens"):
         fused_kda_decode_mtp_dspark(**wide)
     torch.cuda.synchronize()
     assert bool((w["replayssm_g"] == 3.0).all())

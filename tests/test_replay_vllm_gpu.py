@@ -100,7 +100,7 @@ def oracle(layer, x, offsets, slots, rec, out, null_block_id):
 
 
 @pytest.mark.parametrize("layout", ["DS", "SD"])
-@pytest.mark.parametrize("q,heads", [(1, 1), (3, 2), (5, 4), (8, 2)])
+@pytest.mark.parametrize("q,heads", [(1, 1), (3, 2), (5, 4), (8, 2), (11, 2), (16, 1), (21, 2), (32, 2)])
 @pytest.mark.parametrize("index_dtype,null_block_id", [(torch.int32, 0), (torch.int64, -1)])
 def test_replay_verify_paged(layout, q, heads, index_dtype, null_block_id):
     gen = torch.Generator().manual_seed(41 + q + heads)
@@ -170,10 +170,6 @@ def test_replay_verify_skips_malformed_intervals_and_rejects_bad_arguments():
         kda_replay_verify(**args, conv_state=layer.conv, checkpoint_state=layer.state, records=big,
                           query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS",
                           out=big.rawv.view(-1)[:16 * heads * D].view(16, heads * D))
-    wide = records_filled(4, heads, 9)
-    with pytest.raises(NotImplementedError, match="up to 8 tokens"):
-        kda_replay_verify(**args, conv_state=pages(6, heads, 9, "DS", gen).conv, checkpoint_state=layer.state, records=wide,
-                          query_start_loc=vector(offsets), state_indices=vector(slots), conv_state_layout="DS")
 
 
 # ---- commit --------------------------------------------------------------------------------------------
