@@ -331,6 +331,17 @@ int pla_kda_prefill_launch(
     void* o, void* workspace, int64_t workspace_bytes,
     int H, int K, int V, int act_dtype, void* stream);
 
+/*
+ * Rows of the 128-row state tile a wavefront owns (8, 16 or 32) that a k-last launch with
+ * rows_per_wave = 0 takes for a shape: the row count the auto-tuner measured for the nearest batch size
+ * of the same (kernel, heads, dtypes) if the built-in table holds the shape, else the size thresholds.
+ * The table is compiled in from pla_amd/lut/ (the reference compiles its dispatch from
+ * lut/tuned_result_<device>.csv: scripts/decode/generate_kernel_instantiations.py; tuner
+ * scripts/decode/auto_tune.py).  kernel: 0 = k_last, 1 = k_last_packed, 2 = k_last_mtp; tree: 1 for the
+ * eagle-tree mode; dtypes are PLA_* codes.  Host only, no GPU call.  Returns 0 for invalid arguments.
+ */
+int pla_tuned_rows_per_wave(int kernel, int tree, int act_dtype, int state_dtype, int H, int HV, int B);
+
 #ifdef __cplusplus
 }
 #endif

@@ -101,6 +101,8 @@ def load():
     lib.pla_gdn_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int, _c_int]
     lib.pla_kda_prefill_workspace_bytes.restype = _c_i64
     lib.pla_kda_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int]
+    lib.pla_tuned_rows_per_wave.restype = _c_int
+    lib.pla_tuned_rows_per_wave.argtypes = [_c_int] * 7
     for name, argtypes in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = _c_int

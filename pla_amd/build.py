@@ -46,6 +46,8 @@ def build_library(verbose=True):
     """Compile every HIP source and link the shared library. Always recompiles."""
     os.makedirs(LIB_DIR, exist_ok=True)
     os.makedirs(OBJ_DIR, exist_ok=True)
+    from .autotune import write_header
+    write_header()                       # the tuned table is compiled in from pla_amd/lut/*.csv
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(_compile, SOURCES))
     tmp = LIB_PATH + ".tmp"

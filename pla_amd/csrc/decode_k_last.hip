@@ -19,6 +19,9 @@
 
 #include "decode_common.h"
 #include "readonce_verify.h"
+#include "tuned_table.h"
+
+#include <type_traits>
 
 namespace pla {
 
@@ -36,6 +39,7 @@ struct KLastParams {
   int B, H, HV;
   int use_qk_l2norm, disable_state_update;
   const int32_t* num_accepted; int64_t stride_h0_indices_seq; int is_sglang;
+  int tuned_kernel;         // host only: which rows of the tuned table apply (TunedKernel)
 };
 
 // READONCE (verify of up to four draft tokens that writes no state, no snapshots and follows no tree):
@@ -523,11 +527,15 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
 // Measured on MI355X (packed GDN decode, HV = 32, us per step at 8 / 16 / 32 rows per wavefront):
 //   32 tiles 3.9 / 4.6 / 6.0    128 tiles 5.2 / 5.6 / 6.9     256 tiles 8.2 / 7.8 / 9.2
 //   512 tiles 15.8 / 15.4 / 14.8    2048 tiles 53.5 / 53.5 / 50.9    8192 tiles 207.6 / 205.8 / 190.3
-static int pick_rows_per_wave(int tiles, bool mtp) {
-  (void)mtp;
+static int pick_rows_per_wave(int tiles) {
   if (tiles >= 512) return 32;
   if (tiles >= 192) return 16;
   return 8;
+}
+// A shape the auto-tuner has measured takes its tuned row count, every other shape the thresholds above.
+static int pick_rows_per_wave(int kernel, int tree, int act_dtype, int state_dtype, int H, int HV, int B) {
+  const int tuned = tuned_rows_per_wave(kTunedRows, kTunedRowCount, kernel, tree, act_dtype, state_dtype, H, HV, B);
+  return tuned > 0 ? tuned : pick_rows_per_wave(B * HV);
 }
 
 template <typename act_t, bool IS_KDA, bool MTP, typename state_t>
@@ -585,7 +593,10 @@ static int launch_decode(const DecodeParams& d, unsigned tiles, int rpw, hipStre
 
 template <typename state_t>
 static int run_k_last_typed(const KLastParams& p, bool is_kda, bool mtp, int act_dtype, int rows_per_wave, void* stream) {
-  const int rpw = rows_per_wave > 0 ? rows_per_wave : pick_rows_per_wave(p.B * p.HV, mtp);
+  const int rpw = rows_per_wave > 0 ? rows_per_wave
+                                    : pick_rows_per_wave(p.tuned_kernel, p.parents != nullptr, act_dtype,
+                                                         std::is_same<state_t, float>::value ? PLA_F32 : PLA_BF16,
+                                                         p.H, p.HV, p.B);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool lean = !mtp && p.T_max == 1 && p.alog_dtype == PLA_F32 && p.gate_mode == PLA_GATE_SOFTPLUS &&
                     !p.dt_bias_is_f32 && !p.beta_is_activated && p.h0 != nullptr;
@@ -650,6 +661,7 @@ extern "C" int pla_k_last_packed_launch(
   p.stride_a = stride_a; p.stride_q = p.stride_k = p.stride_v = stride_qkv; p.stride_b = stride_b;
   p.h0_slot_stride = h0_slot_stride; p.B = B; p.H = H; p.HV = HV;
   p.use_qk_l2norm = use_qk_l2norm; p.disable_state_update = 0; p.is_sglang = is_sglang;
+  p.tuned_kernel = TUNED_K_LAST_PACKED;
   return run_k_last(p, is_kda != 0, false, act_dtype, state_dtype, rows_per_wave, stream);
 }
 
@@ -702,7 +714,13 @@ extern "C" int pla_k_last_launch(
   p.num_accepted = num_accepted; p.stride_h0_indices_seq = stride_h0_indices_seq; p.is_sglang = is_sglang;
   const bool mtp = T_max > 1 || disable_state_update || cache != nullptr || cache_indices != nullptr ||
                    parents != nullptr || stride_h0_indices_seq > 0;
+  p.tuned_kernel = mtp ? TUNED_K_LAST_MTP : TUNED_K_LAST;
   return run_k_last(p, is_kda != 0, mtp, act_dtype, state_dtype, rows_per_wave, stream);
+}
+
+extern "C" int pla_tuned_rows_per_wave(int kernel, int tree, int act_dtype, int state_dtype, int H, int HV, int B) {
+  if (kernel < TUNED_K_LAST || kernel > TUNED_K_LAST_MTP || H <= 0 || HV <= 0 || B <= 0) return 0;
+  return pick_rows_per_wave(kernel, tree != 0, act_dtype, state_dtype, H, HV, B);
 }
 
 static int launch_fold(const FoldParams& p, int act_dtype, void* stream) {
@@ -716,7 +734,7 @@ static int launch_fold(const FoldParams& p, int act_dtype, void* stream) {
               "state and record tensors require 16-byte alignment");
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const int rpw = pick_rows_per_wave((int)tiles, true);
+  const int rpw = pick_rows_per_wave((int)tiles);
   const dim3 block(256);
   if (act_dtype == PLA_BF16) {
     if (rpw == 32) hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 32>), dim3(tiles, 1), block, 0, s, p);
