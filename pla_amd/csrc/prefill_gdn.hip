@@ -62,8 +62,8 @@ struct GdnPrefillParams {
 
 // ---------------------------------------------------------------------------------------------
 // grid (chunk, H + 1), 256 threads.  blockIdx.y < H: L2 norm of q and k of one head for the
-// chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing) and
-// the transposed K tile; blockIdx.y == H: gate, beta and the chunk-local cumulative log-decay.
+// chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing);
+// blockIdx.y == H: gate, beta and the chunk-local cumulative log-decay.
 template <typename act_t>
 __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
   const int cb = staged_chunk(p.stg, p.stage, blockIdx.x, p.seq_chunk_off[p.N]);
