@@ -50,6 +50,9 @@ struct ReplayVerifyParams {
   // intervals are skipped (src/decode/kda_replayssm/kda_mtp_verify.cu:721-741).
   int native, null_block_id, slots, tokens;
   int64_t state_slot;
+  // Scratch windows with the layout [row, step, channel, 3] (window contiguous, channel pitch 3) and
+  // 16-byte aligned rows: records and windows leave through LDS as 16-byte vectors.
+  int wide_stores;
 };
 
 __device__ __forceinline__ int64_t index_at(const void* p, int wide, int64_t i) {
@@ -101,6 +104,13 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   __shared__ __align__(16) float sC[TMAX][TMAX];    // sC[t][j] = c_{j,t}
   float (*const sW)[128] = sQ;
   __shared__ float sBeta[TMAX], sNorm[2][2][TMAX], sSq[4][TMAX];
+  // Staging of what the workgroup writes besides o (draft windows of up to eight tokens): the raw q / k / v
+  // channel sequences [state taps, tokens] the conv windows are cut from, and the log-decay records.
+  constexpr bool STAGED = TMAX <= 8;
+  constexpr int SEQ = TMAX + 3;
+  __shared__ __align__(16) uint16_t sSeq[STAGED ? 3 : 1][STAGED ? 128 : 1][STAGED ? SEQ : 1];
+  __shared__ __align__(16) float sG[STAGED ? TMAX : 1][STAGED ? 128 : 1];
+  const bool staged = STAGED && p.wide_stores;
 
   // Small inputs first, the state tile after them: memory returns in issue order, so the convolution
   // starts as soon as its inputs are there while the 64 KiB tile is still in flight.  Wavefronts 0-1
@@ -127,6 +137,20 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
   }
   const float eA = __expf(p.a_log[h]);
   const float bias = p.dt_bias[ch];
+  if constexpr (STAGED) {
+    if (staged) {
+#pragma unroll
+      for (int j = 0; j < 3; ++j) {
+        sSeq[ia][i128][j] = ta[j];
+        if (qk_side) sSeq[1][i128][j] = tb[j];
+      }
+#pragma unroll
+      for (int t = 0; t < TMAX; ++t) {
+        sSeq[ia][i128][3 + t] = xa[t];
+        if (qk_side) sSeq[1][i128][3 + t] = xb[t];
+      }
+    }
+  }
 
   // state tile, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
   const Tile<float> h_tile(p.h0 + slot * p.state_slot + (int64_t)h * 16384);
@@ -150,11 +174,13 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       const float k = conv_step(ck, bf(xb[t]), cwb);
       sQ[t][tid] = q;
       sK[t][tid] = k;
-      p.ring_rawk[(ring_row + t) * 128 + tid] = to_bf(k);
+      if (!staged) {
+        p.ring_rawk[(ring_row + t) * 128 + tid] = to_bf(k);
 #pragma unroll
-      for (int j = 0; j < 3; ++j) {
-        p.ic_q[srow * p.ic[0][0] + t * p.ic[0][1] + ch * p.ic[0][2] + j * p.ic[0][3]] = to_bf(cq[j]);
-        p.ic_k[srow * p.ic[1][0] + t * p.ic[1][1] + ch * p.ic[1][2] + j * p.ic[1][3]] = to_bf(ck[j]);
+        for (int j = 0; j < 3; ++j) {
+          p.ic_q[srow * p.ic[0][0] + t * p.ic[0][1] + ch * p.ic[0][2] + j * p.ic[0][3]] = to_bf(cq[j]);
+          p.ic_k[srow * p.ic[1][0] + t * p.ic[1][1] + ch * p.ic[1][2] + j * p.ic[1][3]] = to_bf(ck[j]);
+        }
       }
       const float q2 = wave64_allreduce(q * q), k2 = wave64_allreduce(k * k);
       if (lane == 0) { sNorm[0][wave][t] = q2; sNorm[1][wave][t] = k2; }
@@ -166,12 +192,16 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       if (t >= n_tok) break;
       const float v = conv_step(cv, bf(xa[t]), cwa);
       sV[t][i128] = v;
-      p.ring_rawv[(ring_row + t) * 128 + i128] = to_bf(v);
-#pragma unroll
-      for (int j = 0; j < 3; ++j)
-        p.ic_v[srow * p.ic[2][0] + t * p.ic[2][1] + ch * p.ic[2][2] + j * p.ic[2][3]] = to_bf(cv[j]);
       const float gk = p.lower_bound * fast_sigmoid(eA * (bf(xb[t]) + bias));
-      p.ring_g[(ring_row + t) * 128 + i128] = gk;
+      if (!staged) {
+        p.ring_rawv[(ring_row + t) * 128 + i128] = to_bf(v);
+#pragma unroll
+        for (int j = 0; j < 3; ++j)
+          p.ic_v[srow * p.ic[2][0] + t * p.ic[2][1] + ch * p.ic[2][2] + j * p.ic[2][3]] = to_bf(cv[j]);
+        p.ring_g[(ring_row + t) * 128 + i128] = gk;
+      } else if constexpr (STAGED) {
+        sG[t][i128] = gk;
+      }
       sD[t][i128] = __expf(gk);
       if (i128 == 0) {
         const float b = fast_sigmoid(bf(xc[t]));
@@ -311,6 +341,42 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
           make_uint2(pack2<bf16_t>(val[0], val[1]), pack2<bf16_t>(val[2], val[3]));
     }
   }
+
+  // Records and windows last: nothing in this workgroup waits for them.
+  if constexpr (STAGED) {
+    if (staged) {
+      // Per token 208 vectors of 16 bytes.  Wavefront 0: post-conv k and v as bf16 (lanes 0-15, 16-31) and
+      // the log-decay (lanes 32-63); wavefront 1 + x: the window of tensor x (q, k, v) after the token,
+      // 48 vectors = 128 channels x 3 taps, taps t + 1 .. t + 3 of the channel's sequence.
+      if (wave == 0) {
+        for (int t = 0; t < n_tok; ++t) {
+          if (lane < 32) {
+            const bool is_v = lane >= 16;
+            const float* src = (is_v ? sV[t] : sK[t]) + 8 * (lane & 15);
+            const float4 a = *reinterpret_cast<const float4*>(src), b = *reinterpret_cast<const float4*>(src + 4);
+            uint16_t* dst = (is_v ? p.ring_rawv : p.ring_rawk) + (ring_row + t) * 128 + 8 * (lane & 15);
+            *reinterpret_cast<uint4*>(dst) = make_uint4(pack2<bf16_t>(a.x, a.y), pack2<bf16_t>(a.z, a.w),
+                                                        pack2<bf16_t>(b.x, b.y), pack2<bf16_t>(b.z, b.w));
+          } else {
+            *reinterpret_cast<float4*>(p.ring_g + (ring_row + t) * 128 + 4 * (lane - 32)) =
+                *reinterpret_cast<const float4*>(&sG[t][4 * (lane - 32)]);
+          }
+        }
+      } else if (lane < 48) {
+        const int x = wave - 1;
+        const uint16_t* src[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) src[e] = &sSeq[x][(8 * lane + e) / 3][1 + (8 * lane + e) % 3];
+        uint16_t* const dst = (x == 0 ? p.ic_q : x == 1 ? p.ic_k : p.ic_v) + srow * p.ic[x][0] + (int64_t)h * 384 + 8 * lane;
+        for (int t = 0; t < n_tok; ++t) {
+          uint32_t w[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = (uint32_t)src[2 * e][t] | ((uint32_t)src[2 * e + 1][t] << 16);
+          *reinterpret_cast<uint4*>(dst + t * p.ic[x][1]) = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+      }
+    }
+  }
 }
 
 // One thread per channel: copies the window of the selected step into the destination slot.
@@ -350,6 +416,15 @@ static int launch_replay_verify(ReplayVerifyParams& p, const int64_t* strides, i
               "fused output norm requires an aligned gate (token stride a multiple of 4), a weight and eps >= 0");
   for (int i = 0; i < 26; ++i) PLA_REQUIRE(strides[i] > 0, "stride %d must be positive", i);
   p.T = t_loop;
+  p.wide_stores = 1;
+  {
+    void* const windows[3] = {p.ic_q, p.ic_k, p.ic_v};
+    for (int x = 0; x < 3; ++x)
+      if (strides[14 + 4 * x + 2] != 3 || strides[14 + 4 * x + 3] != 1 || strides[14 + 4 * x] % 8 != 0 ||
+          strides[14 + 4 * x + 1] % 8 != 0 || !aligned_at(windows[x], 16))
+        p.wide_stores = 0;
+    if (!aligned_at(p.ring_rawk, 16) || !aligned_at(p.ring_rawv, 16) || !aligned_at(p.ring_g, 16)) p.wide_stores = 0;
+  }
   p.sx_q = strides[0]; p.sx_k = strides[1]; p.sx_v = strides[2]; p.sg = strides[3]; p.sbeta = strides[4];
   for (int t = 0; t < 3; ++t)
     for (int j = 0; j < 3; ++j) p.cs[t][j] = strides[5 + 3 * t + j];
