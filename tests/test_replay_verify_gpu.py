@@ -74,6 +74,18 @@ def test_verify_layouts_indices_and_padding(index_dtype, strided):
     assert torch.count_nonzero(out[0, 4:8]) > 0
 
 
+@pytest.mark.parametrize("T", [3, 8])
+def test_verify_with_transposed_scratch_windows(T):
+    """Scratch windows stored [row, step, 3, channels] (window-major) take the per-thread stores instead of
+    the 16-byte vectors of the [row, step, channels, 3] layout: same results."""
+    w = kda_replay_verify(3, 4, T, seed=90 + T, onorm=True)
+    for key in WIN_KEYS:
+        rows, steps, dim, taps = w[key].shape
+        w[key] = torch.zeros(rows, steps, taps, dim, dtype=torch.bfloat16, device="cuda").transpose(2, 3)
+        assert w[key].stride(3) == dim and w[key].stride(2) == 1
+    _check(w)
+
+
 def test_verify_rejects_bad_arguments():
     w = kda_replay_verify(2, 4, 4, seed=1)
     bad = dict(w)
