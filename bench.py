@@ -336,6 +336,47 @@ def bench_replay_verify(device, steps=100, N=64, H=32, T=4):
             "commit_us": round(us_commit, 2)}
 
 
+def bench_replay_paged(device, steps=100, N=64, H=32, Q=4, layout="SD"):
+    """The same verify + commit through the request-row (vLLM) contract: paged conv history + FP32 checkpoints,
+    records per request row, device-side commit plan, fold into the final slot, conv windows into the paged history."""
+    import torch
+    from pla_amd.decode.kda_replayssm_vllm import KDAReplayCommitContext, kda_replay_verify
+    from pla_amd.workloads import kda_replay_paged
+    w = kda_replay_paged(N, H, Q, slots=1024, layout=layout, seed=606, device=device)
+    out = torch.empty(w.tokens, H * 128, dtype=torch.bfloat16, device=device)
+
+    def timed(fn):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            fn()
+        for _ in range(10):
+            graph.replay()
+        torch.cuda.synchronize()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(steps):
+            graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / steps * 1e3
+
+    us_verify = timed(lambda: kda_replay_verify(out=out, **w.verify))
+    ctx = KDAReplayCommitContext.create([w.layer], Q, N, layout, 0)
+    g = torch.Generator().manual_seed(7)
+    sampled = torch.randint(0, Q + 1, (N,), generator=g).to(torch.int32).to(device)
+    us_commit = timed(lambda: ctx.commit(sampled, w.source, w.offsets, token_capacity=w.tokens))
+    touched = int((sampled > 0).sum())
+    return {"workload": "request-row KDA replay verify + commit over paged checkpoints (%s pages), B=%d, H=%d, %d draft tokens"
+                        % (layout, N, H, Q),
+            "verify_us": round(us_verify, 2), "verify_state_read_GBps": round(N * H * 65536 / us_verify / 1e3, 1),
+            "commit_us": round(us_commit, 2), "commit_state_GBps": round(touched * H * 131072 / us_commit / 1e3, 1)}
+
+
 def cpu_baseline_decode(w, sample_requests=32, reps=5):
     """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
     sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
@@ -427,6 +468,7 @@ def main():
         result["other_decode"].update(bf16_pool)
         result["decode_mega"] = bench_decode_mega(device)
         result["replay_verify"] = bench_replay_verify(device)
+        result["replay_paged"] = bench_replay_paged(device)
         torch.cuda.empty_cache()
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
         torch.cuda.empty_cache()

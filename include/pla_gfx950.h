@@ -112,12 +112,13 @@ int pla_k_last_launch(
  * Accepted-prefix commit: replays accept_lens[n] recorded tokens of request n into
  * its FP32 state, in place.  Replaces launch_fold
  * (src/decode/kda_replayssm/kda_mtp_abi.h:165-176; kernel
- * src/decode/kda_replayssm/kda_mtp_fold.cu:256-545), single layer per call.
+ * src/decode/kda_replayssm/kda_mtp_fold.cu:256-545), all layers in one launch.
  *
- *   h0    [slots,HV,128,128] float32, slot pitch h0_slot_stride
- *   rawk  [slots,H,L,128]  act dtype (pre-normalisation; L2-normalised inside)
- *   rawv  [slots,HV,L,128] act dtype
- *   gk    [slots,HV,L,128] float32 log-decay;  beta [slots,HV,L] float32
+ *   h0    [layers,slots,HV,128,128] float32, slot pitch h0_slot_stride, layer pitch h0_layer_stride
+ *   rawk  [layers,slots,H,L,128]  act dtype (pre-normalisation; L2-normalised inside)
+ *   rawv  [layers,slots,HV,L,128] act dtype
+ *   gk    [layers,slots,HV,L,128] float32 log-decay;  beta [layers,slots,HV,L] float32
+ *         (every tensor with its own slot and layer pitch, in elements; layers >= 1)
  *   slot_idx, accept_lens [B] int32.  slot <= null_block_id or accept_len <= 0 => untouched.
  *   track_idx, track_step [B] int32 or both NULL: the state after step track_step[n] (0-based) is also
  *         stored to slot track_idx[n] when that slot is > null_block_id.
@@ -128,6 +129,8 @@ int pla_kda_fold_launch(
     const int32_t* track_idx, const int32_t* track_step,
     int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
     int64_t gk_slot_stride, int64_t beta_slot_stride,
+    int layers, int64_t h0_layer_stride, int64_t rawv_layer_stride, int64_t rawk_layer_stride,
+    int64_t gk_layer_stride, int64_t beta_layer_stride,
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
 
 /*

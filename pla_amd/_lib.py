@@ -32,6 +32,7 @@ SIGNATURES = {
     "pla_kda_fold_launch": [
         _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
         _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
+        _c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
     "pla_kda_fold_native_launch": [
         _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,

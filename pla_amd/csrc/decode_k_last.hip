@@ -463,6 +463,8 @@ struct FoldParams {
   // records indexed by the request row instead of the slot; slots > 0 bounds every slot id.
   const int32_t* final_idx; const int32_t* track_idx; const int32_t* track_step;
   int track_is_len, records_by_request, slots;
+  // blockIdx.z selects the layer: every tensor has a layer pitch (elements of its own type).
+  int64_t h0_layer_stride, rawv_layer_stride, rawk_layer_stride, gk_layer_stride, beta_layer_stride;
 };
 
 template <typename act_t, int RPW>
@@ -489,15 +491,19 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
 
   // Each wavefront reads its rows of the source tile before it writes any of them, so the destinations
   // may alias the source slot.
-  const Tile<float> h_tile(p.h0 + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
+  const int64_t layer = blockIdx.z;
+  float* const pool = p.h0 + layer * p.h0_layer_stride;
+  const Tile<float> h_tile(pool + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
   float s[R][4];
   load_state<R>(h_tile, lane_off, s);
   const int64_t rec = p.records_by_request ? i_n : slot;
-  const act_t* const kp = reinterpret_cast<const act_t*>(p.rawk) + rec * p.rawk_slot_stride + (int64_t)i_h * p.L * 128;
-  const act_t* const vp = reinterpret_cast<const act_t*>(p.rawv) + rec * p.rawv_slot_stride + (int64_t)i_hv * p.L * 128 + rowbase;
-  const float* const gp = p.gk + rec * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
-  const float* const bp = p.beta + rec * p.beta_slot_stride + (int64_t)i_hv * p.L;
+  const act_t* const kp = reinterpret_cast<const act_t*>(p.rawk) + layer * p.rawk_layer_stride + rec * p.rawk_slot_stride +
+                          (int64_t)i_h * p.L * 128;
+  const act_t* const vp = reinterpret_cast<const act_t*>(p.rawv) + layer * p.rawv_layer_stride + rec * p.rawv_slot_stride +
+                          (int64_t)i_hv * p.L * 128 + rowbase;
+  const float* const gp = p.gk + layer * p.gk_layer_stride + rec * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
+  const float* const bp = p.beta + layer * p.beta_layer_stride + rec * p.beta_slot_stride + (int64_t)i_hv * p.L;
 
   for (int t = 0; t < n_acc; ++t) {
     float kv[4], gv[4], dec[4], vv[R], unused[R];
@@ -514,9 +520,9 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
     for (int e = 0; e < 4; ++e) { kv[e] *= kn; dec[e] = __expf(gv[e]); }
     delta_rows<R, true, false>(s, dec, 1.f, kv, kv, vv, bp[t], unused);
     if (tracked && t == track_at)
-      store_state<R>(Tile<float>(p.h0 + (int64_t)track_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
+      store_state<R>(Tile<float>(pool + (int64_t)track_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
   }
-  store_state<R>(Tile<float>(p.h0 + (int64_t)final_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
+  store_state<R>(Tile<float>(pool + (int64_t)final_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
 }
 
 // ---- host side ---------------------------------------------------------------
@@ -723,7 +729,7 @@ extern "C" int pla_tuned_rows_per_wave(int kernel, int tree, int act_dtype, int 
   return pick_rows_per_wave(kernel, tree != 0, act_dtype, state_dtype, H, HV, B);
 }
 
-static int launch_fold(const FoldParams& p, int act_dtype, void* stream) {
+static int launch_fold(const FoldParams& p, int act_dtype, void* stream, int layers = 1) {
   PLA_REQUIRE(p.h0 && p.rawv && p.rawk && p.gk && p.beta && p.slot_idx && p.accept_lens, "null tensor pointer");
   PLA_REQUIRE(p.B > 0 && p.L > 0, "fold requires B > 0 and L > 0");
   PLA_REQUIRE(p.H > 0 && p.HV >= p.H && p.HV % p.H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", p.H, p.HV);
@@ -732,18 +738,22 @@ static int launch_fold(const FoldParams& p, int act_dtype, void* stream) {
   PLA_REQUIRE(aligned(p.h0, 16) && p.h0_slot_stride % 4 == 0 && aligned(p.gk, 16) && p.gk_slot_stride % 4 == 0 &&
               aligned(p.rawk, 8) && p.rawk_slot_stride % 4 == 0 && aligned(p.rawv, 16) && p.rawv_slot_stride % 8 == 0,
               "state and record tensors require 16-byte alignment");
+  PLA_REQUIRE(layers >= 1 && layers <= 65535, "fold takes 1..65535 layers per launch, got %d", layers);
+  PLA_REQUIRE(layers == 1 || (p.h0_layer_stride % 4 == 0 && p.gk_layer_stride % 4 == 0 && p.rawk_layer_stride % 4 == 0 &&
+                              p.rawv_layer_stride % 8 == 0), "layer pitches require 16-byte alignment");
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  const int rpw = pick_rows_per_wave((int)tiles);
+  const int rpw = pick_rows_per_wave((int)tiles * layers);
   const dim3 block(256);
+  const unsigned z = (unsigned)layers;
   if (act_dtype == PLA_BF16) {
-    if (rpw == 32) hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 32>), dim3(tiles, 1), block, 0, s, p);
-    else if (rpw == 16) hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 16>), dim3(tiles, 2), block, 0, s, p);
-    else hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 8>), dim3(tiles, 4), block, 0, s, p);
+    if (rpw == 32) hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 32>), dim3(tiles, 1, z), block, 0, s, p);
+    else if (rpw == 16) hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 16>), dim3(tiles, 2, z), block, 0, s, p);
+    else hipLaunchKernelGGL((kda_fold_kernel<bf16_t, 8>), dim3(tiles, 4, z), block, 0, s, p);
   } else {
-    if (rpw == 32) hipLaunchKernelGGL((kda_fold_kernel<f16_t, 32>), dim3(tiles, 1), block, 0, s, p);
-    else if (rpw == 16) hipLaunchKernelGGL((kda_fold_kernel<f16_t, 16>), dim3(tiles, 2), block, 0, s, p);
-    else hipLaunchKernelGGL((kda_fold_kernel<f16_t, 8>), dim3(tiles, 4), block, 0, s, p);
+    if (rpw == 32) hipLaunchKernelGGL((kda_fold_kernel<f16_t, 32>), dim3(tiles, 1, z), block, 0, s, p);
+    else if (rpw == 16) hipLaunchKernelGGL((kda_fold_kernel<f16_t, 16>), dim3(tiles, 2, z), block, 0, s, p);
+    else hipLaunchKernelGGL((kda_fold_kernel<f16_t, 8>), dim3(tiles, 4, z), block, 0, s, p);
   }
   return check_launch("kda_fold_kernel launch");
 }
@@ -754,11 +764,14 @@ extern "C" int pla_kda_fold_launch(
     const int32_t* track_idx, const int32_t* track_step,
     int64_t h0_slot_stride, int64_t rawv_slot_stride, int64_t rawk_slot_stride,
     int64_t gk_slot_stride, int64_t beta_slot_stride,
+    int layers, int64_t h0_layer_stride, int64_t rawv_layer_stride, int64_t rawk_layer_stride,
+    int64_t gk_layer_stride, int64_t beta_layer_stride,
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream) {
   FoldParams p{h0, rawv, rawk, gk, beta, slot_idx, accept_lens,
                h0_slot_stride, rawv_slot_stride, rawk_slot_stride, gk_slot_stride, beta_slot_stride,
-               B, H, HV, L, null_block_id, nullptr, track_idx, track_step, 0, 0, 0};
-  return launch_fold(p, act_dtype, stream);
+               B, H, HV, L, null_block_id, nullptr, track_idx, track_step, 0, 0, 0,
+               h0_layer_stride, rawv_layer_stride, rawk_layer_stride, gk_layer_stride, beta_layer_stride};
+  return launch_fold(p, act_dtype, stream, layers);
 }
 
 extern "C" int pla_kda_fold_native_launch(

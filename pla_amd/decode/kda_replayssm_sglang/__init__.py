@@ -37,7 +37,7 @@ def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, ac
     temporal [layers, slots, HV, 128, 128] float32; rawv [layers, slots, HV, L, 128] and
     rawk [layers, slots, H, L, 128] in bf16/fp16; gk [layers, slots, HV, L, 128] float32
     log-decay; beta [layers, slots, HV, L] float32; indices / lengths int32 [B].
-    One launch per layer on the current stream.
+    One launch for all layers on the current stream.
     """
     if temporal.dim() != 5 or temporal.dtype != torch.float32:
         raise RuntimeError("temporal must be float32 [layers, slots, HV, V, K]")
@@ -69,11 +69,13 @@ def fold_accepted_prefix(temporal, rawv, rawk, gk, beta, state_batch_indices, ac
         raise RuntimeError("temporal slots must be dense [HV, V, K]")
     stream = _lib.current_stream(temporal.device)
     act = _lib.dtype_code(rawk.dtype)
-    for layer in range(layers):
-        _lib.call("pla_kda_fold_launch", temporal[layer].data_ptr(), rawv[layer].data_ptr(), rawk[layer].data_ptr(),
-                  gk[layer].data_ptr(), beta[layer].data_ptr(), state_batch_indices.data_ptr(),
-                  accept_lens.data_ptr(), _lib.ptr(track_indices), _lib.ptr(track_steps), temporal.stride(1), rawv.stride(1), rawk.stride(1), gk.stride(1),
-                  beta.stride(1), B, H, HV, L, int(null_block_id), act, stream)
+    if layers == 0 or B == 0:
+        return
+    _lib.call("pla_kda_fold_launch", temporal.data_ptr(), rawv.data_ptr(), rawk.data_ptr(), gk.data_ptr(), beta.data_ptr(),
+              state_batch_indices.data_ptr(), accept_lens.data_ptr(), _lib.ptr(track_indices), _lib.ptr(track_steps),
+              temporal.stride(1), rawv.stride(1), rawk.stride(1), gk.stride(1), beta.stride(1),
+              layers, temporal.stride(0), rawv.stride(0), rawk.stride(0), gk.stride(0), beta.stride(0),
+              B, H, HV, L, int(null_block_id), act, stream)
 
 
 def _index(t):
@@ -164,7 +166,7 @@ def fused_kda_decode_mtp_dspark(*, x_q, x_k, x_v, w_q, w_k, w_v, cs_q, cs_k, cs_
     [slots, H*128, 3] and windows bf16 [rows, steps, H*128, 3] with any positive strides; state float32
     [slots, H, 128, 128], rings [slots, H, L, 128] (bf16 rawv / rawk, float32 g) and [slots, H, L] (float32
     beta), ``out`` bf16, all contiguous; index tensors int32 or int64.  ``T`` must be ``N`` times the draft
-    window, which is limited to 8 tokens here.
+    window (at most 32 tokens, as in the reference).
     """
     rings = (replayssm_rawv, replayssm_rawk, replayssm_g, replayssm_beta)
     if any(r is None for r in rings):

@@ -299,3 +299,43 @@ def kda_replay_verify(N, H, num_draft, seed=0, device="cuda", ring_len=None, slo
         out.update(onorm_gate=onorm_gate, onorm_weight=(torch.rand(D, generator=g) * 0.5 + 0.75).to(device),
                    onorm_eps=1e-6)
     return out
+
+
+def kda_replay_paged(N, H, Q, slots=None, layout="DS", seed=0, device="cuda", lower_bound=-5.0, history=None):
+    """Request-row (vLLM-style) KDA replay workload: ``N`` requests of ``Q`` draft tokens over paged caches.
+
+    Every page holds the conv history of the 3*H*128 channels (``DS`` = [channels, history], ``SD`` =
+    [history, channels]) followed by the FP32 checkpoint [H, 128, 128], as the reference's test lays its
+    pages out (tests/test_kda_replayssm_vllm.py:45-96).  Returns a namespace with the keyword arguments of
+    ``kda_replay_verify`` (``verify``), the layer object a ``KDAReplayCommitContext`` takes (``layer``) and
+    the index vectors."""
+    from types import SimpleNamespace
+    from .decode.kda_replayssm_vllm import KDAReplayRecords
+    device = torch.device(device)
+    g = _gen(seed)
+    slots = slots or 2 * N + 1
+    c = 3 * H * D
+    history = history or Q + 2
+    conv_shape = (c, history) if layout == "DS" else (history, c)
+    state_offset = ((c * history * 2 + 15) // 16) * 16
+    page_bytes = ((state_offset + H * D * D * 4 + 255) // 256) * 256
+    raw = torch.zeros(slots * page_bytes, dtype=torch.uint8, device=device)
+    conv = raw.view(torch.bfloat16).as_strided((slots, *conv_shape), (page_bytes // 2, *torch.empty(conv_shape).stride()))
+    state = raw.view(torch.float32).as_strided((slots, H, D, D), (page_bytes // 4, D * D, D, 1), state_offset // 4)
+    for s0 in range(0, slots, 64):                      # bounded host staging
+        n = min(64, slots - s0)
+        conv[s0:s0 + n].copy_((torch.randn(n, *conv_shape, generator=g) * 0.2).to(torch.bfloat16))
+        state[s0:s0 + n].copy_(torch.randn(n, H, D, D, generator=g) * 0.1)
+    T = N * Q
+    rows = (torch.randn(T, 4 * H * D + H, generator=g) * 0.4).to(torch.bfloat16).to(device)
+    hd = H * D
+    records = KDAReplayRecords.allocate(N, H, Q, device)
+    source = (1 + torch.randperm(slots - 1, generator=g)[:N]).to(torch.int32).to(device)      # slot 0 is the null block
+    offsets = torch.arange(0, T + 1, Q, dtype=torch.int32, device=device)
+    verify = dict(mixed_qkv=rows[:, :3 * hd], raw_g=rows[:, 3 * hd:4 * hd], raw_beta=rows[:, 4 * hd:],
+                  conv_weight=(torch.randn(3 * hd, 4, generator=g) * 0.2).to(device),
+                  A_log=(torch.randn(H, generator=g) * 0.1).to(device), dt_bias=(torch.randn(hd, generator=g) * 0.2).to(device),
+                  lower_bound=lower_bound, conv_state=conv, checkpoint_state=state, records=records,
+                  query_start_loc=offsets, state_indices=source, conv_state_layout=layout, null_block_id=0)
+    layer = SimpleNamespace(kv_cache=(conv, state), replay_records=records)
+    return SimpleNamespace(verify=verify, layer=layer, source=source, offsets=offsets, raw=raw, tokens=T)

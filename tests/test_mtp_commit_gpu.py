@@ -73,16 +73,23 @@ def test_config2_kda_mtp_verify_and_commit(B, slots):
     assert torch.equal(m["backing"][~touched], before[~touched])
 
 
-def test_commit_null_slots_and_clamped_lengths():
+@pytest.mark.parametrize("layers,padded", [(2, False), (3, True)])
+def test_commit_null_slots_and_clamped_lengths(layers, padded):
+    """All layers fold in one launch; with `padded` every tensor is a view with a layer pitch larger than its
+    extent (two spare slots per layer), whose spare slots must stay untouched."""
     from pla_amd.decode.kda_replayssm_sglang import fold_accepted_prefix
     g = torch.Generator().manual_seed(5)
-    layers, slots, H, HV, L = 2, 6, 2, 4, 3
+    slots, H, HV, L = 6, 2, 4, 3
     dev = "cuda"
-    temporal = (torch.randn(layers, slots, HV, 128, 128, generator=g) * 0.1).to(dev)
-    rawk = torch.randn(layers, slots, H, L, 128, generator=g).bfloat16().to(dev)
-    rawv = torch.randn(layers, slots, HV, L, 128, generator=g).bfloat16().to(dev)
-    gk = (-torch.rand(layers, slots, HV, L, 128, generator=g)).to(dev)
-    beta = torch.rand(layers, slots, HV, L, generator=g).to(dev)
+    spare = 2 if padded else 0
+    view = lambda t: t[:, :slots]
+    temporal_all = (torch.randn(layers, slots + spare, HV, 128, 128, generator=g) * 0.1).to(dev)
+    rawk_all = torch.randn(layers, slots + spare, H, L, 128, generator=g).bfloat16().to(dev)
+    rawv_all = torch.randn(layers, slots + spare, HV, L, 128, generator=g).bfloat16().to(dev)
+    gk_all = (-torch.rand(layers, slots + spare, HV, L, 128, generator=g)).to(dev)
+    beta_all = torch.rand(layers, slots + spare, HV, L, generator=g).to(dev)
+    temporal, rawk, rawv, gk, beta = (view(t) for t in (temporal_all, rawk_all, rawv_all, gk_all, beta_all))
+    spare_before = temporal_all[:, slots:].clone()
     idx = torch.tensor([4, 0, -1, 2], dtype=torch.int32, device=dev)
     acc = torch.tensor([2, 0, 3, 99], dtype=torch.int32, device=dev)      # 99 is clamped to L
     before = temporal.clone()
@@ -94,6 +101,7 @@ def test_commit_null_slots_and_clamped_lengths():
         assert torch.equal(temporal[layer, [0, 1, 3, 5]], before[layer, [0, 1, 3, 5]])
         for slot in (4, 2):
             assert rel_l2(temporal[layer, slot], exp[slot]) <= 1e-4
+    assert torch.equal(temporal_all[:, slots:], spare_before)
     # with null_block_id = 0 slot 0 would be a null block as well; here slot 0 had accept 0 anyway
     temporal.copy_(before)
     fold_accepted_prefix(temporal, rawv, rawk, gk, beta, idx, acc, null_block_id=4)
