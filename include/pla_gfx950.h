@@ -134,19 +134,42 @@ int pla_kda_fold_launch(
     int B, int H, int HV, int L, int null_block_id, int act_dtype, void* stream);
 
 /*
- * The fold of one layer driven by a commit plan over paged checkpoints with request-row records (vLLM
- * ReplaySSM).  Replaces launch_fold_native (src/decode/kda_replayssm/kda_mtp_abi.h:139-144) for one layer:
- * request n replays lengths[n] tokens of records row n from state[source[n]] and stores the result to
+ * Layer table of the paged (vLLM ReplaySSM) commit: device memory, PLA_LAYER_TABLE_ENTRIES int64 per layer
+ * (the reference passes a table of layer descriptors the same way: `const int64_t* layers`,
+ * src/decode/kda_replayssm/kda_mtp_abi.h:139-150).  Entries of layer l:
+ *   0 checkpoint pool (float*, [slots,H,128,128]), 1 its slot pitch in floats,
+ *   2 rawv, 3 rawk (bf16 [R,H,Q,128], dense), 4 gate (float [R,H,Q,128]), 5 beta (float [R,H,Q]),
+ *   6 conv history (bf16*), 7-9 its slot / channel / tap pitches in elements,
+ *   10 record windows (bf16*, [R,Q,channels,3]), 11-14 their row / step / channel / tap pitches, 15 unused.
+ * Pools and records need 16-byte aligned bases, slot pitches a multiple of 4 floats.
+ */
+#define PLA_LAYER_TABLE_ENTRIES 16
+
+/*
+ * The fold of all layers driven by a commit plan over paged checkpoints with request-row records.  Replaces
+ * launch_fold_native (src/decode/kda_replayssm/kda_mtp_abi.h:139-144): in every layer, request n replays
+ * lengths[n] tokens of records row n from state[source[n]] and stores the result to
  * state[final_indices[n]]; when boundary_lengths[n] > 0 the state after that many tokens also goes to
  * state[boundary_indices[n]].  Destinations may equal the source slot.  Requests with lengths[n] <= 0 or a
- * source / final slot outside (null_block_id, slots) are skipped.  Records: rawv, rawk [R,H,Q,128] bf16,
- * gate [R,H,Q,128], beta [R,H,Q] float32, dense.
+ * source / final slot outside (null_block_id, slots) are skipped.
  */
 int pla_kda_fold_native_launch(
-    float* state, int64_t state_slot_stride, const void* rawv, const void* rawk, const float* gate, const float* beta,
+    const int64_t* layer_table, int layers,
     const int32_t* source, const int32_t* lengths, const int32_t* final_indices,
     const int32_t* boundary_indices, const int32_t* boundary_lengths,
     int batch, int heads, int Q, int slots, int null_block_id, void* stream);
+
+/*
+ * The conv part of the same commit, all layers in one launch.  Replaces launch_conv_native
+ * (src/decode/kda_replayssm/kda_mtp_abi.h:146-150): request n copies the record window after its
+ * boundary_lengths[n]-th token into the conv history of slot boundary_indices[n] (when that length is
+ * positive), then the window after its lengths[n]-th token into slot final_indices[n]; destinations
+ * outside [0, slots) are skipped.  channels = 3 * H * 128, rows = record rows R.
+ */
+int pla_kda_conv_native_launch(
+    const int64_t* layer_table, int layers, const int32_t* lengths, const int32_t* final_indices,
+    const int32_t* boundary_indices, const int32_t* boundary_lengths,
+    int batch, int channels, int Q, int rows, int slots, void* stream);
 
 /*
  * Fused KDA decode step (one token per request): width-4 causal conv1d update + SiLU on the packed

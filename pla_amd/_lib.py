@@ -35,7 +35,10 @@ SIGNATURES = {
         _c_int, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
     "pla_kda_fold_native_launch": [
-        _c_p, _c_i64, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_int, _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_kda_conv_native_launch": [
+        _c_p, _c_int, _c_p, _c_p, _c_p, _c_p,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
     "pla_kda_decode_mega_launch": [
         _c_int, _c_int, _c_int, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p, _c_p,

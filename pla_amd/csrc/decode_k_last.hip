@@ -463,8 +463,10 @@ struct FoldParams {
   // records indexed by the request row instead of the slot; slots > 0 bounds every slot id.
   const int32_t* final_idx; const int32_t* track_idx; const int32_t* track_step;
   int track_is_len, records_by_request, slots;
-  // blockIdx.z selects the layer: every tensor has a layer pitch (elements of its own type).
+  // blockIdx.z selects the layer: every tensor has a layer pitch (elements of its own type), or, with a
+  // layer table (device memory, PLA_LAYER_TABLE_ENTRIES int64 per layer), its own base pointers.
   int64_t h0_layer_stride, rawv_layer_stride, rawk_layer_stride, gk_layer_stride, beta_layer_stride;
+  const int64_t* layer_table;
 };
 
 template <typename act_t, int RPW>
@@ -492,18 +494,32 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
   // Each wavefront reads its rows of the source tile before it writes any of them, so the destinations
   // may alias the source slot.
   const int64_t layer = blockIdx.z;
-  float* const pool = p.h0 + layer * p.h0_layer_stride;
-  const Tile<float> h_tile(pool + (int64_t)slot * p.h0_slot_stride + (int64_t)i_hv * 16384);
+  float* pool = p.h0 + layer * p.h0_layer_stride;
+  int64_t h0_slot_stride = p.h0_slot_stride;
+  const void* rawk = p.rawk;
+  const void* rawv = p.rawv;
+  const float* gk = p.gk;
+  const float* beta = p.beta;
+  if (p.layer_table != nullptr) {
+    const int64_t* const e = p.layer_table + layer * PLA_LAYER_TABLE_ENTRIES;
+    pool = reinterpret_cast<float*>(e[0]);
+    h0_slot_stride = e[1];
+    rawv = reinterpret_cast<const void*>(e[2]);
+    rawk = reinterpret_cast<const void*>(e[3]);
+    gk = reinterpret_cast<const float*>(e[4]);
+    beta = reinterpret_cast<const float*>(e[5]);
+  }
+  const Tile<float> h_tile(pool + (int64_t)slot * h0_slot_stride + (int64_t)i_hv * 16384);
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;
   float s[R][4];
   load_state<R>(h_tile, lane_off, s);
   const int64_t rec = p.records_by_request ? i_n : slot;
-  const act_t* const kp = reinterpret_cast<const act_t*>(p.rawk) + layer * p.rawk_layer_stride + rec * p.rawk_slot_stride +
+  const act_t* const kp = reinterpret_cast<const act_t*>(rawk) + layer * p.rawk_layer_stride + rec * p.rawk_slot_stride +
                           (int64_t)i_h * p.L * 128;
-  const act_t* const vp = reinterpret_cast<const act_t*>(p.rawv) + layer * p.rawv_layer_stride + rec * p.rawv_slot_stride +
+  const act_t* const vp = reinterpret_cast<const act_t*>(rawv) + layer * p.rawv_layer_stride + rec * p.rawv_slot_stride +
                           (int64_t)i_hv * p.L * 128 + rowbase;
-  const float* const gp = p.gk + layer * p.gk_layer_stride + rec * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
-  const float* const bp = p.beta + layer * p.beta_layer_stride + rec * p.beta_slot_stride + (int64_t)i_hv * p.L;
+  const float* const gp = gk + layer * p.gk_layer_stride + rec * p.gk_slot_stride + (int64_t)i_hv * p.L * 128;
+  const float* const bp = beta + layer * p.beta_layer_stride + rec * p.beta_slot_stride + (int64_t)i_hv * p.L;
 
   for (int t = 0; t < n_acc; ++t) {
     float kv[4], gv[4], dec[4], vv[R], unused[R];
@@ -520,9 +536,9 @@ __global__ __launch_bounds__(256) void kda_fold_kernel(const FoldParams p) {
     for (int e = 0; e < 4; ++e) { kv[e] *= kn; dec[e] = __expf(gv[e]); }
     delta_rows<R, true, false>(s, dec, 1.f, kv, kv, vv, bp[t], unused);
     if (tracked && t == track_at)
-      store_state<R>(Tile<float>(pool + (int64_t)track_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
+      store_state<R>(Tile<float>(pool + (int64_t)track_slot * h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
   }
-  store_state<R>(Tile<float>(pool + (int64_t)final_slot * p.h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
+  store_state<R>(Tile<float>(pool + (int64_t)final_slot * h0_slot_stride + (int64_t)i_hv * 16384), lane_off, s);
 }
 
 // ---- host side ---------------------------------------------------------------
@@ -730,13 +746,14 @@ extern "C" int pla_tuned_rows_per_wave(int kernel, int tree, int act_dtype, int 
 }
 
 static int launch_fold(const FoldParams& p, int act_dtype, void* stream, int layers = 1) {
-  PLA_REQUIRE(p.h0 && p.rawv && p.rawk && p.gk && p.beta && p.slot_idx && p.accept_lens, "null tensor pointer");
+  PLA_REQUIRE((p.layer_table || (p.h0 && p.rawv && p.rawk && p.gk && p.beta)) && p.slot_idx && p.accept_lens, "null tensor pointer");
   PLA_REQUIRE(p.B > 0 && p.L > 0, "fold requires B > 0 and L > 0");
   PLA_REQUIRE(p.H > 0 && p.HV >= p.H && p.HV % p.H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", p.H, p.HV);
   PLA_REQUIRE(act_dtype == PLA_BF16 || act_dtype == PLA_F16, "record dtype must be bf16 or fp16");
   PLA_REQUIRE((p.track_idx == nullptr) == (p.track_step == nullptr), "track indices and steps must be given together");
-  PLA_REQUIRE(aligned(p.h0, 16) && p.h0_slot_stride % 4 == 0 && aligned(p.gk, 16) && p.gk_slot_stride % 4 == 0 &&
-              aligned(p.rawk, 8) && p.rawk_slot_stride % 4 == 0 && aligned(p.rawv, 16) && p.rawv_slot_stride % 8 == 0,
+  PLA_REQUIRE(p.layer_table != nullptr ||
+              (aligned(p.h0, 16) && p.h0_slot_stride % 4 == 0 && aligned(p.gk, 16) && p.gk_slot_stride % 4 == 0 &&
+               aligned(p.rawk, 8) && p.rawk_slot_stride % 4 == 0 && aligned(p.rawv, 16) && p.rawv_slot_stride % 8 == 0),
               "state and record tensors require 16-byte alignment");
   PLA_REQUIRE(layers >= 1 && layers <= 65535, "fold takes 1..65535 layers per launch, got %d", layers);
   PLA_REQUIRE(layers == 1 || (p.h0_layer_stride % 4 == 0 && p.gk_layer_stride % 4 == 0 && p.rawk_layer_stride % 4 == 0 &&
@@ -775,16 +792,16 @@ extern "C" int pla_kda_fold_launch(
 }
 
 extern "C" int pla_kda_fold_native_launch(
-    float* state, int64_t state_slot_stride, const void* rawv, const void* rawk, const float* gate, const float* beta,
+    const int64_t* layer_table, int layers,
     const int32_t* source, const int32_t* lengths, const int32_t* final_indices,
     const int32_t* boundary_indices, const int32_t* boundary_lengths,
     int batch, int heads, int Q, int slots, int null_block_id, void* stream) {
-  PLA_REQUIRE(final_indices && boundary_indices && boundary_lengths, "null plan pointer");
+  PLA_REQUIRE(layer_table && final_indices && boundary_indices && boundary_lengths, "null table or plan pointer");
   PLA_REQUIRE(slots > 0 && (null_block_id == -1 || null_block_id == 0), "paged fold requires slots > 0 and null_block_id -1 or 0");
   if (batch == 0) return 0;
-  FoldParams p{state, rawv, rawk, gate, beta, source, lengths,
-               state_slot_stride, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128,
+  FoldParams p{nullptr, nullptr, nullptr, nullptr, nullptr, source, lengths,
+               0, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128, (int64_t)heads * Q * 128,
                (int64_t)heads * Q, batch, heads, heads, Q, null_block_id,
-               final_indices, boundary_indices, boundary_lengths, 1, 1, slots};
-  return launch_fold(p, PLA_BF16, stream);
+               final_indices, boundary_indices, boundary_lengths, 1, 1, slots, 0, 0, 0, 0, 0, layer_table};
+  return launch_fold(p, PLA_BF16, stream, layers);
 }

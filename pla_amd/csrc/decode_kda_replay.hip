@@ -397,6 +397,33 @@ __global__ __launch_bounds__(256) void conv_window_scatter_kernel(
   for (int w = 0; w < km1; ++w) dp[w * d_win] = sp[w * s_win];
 }
 
+// Conv windows of a commit plan into the paged conv histories of all layers: request r copies the window
+// after its boundary_lengths[r]-th token to slot boundary[r] (if any) and then the window after its
+// lengths[r]-th token to slot final[r]; one thread per channel does both, in this order.  Layer pointers
+// and strides come from the layer table (entries 6-14).
+__global__ __launch_bounds__(256) void conv_window_native_kernel(
+    const int64_t* layer_table, const int32_t* lengths, const int32_t* final_idx, const int32_t* boundary_idx,
+    const int32_t* boundary_lengths, int channels, int steps, int rows, int slots) {
+  const int r = blockIdx.x;
+  const int d = blockIdx.z * 256 + threadIdx.x;
+  if (d >= channels || r >= rows) return;
+  const int64_t* const e = layer_table + (int64_t)blockIdx.y * PLA_LAYER_TABLE_ENTRIES;
+  uint16_t* const conv = reinterpret_cast<uint16_t*>(e[6]);
+  const uint16_t* const win = reinterpret_cast<const uint16_t*>(e[10]);
+  const int64_t c_slot = e[7], c_ch = e[8], c_tap = e[9], w_row = e[11], w_step = e[12], w_ch = e[13], w_tap = e[14];
+  const int count[2] = {boundary_lengths[r], lengths[r]};
+  const int dest[2] = {boundary_idx[r], final_idx[r]};
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int step = count[i] - 1;
+    if (step < 0 || step >= steps || dest[i] < 0 || dest[i] >= slots) continue;
+    const uint16_t* sp = win + r * w_row + step * w_step + d * w_ch;
+    uint16_t* dp = conv + dest[i] * c_slot + d * c_ch;
+#pragma unroll
+    for (int w = 0; w < 3; ++w) dp[w * c_tap] = sp[w * w_tap];
+  }
+}
+
 static bool aligned_at(const void* ptr, size_t a) { return (reinterpret_cast<uintptr_t>(ptr) % a) == 0; }
 
 }  // namespace pla
@@ -540,4 +567,19 @@ extern "C" int pla_conv_window_scatter_launch(
         (const uint32_t*)src, (uint32_t*)dst, dst_idx, dst_idx_wide, step_idx, step_idx_wide, dim, km1,
         src_s0, src_s1, src_s2, src_s3, src_s4, dst_s0, dst_s1, dst_s2, dst_s3, src_reqs, src_steps, dst_reqs);
   return check_launch("conv_window_scatter_kernel");
+}
+
+extern "C" int pla_kda_conv_native_launch(
+    const int64_t* layer_table, int layers, const int32_t* lengths, const int32_t* final_indices,
+    const int32_t* boundary_indices, const int32_t* boundary_lengths,
+    int batch, int channels, int Q, int rows, int slots, void* stream) {
+  using namespace pla;
+  PLA_REQUIRE(layer_table && lengths && final_indices && boundary_indices && boundary_lengths, "null table or plan pointer");
+  PLA_REQUIRE(layers >= 1 && layers <= 65535 && channels > 0 && Q >= 1 && slots > 0 && batch <= rows,
+              "conv commit requires 1..65535 layers, channels > 0, Q >= 1, slots > 0 and batch <= record rows");
+  if (batch == 0) return 0;
+  const dim3 grid((unsigned)batch, (unsigned)layers, (unsigned)((channels + 255) / 256)), block(256);
+  conv_window_native_kernel<<<grid, block, 0, static_cast<hipStream_t>(stream)>>>(
+      layer_table, lengths, final_indices, boundary_indices, boundary_lengths, channels, Q, rows, slots);
+  return check_launch("conv_window_native_kernel");
 }

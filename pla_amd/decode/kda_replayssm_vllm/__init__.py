@@ -291,9 +291,21 @@ class KDAReplayCommitContext:
             views.append((ds, state, records))
         self = cls()
         self._layers, self._views = layers, tuple(views)
+        # one row of base pointers and pitches per layer (include/pla_gfx950.h: PLA_LAYER_TABLE_ENTRIES), so
+        # that one fold launch and one conv launch serve every layer
+        table = []
+        for ds, state, records in views:
+            win = records.conv
+            _need(state.data_ptr() % 16 == 0 and state.stride(0) % 4 == 0
+                  and all(t.data_ptr() % 16 == 0 for t in (records.rawv, records.rawk, records.g, records.beta)),
+                  "checkpoint pools and records require 16-byte alignment")
+            table.append([state.data_ptr(), state.stride(0), records.rawv.data_ptr(), records.rawk.data_ptr(),
+                          records.g.data_ptr(), records.beta.data_ptr(), ds.data_ptr(), *ds.stride(),
+                          win.data_ptr(), *win.stride(), 0])
+        self._table = torch.tensor(table, dtype=torch.int64).to(device)
+        self._channels, self._rows = views[0][0].size(1), views[0][2].conv.size(0)
         self._candidate = torch.zeros((4, max_num_reqs), dtype=torch.int32, device=device)
         self._buffer = torch.zeros_like(self._candidate)
-        self._steps = torch.zeros((2, max_num_reqs), dtype=torch.int32, device=device)
         self.plan = KDAReplayCommitPlan(*self._buffer.unbind(0))
         self._heads, self._slots = heads, slots
         self._q, self._capacity, self._null = spec_query_len, max_num_reqs, null_block_id
@@ -357,16 +369,10 @@ class KDAReplayCommitContext:
             if N == 0:
                 return self.plan
             lens, final, boundary, bc = (t[:N] for t in self._buffer.unbind(0))
-            torch.sub(lens, 1, out=self._steps[0, :N])          # window of the last committed token
-            torch.sub(bc, 1, out=self._steps[1, :N])            # -1 (skipped) without a boundary
-            for ds, state, records in self._views:
-                _lib.call("pla_kda_fold_native_launch", state.data_ptr(), state.stride(0), records.rawv.data_ptr(),
-                          records.rawk.data_ptr(), records.g.data_ptr(), records.beta.data_ptr(),
-                          source32.data_ptr(), lens.data_ptr(), final.data_ptr(), boundary.data_ptr(), bc.data_ptr(),
-                          N, self._heads, self._q, self._slots, self._null, stream)
-                win = records.conv
-                for dst_idx, steps in ((boundary, self._steps[1, :N]), (final, self._steps[0, :N])):
-                    _lib.call("pla_conv_window_scatter_launch", 2, 3, win.data_ptr(), ds.data_ptr(),
-                              dst_idx.data_ptr(), 0, steps.data_ptr(), 0, 1, ds.size(1), N,
-                              0, *win.stride(), 0, *ds.stride(), win.size(0), win.size(1), self._slots, stream)
+            plan = (lens.data_ptr(), final.data_ptr(), boundary.data_ptr(), bc.data_ptr())
+            nlayers = len(self._views)
+            _lib.call("pla_kda_fold_native_launch", self._table.data_ptr(), nlayers, source32.data_ptr(), *plan,
+                      N, self._heads, self._q, self._slots, self._null, stream)
+            _lib.call("pla_kda_conv_native_launch", self._table.data_ptr(), nlayers, *plan,
+                      N, self._channels, self._q, self._rows, self._slots, stream)
         return self.plan
