@@ -308,17 +308,20 @@ int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV);
  * (src/prefill/flashqla/host/torch_extension_cute.cc:60-148: chunk_local_cumsum_qk_norm_gated,
  * kkt_solve, fused_fwd) with one call that runs all stages on `stream`.
  *
- *   q,k [T,H,128], v [T,HV,128] bf16 with token pitches stride_q/k/v (views into a packed
- *       Q|K|V row are fine); a,b [T,HV] raw gate / beta logits (pitches stride_a/b) with
+ *   q,k [T,H,128], v [T,HV,128] in the activation dtype (act_dtype: PLA_BF16 or PLA_F16) with token
+ *       pitches stride_q/k/v (views into a packed Q|K|V row are fine); a,b [T,HV] raw gate / beta
+ *       logits in the same dtype (pitches stride_a/b) with
  *       A_log, dt_bias [HV] float32:  g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b);
  *       or g_in, beta_in [T,HV] float32 (log-decay per token, activated beta) instead.
- *   normalize_qk: L2-normalise q and k (eps 1e-6 inside the root) and round to bf16 first.
+ *   normalize_qk: L2-normalise q and k (eps 1e-6 inside the root) and round to the activation dtype first.
+ *   The matrix products take fp16 operands with FP32 accumulation: magnitudes above 65504 in v, the
+ *       state or the intermediate products are outside the supported range.
  *   cu_seqlens [N+1] int32; tokens at and beyond cu_seqlens[N] are padding: their rows of o
  *       are set to zero and they never touch a state.  Empty sequences keep their state.
  *   h0 / ht: k-last FP32 state [slots,HV,128,128] read at h0_indices[n] (or n when the index
  *       array is NULL; zero state when h0 is NULL) and written at ht_indices[n].  h0 == ht with
  *       the same indices updates an indexed pool in place.
- *   o [T,HV,128] bf16 dense.   gcum_out / beta_out: optional [T,HV] float32 copies of the
+ *   o [T,HV,128] activation dtype, dense.   gcum_out / beta_out: optional [T,HV] float32 copies of the
  *       chunk-local cumulative log-decay and of beta (NULL keeps them in the workspace).
  */
 int pla_gdn_prefill_launch(

@@ -92,8 +92,8 @@ def unsupported_reason(case):
             return f"the fused KDA decode step supports H in {_MEGA_HEADS}"
         if case.get("seqlen_q", 1) > 32:
             return "the KDA verify handles up to 32 draft tokens"
-    if case["phase"] == "P" and case.get("dtype") != "bf16":
-        return "prefill takes bf16 activations"
+    if case["phase"] == "P" and case["op"] == "kda_attn" and case.get("dtype") != "bf16":
+        return "KDA prefill takes bf16 activations"
     return None
 
 

@@ -37,4 +37,16 @@ __device__ __forceinline__ bf16x8_t round8(f32x4_t a, f32x4_t b) {
   return __builtin_convertvector(x, bf16x8_t);
 }
 
+// The same instruction shape with fp16 operands (v_mfma_f32_16x16x32_f16, same rate).  Operands travel as
+// eight 16-bit lanes in a bf16x8_t container (loads, LDS reads and transposing reads do not care what the
+// bits mean); half8 rounds two accumulator quads to fp16 (round to nearest even, 11 significant bits).
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f32x4_t mfma16h(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ bf16x8_t half8(f32x4_t a, f32x4_t b) {
+  const f32x8_t x = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+  return __builtin_bit_cast(bf16x8_t, __builtin_convertvector(x, f16x8_t));
+}
+
 }  // namespace pla

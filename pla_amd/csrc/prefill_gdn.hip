@@ -12,19 +12,24 @@
 // scripts/prefill/flashqla/private/ref_gdr.py:78-298; kernels
 // src/prefill/flashqla/kernels/chunk_cumsum_cute.cu:232-330, kkt_solve_cute_impl.cuh:34-60,
 // fused_fwd_cute.cu:34-66).  Because the gate is a scalar per (token, head) every decay is a
-// row or column scaling of a GEMM result, so the bf16 MFMA operands q, k, v stay exact;
-// the FP32 quantities that feed the state (S, X, W, U) are split into bf16 hi + lo parts
-// (16 mantissa bits), which keeps the FP32 final state within 1e-5 of a float64 evaluation.
+// row or column scaling of a GEMM result, and every factor lies in (0, 1].  All MFMA operands are
+// fp16 (v_mfma_f32_16x16x32_f16, the rate of the bf16 instruction): normalised q / k (rounded to the
+// activation dtype first, as the reference does, which fp16 then holds exactly) and the FP32
+// quantities S, X, W, U, P rounded once to fp16 (11 significant bits; accumulation and the state stay
+// FP32).  A float64 simulation of these rounding points over 8192 tokens gives a final-state rel-L2
+// of 3.7e-4 .. 4.8e-4 from strong decay to none at all (bound 1e-3), against 2.3e-3 .. 3.8e-3 for single
+// bf16 operands, which therefore need hi + lo pairs (1.75 x the MFMAs and six VALU operations per
+// element pair instead of one).  Operands beyond the fp16 range (|x| > 65504) are not supported.
 //
 // Kernels:
 //   chunk_map_kernel         chunk table from cu_seqlens (device side, graph-capturable)
 //   gdn_prep_kernel          gate, beta, chunk-local cumsum and per-chunk decay-factor tiles, q/k L2
-//                            norm (rounded to bf16)
+//                            norm (rounded to the activation dtype, stored as fp16)
 //   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
-//                            forward substitution in LDS, W (hi/lo) and P to the workspace
+//                            forward substitution in LDS, W and P (fp16) to the workspace
 //   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), four wavefronts each owning a
 //                            32-wide V slice of S^T in MFMA accumulator layout; the chain
-//                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_bf16 with every
+//                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_f16 with every
 //                            intermediate staying in registers (an accumulator tile is already a
 //                            valid B operand of the next product); A operands come from LDS tiles
 //                            filled by asynchronous global -> LDS copies one chunk ahead.
@@ -51,7 +56,7 @@ struct GdnPrefillParams {
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
   uint16_t* qn; uint16_t* kn;
   float* gcum; float* beta;
-  uint16_t* Whi; uint16_t* Wlo; uint16_t* P;
+  uint16_t* W; uint16_t* P;                           // fp16 [chunk, HV, 64, 64]
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
   SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
   StageTable stg;        // pipelined preparation and sweep (stg.stages > 0)
@@ -145,8 +150,10 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
     }
     if (j < len) {
       const int64_t t = t0 + j;
-      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2<bf16_t>(q0, q1);
-      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2<bf16_t>(k0, k1);
+      // rounded to the activation dtype (the reference's operand), then held as fp16
+      const uint32_t qa = pack2<act_t>(q0, q1), ka = pack2<act_t>(k0, k1);
+      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2<f16_t>(lo16<act_t>(qa), hi16<act_t>(qa));
+      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2<f16_t>(lo16<act_t>(ka), hi16<act_t>(ka));
     }
   }
 }
@@ -197,7 +204,7 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
     for (int ni = 0; ni <= mi; ++ni) {
       f32x4_t kk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < 4; ++s) kk = mfma16(Kop[mi][s], Kop[ni][s], kk);
+      for (int s = 0; s < 4; ++s) kk = mfma16h(Kop[mi][s], Kop[ni][s], kk);
       const int j = 16 * ni + r16;
       const float Gj = Gs[j];
 #pragma unroll
@@ -231,13 +238,13 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
       }
       f32x4_t qk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < 4; ++s) qk = mfma16(Qop[s], Kop[ni][s], qk);
+      for (int s = 0; s < 4; ++s) qk = mfma16h(Qop[s], Kop[ni][s], qk);
       const float Gj = Gs[j];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * mi + 4 * kb + r;
         const float gam = i >= j ? __expf(Gs[i] - Gj) : 0.f;
-        Pt[i * 64 + j] = from_float<bf16_t>(p.scale * qk[r] * gam).bits;
+        Pt[i * 64 + j] = from_float<f16_t>(p.scale * qk[r] * gam).bits;
       }
     }
   }
@@ -260,14 +267,9 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
     }
     x[i] = (a0 + a1) + (a2 + a3);
   }
-  uint16_t* const Wh = p.Whi + ((int64_t)cb * p.HV + hv) * 4096;
-  uint16_t* const Wl = p.Wlo + ((int64_t)cb * p.HV + hv) * 4096;
+  uint16_t* const Wt = p.W + ((int64_t)cb * p.HV + hv) * 4096;
 #pragma unroll
-  for (int i = 0; i < CHUNK; ++i) {
-    const bf16_t hi = from_float<bf16_t>(x[i]);
-    Wh[i * 64 + lane] = hi.bits;
-    Wl[i * 64 + lane] = from_float<bf16_t>(x[i] - to_float(hi)).bits;
-  }
+  for (int i = 0; i < CHUNK; ++i) Wt[i * 64 + lane] = from_float<f16_t>(x[i]).bits;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -314,8 +316,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tWh[CHUNK * PITCH64];
-  __shared__ __align__(16) uint16_t tWl[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
   __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
   // decay factors by chunk parity: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
@@ -346,8 +347,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-  const char* const wh_b = reinterpret_cast<const char*>(p.Whi) + ((int64_t)c_begin * p.HV + hv) * 8192;
-  const char* const wl_b = reinterpret_cast<const char*>(p.Wlo) + ((int64_t)c_begin * p.HV + hv) * 8192;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 8192;
   const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
   const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
 
@@ -379,10 +379,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       }
     }
   };
-  auto issue_w = [&](int c) {
-    plan_w.issue(tWh, wh_b + (int64_t)c * p.HV * 8192, wave);
-    plan_w.issue(tWl, wl_b + (int64_t)c * p.HV * 8192, wave);
-  };
+  auto issue_w = [&](int c) { plan_w.issue(tW, w_b + (int64_t)c * p.HV * 8192, wave); };
   auto issue_p = [&](int c) { plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave); };
   auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
     if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
@@ -435,10 +432,10 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
     float4 eg[4];
     uint16_t vraw[NB][16];
-    bf16x8_t wh[2][4], wl[2][4];
-    HiLo sb[2][NB];
+    bf16x8_t wa[2][4];
+    bf16x8_t sb[2][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = split8(St[nb][0], St[nb][1]);
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
@@ -462,37 +459,22 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wh[s2][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s2, kb);
-            wl[s2][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s2, kb);
-          }
+          for (int mi = 0; mi < 4; ++mi) wa[s2][mi] = operand_from(&tW[(16 * mi + r16) * PITCH64], s2, kb);
       }
       __builtin_amdgcn_sched_barrier(0);
-      // the split of the next step's state slice is interleaved with this step's MFMAs (one MFMA
-      // issues together with about two VALU instructions in its 16 cycles)
+      // the next step's state slice is rounded underneath this step's MFMAs
       if (s < 3) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = split8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[s & 1][nb].hi, QS[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(ka[s & 1][mi], sb[s & 1][nb].lo, KS[nb][mi]);
-      if (s < 3) {
-#pragma unroll
-        for (int i = 0; i < 12 * NB; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);   // three VALU
-        }
-      }
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
       __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - e^{G} (.) KS
@@ -514,21 +496,13 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      HiLo xb[NB];
+      bf16x8_t xb[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = split8(X[nb][2 * s], X[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].hi, U[nb][mi]);
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8(X[nb][2 * s], X[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wl[s][mi], xb[nb].hi, U[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
     }
 
     // barrier B: P of this chunk has landed; Q, V, W and the other K tile are free for the next chunk
@@ -569,23 +543,19 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      HiLo ub[NB];
+      bf16x8_t ub[NB];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
                             U[nb][2 * s][3] * dg[s][0].w};
         const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
                             U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
-        ub[nb] = split8(u0, u1);
+        ub[nb] = half8(u0, u1);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(kt[s][mc], ub[nb].hi, St[nb][mc]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(kt[s][mc], ub[nb].lo, St[nb][mc]);
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb], St[nb][mc]);
     }
 
     // O = scale e^{G} (.) QS + P U -> O tile
@@ -599,11 +569,11 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     for (int s = 0; s < 2; ++s) {
       bf16x8_t ur[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ur[nb] = round8(U[nb][2 * s], U[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(pa[s][mi], ur[nb], QS[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
     }
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -631,7 +601,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 }
 
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, Whi, Wlo, P;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, W, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -650,8 +620,7 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
   L.gtile = take((size_t)L.NC_max * HV * 256 * 4);
-  L.Whi = take((size_t)L.NC_max * HV * 4096 * 2);
-  L.Wlo = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.W = take((size_t)L.NC_max * HV * 4096 * 2);
   L.P = take((size_t)L.NC_max * HV * 4096 * 2);
   L.seg_chunks = pick_segment_chunks(T, N, HV);
   L.max_segments = max_segments(T, N, L.seg_chunks);
@@ -697,7 +666,8 @@ extern "C" int pla_gdn_prefill_launch(
   PLA_REQUIRE(K == 128 && V == 128, "GDN prefill requires head_dim K == V == 128, got K=%d, V=%d", K, V);
   PLA_REQUIRE(T > 0 && N > 0, "GDN prefill needs at least one token and one sequence");
   PLA_REQUIRE(H > 0 && HV >= H && HV % H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", H, HV);
-  PLA_REQUIRE(act_dtype == PLA_BF16, "GDN prefill takes bf16 activations (the MFMA operands are bf16)");
+  PLA_REQUIRE(act_dtype == PLA_BF16 || act_dtype == PLA_F16, "GDN prefill takes bf16 or fp16 activations");
+  const bool half_act = act_dtype == PLA_F16;
   PLA_REQUIRE(q && k && v && o && cu_seqlens && workspace, "null tensor pointer");
   PLA_REQUIRE((g_in != nullptr) == (beta_in != nullptr), "g and beta must be given together");
   PLA_REQUIRE(g_in != nullptr || (a && b && A_log && dt_bias), "raw gating needs a, b, A_log and dt_bias");
@@ -727,8 +697,7 @@ extern "C" int pla_gdn_prefill_launch(
   p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
   p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
   p.gtile = reinterpret_cast<float*>(ws + L.gtile);
-  p.Whi = reinterpret_cast<uint16_t*>(ws + L.Whi);
-  p.Wlo = reinterpret_cast<uint16_t*>(ws + L.Wlo);
+  p.W = reinterpret_cast<uint16_t*>(ws + L.W);
   p.P = reinterpret_cast<uint16_t*>(ws + L.P);
   p.H = H; p.HV = HV; p.NC_max = L.NC_max;
 
@@ -764,16 +733,21 @@ extern "C" int pla_gdn_prefill_launch(
   const bool ok = launch_pipeline(
       s, L.stages, segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
       [&](hipStream_t ps) {
-        hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
+        if (half_act) hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
+        else hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
         hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
       },
-      [&](unsigned grid) { hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3(grid), dim3(256), 0, s, p); });
+      [&](unsigned grid) {
+        if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2>), dim3(grid), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3(grid), dim3(256), 0, s, p);
+      });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+    if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
   }
   return check_launch("gdn prefill launch");
 }

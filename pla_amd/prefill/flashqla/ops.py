@@ -78,8 +78,8 @@ def chunk_gated_delta_rule_fwd(
         raise ValueError("raw gating is fused with q/k normalisation: pass normalize_qk=True")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.size(0) != 1:
         raise ValueError("q, k, v must be packed as [1, T, heads, dim]")
-    if q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise ValueError("q, k, v must be bf16")
+    if q.dtype not in (torch.bfloat16, torch.float16) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise ValueError("q, k, v must share bf16 or fp16")
     num_tokens, Hg, H = q.size(1), k.size(2), v.size(2)
     if q.shape != k.shape or v.size(1) != num_tokens:
         raise ValueError("q/k shapes and q/k/v token dimensions must match")

@@ -53,7 +53,7 @@ def _check(w, fast=False):
     exp_o, exp_final = _oracle_workload(w, fast)
     g_cum, A, o, none, final = _run_workload(w)
     torch.cuda.synchronize()
-    assert none is None and o.shape == (1, m["T"], m["HV"], 128) and o.dtype == torch.bfloat16
+    assert none is None and o.shape == (1, m["T"], m["HV"], 128) and o.dtype == w["packed_qkv"].dtype
     torch.testing.assert_close(o[0].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
     idx = w["initial_state_indices"].cpu().tolist()
     worst = max(rel_l2(final[n], exp_final[n]) for n in range(len(idx)))
@@ -75,6 +75,17 @@ def _check(w, fast=False):
 def test_gdn_prefill_small(lengths, tail_pad, H, HV):
     from pla_amd.workloads import gdn_prefill_packed
     w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=sum(lengths) + H, tail_pad=tail_pad)
+    _check(w, fast=sum(lengths) > 3000)
+
+
+@pytest.mark.parametrize("lengths,tail_pad", [([17], 3), ([200, 0, 33, 2049], 5), ([5555], 0)])
+def test_gdn_prefill_fp16_activations(lengths, tail_pad):
+    """fp16 q / k / v / gates (the reference's FlashQLA takes both,
+    src/prefill/flashqla/host/torch_extension_cute.cc:348-349): the oracle rounds the normalised q / k to fp16,
+    as the kernel does; same tolerances as bf16."""
+    from pla_amd.workloads import gdn_prefill_packed
+    w = gdn_prefill_packed(lengths, H=2, HV=4, pool_slots=len(lengths) + 3, seed=7 + sum(lengths), tail_pad=tail_pad,
+                           dtype=torch.float16)
     _check(w, fast=sum(lengths) > 3000)
 
 
