@@ -50,7 +50,7 @@ constexpr int PITCH64 = 72;
 __device__ __forceinline__ int solve_slot(int j) { return 16 * (j & 3) + 4 * (j >> 4) + ((j >> 2) & 3); }
 
 __device__ __forceinline__ void solve_store_w(const float (*L)[68], const float* beta, int wave, int lane,
-                                              uint16_t* Wh, uint16_t* Wl) {
+                                              uint16_t* W) {
   const int col = 16 * wave + (lane >> 2), part = lane & 3;
   const float bcol = beta[col];
   float xs[16];
@@ -87,9 +87,7 @@ __device__ __forceinline__ void solve_store_w(const float (*L)[68], const float*
 #pragma unroll
   for (int t = 0; t < 16; ++t) {
     const int l = 16 * (t >> 2) + 4 * (t & 3) + part;
-    const bf16_t hi = from_float<bf16_t>(xs[t]);
-    Wh[l * 64 + col] = hi.bits;
-    Wl[l * 64 + col] = from_float<bf16_t>(xs[t] - to_float(hi)).bits;
+    W[l * 64 + col] = from_float<f16_t>(xs[t]).bits;              // fp16: the sweeps' operand type
   }
 }
 

@@ -11,16 +11,18 @@
 // (reference pipeline: src/prefill/flashkdapro/tc01/fla/runtime.cc:474-545 - gate, token, inter,
 // recompute, recurrence, output; public contract pla/prefill/flashkdapro/ops.py:68-219).
 // The gate cannot be factored out of the products here, so the decayed operands are formed in
-// FP32 and split into bf16 hi + lo parts wherever they feed the state.  Overflow never occurs:
-// every exponent is <= 0 except inside a 16-row diagonal block of M / P, where the reference row
+// FP32.  In M / P every exponent is <= 0 except inside a 16-row diagonal block, where the reference row
 // is the block's first row and the exponent is bounded by 15 tokens of decay (|lower_bound| <= 5
 // gives e^75, well inside the bf16 / FP32 range) - the same sub-chunk scheme as the reference's
-// FLA kernels (scripts/prefill/private/ref/chunk_intra.py:170-202).
+// FLA kernels (scripts/prefill/private/ref/chunk_intra.py:170-202); those operands are split into
+// bf16 hi + lo parts (bf16 has the range, the pair the precision).  The operands of the sequential
+// sweep (k e^{G}, q e^{G}, k e^{G_last - G}, W, P, S, X, U) all carry factors in (0, 1] and go to the
+// MFMA as fp16, rounded once.
 //
 // Kernels:
 //   kda_prep_solve_kernel   one workgroup per (chunk, head): q/k L2 norm (rounded to bf16), lower-bound
-//                           gate, cumulative decay, decayed operand tiles, M / P on MFMA, FP32 forward
-//                           substitution, W (hi/lo)
+//                           gate, cumulative decay, decayed operand tiles (fp16), M / P on MFMA, FP32
+//                           forward substitution, W and P (fp16)
 //   kda_chunk_seq_kernel    one workgroup per (sequence, head) or segment sweep, four wavefronts x 32 V
 //                           columns, same register-chained MFMA pipeline and asynchronous LDS tile
 //                           copies as the GDN kernel
@@ -39,9 +41,9 @@ struct KdaPrefillParams {
   float* ht; const int32_t* ht_indices; int64_t ht_slot_stride;
   void* o;
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
-  uint16_t* Khi; uint16_t* Klo; uint16_t* Qh;      // [chunk, H, 64, 128]: k e^{G} (hi, lo), scale q e^{G}
-  uint16_t* KtH; uint16_t* KtL;                    // [chunk, H, 128, 64]: (k e^{G_last - G})^T (hi, lo)
-  uint16_t* Whi; uint16_t* Wlo; uint16_t* P;       // [chunk, H, 64, 64]
+  // operand tiles of the sweeps, fp16 (every factor lies in (0, 1]; values below 6e-8 vanish)
+  uint16_t* Kg; uint16_t* Qg; uint16_t* Kt;        // [chunk, H, 64, 128]: k e^{G}, scale q e^{G}, k e^{G_last - G}
+  uint16_t* W; uint16_t* P;                        // [chunk, H, 64, 64]
   float* eGlast;                                   // [chunk, H, 128]: e^{G_last}
   SegmentTable seg;                                // split long sequences (seg.seg_chunks > 0)
   StageTable stg;                                  // pipelined preparation and sweep (stg.stages > 0)
@@ -180,9 +182,10 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #ifdef PLA_PROF
   tk[2] = clock64();
 #endif
-  // ---- phase 2: decayed operand tiles for the sequential kernel -------------------------------
+  // ---- phase 2: decayed operand tiles for the sequential kernel (fp16, row major) ---------------
   {
-    // row-major tiles: thread handles row j, eight channels, twice
+    // thread handles row j, eight channels, four times
+    const float* const glast = &sh.G[CHUNK - 1][0];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int vec = tid + 256 * u;                // 1024 vectors: 64 rows x 16
@@ -190,37 +193,20 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       const uint4 kx = *reinterpret_cast<const uint4*>(&sh.Kn[j][c0]);
       const uint4 qx = *reinterpret_cast<const uint4*>(&sh.Qn[j][c0]);
       const uint32_t kwv[4] = {kx.x, kx.y, kx.z, kx.w}, qwv[4] = {qx.x, qx.y, qx.z, qx.w};
-      uint32_t khi[4], klo[4], qh[4];
+      uint32_t kg[4], qg[4], kt[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float e0 = __expf(sh.G[j][c0 + 2 * e]), e1 = __expf(sh.G[j][c0 + 2 * e + 1]);
-        const float a0 = lo16<bf16_t>(kwv[e]) * e0, a1 = hi16<bf16_t>(kwv[e]) * e1;
-        khi[e] = pack2<bf16_t>(a0, a1);
-        klo[e] = pack2<bf16_t>(a0 - lo16<bf16_t>(khi[e]), a1 - hi16<bf16_t>(khi[e]));
-        qh[e] = pack2<bf16_t>(p.scale * lo16<bf16_t>(qwv[e]) * e0, p.scale * hi16<bf16_t>(qwv[e]) * e1);
+        const float g0 = sh.G[j][c0 + 2 * e], g1 = sh.G[j][c0 + 2 * e + 1];
+        const float e0 = __expf(g0), e1 = __expf(g1);
+        const float k0 = lo16<bf16_t>(kwv[e]), k1 = hi16<bf16_t>(kwv[e]);
+        kg[e] = pack2<f16_t>(k0 * e0, k1 * e1);
+        qg[e] = pack2<f16_t>(p.scale * lo16<bf16_t>(qwv[e]) * e0, p.scale * hi16<bf16_t>(qwv[e]) * e1);
+        kt[e] = pack2<f16_t>(k0 * __expf(glast[c0 + 2 * e] - g0), k1 * __expf(glast[c0 + 2 * e + 1] - g1));
       }
       const int64_t off = tile * 8192 + (int64_t)j * 128 + c0;
-      *reinterpret_cast<uint4*>(p.Khi + off) = make_uint4(khi[0], khi[1], khi[2], khi[3]);
-      *reinterpret_cast<uint4*>(p.Klo + off) = make_uint4(klo[0], klo[1], klo[2], klo[3]);
-      *reinterpret_cast<uint4*>(p.Qh + off) = make_uint4(qh[0], qh[1], qh[2], qh[3]);
-    }
-    // transposed tile (k e^{G_last - G})^T: thread (c, half) gathers 32 tokens of channel c
-    const int c = tid >> 1, half = tid & 1;
-    const float gl = sh.G[CHUNK - 1][c];
-    uint32_t th[16], tl[16];
-#pragma unroll
-    for (int jj = 0; jj < 16; ++jj) {
-      const int j0 = 32 * half + 2 * jj;
-      const float a0 = to_float(bf16_t{sh.Kn[j0][c]}) * __expf(gl - sh.G[j0][c]);
-      const float a1 = to_float(bf16_t{sh.Kn[j0 + 1][c]}) * __expf(gl - sh.G[j0 + 1][c]);
-      th[jj] = pack2<bf16_t>(a0, a1);
-      tl[jj] = pack2<bf16_t>(a0 - lo16<bf16_t>(th[jj]), a1 - hi16<bf16_t>(th[jj]));
-    }
-    const int64_t off = tile * 8192 + (int64_t)c * CHUNK + 32 * half;
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      reinterpret_cast<uint4*>(p.KtH + off)[x] = make_uint4(th[4 * x], th[4 * x + 1], th[4 * x + 2], th[4 * x + 3]);
-      reinterpret_cast<uint4*>(p.KtL + off)[x] = make_uint4(tl[4 * x], tl[4 * x + 1], tl[4 * x + 2], tl[4 * x + 3]);
+      *reinterpret_cast<uint4*>(p.Kg + off) = make_uint4(kg[0], kg[1], kg[2], kg[3]);
+      *reinterpret_cast<uint4*>(p.Qg + off) = make_uint4(qg[0], qg[1], qg[2], qg[3]);
+      *reinterpret_cast<uint4*>(p.Kt + off) = make_uint4(kt[0], kt[1], kt[2], kt[3]);
     }
   }
 
@@ -266,7 +252,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * bi + 4 * kb + r;
         sh.L[i][solve_slot(j)] = i > j ? sh.B[i] * m[r] : 0.f;
-        Pt[i * 64 + j] = from_float<bf16_t>(i >= j ? p.scale * pq[r] : 0.f).bits;
+        Pt[i * 64 + j] = from_float<f16_t>(i >= j ? p.scale * pq[r] : 0.f).bits;
       }
     }
   }
@@ -276,7 +262,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   tk[4] = clock64();
 #endif
   // ---- phase 4: W = L^-1 diag(beta), forward substitution on all four wavefronts ----------------
-  solve_store_w(sh.L, sh.B, wave, lane, p.Whi + tile * 4096, p.Wlo + tile * 4096);
+  solve_store_w(sh.L, sh.B, wave, lane, p.W + tile * 4096);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -284,21 +270,25 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 // SIMD), each owning two 16-column blocks of V that share every A operand.  S^T stays in MFMA
 // accumulator layout (an accumulator tile pair is already a valid B operand of the next product); the
 // A operands come from LDS tiles filled by asynchronous global -> LDS copies.  Every tile is single
-// buffered (149 KB of LDS) and there are two barriers per chunk; a tile's next version is requested at
-// the barrier after its last use and has half a chunk of compute time to land:
+// buffered (104 KB of LDS) and there are two barriers per chunk; a tile's next version is requested at
+// the barrier after its last use and has half a chunk of compute time to land.  Every operand is fp16
+// (v_mfma_f32_16x16x32_f16), rounded once: the decayed tiles hold factors in (0, 1], and a float64
+// simulation of these rounding points gives a final-state rel-L2 of 2.5e-4 .. 4.8e-4 from strong to weak
+// decay (bound 1e-3; 2.6e-3 .. 3.8e-3 with single bf16 operands, which therefore needed hi + lo pairs):
 //
-//   barrier A   K e^G (hi, lo), scale Q e^G, V, W (hi, lo) of chunk c landed
-//               flush O(c-1); issue (K e^{G_last-G})^T (hi, lo), P, e^{G_last} of chunk c
-//               KS = (K e^G) S^T (three split passes), QS = (scale Q e^G) S^T, X = V - KS, U = W X
+//   barrier A   K e^G, scale Q e^G, V, W of chunk c landed
+//               flush O(c-1); issue K e^{G_last-G}, P, e^{G_last} of chunk c
+//               KS = (K e^G) S^T, QS = (scale Q e^G) S^T, X = V - KS, U = W X
 //   barrier B   the tiles issued at A landed; issue the first group for chunk c+1
 //               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U,  O = QS + P U -> O tile
+// The K e^{G_last-G} tile is stored row major like the others; its transposed operands come from
+// ds_read_b64_tr_b16.
 //
 // Every wait is for all outstanding copies: what is in flight at a barrier is what the next half needs.
 __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2, WAVES = 4;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
-  using CopyKt = TileCopy<128, 2 * PITCH64, 128, WAVES>;          // 128 x 64 tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -319,15 +309,12 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int n_chunks = c_end - c_begin;
 
   // distinct LDS objects, 16-byte aligned, filled in 1 KiB pieces
-  __shared__ __align__(16) uint16_t tKh[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tKl[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tK[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tKtH[128 * PITCH64];
-  __shared__ __align__(16) uint16_t tKtL[128 * PITCH64];
-  __shared__ __align__(16) uint16_t tWh[CHUNK * PITCH64];
-  __shared__ __align__(16) uint16_t tWl[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tKt[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
   __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
   __shared__ __align__(16) float tE[128];            // e^{G_last} of the chunk
 
@@ -351,13 +338,10 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   }
 
   const int64_t tile0 = (int64_t)c_begin * p.H + h;                       // chunk tiles are [chunk, H, ...]
-  const char* const kh_b = reinterpret_cast<const char*>(p.Khi) + tile0 * 16384;
-  const char* const kl_b = reinterpret_cast<const char*>(p.Klo) + tile0 * 16384;
-  const char* const qh_b = reinterpret_cast<const char*>(p.Qh) + tile0 * 16384;
-  const char* const th_b = reinterpret_cast<const char*>(p.KtH) + tile0 * 16384;
-  const char* const tl_b = reinterpret_cast<const char*>(p.KtL) + tile0 * 16384;
-  const char* const wh_b = reinterpret_cast<const char*>(p.Whi) + tile0 * 8192;
-  const char* const wl_b = reinterpret_cast<const char*>(p.Wlo) + tile0 * 8192;
+  const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
+  const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
+  const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 16384;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 8192;
   const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
   const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
@@ -366,15 +350,12 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
   CopyWide plan_k, plan_v;
   CopyNarrow plan_w;
-  CopyKt plan_kt;
   plan_k.plan(256, CHUNK - 1, wave, lane);
   plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
   plan_w.plan(128, CHUNK - 1, wave, lane);
-  plan_kt.plan(128, 127, wave, lane);
-  auto issue_first = [&](int c) {                    // K e^G (hi, lo), scale Q e^G, V, W (hi, lo)
-    plan_k.issue(tKh, kh_b + c * big_step, wave);
-    plan_k.issue(tKl, kl_b + c * big_step, wave);
-    plan_k.issue(tQ, qh_b + c * big_step, wave);
+  auto issue_first = [&](int c) {                    // K e^G, scale Q e^G, V, W
+    plan_k.issue(tK, kg_b + c * big_step, wave);
+    plan_k.issue(tQ, qg_b + c * big_step, wave);
     if (!zero_v) {
       const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
       const int len = chunk_len(c);
@@ -386,12 +367,10 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
         tail_v.issue(tV, vs, wave);
       }
     }
-    plan_w.issue(tWh, wh_b + c * small_step, wave);
-    plan_w.issue(tWl, wl_b + c * small_step, wave);
+    plan_w.issue(tW, w_b + c * small_step, wave);
   };
-  auto issue_second = [&](int c) {                   // (K e^{G_last-G})^T (hi, lo), P, e^{G_last}
-    plan_kt.issue(tKtH, th_b + c * big_step, wave);
-    plan_kt.issue(tKtL, tl_b + c * big_step, wave);
+  auto issue_second = [&](int c) {                   // K e^{G_last-G}, P, e^{G_last}
+    plan_k.issue(tKt, kt_b + c * big_step, wave);
     plan_w.issue(tP, pp_b + c * small_step, wave);
     if (wave == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
   };
@@ -417,11 +396,10 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
     // barrier A
     wait_vmcnt<0>();
     __syncthreads();
-    bf16x8_t kh[2][4], kl[2][4], qa[2][4];
+    bf16x8_t ka[2][4], qa[2][4];
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
-      kh[0][mi] = operand_from(&tKh[(16 * mi + r16) * PITCH128], 0, kb);
-      kl[0][mi] = operand_from(&tKl[(16 * mi + r16) * PITCH128], 0, kb);
+      ka[0][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], 0, kb);
       qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -434,17 +412,16 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
     uint16_t vraw[NB][16];
-    bf16x8_t wh[2][4], wl[2][4];
-    HiLo sb[2][NB];
+    bf16x8_t wa[2][4];
+    bf16x8_t sb[2][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = split8(St[nb][0], St[nb][1]);
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          kh[(s + 1) & 1][mi] = operand_from(&tKh[(16 * mi + r16) * PITCH128], s + 1, kb);
-          kl[(s + 1) & 1][mi] = operand_from(&tKl[(16 * mi + r16) * PITCH128], s + 1, kb);
+          ka[(s + 1) & 1][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], s + 1, kb);
           qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
         }
       } else {
@@ -460,40 +437,22 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wh[s2][mi] = operand_from(&tWh[(16 * mi + r16) * PITCH64], s2, kb);
-            wl[s2][mi] = operand_from(&tWl[(16 * mi + r16) * PITCH64], s2, kb);
-          }
+          for (int mi = 0; mi < 4; ++mi) wa[s2][mi] = operand_from(&tW[(16 * mi + r16) * PITCH64], s2, kb);
       }
       __builtin_amdgcn_sched_barrier(0);
-      // the split of the next step's state slice is interleaved with this step's MFMAs
+      // the next step's state slice is rounded underneath this step's MFMAs
       if (s < 3) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = split8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kh[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(qa[s & 1][mi], sb[s & 1][nb].hi, QS[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kl[s & 1][mi], sb[s & 1][nb].hi, KS[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16(kh[s & 1][mi], sb[s & 1][nb].lo, KS[nb][mi]);
-      if (s < 3) {
-#pragma unroll
-        for (int i = 0; i < 16 * NB; ++i) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);   // two VALU
-        }
-      }
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
       __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - KS
@@ -512,32 +471,23 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
       for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      HiLo xb[NB];
+      bf16x8_t xb[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = split8(X[nb][2 * s], X[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].hi, U[nb][mi]);
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8(X[nb][2 * s], X[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wl[s][mi], xb[nb].hi, U[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16(wh[s][mi], xb[nb].lo, U[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
     }
 
     // barrier B
     wait_vmcnt<0>();
     __syncthreads();
-    bf16x8_t th[8], tl[8];
+    bf16x8_t kt[2][8];
 #pragma unroll
-    for (int mc = 0; mc < 8; ++mc) {
-      th[mc] = operand_from(&tKtH[(16 * mc + r16) * PITCH64], 0, kb);
-      tl[mc] = operand_from(&tKtL[(16 * mc + r16) * PITCH64], 0, kb);
-    }
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tKt, s, mc, kb, r16);
     float4 eg[8];
 #pragma unroll
     for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
@@ -554,33 +504,20 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
       if (s == 1) {
-        // second contraction step: its operands and those of the output product are requested together
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) {
-          th[mc] = operand_from(&tKtH[(16 * mc + r16) * PITCH64], 1, kb);
-          tl[mc] = operand_from(&tKtL[(16 * mc + r16) * PITCH64], 1, kb);
-        }
+        // the last step's MFMAs cover the reads for the output product
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
           for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
         __builtin_amdgcn_sched_barrier(0);
       }
-      HiLo ub[NB];
+      bf16x8_t ub[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ub[nb] = split8(U[nb][2 * s], U[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(th[mc], ub[nb].hi, St[nb][mc]);
+      for (int nb = 0; nb < NB; ++nb) ub[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(tl[mc], ub[nb].hi, St[nb][mc]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16(th[mc], ub[nb].lo, St[nb][mc]);
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb], St[nb][mc]);
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -589,11 +526,11 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
     for (int s = 0; s < 2; ++s) {
       bf16x8_t ur[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ur[nb] = round8(U[nb][2 * s], U[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16(pa[s][mi], ur[nb], QS[nb][mi]);
+        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
     }
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -621,7 +558,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 }
 
 struct KdaWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Khi, Klo, Qh, KtH, KtL, Whi, Wlo, P, eGlast;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Kg, Qg, Kt, W, P, eGlast;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -636,8 +573,8 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   L.chunk_tok = take((size_t)L.NC_max * 4);
   L.chunk_len = take((size_t)L.NC_max * 4);
   const size_t big = (size_t)L.NC_max * H * 8192 * 2, small = (size_t)L.NC_max * H * 4096 * 2;
-  L.Khi = take(big); L.Klo = take(big); L.Qh = take(big); L.KtH = take(big); L.KtL = take(big);
-  L.Whi = take(small); L.Wlo = take(small); L.P = take(small);
+  L.Kg = take(big); L.Qg = take(big); L.Kt = take(big);
+  L.W = take(small); L.P = take(small);
   L.eGlast = take((size_t)L.NC_max * H * 128 * 4);
   L.seg_chunks = pick_segment_chunks(T, N, H);
   L.max_segments = max_segments(T, N, L.seg_chunks);
@@ -708,10 +645,9 @@ extern "C" int pla_kda_prefill_launch(
   p.chunk_seq = reinterpret_cast<int32_t*>(ws + L.chunk_seq);
   p.chunk_tok = reinterpret_cast<int32_t*>(ws + L.chunk_tok);
   p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
-  p.Khi = reinterpret_cast<uint16_t*>(ws + L.Khi); p.Klo = reinterpret_cast<uint16_t*>(ws + L.Klo);
-  p.Qh = reinterpret_cast<uint16_t*>(ws + L.Qh);
-  p.KtH = reinterpret_cast<uint16_t*>(ws + L.KtH); p.KtL = reinterpret_cast<uint16_t*>(ws + L.KtL);
-  p.Whi = reinterpret_cast<uint16_t*>(ws + L.Whi); p.Wlo = reinterpret_cast<uint16_t*>(ws + L.Wlo);
+  p.Kg = reinterpret_cast<uint16_t*>(ws + L.Kg); p.Qg = reinterpret_cast<uint16_t*>(ws + L.Qg);
+  p.Kt = reinterpret_cast<uint16_t*>(ws + L.Kt);
+  p.W = reinterpret_cast<uint16_t*>(ws + L.W);
   p.P = reinterpret_cast<uint16_t*>(ws + L.P);
   p.eGlast = reinterpret_cast<float*>(ws + L.eGlast);
   p.H = H; p.NC_max = L.NC_max;
