@@ -268,13 +268,16 @@ struct SweepRole {
   int n, head, c_begin, c_end;
   const float* init;      // [V, K] tile the state starts from (nullptr: zero)
   float* fin;             // [V, K] tile that receives the state at the end (nullptr: none)
+  float* keep_init;       // [V, K] tile that receives a copy of the start state (nullptr: none)
   bool zero_v, write_o, active;
 };
 __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, const int32_t* seq_chunk_off,
                                                   const SegmentTable& seg, const StageTable& stg, int stage,
                                                   const float* h0, const int32_t* h0_indices,
                                                   int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
-                                                  int64_t ht_slot_stride) {
+                                                  int64_t ht_slot_stride, bool resweep_first = false) {
+  // resweep_first: the first sweep publishes no output at all (first segments keep a copy of their start
+  // state and only deliver the state they end in), the second sweep runs every segment with output.
   SweepRole r{};
   r.write_o = true;
   auto state_in = [&](int n, int head) -> const float* {
@@ -312,6 +315,7 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
         r.init = state_in(r.n, r.head);
         r.fin = last ? state_out(r.n, r.head) : seg.B + tile;   // B of a first segment: the state entering the second
         carry = seg.B + tile;
+        if (resweep_first) { r.write_o = false; r.keep_init = seg.S + tile; }
       } else {
         r.write_o = false;
         if (from_identity) { r.init = seg.identity; r.zero_v = true; r.fin = seg.M + tile; }
@@ -319,8 +323,8 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
         carry = r.fin;
       }
     } else {
-      if (first) return r;
-      r.init = seg.S + tile;                          // the final state came out of the combine step
+      if (first && !resweep_first) return r;
+      r.init = seg.S + tile;                          // the state entering the segment (combine step, or kept copy)
     }
   }
   if (carry != nullptr && stg.stages > 0) {

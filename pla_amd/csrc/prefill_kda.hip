@@ -285,7 +285,11 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 // ds_read_b64_tr_b16.
 //
 // Every wait is for all outstanding copies: what is in flight at a barrier is what the next half needs.
-__global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
+//
+// WRITE_O = false is the first sweep over segments (affine summaries only): without the query, output and
+// P tiles the workgroup holds 60 KB of LDS and at most 256 registers per lane, so two of them share a CU.
+template <bool WRITE_O>
+__global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2, WAVES = 4;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
@@ -296,12 +300,12 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
 
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const float* const init = role.init;
   float* const fin = role.fin;
-  const bool zero_v = role.zero_v, write_o = role.write_o;
+  const bool zero_v = role.zero_v, write_o = WRITE_O && role.write_o;
   const int chunk_in_seq = c_begin - p.seq_chunk_off[n];
   const int seq_start = p.cu_seqlens[n] + chunk_in_seq * CHUNK;
   const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
@@ -310,12 +314,12 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 
   // distinct LDS objects, 16-byte aligned, filled in 1 KiB pieces
   __shared__ __align__(16) uint16_t tK[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tKt[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
-  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
   __shared__ __align__(16) float tE[128];            // e^{G_last} of the chunk
 
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
@@ -333,6 +337,15 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
+  if (role.keep_init != nullptr) {                   // a first segment that is swept again later: keep its start state
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
   if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
     for (int i = tid; i < CHUNK * PITCH128 / 2; i += 256) reinterpret_cast<uint32_t*>(tV)[i] = 0u;
   }
@@ -355,7 +368,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   plan_w.plan(128, CHUNK - 1, wave, lane);
   auto issue_first = [&](int c) {                    // K e^G, scale Q e^G, V, W
     plan_k.issue(tK, kg_b + c * big_step, wave);
-    plan_k.issue(tQ, qg_b + c * big_step, wave);
+    if constexpr (WRITE_O) plan_k.issue(tQ, qg_b + c * big_step, wave);
     if (!zero_v) {
       const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
       const int len = chunk_len(c);
@@ -371,7 +384,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
   };
   auto issue_second = [&](int c) {                   // K e^{G_last-G}, P, e^{G_last}
     plan_k.issue(tKt, kt_b + c * big_step, wave);
-    plan_w.issue(tP, pp_b + c * small_step, wave);
+    if constexpr (WRITE_O) plan_w.issue(tP, pp_b + c * small_step, wave);
     if (wave == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
   };
   // coalesced write of a finished output tile
@@ -400,7 +413,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
       ka[0][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], 0, kb);
-      qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
+      if constexpr (WRITE_O) qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (ci > 0) flush_output(ci - 1);
@@ -422,7 +435,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
           ka[(s + 1) & 1][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], s + 1, kb);
-          qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
+          if constexpr (WRITE_O) qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
         }
       } else {
         // the last step's MFMAs cover the reads for X and for U = W X
@@ -449,10 +462,12 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
+      if constexpr (WRITE_O) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
+          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - KS
@@ -503,7 +518,7 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
     bf16x8_t pa[2][4];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      if (s == 1) {
+      if (WRITE_O && s == 1) {
         // the last step's MFMAs cover the reads for the output product
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
@@ -521,27 +536,30 @@ __global__ __launch_bounds__(256) void kda_chunk_seq_kernel(const KdaPrefillPara
       __builtin_amdgcn_sched_barrier(0);
     }
 
-    // O = QS + P U -> O tile
+    if constexpr (WRITE_O) {
+      // O = QS + P U -> O tile
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      bf16x8_t ur[NB];
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t ur[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
+        for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
-    }
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-        orow[0] = from_float<bf16_t>(QS[nb][mi][0]).bits;
-        orow[PITCH128] = from_float<bf16_t>(QS[nb][mi][1]).bits;
-        orow[2 * PITCH128] = from_float<bf16_t>(QS[nb][mi][2]).bits;
-        orow[3 * PITCH128] = from_float<bf16_t>(QS[nb][mi][3]).bits;
+          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
       }
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+          orow[0] = from_float<bf16_t>(QS[nb][mi][0]).bits;
+          orow[PITCH128] = from_float<bf16_t>(QS[nb][mi][1]).bits;
+          orow[2 * PITCH128] = from_float<bf16_t>(QS[nb][mi][2]).bits;
+          orow[3 * PITCH128] = from_float<bf16_t>(QS[nb][mi][3]).bits;
+        }
+  
+    }
   }
   __syncthreads();
   if (n_chunks > 0) flush_output(n_chunks - 1);
@@ -684,13 +702,17 @@ extern "C" int pla_kda_prefill_launch(
   const bool ok = launch_pipeline(
       s, L.stages, segmented, (unsigned)N * H, (unsigned)L.max_segments * H, &p.pass, &p.stage,
       [&](hipStream_t ps) { hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, ps, p); },
-      [&](unsigned grid) { hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3(grid), dim3(256), 0, s, p); });
+      [&](unsigned grid) {
+        // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
+        if (p.pass == 1) hipLaunchKernelGGL(kda_chunk_seq_kernel<false>, dim3(grid), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(kda_chunk_seq_kernel<true>, dim3(grid), dim3(256), 0, s, p);
+      });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(kda_chunk_seq_kernel<true>, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
