@@ -93,9 +93,6 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   __shared__ KdaPrepShared sh;
   const int64_t tile = (int64_t)cb * p.H + h;
 
-#ifdef PLA_PROF
-  long long tk[6]; tk[0] = clock64();
-#endif
   // ---- phase 1: normalised q / k, per-channel log-decay, beta ---------------------------------
   {
     // q, k: thread handles eight channels of rows tid / 16 + 16 u (a row is one 16-lane DPP row, so its
@@ -109,6 +106,22 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       qv[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128 + nc0);
       kv[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + nc0);
     }
+    // gate: thread handles eight channels of rows tid / 16 + 16 u; requested together with q and k, so the
+    // phase costs one trip to memory
+    const int gc0 = 8 * (tid & 15);
+    uint4 graw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int j = (tid >> 4) + 16 * u;
+      graw[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.g) +
+                                                (int64_t)(t0 + (j < len ? j : 0)) * p.stride_g + h * 128 + gc0);
+    }
+    float dtb[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) dtb[e] = p.dt_bias[h * 128 + gc0 + e];
+    const float a_log = p.A_log[h];
+    float braw = 0.f;
+    if (tid < len) braw = to_float(reinterpret_cast<const bf16_t*>(p.beta)[(int64_t)(t0 + tid) * p.stride_beta + h]);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = nrow + 16 * u;
@@ -131,19 +144,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       *reinterpret_cast<uint4*>(&sh.Qn[j][nc0]) = make_uint4(qo[0], qo[1], qo[2], qo[3]);
       *reinterpret_cast<uint4*>(&sh.Kn[j][nc0]) = make_uint4(ko[0], ko[1], ko[2], ko[3]);
     }
-    // gate: thread handles eight channels of rows tid / 16 + 16 u; all four 16-byte loads are in flight at once
-    const float eA = expf(p.A_log[h]);
-    const int gc0 = 8 * (tid & 15);
-    uint4 graw[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int j = (tid >> 4) + 16 * u;
-      graw[u] = *reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(p.g) +
-                                                (int64_t)(t0 + (j < len ? j : 0)) * p.stride_g + h * 128 + gc0);
-    }
-    float dtb[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) dtb[e] = p.dt_bias[h * 128 + gc0 + e];
+    const float eA = expf(a_log);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = (tid >> 4) + 16 * u;
@@ -157,18 +158,10 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       }
     }
     if (tid < CHUNK) {
-      float bt = 0.f;
-      if (tid < len) {
-        const float braw = to_float(reinterpret_cast<const bf16_t*>(p.beta)[(int64_t)(t0 + tid) * p.stride_beta + h]);
-        bt = 1.0f / (1.0f + expf(-braw));
-      }
-      sh.B[tid] = bt;
+      sh.B[tid] = tid < len ? 1.0f / (1.0f + expf(-braw)) : 0.f;
     }
   }
   __syncthreads();
-#ifdef PLA_PROF
-  tk[1] = clock64();
-#endif
   if (tid < 128) {
     float cum = 0.f;
     for (int j = 0; j < CHUNK; ++j) {
@@ -179,9 +172,6 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   }
   __syncthreads();
 
-#ifdef PLA_PROF
-  tk[2] = clock64();
-#endif
   // ---- phase 2: decayed operand tiles for the sequential kernel (fp16, row major) ---------------
   {
     // thread handles row j, eight channels, four times
@@ -210,9 +200,6 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
     }
   }
 
-#ifdef PLA_PROF
-  tk[3] = clock64();
-#endif
   // ---- phase 3: M and P, wavefront w owns row block w (reference row = first row of the block) --
   {
     const int bi = wave;
@@ -258,9 +245,6 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   }
   __syncthreads();
 
-#ifdef PLA_PROF
-  tk[4] = clock64();
-#endif
   // ---- phase 4: W = L^-1 diag(beta), forward substitution on all four wavefronts ----------------
   solve_store_w(sh.L, sh.B, wave, lane, p.W + tile * 4096);
 }
