@@ -52,18 +52,21 @@ struct KdaPrefillParams {
   int H, NC_max;
 };
 
-// 69 KB, so that two workgroups share a CU.  L takes over Qn's storage once every wavefront has
-// formed its q operands (a barrier in phase 3 separates the two uses).
+// 52 KB, so that three workgroups share a CU.  The normalised q never goes through LDS: the thread that
+// normalised a piece of it also forms that piece of the decayed tile, and the wavefront that needs a row block
+// as an MFMA operand reads those rows again (they were fetched a moment ago) and scales them by the row's
+// inverse norm.  L takes over Kn's storage once every wavefront is done with its k operands (the M blocks wait
+// in registers for the barrier).
 struct __align__(16) KdaPrepShared {
   float G[CHUNK][132];
-  uint16_t Kn[CHUNK][PITCH128];
   union {
-    uint16_t Qn[CHUNK][PITCH128];
+    uint16_t Kn[CHUNK][PITCH128];
     float L[CHUNK][68];
   };
   float B[CHUNK];
+  float QI[CHUNK];         // 1 / |q_row|
 };
-static_assert(sizeof(float[CHUNK][68]) <= sizeof(uint16_t[CHUNK][PITCH128]), "L must fit into Qn's storage");
+static_assert(sizeof(float[CHUNK][68]) <= sizeof(uint16_t[CHUNK][PITCH128]), "L must fit into Kn's storage");
 
 // Eight decayed elements of a bf16 row: x[c] * exp(sign * (G[c] - R[c])) for the lane's two
 // channel quads of contraction step s.
@@ -93,6 +96,8 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
   __shared__ KdaPrepShared sh;
   const int64_t tile = (int64_t)cb * p.H + h;
 
+  uint32_t qn[4][4], kn[4][4];   // normalised bf16 pairs of rows tid / 16 + 16 u, channels 8 (tid % 16) .. + 7
+  uint2 qraw[4][2];
   // ---- phase 1: normalised q / k, per-channel log-decay, beta ---------------------------------
   {
     // q, k: thread handles eight channels of rows tid / 16 + 16 u (a row is one 16-lane DPP row, so its
@@ -122,6 +127,16 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
     const float a_log = p.A_log[h];
     float braw = 0.f;
     if (tid < len) braw = to_float(reinterpret_cast<const bf16_t*>(p.beta)[(int64_t)(t0 + tid) * p.stride_beta + h]);
+    // the q rows of this wavefront's row block in MFMA operand layout (phase 3), raw
+    {
+      const int i_row = 16 * wave + r16;
+      const uint16_t* qrow = reinterpret_cast<const uint16_t*>(p.q) + (int64_t)(t0 + (i_row < len ? i_row : 0)) * p.stride_q + h * 128;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        qraw[s][0] = *reinterpret_cast<const uint2*>(qrow + 32 * s + 4 * kb);
+        qraw[s][1] = *reinterpret_cast<const uint2*>(qrow + 32 * s + 4 * kb + 16);
+      }
+    }
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       const int j = nrow + 16 * u;
@@ -135,14 +150,13 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       }
       const float qi = rsqrtf(row16_allreduce(qs) + 1e-6f), ki = rsqrtf(row16_allreduce(ks) + 1e-6f);
       const bool ok = j < len;
-      uint32_t qo[4], ko[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        qo[e] = ok ? pack2<bf16_t>(lo16<bf16_t>(qw[e]) * qi, hi16<bf16_t>(qw[e]) * qi) : 0u;
-        ko[e] = ok ? pack2<bf16_t>(lo16<bf16_t>(kw[e]) * ki, hi16<bf16_t>(kw[e]) * ki) : 0u;
+        qn[u][e] = ok ? pack2<bf16_t>(lo16<bf16_t>(qw[e]) * qi, hi16<bf16_t>(qw[e]) * qi) : 0u;
+        kn[u][e] = ok ? pack2<bf16_t>(lo16<bf16_t>(kw[e]) * ki, hi16<bf16_t>(kw[e]) * ki) : 0u;
       }
-      *reinterpret_cast<uint4*>(&sh.Qn[j][nc0]) = make_uint4(qo[0], qo[1], qo[2], qo[3]);
-      *reinterpret_cast<uint4*>(&sh.Kn[j][nc0]) = make_uint4(ko[0], ko[1], ko[2], ko[3]);
+      *reinterpret_cast<uint4*>(&sh.Kn[j][nc0]) = make_uint4(kn[u][0], kn[u][1], kn[u][2], kn[u][3]);
+      if ((tid & 15) == 0) sh.QI[j] = ok ? qi : 0.f;
     }
     const float eA = expf(a_log);
 #pragma unroll
@@ -174,15 +188,12 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 
   // ---- phase 2: decayed operand tiles for the sequential kernel (fp16, row major) ---------------
   {
-    // thread handles row j, eight channels, four times
     const float* const glast = &sh.G[CHUNK - 1][0];
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const int vec = tid + 256 * u;                // 1024 vectors: 64 rows x 16
-      const int j = vec >> 4, c0 = 8 * (vec & 15);
-      const uint4 kx = *reinterpret_cast<const uint4*>(&sh.Kn[j][c0]);
-      const uint4 qx = *reinterpret_cast<const uint4*>(&sh.Qn[j][c0]);
-      const uint32_t kwv[4] = {kx.x, kx.y, kx.z, kx.w}, qwv[4] = {qx.x, qx.y, qx.z, qx.w};
+      const int j = (tid >> 4) + 16 * u, c0 = 8 * (tid & 15);   // the rows and channels this thread normalised
+      const uint32_t* const kwv = kn[u];
+      const uint32_t* const qwv = qn[u];
       uint32_t kg[4], qg[4], kt[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -212,11 +223,25 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       f32x4_t a, b;
       decayed8(&sh.Kn[i_row][0], &sh.G[i_row][0], R, 1.0f, s, kb, a, b);
       Al[s] = split8(a, b);
-      decayed8(&sh.Qn[i_row][0], &sh.G[i_row][0], R, 1.0f, s, kb, a, b);
+      // the same normalised bf16 values as phase 1 formed: raw q times the row's inverse norm, rounded to bf16
+      const float qi = sh.QI[i_row];
+      const uint2 x0 = qraw[s][0], x1 = qraw[s][1];
+      const uint32_t n0 = pack2<bf16_t>(lo16<bf16_t>(x0.x) * qi, hi16<bf16_t>(x0.x) * qi);
+      const uint32_t n1 = pack2<bf16_t>(lo16<bf16_t>(x0.y) * qi, hi16<bf16_t>(x0.y) * qi);
+      const uint32_t n2 = pack2<bf16_t>(lo16<bf16_t>(x1.x) * qi, hi16<bf16_t>(x1.x) * qi);
+      const uint32_t n3 = pack2<bf16_t>(lo16<bf16_t>(x1.y) * qi, hi16<bf16_t>(x1.y) * qi);
+      const int c0 = 32 * s + 4 * kb, c1 = c0 + 16;
+      const float4 g0 = *reinterpret_cast<const float4*>(&sh.G[i_row][c0]), g1 = *reinterpret_cast<const float4*>(&sh.G[i_row][c1]);
+      const float4 r0 = *reinterpret_cast<const float4*>(R + c0), r1 = *reinterpret_cast<const float4*>(R + c1);
+      a = f32x4_t{lo16<bf16_t>(n0) * __expf(g0.x - r0.x), hi16<bf16_t>(n0) * __expf(g0.y - r0.y),
+                  lo16<bf16_t>(n1) * __expf(g0.z - r0.z), hi16<bf16_t>(n1) * __expf(g0.w - r0.w)};
+      b = f32x4_t{lo16<bf16_t>(n2) * __expf(g1.x - r1.x), hi16<bf16_t>(n2) * __expf(g1.y - r1.y),
+                  lo16<bf16_t>(n3) * __expf(g1.z - r1.z), hi16<bf16_t>(n3) * __expf(g1.w - r1.w)};
       Ql[s] = round8(a, b);
     }
-    __syncthreads();                     // Qn is dead from here on: L reuses its storage
     uint16_t* const Pt = p.P + tile * 4096;
+    f32x4_t mblock[4];
+#pragma unroll
     for (int bj = 0; bj < 4; ++bj) {
       const int j = 16 * bj + r16;
       if (bj > bi) {
@@ -235,11 +260,22 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
         m = mfma16(Al[s].hi, Br.lo, m);
         pq = mfma16(Ql[s], Br.hi, pq);
       }
+      mblock[bj] = m;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * bi + 4 * kb + r;
-        sh.L[i][solve_slot(j)] = i > j ? sh.B[i] * m[r] : 0.f;
         Pt[i * 64 + j] = from_float<f16_t>(i >= j ? p.scale * pq[r] : 0.f).bits;
+      }
+    }
+    __syncthreads();                     // Kn is dead from here on: L reuses its storage
+#pragma unroll
+    for (int bj = 0; bj < 4; ++bj) {
+      if (bj > bi) continue;
+      const int j = 16 * bj + r16;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * bi + 4 * kb + r;
+        sh.L[i][solve_slot(j)] = i > j ? sh.B[i] * mblock[bj][r] : 0.f;
       }
     }
   }
