@@ -60,3 +60,20 @@ def offsets(cu, capacity, raw=None, *, reference=None):
     device_values = _offset_values(cu.detach().cpu().tolist(), capacity, cu.numel())
     if host is not None:
         check(host == device_values, "raw_cu_seqlens must equal device cu_seqlens")
+
+
+_OPERAND_MAX = 65504.0          # largest finite fp16: the matrix products take fp16 operands
+
+
+def operand_range(reference, **tensors):
+    """The prefill products round their operands (v, the state, intermediate products) to fp16, so values
+    beyond +-65504 or non-finite ones would turn into infinities inside the kernels.  Checks the named
+    tensors (``None`` entries are skipped) outside stream capture; no-op unless the mode is on."""
+    if not enabled() or _capturing(reference):
+        return
+    for name, t in tensors.items():
+        if t is None or t.numel() == 0:
+            continue
+        peak = float(t.detach().abs().max().float())          # NaN propagates through max
+        check(peak == peak and peak <= _OPERAND_MAX,
+              f"{name} must be finite and within the fp16 operand range (|x| <= 65504), got max |x| = {peak}")

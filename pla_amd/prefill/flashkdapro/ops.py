@@ -98,6 +98,7 @@ def flashkda_fwd(
         raise ValueError("A_log must be [H]")
 
     _sanity.offsets(cu_seqlens, T, raw_cu_seqlens, reference=q)
+    _sanity.operand_range(q, v=v, initial_state=initial_state)
     if cu_seqlens is None:
         cu32 = torch.tensor([0, T], dtype=torch.int32, device=q.device)
     else:

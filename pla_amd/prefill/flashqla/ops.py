@@ -97,6 +97,7 @@ def chunk_gated_delta_rule_fwd(
 
     _sanity.offsets(cu_seqlens, num_tokens,
                     raw_cu_seqlens.tolist() if isinstance(raw_cu_seqlens, torch.Tensor) else raw_cu_seqlens, reference=q)
+    _sanity.operand_range(q, v=v, initial_state=initial_state)
     if cu_seqlens is None:
         cu_seqlens = torch.tensor([0, num_tokens], dtype=torch.int32, device=q.device)
     cu32 = cu_seqlens.to(device=q.device, dtype=torch.int32).contiguous()

@@ -123,3 +123,11 @@ def test_prefill_sanity_mode_checks_offsets(monkeypatch):
             (None, 7, (0, 6), r"must be \[0,T\]")):
         with pytest.raises(AssertionError, match=r"PLA_SANITY_CHECK \[prefill\]: .*" + msg):
             _sanity.offsets(bad_cu, cap, raw)
+    # operands of the fp16 matrix products: finite and within +-65504
+    ref = torch.zeros(1)
+    _sanity.operand_range(ref, v=torch.tensor([1.0, -65504.0]), initial_state=None)
+    for bad in (torch.tensor([7e4]), torch.tensor([float("nan")]), torch.tensor([float("-inf")])):
+        with pytest.raises(AssertionError, match=r"PLA_SANITY_CHECK \[prefill\]: v must be finite and within the fp16"):
+            _sanity.operand_range(ref, v=bad)
+    monkeypatch.delenv("PLA_SANITY_CHECK")
+    _sanity.operand_range(ref, v=torch.tensor([7e4]))                                 # off: nothing is checked
