@@ -117,23 +117,36 @@ def flashkda_fwd(
     if indexed and (state_indices.dtype != torch.int32 or state_indices.dim() != 1 or state_indices.numel() != N
                     or not state_indices.is_contiguous()):
         raise ValueError("state_indices must be contiguous int32 [N]")
+    staged = False
     for name, t in (("initial_state", initial_state), ("final_state", final_state)):
         if t is None:
             continue
-        if t.dtype != torch.float32:
-            raise ValueError(f"{name} must be fp32 in this build (states are not rounded to bf16)")
+        if t.dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError(f"{name} must be fp32 or bf16")
         if t.dim() != 4 or t.size(1) != H or t.size(2) != DV or t.size(3) != DK:
             raise ValueError(f"{name} must be [N, H, DV, DK]")
-        if not t[0].is_contiguous() or t.stride(0) % 4 != 0:
-            raise ValueError(f"{name} slots must be dense [H, DV, DK]")
         if not indexed and t.size(0) < N:
             raise ValueError(f"{name} must hold at least N states")
+        # the kernels read and write dense FP32 slots; anything else goes through a dense FP32 copy
+        staged = staged or t.dtype != torch.float32 or not t[0].is_contiguous() or t.stride(0) % 4 != 0 or t.data_ptr() % 16 != 0
+    if initial_state is not None and final_state is not None and initial_state.dtype != final_state.dtype:
+        raise ValueError("initial_state and final_state must have the same dtype")
     if final_state is not None and final_state.data_ptr() == out.data_ptr():
         raise ValueError("final_state must not share storage with out")
-    if final_state is not None and initial_state is not None and final_state is not initial_state \
-            and final_state.data_ptr() != initial_state.data_ptr():
-        # empty sequences publish their incoming state unchanged
-        pass
+    if staged:
+        # As the reference does for layouts its kernels do not consume in place: the states are materialised
+        # once before the first kernel (exactly: bf16 widens to FP32) and written back after the last one
+        # (bf16 states are rounded once, at the end).  Sequences of length zero publish their incoming state.
+        rows = state_indices.long() if indexed else slice(0, N)
+        init32 = None if initial_state is None else initial_state[rows].to(torch.float32).contiguous()
+        fin32 = None
+        if final_state is not None:
+            fin32 = torch.empty(N, H, DV, DK, dtype=torch.float32, device=q.device)
+        flashkda_fwd(q, k, v, g, beta, A_log, dt_bias, out, scale=scale, lower_bound=lower_bound, initial_state=init32,
+                     final_state=fin32, cu_seqlens=cu_seqlens, raw_cu_seqlens=raw_cu_seqlens)
+        if final_state is not None:
+            final_state[rows] = fin32.to(final_state.dtype)
+        return None
 
     lib = _lib.load()
     nbytes = lib.pla_kda_prefill_workspace_bytes(T, N, H)

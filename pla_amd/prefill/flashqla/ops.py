@@ -118,8 +118,45 @@ def chunk_gated_delta_rule_fwd(
             raise ValueError("raw_cu_seqlens must be monotone offsets matching cu_seqlens")
 
     indexed = initial_state_indices is not None
-    if final_state_dtype is not None and final_state_dtype != torch.float32:
-        raise ValueError("this build keeps FP32 states: final_state_dtype must be float32")
+    # One dtype covers the incoming state, the indexed pool and the returned state (reference rule,
+    # pla/prefill/flashqla/ops.py:440-451): final_state_dtype selects it, must agree with initial_state when
+    # one is given, and defaults to that dtype, or to fp32 without an incoming state.
+    if final_state_dtype is None:
+        state_dtype = initial_state.dtype if initial_state is not None else torch.float32
+    else:
+        if final_state_dtype not in (torch.float32, torch.bfloat16):
+            raise ValueError("final_state_dtype must be fp32 or bf16")
+        if initial_state is not None and final_state_dtype != initial_state.dtype:
+            raise ValueError("final_state_dtype must match the initial_state dtype")
+        state_dtype = final_state_dtype
+    if state_dtype == torch.bfloat16:
+        # The kernels keep FP32 states: bf16 states are widened before the first kernel (exactly) and rounded
+        # once after the last one; an indexed bf16 pool is updated in place at its indexed slots.
+        if initial_state is not None and (initial_state.ndim != 4 or initial_state.size(1) != H
+                                          or initial_state.size(2) != DV or initial_state.size(3) != DK):
+            raise ValueError("initial_state must be [num_states,H,DV,DK] (k-last)")
+        if indexed:
+            idx = initial_state_indices
+            if initial_state is None:
+                raise ValueError("indexed initial_state must be given")
+            if (idx.device != q.device or idx.dtype != torch.int32 or not idx.is_contiguous()
+                    or idx.ndim != 1 or idx.numel() != batch):
+                raise ValueError("initial_state_indices must be contiguous int32 [batch] on q.device")
+            init32 = initial_state[idx.long()].to(torch.float32)
+        else:
+            if initial_state is not None and initial_state.size(0) < batch:
+                raise ValueError("initial_state must be [num_states>=batch,H,DV,DK] (k-last)")
+            init32 = None if initial_state is None else initial_state[:batch].to(torch.float32).contiguous()
+        g_cum, ws, o, _, final32 = chunk_gated_delta_rule_fwd(
+            q, k, v, g, beta, scale=scale, initial_state=init32, initial_state_indices=None, cu_seqlens=cu_seqlens,
+            output_final_state=output_final_state or indexed, auto_cp=auto_cp,
+            overlap_warmup_threshold=overlap_warmup_threshold, force_tc01_cp_candidate=force_tc01_cp_candidate,
+            normalize_qk=normalize_qk, raw_cu_seqlens=raw_cu_seqlens, raw_gate_a=raw_gate_a, raw_beta_b=raw_beta_b,
+            A_log=A_log, dt_bias=dt_bias, final_state_dtype=None)
+        final = None if final32 is None else final32.to(torch.bfloat16)
+        if indexed:
+            initial_state[idx.long()] = final
+        return g_cum, ws, o, None, (final if output_final_state else None)
     if indexed:
         if initial_state is None or initial_state.dtype != torch.float32 or not initial_state.is_contiguous():
             raise ValueError("indexed initial_state must be contiguous fp32")

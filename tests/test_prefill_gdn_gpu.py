@@ -116,6 +116,35 @@ def test_gdn_prefill_no_final_state_still_updates_pool_and_chained_calls():
     assert torch.equal(w["initial_state"], pool_full)
 
 
+def test_gdn_prefill_bf16_states():
+    """A bf16 pool (or final_state_dtype=bf16) follows the reference's rule of one dtype for the incoming state,
+    the pool and the returned state (pla/prefill/flashqla/ops.py:440-451): the states are widened to FP32, the
+    FP32 result is rounded once, outputs equal the FP32-state call on the same (representable) values."""
+    from pla_amd.workloads import gdn_prefill_packed
+    w = gdn_prefill_packed([70, 0, 300], H=2, HV=4, pool_slots=6, seed=17)
+    w["initial_state"].copy_(w["initial_state"].bfloat16().float())
+    pool32 = w["initial_state"].clone()
+    _, _, o32, _, final32 = _run_workload(w)
+    after32 = w["initial_state"].clone()
+    pool16 = pool32.bfloat16()
+    w16 = dict(w, initial_state=pool16)
+    _, _, o16, _, final16 = _run_workload(w16)
+    torch.cuda.synchronize()
+    assert final16.dtype == torch.bfloat16 and torch.equal(o16, o32)
+    assert torch.equal(final16, final32.bfloat16()) and torch.equal(pool16, after32.bfloat16())
+    # no incoming state, bf16 result requested
+    call = {k: v for k, v in w.items() if not k.startswith("_") and k not in ("initial_state", "initial_state_indices")}
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    packed = call.pop("packed_qkv")
+    a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+    r32 = gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, **call)
+    r16 = gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, final_state_dtype=torch.bfloat16, **call)
+    torch.cuda.synchronize()
+    assert torch.equal(r16[2], r32[2]) and torch.equal(r16[4], r32[4].bfloat16())
+    with pytest.raises(ValueError, match="must match the initial_state dtype"):
+        _run_workload(dict(w, final_state_dtype=torch.bfloat16))
+
+
 def test_gdn_prefill_split_inputs_and_compact_state():
     """g / beta given explicitly, q/k already normalised, compact (non-indexed) state."""
     from pla_amd.prefill.flashqla import chunk_gated_delta_rule_fwd

@@ -82,6 +82,50 @@ def test_kda_prefill_small(lengths, pad, H):
     assert torch.equal(pool[untouched], before[untouched])
 
 
+def test_kda_prefill_bf16_and_strided_states():
+    """States may be bf16 or arbitrarily strided (pla/prefill/flashkdapro/ops.py:104-118 of the reference): they
+    are staged through dense FP32 copies, so the outputs equal the FP32-state call bit for bit when the bf16
+    initial state holds the same values, and the final state is the FP32 result rounded once."""
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    lengths, H, dev = [0, 17, 300], 2, "cuda"
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=91, pad=2)
+    S0 = S0.bfloat16().float()                                   # representable in both dtypes
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    args = [t.to(dev) for t in (q, k, v, raw, beta, A_log, dt_bias)]
+    out32 = torch.empty(q.shape[0], H, 128, dtype=torch.bfloat16, device=dev)
+    fin32 = torch.empty(len(lengths), H, 128, 128, device=dev)
+    flashkda_fwd(*args, out32, initial_state=S0.to(dev), final_state=fin32, cu_seqlens=cu)
+    # bf16 states
+    out16 = torch.empty_like(out32)
+    init16 = S0.to(dev).bfloat16()
+    fin16 = torch.full((len(lengths), H, 128, 128), 5.0, dtype=torch.bfloat16, device=dev)
+    flashkda_fwd(*args, out16, initial_state=init16, final_state=fin16, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    assert torch.equal(out16, out32) and torch.equal(fin16, fin32.bfloat16())
+    # a bf16 pool with a padded slot pitch, updated in place at the indexed slots only
+    backing = torch.full((6, H * 128 * 128 + 24), 3.0, dtype=torch.bfloat16, device=dev)
+    pool = backing[:, 8:8 + H * 128 * 128].view(6, H, 128, 128)
+    idx = torch.tensor([4, 1, 3], dtype=torch.int32, device=dev)
+    pool[idx.long()] = init16
+    before = backing.clone()
+    outp = torch.empty_like(out32)
+    flashkda_fwd(*args, outp, state_pool=pool, state_indices=idx, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    assert torch.equal(outp, out32) and torch.equal(pool[idx.long()], fin32.bfloat16())
+    untouched = torch.ones_like(backing, dtype=torch.bool)
+    untouched[idx.long(), 8:8 + H * 128 * 128] = False
+    assert torch.equal(backing[untouched], before[untouched])
+    # transposed FP32 states (strided V / K axes)
+    init_t = S0.to(dev).transpose(2, 3).contiguous().transpose(2, 3)
+    fin_t = torch.empty(len(lengths), H, 128, 128, device=dev).transpose(2, 3)
+    outt = torch.empty_like(out32)
+    flashkda_fwd(*args, outt, initial_state=init_t, final_state=fin_t, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    assert torch.equal(outt, out32) and torch.equal(fin_t, fin32)
+    with pytest.raises(ValueError, match="same dtype"):
+        flashkda_fwd(*args, outt, initial_state=init16, final_state=fin32, cu_seqlens=cu)
+
+
 @pytest.mark.parametrize("scenario", ["initial_bits", "weak_decay", "small_update", "fresh_update"])
 def test_kda_prefill_closed_forms(scenario):
     from pla_amd.prefill.flashkdapro import flashkda_fwd
