@@ -2,7 +2,8 @@
 
 Sub-packages mirror the reference's ``pla`` namespace (pla/__init__.py:31-53):
 ``pla_amd.decode``, ``pla_amd.decode.private``, ``pla_amd.decode.kda``,
-``pla_amd.decode.kda_replayssm_sglang``, ``pla_amd.prefill.flashqla`` and
+``pla_amd.decode.kda_replayssm_sglang`` (also under its former name ``kda_mtp_sglang``),
+``pla_amd.decode.kda_replayssm_vllm``, ``pla_amd.prefill.flashqla`` and
 ``pla_amd.prefill.flashkdapro``.  ``import pla_amd as pla`` is the drop-in.
 Sub-packages are imported lazily so that importing the top level never loads
 the native library.

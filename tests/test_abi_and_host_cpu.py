@@ -131,3 +131,29 @@ def test_prefill_sanity_mode_checks_offsets(monkeypatch):
             _sanity.operand_range(ref, v=bad)
     monkeypatch.delenv("PLA_SANITY_CHECK")
     _sanity.operand_range(ref, v=torch.tensor([7e4]))                                 # off: nothing is checked
+
+
+def test_namespace_mirrors_the_reference_packages():
+    """`import pla_amd as pla` gives the reference's sub-packages and public names for the path
+    (pla/decode/__init__.py:63-66, pla/decode/kda/__init__.py:51-52, pla/decode/private/__init__.py:46-47,
+    pla/decode/kda_mtp_sglang/__init__.py:35-41, pla/decode/kda_replayssm_vllm/__init__.py,
+    pla/prefill/flashqla/__init__.py:48, pla/prefill/flashkdapro/__init__.py:39)."""
+    import importlib
+    expected = {
+        "decode": ["fused_sigmoid_gating_delta_rule_forward_k_last", "fused_sigmoid_gating_delta_rule_forward_k_last_packed"],
+        "decode.private": ["fused_sigmoid_gating_delta_rule_forward_k_last_tunable",
+                           "fused_sigmoid_gating_delta_rule_forward_k_last_packed_tunable"],
+        "decode.kda": ["fused_recurrent_kda", "fused_kda_decode_mega_forward"],
+        "decode.kda_replayssm_sglang": ["fused_kda_decode_mtp_dspark", "commit_kda_replayssm_after_verify"],
+        "decode.kda_mtp_sglang": ["fused_kda_decode_mtp_dspark", "commit_kda_replayssm_after_verify"],
+        "decode.kda_replayssm_vllm": ["KDAReplayRecords", "KDAReplayCommitPlan", "KDAReplayCommitContext", "kda_replay_verify"],
+        "prefill.flashqla": ["chunk_gated_delta_rule_fwd", "gdn_prefill_packed_qkv_fwd"],
+        "prefill.flashkdapro": ["flashkda_fwd"],
+    }
+    for sub, names in expected.items():
+        mod = importlib.import_module("pla_amd." + sub)
+        for name in names:
+            assert callable(getattr(mod, name)), (sub, name)
+    a = importlib.import_module("pla_amd.decode.kda_mtp_sglang")
+    b = importlib.import_module("pla_amd.decode.kda_replayssm_sglang")
+    assert a.fused_kda_decode_mtp_dspark is b.fused_kda_decode_mtp_dspark
