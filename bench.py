@@ -159,6 +159,42 @@ def bench_prefill(steps, warmup, device):
                                    "chunk map + prep + gram/solve + sequential kernels"))
 
 
+# GDN prefill shapes the reference publishes timings for (reports/prefill_bench_20260911.json, family gdn,
+# num_v_heads 32 / 16 q/k heads, bf16, measured by its authors on a ZW-M890P PPU): lengths -> published ms
+REFERENCE_GDN_PREFILL_MS = (([2048] * 8, 1.4865), ([4096] * 4, 1.5035), ([16384], 2.241))
+
+
+def bench_prefill_reference_shapes(steps, device):
+    """The batch x length shapes of the reference's own prefill report, next to its published times (other
+    hardware: a ratio of two machines, not a like-for-like comparison)."""
+    import torch
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from pla_amd.workloads import gdn_prefill_packed
+    rows = []
+    for lengths, published_ms in REFERENCE_GDN_PREFILL_MS:
+        w = gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=len(lengths) + 2, seed=1, device=device)
+        call = {k: v for k, v in w.items() if not k.startswith("_")}
+        packed = call.pop("packed_qkv")
+        a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+        run = lambda: gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, **call)
+        for _ in range(3):
+            run()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(steps):
+            run()
+        end.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(end) / steps
+        rows.append({"shape": "%d x %d tokens" % (len(lengths), lengths[0]), "ms_per_call": round(ms, 4),
+                     "tokens_per_s": round(sum(lengths) / ms * 1e3, 1), "reference_ppu_ms": published_ms,
+                     "reference_ms_over_ours": round(published_ms / ms, 2)})
+        del w, call, packed
+        torch.cuda.empty_cache()
+    return rows
+
+
 def bench_prefill_kda(steps, device):
     """Config 4: KDA chunk-64 prefill of one 65 536-token sequence, 32 heads (32 independent chains)."""
     import torch
@@ -473,6 +509,7 @@ def main():
         torch.cuda.empty_cache()
         result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
         torch.cuda.empty_cache()
+        result["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 20, 5), device)
         result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
     if args.copy_calibration:
         result["copy_calibration"] = copy_calibration(device)
