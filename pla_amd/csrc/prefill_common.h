@@ -41,53 +41,102 @@ constexpr int PITCH128 = 136;
 constexpr int PITCH64 = 72;
 
 // ---------------------------------------------------------------------------------------------
-// W = L^-1 diag(beta) for a unit lower triangular 64 x 64 L, by forward substitution on the four
-// wavefronts of a workgroup.  Wavefront w owns columns 16 w .. 16 w + 15; the four lanes of a quad share
-// one column and split each row's dot product by l mod 4: lane part p keeps x_l for l = 16 m + 4 e + p
-// in xs[4 m + e], and column j of L is stored at solve_slot(j), which makes those columns contiguous.
-// A row costs ceil(i / 16) float4 reads and 4 ceil(i / 16) FMAs per lane plus a two-step quad
-// reduction.  L must hold zeros on and above the diagonal of every diagonal 16 x 16 block it touches.
-__device__ __forceinline__ int solve_slot(int j) { return 16 * (j & 3) + 4 * (j >> 4) + ((j >> 2) & 3); }
+// W = (I + L)^-1 diag(beta) for a strictly lower triangular 64 x 64 L (FP32, in LDS) on ONE wavefront, by
+// 16 x 16 blocks with the off-diagonal blocks on MFMA.  With N = (I + L)^-1: the diagonal blocks D_a = (I + L_aa)^-1 come from forward substitution over 16 rows
+// (lane 16 a + j owns column j of D_a), the others from N_ab = -D_a sum_{b <= c < a} L_ac N_cb in order of
+// a - b = 1, 2, 3 (13 products of 16 x 16 x 16 or 16 x 16 x 32).  FP32 values cross the MFMA as bf16
+// hi/lo pairs (hi.hi + hi.lo + lo.hi, error ~2^-16 per product).  L is used as workspace: D_a replaces
+// L_aa, D_b^T is parked in the unused block (b, b + 1) where lanes read it as a B operand, N_ab replaces
+// L_ab, and the fp16 tile leaves in 16-byte pieces (8 rows of 128 bytes per store instruction).  Only the
+// strictly lower triangle of L is read.
+__device__ __forceinline__ f32x4_t mfma_hilo(const HiLo& a, const HiLo& b, f32x4_t c) {
+  c = mfma16(a.lo, b.hi, c);
+  c = mfma16(a.hi, b.lo, c);
+  return mfma16(a.hi, b.hi, c);
+}
 
-__device__ __forceinline__ void solve_store_w(const float (*L)[68], const float* beta, int wave, int lane,
-                                              uint16_t* W) {
-  const int col = 16 * wave + (lane >> 2), part = lane & 3;
-  const float bcol = beta[col];
-  float xs[16];
+__device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const float* beta, int lane, uint16_t* W) {
+  const int r16 = lane & 15, kb = lane >> 4;
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  {
+    // diagonal blocks: x_i = [i == j] - sum_{l < i} L_aa[i][l] x_l
+    const int a = kb, j = r16;
+    float x[16];
 #pragma unroll
-  for (int t = 0; t < 16; ++t) xs[t] = 0.f;
-  // the L values of row i + 2 are requested while row i is reduced: they do not depend on x
-  float4 ahead[2][4];
+    for (int i = 0; i < 16; ++i) {
+      float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-  for (int i = 1; i < 3; ++i) ahead[i & 1][0] = *reinterpret_cast<const float4*>(&L[i][16 * part]);
-#pragma unroll
-  for (int i = 0; i < CHUNK; ++i) {
-    float4 row[4];
-#pragma unroll
-    for (int m = 0; 16 * m < i; ++m) row[m] = ahead[i & 1][m];
-    if (i + 2 < CHUNK) {
-#pragma unroll
-      for (int m = 0; 16 * m < i + 2; ++m)
-        ahead[i & 1][m] = *reinterpret_cast<const float4*>(&L[i + 2][16 * part + 4 * m]);
+      for (int l4 = 0; l4 < i; l4 += 4) {
+        const float4 row = *reinterpret_cast<const float4*>(&L[16 * a + i][16 * a + l4]);
+        acc0 = fmaf(row.x, x[l4], acc0);
+        if (l4 + 1 < i) acc1 = fmaf(row.y, x[l4 + 1], acc1);
+        if (l4 + 2 < i) acc0 = fmaf(row.z, x[l4 + 2], acc0);
+        if (l4 + 3 < i) acc1 = fmaf(row.w, x[l4 + 3], acc1);
+      }
+      x[i] = (i == j ? 1.f : 0.f) - (acc0 + acc1);
     }
-    float acc = 0.f, acc2 = 0.f;
+    // all reads of L_aa are done (one wavefront, LDS operations complete in order)
 #pragma unroll
-    for (int m = 0; 16 * m < i; ++m) {
-      acc = fmaf(row[m].x, xs[4 * m + 0], acc);
-      acc2 = fmaf(row[m].y, xs[4 * m + 1], acc2);
-      acc = fmaf(row[m].z, xs[4 * m + 2], acc);
-      acc2 = fmaf(row[m].w, xs[4 * m + 3], acc2);
+    for (int i = 0; i < 16; ++i) L[16 * a + i][16 * a + j] = x[i];
+    if (a < 3) {
+#pragma unroll
+      for (int i4 = 0; i4 < 16; i4 += 4)
+        *reinterpret_cast<float4*>(&L[16 * a + j][16 * (a + 1) + i4]) = make_float4(x[i4], x[i4 + 1], x[i4 + 2], x[i4 + 3]);
     }
-    acc += acc2;
-    acc += dpp_mov<0xB1>(acc);    // quad_perm [1,0,3,2]
-    acc += dpp_mov<0x4E>(acc);    // quad_perm [2,3,0,1]
-    const float xi = (i == col ? bcol : 0.f) - acc;
-    if (part == (i & 3)) xs[4 * (i >> 4) + ((i & 15) >> 2)] = xi;
   }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // operands: A = rows of L (blocks c0 and, if c1 >= 0, c1 of block row a); lane (m, kb) holds columns 4 kb .. 4 kb + 3 of each
+  auto quad = [&](int row, int col) {
+    const float4 t = *reinterpret_cast<const float4*>(&L[row][col]);
+    return f32x4_t{t.x, t.y, t.z, t.w};
+  };
+  auto a_rows = [&](int a, int c0, int c1) {
+    return split8(quad(16 * a + r16, 16 * c0 + 4 * kb), c1 >= 0 ? quad(16 * a + r16, 16 * c1 + 4 * kb) : zero);
+  };
+  auto negate = [](f32x4_t t) { return f32x4_t{-t.x, -t.y, -t.z, -t.w}; };
+  // D_b as a B operand half: rows 4 kb .. 4 kb + 3 of column r16, read from the transposed copy
+  const f32x4_t D0 = quad(r16, 16 + 4 * kb), D1 = quad(16 + r16, 32 + 4 * kb), D2 = quad(32 + r16, 48 + 4 * kb);
+  const HiLo AD1 = a_rows(1, 1, -1), AD2 = a_rows(2, 2, -1), AD3 = a_rows(3, 3, -1);
+  const HiLo A32 = a_rows(3, 2, -1);
+  // a - b = 1
+  const f32x4_t Y10 = mfma_hilo(a_rows(1, 0, -1), split8(D0, zero), zero);
+  const f32x4_t Y21 = mfma_hilo(a_rows(2, 1, -1), split8(D1, zero), zero);
+  const f32x4_t Y32 = mfma_hilo(A32, split8(D2, zero), zero);
+  const f32x4_t X10 = negate(mfma_hilo(AD1, split8(Y10, zero), zero));
+  const f32x4_t X21 = negate(mfma_hilo(AD2, split8(Y21, zero), zero));
+  const f32x4_t X32 = negate(mfma_hilo(AD3, split8(Y32, zero), zero));
+  // a - b = 2
+  const HiLo B0 = split8(D0, X10);                        // [D_0; N_10], shared by N_20 and N_30
+  const f32x4_t Y20 = mfma_hilo(a_rows(2, 0, 1), B0, zero);
+  const f32x4_t Y31 = mfma_hilo(a_rows(3, 1, 2), split8(D1, X21), zero);
+  const f32x4_t X20 = negate(mfma_hilo(AD2, split8(Y20, zero), zero));
+  const f32x4_t X31 = negate(mfma_hilo(AD3, split8(Y31, zero), zero));
+  // a - b = 3
+  f32x4_t Y30 = mfma_hilo(a_rows(3, 0, 1), B0, zero);
+  Y30 = mfma_hilo(A32, split8(X20, zero), Y30);
+  const f32x4_t X30 = negate(mfma_hilo(AD3, split8(Y30, zero), zero));
+  // N_ab replaces L_ab (accumulator layout: lane (n, kb) holds rows 4 kb + r of column n)
+  auto put = [&](int a, int b, f32x4_t t) {
 #pragma unroll
-  for (int t = 0; t < 16; ++t) {
-    const int l = 16 * (t >> 2) + 4 * (t & 3) + part;
-    W[l * 64 + col] = from_float<f16_t>(xs[t]).bits;              // fp16: the sweeps' operand type
+    for (int r = 0; r < 4; ++r) L[16 * a + 4 * kb + r][16 * b + r16] = t[r];
+  };
+  put(1, 0, X10); put(2, 1, X21); put(3, 2, X32); put(2, 0, X20); put(3, 1, X31); put(3, 0, X30);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // W[i][j] = N[i][j] beta_j for j <= i, zero above: lane -> row 8 pass + lane / 8, columns 8 (lane % 8) ..
+  const int c8 = 8 * (lane & 7);
+  const float4 b0 = *reinterpret_cast<const float4*>(&beta[c8]), b1 = *reinterpret_cast<const float4*>(&beta[c8 + 4]);
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int i = 8 * pass + (lane >> 3);
+    const float4 lo = *reinterpret_cast<const float4*>(&L[i][c8]), hi = *reinterpret_cast<const float4*>(&L[i][c8 + 4]);
+    const float w[8] = {lo.x * b0.x, lo.y * b0.y, lo.z * b0.z, lo.w * b0.w, hi.x * b1.x, hi.y * b1.y, hi.z * b1.z, hi.w * b1.w};
+    uint32_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      packed[e] = pack2<f16_t>(c8 + 2 * e <= i ? w[2 * e] : 0.f, c8 + 2 * e + 1 <= i ? w[2 * e + 1] : 0.f);
+    *reinterpret_cast<uint4*>(W + i * 64 + c8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
   }
 }
 
@@ -228,10 +277,13 @@ __device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((i
 // writes its own chunk ids.
 static __global__ void stage_map_kernel(const int32_t* starts, const int32_t* counts, const int32_t* n_items_ptr,
                                         int n_items_max, int NC_max, StageTable t) {
-  extern __shared__ int32_t pair_begin[];              // [stages * n_items_max + 1]
+  extern __shared__ int32_t pair_begin[];              // [stages * n_items_max + 1], then n_items_max chunk counts
   const int S = t.stages;
   const int n_items = n_items_ptr ? min(*n_items_ptr, n_items_max) : n_items_max;
-  auto count_of = [&](int i) { return counts ? counts[i] : starts[i + 1] - starts[i]; };
+  int32_t* const count = pair_begin + S * n_items_max + 1;
+  for (int i = threadIdx.x; i < n_items; i += blockDim.x) count[i] = counts ? counts[i] : starts[i + 1] - starts[i];
+  __syncthreads();
+  auto count_of = [&](int i) { return count[i]; };
   if (threadIdx.x == 0) {
     int k = 0;
     for (int s = 0; s < S; ++s) {
@@ -473,7 +525,8 @@ static inline SideStream* side_stream() {
 // times.)
 inline int pick_stages(int T, int N, int heads, int seg_chunks) {
   if (seg_chunks > 0) return 0;
-  return ((int64_t)N * heads >= 128 && T / CHUNK >= 16 * N) ? MAX_STAGES : 0;
+  // (the stage map keeps (stages + 1) counters per sequence in LDS: at most 2048 sequences)
+  return ((int64_t)N * heads >= 128 && T / CHUNK >= 16 * N && N <= 2048) ? MAX_STAGES : 0;
 }
 
 // Launch order of a prefill call, shared by both paths.  `prepare(stream)` launches the per-chunk

@@ -25,8 +25,8 @@
 //   chunk_map_kernel         chunk table from cu_seqlens (device side, graph-capturable)
 //   gdn_prep_kernel          gate, beta, chunk-local cumsum and per-chunk decay-factor tiles, q/k L2
 //                            norm (rounded to the activation dtype, stored as fp16)
-//   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, FP32
-//                            forward substitution in LDS, W and P (fp16) to the workspace
+//   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, the inverse of
+//                            I + L by 16 x 16 blocks in LDS, W and P (fp16) to the workspace
 //   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), four wavefronts each owning a
 //                            32-wide V slice of S^T in MFMA accumulator layout; the chain
 //                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_f16 with every
@@ -66,9 +66,9 @@ struct GdnPrefillParams {
 };
 
 // ---------------------------------------------------------------------------------------------
-// grid (chunk, H + 1), 256 threads.  blockIdx.y < H: L2 norm of q and k of one head for the
-// chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing);
-// blockIdx.y == H: gate, beta and the chunk-local cumulative log-decay.
+// grid (chunk, 1 + H), 256 threads.  blockIdx.y == 0: gate, beta and the chunk-local cumulative log-decay
+// (the longest workgroups, so they are dispatched first); blockIdx.y - 1 = head: L2 norm of q and k of
+// that head for the chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing).
 template <typename act_t>
 __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
   const int cb = staged_chunk(p.stg, p.stage, blockIdx.x, p.seq_chunk_off[p.N]);
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
     float g[CHUNK][129];              // per-token log-decay of up to 128 value heads
   } sh;
 
-  if ((int)blockIdx.y == p.H) {
+  if (blockIdx.y == 0) {
     for (int hv0 = 0; hv0 < p.HV; hv0 += 128) {
       const int nh = min(128, p.HV - hv0);
       for (int idx = threadIdx.x; idx < CHUNK * nh; idx += 256) {
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
     return;
   }
 
-  const int h = blockIdx.y;
+  const int h = (int)blockIdx.y - 1;
   uint32_t qw[16], kw[16];
 #pragma unroll
   for (int x = 0; x < 16; ++x) {
@@ -159,20 +159,27 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
 }
 
 // ---------------------------------------------------------------------------------------------
-// One wavefront per (chunk, value head).
-__global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillParams p) {
-  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / p.HV, p.seq_chunk_off[p.N]);
-  const int hv = blockIdx.x % p.HV;
+// One wavefront per (chunk, value head); the WAVES wavefronts of a workgroup take consecutive value heads
+// of one q/k head, so their K and Q rows meet in the CU's cache instead of crossing HBM once per value head.
+template <int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPrefillParams p) {
+  const int groups = p.HV / WAVES;
+  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
   if (cb < 0) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int hv = (blockIdx.x % groups) * WAVES + wave;
   const int h = hv / (p.HV / p.H);
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
 
-  __shared__ float Lm[CHUNK][68];
-  __shared__ float Gs[CHUNK];
-  __shared__ float Bs[CHUNK];
+  __shared__ __align__(16) float Lm_all[WAVES][CHUNK][68];
+  __shared__ __align__(16) float Gs_all[WAVES][CHUNK];
+  __shared__ __align__(16) float Bs_all[WAVES][CHUNK];
+  float (*const Lm)[68] = Lm_all[wave];
+  float* const Gs = Gs_all[wave];
+  float* const Bs = Bs_all[wave];
 
   {
     const bool ok = lane < len;
@@ -181,20 +188,29 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
     Bs[lane] = ok ? p.beta[(int64_t)(t0 + lane) * p.HV + hv] : 0.f;
   }
 
-  // K operands: 4 row blocks x 4 contraction steps (rows beyond the chunk are zero)
+  // K and Q operands: 4 row blocks x 4 contraction steps (rows beyond the chunk are zero).  All 32 loads of a
+  // lane are requested before the first use: the LDS tile limits a SIMD to two wavefronts, which hide no
+  // memory latency, and leaves them 256 registers each.
   const uint4 zero4 = make_uint4(0, 0, 0, 0);
-  bf16x8_t Kop[4][4];
+  bf16x8_t Kop[4][4], Qop[4][4];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
     const int row = 16 * mb + r16;
     const bool ok = row < len;
     const uint16_t* kr = p.kn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
+    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       const bf16x8_t kz = operand_from(kr, s, kb);
       Kop[mb][s] = ok ? kz : __builtin_bit_cast(bf16x8_t, zero4);
     }
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const bf16x8_t qz = operand_from(qr, s, kb);
+      Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
+    }
   }
+  __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
 
   // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
@@ -215,61 +231,57 @@ __global__ __launch_bounds__(64) void gdn_gram_solve_kernel(const GdnPrefillPara
     }
   }
 
-  // P = scale * tril(q_i . k_j e^{G_i - G_j}); one row block of Q at a time keeps registers low
-  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
+  // P = scale * tril(q_i . k_j e^{G_i - G_j}), kept as packed fp16 until the solve has released the LDS tile
+  uint32_t Ppk[10][2];
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi) {
-    const int row = 16 * mi + r16;
-    const bool ok = row < len;
-    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
-    bf16x8_t Qop[4];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const bf16x8_t qz = operand_from(qr, s, kb);
-      Qop[s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
-    }
-#pragma unroll
-    for (int ni = 0; ni < 4; ++ni) {
+    for (int ni = 0; ni <= mi; ++ni) {
       const int j = 16 * ni + r16;
-      if (ni > mi) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Pt[(16 * mi + 4 * kb + r) * 64 + j] = 0;
-        continue;
-      }
       f32x4_t qk = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int s = 0; s < 4; ++s) qk = mfma16h(Qop[s], Kop[ni][s], qk);
+      for (int s = 0; s < 4; ++s) qk = mfma16h(Qop[mi][s], Kop[ni][s], qk);
       const float Gj = Gs[j];
+      float pv[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * mi + 4 * kb + r;
-        const float gam = i >= j ? __expf(Gs[i] - Gj) : 0.f;
-        Pt[i * 64 + j] = from_float<f16_t>(p.scale * qk[r] * gam).bits;
+        pv[r] = i >= j ? p.scale * qk[r] * __expf(Gs[i] - Gj) : 0.f;
       }
+      Ppk[mi * (mi + 1) / 2 + ni][0] = pack2<f16_t>(pv[0], pv[1]);
+      Ppk[mi * (mi + 1) / 2 + ni][1] = pack2<f16_t>(pv[2], pv[3]);
     }
   }
+
+  // W = (I + L)^-1 diag(beta): 16 x 16 blocks, the off-diagonal ones on MFMA
+  block_inverse_store_w(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * 4096);
   __syncthreads();
 
-  // forward substitution, one column per lane: x_i = beta_j [i == j] - sum_{l < i} L[i][l] x_l
-  float x[CHUNK];
-  const float bj = Bs[lane];
+  // P leaves through the released tile in 16-byte pieces; blocks above the diagonal are never written and read as zero
+  uint16_t* const Ps = reinterpret_cast<uint16_t*>(&Lm[0][0]);          // rows of 136 halves
 #pragma unroll
-  for (int i = 0; i < CHUNK; ++i) {
-    // four independent partial sums keep the FMA pipeline full
-    float a0 = (i == lane) ? bj : 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+  for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-    for (int l4 = 0; l4 < i; l4 += 4) {
-      const float4 row = *reinterpret_cast<const float4*>(&Lm[i][l4]);
-      a0 = fmaf(-row.x, x[l4], a0);
-      if (l4 + 1 < i) a1 = fmaf(-row.y, x[l4 + 1], a1);
-      if (l4 + 2 < i) a2 = fmaf(-row.z, x[l4 + 2], a2);
-      if (l4 + 3 < i) a3 = fmaf(-row.w, x[l4 + 3], a3);
+    for (int ni = 0; ni <= mi; ++ni) {
+      uint16_t* dst = Ps + (16 * mi + 4 * kb) * 136 + 16 * ni + r16;
+      const uint32_t w0 = Ppk[mi * (mi + 1) / 2 + ni][0], w1 = Ppk[mi * (mi + 1) / 2 + ni][1];
+      dst[0] = (uint16_t)w0; dst[136] = (uint16_t)(w0 >> 16); dst[272] = (uint16_t)w1; dst[408] = (uint16_t)(w1 >> 16);
     }
-    x[i] = (a0 + a1) + (a2 + a3);
-  }
-  uint16_t* const Wt = p.W + ((int64_t)cb * p.HV + hv) * 4096;
+  __syncthreads();
+  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
+  const int c8 = 8 * (lane & 7);
 #pragma unroll
-  for (int i = 0; i < CHUNK; ++i) Wt[i * 64 + lane] = from_float<f16_t>(x[i]).bits;
+  for (int pass = 0; pass < 8; ++pass) {
+    const int i = 8 * pass + (lane >> 3);
+    uint4 w = *reinterpret_cast<const uint4*>(Ps + i * 136 + c8);
+    uint32_t* we = reinterpret_cast<uint32_t*>(&w);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (c8 + 2 * e > i) we[e] = 0u;
+      else if (c8 + 2 * e + 1 > i) we[e] &= 0xffffu;
+    }
+    *reinterpret_cast<uint4*>(Pt + i * 64 + c8) = w;
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -726,7 +738,7 @@ extern "C" int pla_gdn_prefill_launch(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = L.stages;
     const int items = segmented ? L.max_segments : N;
-    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * items + 1) * 4, s,
+    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)((L.stages + 1) * items + 1) * 4, s,
                        segmented ? p.seg.seg_c0 : p.seq_chunk_off, segmented ? p.seg.seg_nc : nullptr,
                        segmented ? p.seg.seq_seg_off + N : nullptr, items, L.NC_max, p.stg);
   }
@@ -735,7 +747,10 @@ extern "C" int pla_gdn_prefill_launch(
       [&](hipStream_t ps) {
         if (half_act) hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
         else hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
-        hipLaunchKernelGGL(gdn_gram_solve_kernel, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
+        const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
+        if (ratio % 4 == 0) hipLaunchKernelGGL(gdn_gram_solve_kernel<4>, dim3((unsigned)L.NC_max * (HV / 4)), dim3(256), 0, ps, p);
+        else if (ratio % 2 == 0) hipLaunchKernelGGL(gdn_gram_solve_kernel<2>, dim3((unsigned)L.NC_max * (HV / 2)), dim3(128), 0, ps, p);
+        else hipLaunchKernelGGL(gdn_gram_solve_kernel<1>, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
       },
       [&](unsigned grid) {
         if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2>), dim3(grid), dim3(256), 0, s, p);

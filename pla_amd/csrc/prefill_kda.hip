@@ -21,8 +21,8 @@
 //
 // Kernels:
 //   kda_prep_solve_kernel   one workgroup per (chunk, head): q/k L2 norm (rounded to bf16), lower-bound
-//                           gate, cumulative decay, decayed operand tiles (fp16), M / P on MFMA, FP32
-//                           forward substitution, W and P (fp16)
+//                           gate, cumulative decay, decayed operand tiles (fp16), M / P on MFMA, the
+//                           inverse of I + L by 16 x 16 blocks, W and P (fp16)
 //   kda_chunk_seq_kernel    one workgroup per (sequence, head) or segment sweep, four wavefronts x 32 V
 //                           columns, same register-chained MFMA pipeline and asynchronous LDS tile
 //                           copies as the GDN kernel
@@ -275,14 +275,15 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int i = 16 * bi + 4 * kb + r;
-        sh.L[i][solve_slot(j)] = i > j ? sh.B[i] * mblock[bj][r] : 0.f;
+        sh.L[i][j] = i > j ? sh.B[i] * mblock[bj][r] : 0.f;
       }
     }
   }
   __syncthreads();
 
-  // ---- phase 4: W = L^-1 diag(beta), forward substitution on all four wavefronts ----------------
-  solve_store_w(sh.L, sh.B, wave, lane, p.W + tile * 4096);
+  // ---- phase 4: W = L^-1 diag(beta) by blocks on one wavefront (which one rotates with the workgroup, so
+  // that co-resident workgroups keep different SIMDs busy) -----------------------------------------
+  if (wave == (int)(blockIdx.x & 3)) block_inverse_store_w(sh.L, sh.B, lane, p.W + tile * 4096);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -715,7 +716,7 @@ extern "C" int pla_kda_prefill_launch(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = L.stages;
     const int items = segmented ? L.max_segments : N;
-    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)(L.stages * items + 1) * 4, s,
+    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)((L.stages + 1) * items + 1) * 4, s,
                        segmented ? p.seg.seg_c0 : p.seq_chunk_off, segmented ? p.seg.seg_nc : nullptr,
                        segmented ? p.seg.seq_seg_off + N : nullptr, items, L.NC_max, p.stg);
   }
