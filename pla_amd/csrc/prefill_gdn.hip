@@ -181,13 +181,6 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPre
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
-  {
-    const bool ok = lane < len;
-    const float glast = p.gcum[(int64_t)(t0 + len - 1) * p.HV + hv];
-    Gs[lane] = ok ? p.gcum[(int64_t)(t0 + lane) * p.HV + hv] : glast;
-    Bs[lane] = ok ? p.beta[(int64_t)(t0 + lane) * p.HV + hv] : 0.f;
-  }
-
   // K and Q operands: 4 row blocks x 4 contraction steps (rows beyond the chunk are zero).  All 32 loads of a
   // lane are requested before the first use: the LDS tile limits a SIMD to two wavefronts, which hide no
   // memory latency, and leaves them 256 registers each.
@@ -210,7 +203,15 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPre
       Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
     }
   }
-  __builtin_amdgcn_sched_barrier(0);
+  {
+    // rows beyond the chunk repeat its last log-decay (their K rows are zero) and have beta = 0; requested
+    // after the operands and in the same round trip
+    const int64_t at = (int64_t)(t0 + min(lane, len - 1)) * p.HV + hv;
+    const float gl = p.gcum[at], bl = p.beta[at];
+    __builtin_amdgcn_sched_barrier(0);
+    Gs[lane] = gl;
+    Bs[lane] = lane < len ? bl : 0.f;
+  }
   __syncthreads();
 
   // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
@@ -685,6 +686,8 @@ extern "C" int pla_gdn_prefill_launch(
   PLA_REQUIRE(g_in != nullptr || (a && b && A_log && dt_bias), "raw gating needs a, b, A_log and dt_bias");
   PLA_REQUIRE(((uintptr_t)q % 4 == 0) && ((uintptr_t)k % 4 == 0) && stride_q % 2 == 0 && stride_k % 2 == 0,
               "q/k rows require 4-byte alignment");
+  PLA_REQUIRE((uintptr_t)v % 16 == 0 && stride_v % 8 == 0, "v rows require 16-byte alignment (they are copied to LDS in 16-byte pieces)");
+  PLA_REQUIRE((uintptr_t)o % 16 == 0, "o requires 16-byte alignment");
   const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV);
   PLA_REQUIRE(workspace_bytes >= (int64_t)L.total, "workspace too small: need %zu bytes", L.total);
   PLA_REQUIRE((uintptr_t)workspace % 256 == 0, "workspace requires 256-byte alignment");

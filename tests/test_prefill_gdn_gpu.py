@@ -259,3 +259,31 @@ def test_gdn_prefill_staged_pipeline_in_a_graph():
         assert scratch == scratch
         assert torch.equal(o_graph, o_eager), replay
         assert torch.equal(w["initial_state"], pool_eager), replay
+
+
+def test_gdn_prefill_rows_aligned_to_4_bytes_only():
+    """A packed Q|K|V view whose rows start 4 bytes into a 16-byte piece: q and k are read in place, v (copied to
+    LDS in 16-byte pieces) is materialised by the facade; the results equal those of the aligned buffer."""
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from pla_amd.workloads import gdn_prefill_packed
+    lengths = [130, 0, 77]
+    outs = []
+    for shifted in (False, True):
+        w = gdn_prefill_packed(lengths, H=2, HV=4, pool_slots=6, seed=23)
+        call = {k: v for k, v in w.items() if not k.startswith("_")}
+        packed = call.pop("packed_qkv")
+        if shifted:
+            T, width = packed.shape
+            wide = torch.zeros(T, width + 6, dtype=packed.dtype, device=packed.device)
+            wide[:, 2:2 + width] = packed
+            packed = wide[:, 2:2 + width]
+            assert packed.data_ptr() % 8 == 4 and packed.stride(0) % 4 == 2
+        a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+        g_cum, _, o, _, final = gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, **call)
+        torch.cuda.synchronize()
+        outs.append((o.float().cpu(), final.cpu()))
+    torch.testing.assert_close(outs[1][0], outs[0][0], atol=2e-2, rtol=2e-2)
+    assert max(rel_l2(outs[1][1][n], outs[0][1][n]) for n in range(len(lengths))) <= 1e-3
+    w = gdn_prefill_packed(lengths, H=2, HV=4, pool_slots=6, seed=23)
+    exp_o, exp_final = _oracle_workload(w)
+    torch.testing.assert_close(outs[1][0][0], exp_o.float(), atol=2e-2, rtol=2e-2)
