@@ -205,8 +205,8 @@ struct TileCopy {
 
 // Chunk table from cu_seqlens, built on the device so that no call reads offsets back to the host.
 // Single workgroup.  seq_chunk_off[n] = first chunk of sequence n (seq_chunk_off[N] = total).
-static __global__ void chunk_map_kernel(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,
-                                        int32_t* chunk_seq, int32_t* chunk_tok, int32_t* chunk_len) {
+__device__ __forceinline__ void chunk_map(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,
+                                          int32_t* chunk_seq, int32_t* chunk_tok, int32_t* chunk_len) {
   if (threadIdx.x == 0) {
     int acc = 0;
     for (int n = 0; n < N; ++n) {
@@ -271,13 +271,13 @@ constexpr int MAX_STAGES = 4;
 // Chunks [lo, hi) of an item of `nc` chunks that belong to stage s of S.
 __device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((int64_t)nc * s / S); }
 
-// Single workgroup of 256 threads.  The items are sequences (`counts` null: item i holds chunks
+// Single workgroup of 256 threads with (stages + 1) * n_items_max + 1 words of LDS at `pair_begin`.  The items are sequences (`counts` null: item i holds chunks
 // starts[i] .. starts[i + 1]) or segments (chunks starts[i] .. starts[i] + counts[i]); `n_items` is read
 // on the device.  (Stage, item) pairs count their chunks, a serial prefix places them, then every pair
 // writes its own chunk ids.
-static __global__ void stage_map_kernel(const int32_t* starts, const int32_t* counts, const int32_t* n_items_ptr,
-                                        int n_items_max, int NC_max, StageTable t) {
-  extern __shared__ int32_t pair_begin[];              // [stages * n_items_max + 1], then n_items_max chunk counts
+__device__ __forceinline__ void stage_map(const int32_t* starts, const int32_t* counts, const int32_t* n_items_ptr,
+                                          int n_items_max, int NC_max, StageTable t, int32_t* pair_begin) {
+  // pair_begin: [stages * n_items_max + 1], then n_items_max chunk counts
   const int S = t.stages;
   const int n_items = n_items_ptr ? min(*n_items_ptr, n_items_max) : n_items_max;
   int32_t* const count = pair_begin + S * n_items_max + 1;
@@ -390,8 +390,8 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
   return r;
 }
 
-// Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map_kernel.
-static __global__ void segment_map_kernel(const int32_t* seq_chunk_off, int N, SegmentTable t) {
+// Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map.
+__device__ __forceinline__ void segment_map(const int32_t* seq_chunk_off, int N, SegmentTable t) {
   if (threadIdx.x == 0) {
     int acc = 0;
     for (int n = 0; n < N; ++n) {
@@ -481,13 +481,48 @@ inline int pick_segment_chunks(int T, int N, int heads) {
 }
 inline int max_segments(int T, int N, int seg_chunks) { return seg_chunks > 0 ? T / CHUNK / seg_chunks + N + 1 : 0; }
 
-// Zero the rows of a dense [T, heads, 128] 16-bit output that lie beyond the last sequence.
-static __global__ void zero_tail_kernel(uint16_t* o, const int32_t* cu_seqlens, int N, int T, int heads) {
+// Zero the rows of a dense [T, heads, 128] 16-bit output that lie beyond the last sequence (workgroup `block` of `blocks`).
+__device__ __forceinline__ void zero_tail(uint16_t* o, const int32_t* cu_seqlens, int N, int T, int heads, int block, int blocks) {
   const int64_t first = (int64_t)cu_seqlens[N] * heads * 128;
   const int64_t total = (int64_t)T * heads * 128;
-  for (int64_t i = first + (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x)
+  for (int64_t i = first + (int64_t)block * blockDim.x + threadIdx.x; i < total; i += (int64_t)blocks * blockDim.x)
     o[i] = 0;
+}
+
+// All tables of a call in one launch.  Workgroup 0 builds the chunk table, then (split calls) the segment
+// table, then (pipelined calls) the stage table; each step reads what the previous one wrote, through
+// memory, after a device-scope fence and a barrier of that one workgroup.  The other workgroups zero the
+// output rows beyond the last sequence.  Dynamic LDS: (stages + 1) * stage_items + 1 words.
+constexpr int TABLE_WORKGROUPS = 1 + 64;
+static __global__ __launch_bounds__(256) void prefill_tables_kernel(
+    const int32_t* cu_seqlens, int N, int T, int NC_max, int32_t* seq_chunk_off, int32_t* chunk_seq,
+    int32_t* chunk_tok, int32_t* chunk_len, SegmentTable seg, StageTable stg, int stage_items, uint16_t* o, int heads) {
+  extern __shared__ int32_t table_lds[];
+  if (blockIdx.x > 0) {
+    zero_tail(o, cu_seqlens, N, T, heads, blockIdx.x - 1, gridDim.x - 1);
+    return;
+  }
+  chunk_map(cu_seqlens, N, NC_max, seq_chunk_off, chunk_seq, chunk_tok, chunk_len);
+  const bool segmented = seg.seg_chunks > 0;
+  if (segmented) {
+    __threadfence();
+    __syncthreads();
+    segment_map(seq_chunk_off, N, seg);
+  }
+  if (stg.stages > 0) {
+    __threadfence();
+    __syncthreads();
+    stage_map(segmented ? seg.seg_c0 : seq_chunk_off, segmented ? seg.seg_nc : nullptr,
+              segmented ? seg.seq_seg_off + N : nullptr, stage_items, NC_max, stg, table_lds);
+  }
+}
+inline void launch_tables(hipStream_t s, const int32_t* cu_seqlens, int N, int T, int NC_max, int32_t* seq_chunk_off,
+                          int32_t* chunk_seq, int32_t* chunk_tok, int32_t* chunk_len, const SegmentTable& seg,
+                          const StageTable& stg, int stage_items, void* o, int heads) {
+  const size_t lds = stg.stages > 0 ? (size_t)((stg.stages + 1) * stage_items + 1) * 4 : 0;
+  hipLaunchKernelGGL(prefill_tables_kernel, dim3(TABLE_WORKGROUPS), dim3(256), lds, s, cu_seqlens, N, T, NC_max,
+                     seq_chunk_off, chunk_seq, chunk_tok, chunk_len, seg, stg, stage_items,
+                     reinterpret_cast<uint16_t*>(o), heads);
 }
 
 inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }

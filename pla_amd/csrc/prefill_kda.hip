@@ -692,9 +692,6 @@ extern "C" int pla_kda_prefill_launch(
   p.H = H; p.NC_max = L.NC_max;
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-  hipLaunchKernelGGL(chunk_map_kernel, dim3(1), dim3(256), 0, s, cu_seqlens, N, L.NC_max, p.seq_chunk_off,
-                     p.chunk_seq, p.chunk_tok, p.chunk_len);
-  hipLaunchKernelGGL(zero_tail_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint16_t*>(o), cu_seqlens, N, T, H);
   const bool segmented = L.seg_chunks > 0;
   if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
@@ -708,18 +705,15 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.identity = reinterpret_cast<float*>(ws + L.identity);
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
-    hipLaunchKernelGGL(segment_map_kernel, dim3(1), dim3(256), 0, s, p.seq_chunk_off, N, p.seg);
   }
   if (L.stages > 0) {
     p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
     p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = L.stages;
-    const int items = segmented ? L.max_segments : N;
-    hipLaunchKernelGGL(stage_map_kernel, dim3(1), dim3(256), (size_t)((L.stages + 1) * items + 1) * 4, s,
-                       segmented ? p.seg.seg_c0 : p.seq_chunk_off, segmented ? p.seg.seg_nc : nullptr,
-                       segmented ? p.seg.seq_seg_off + N : nullptr, items, L.NC_max, p.stg);
   }
+  launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
+                segmented ? L.max_segments : N, o, H);
   const bool ok = launch_pipeline(
       s, L.stages, segmented, (unsigned)N * H, (unsigned)L.max_segments * H, &p.pass, &p.stage,
       [&](hipStream_t ps) { hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, ps, p); },
