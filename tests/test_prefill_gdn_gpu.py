@@ -71,7 +71,7 @@ def _check(w, fast=False):
 
 @pytest.mark.parametrize("lengths,tail_pad", [([64], 0), ([1], 0), ([17], 3), ([63, 65, 128], 0),
                                               ([200, 0, 33, 2049], 5), ([5555], 0)])
-@pytest.mark.parametrize("H,HV", [(2, 4), (4, 4)])
+@pytest.mark.parametrize("H,HV", [(2, 4), (4, 4), (1, 3)])
 def test_gdn_prefill_small(lengths, tail_pad, H, HV):
     from pla_amd.workloads import gdn_prefill_packed
     w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=sum(lengths) + H, tail_pad=tail_pad)
