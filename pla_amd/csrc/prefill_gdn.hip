@@ -304,16 +304,20 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPre
 //
 // Every wait is for all outstanding copies (s_waitcnt vmcnt(0)): whatever is in flight at a barrier is
 // exactly what the next half needs.
-template <typename act_t, int NB>
-__global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
+//
+// WRITE_O = false is the first sweep over segments (affine summaries only): without the query, output and P
+// tiles (62 KB of LDS) two workgroups share a CU and every chain of that sweep is resident at once.  First
+// segments then keep a copy of their start state and are swept again, with output, in the second sweep.
+template <typename act_t, int NB, bool WRITE_O>
+__global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
   constexpr int WAVES = 8 / NB;                            // NB 16-column blocks of V per wavefront
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
-  const bool zero_v = role.zero_v, write_o = role.write_o;
+  const bool zero_v = role.zero_v, write_o = WRITE_O && role.write_o;
   const int h = hv / (p.HV / p.H);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -326,11 +330,11 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 
   // distinct LDS objects: the compiler tracks outstanding direct-to-LDS loads per object
   __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];      // by chunk parity: the state update reads it last
-  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tO[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
-  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
   // decay factors by chunk parity: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
 
@@ -350,6 +354,16 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 #pragma unroll
         for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       }
+  }
+
+  if (role.keep_init != nullptr) {                   // a first segment that is swept again later: keep its start state
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
   }
 
   if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
@@ -379,13 +393,13 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     const int len = chunk_len(c);
     if (len == CHUNK) {
       plan_kq.issue(tK[c & 1], ks, wave);
-      plan_kq.issue(tQ, qs, wave);
+      if constexpr (WRITE_O) plan_kq.issue(tQ, qs, wave);
       if (!zero_v) plan_v.issue(tV, vs, wave);
     } else {
       CopyWide tail_kq, tail_v;
       tail_kq.plan((uint32_t)tok_pitch_b, len - 1, wave, lane);
       tail_kq.issue(tK[c & 1], ks, wave);
-      tail_kq.issue(tQ, qs, wave);
+      if constexpr (WRITE_O) tail_kq.issue(tQ, qs, wave);
       if (!zero_v) {
         tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
         tail_v.issue(tV, vs, wave);
@@ -393,7 +407,9 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     }
   };
   auto issue_w = [&](int c) { plan_w.issue(tW, w_b + (int64_t)c * p.HV * 8192, wave); };
-  auto issue_p = [&](int c) { plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave); };
+  auto issue_p = [&](int c) {
+    if constexpr (WRITE_O) plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave);
+  };
   auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
     if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
   };
@@ -402,7 +418,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
   const int krow = tid >> 4, kcv = tid & 15;
   uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
   auto flush_output = [&](int c) {
-    if (!write_o) return;
+    if (!WRITE_O || !write_o) return;
     const int len = chunk_len(c);
     uint16_t* dst = o_b + (int64_t)c * CHUNK * p.HV * 128;
 #pragma unroll
@@ -431,7 +447,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
       ka[0][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], 0, kb);
-      qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
+      if constexpr (WRITE_O) qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (ci > 0) flush_output(ci - 1);
@@ -455,7 +471,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
           ka[(s + 1) & 1][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], s + 1, kb);
-          qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
+          if constexpr (WRITE_O) qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
         }
       } else {
         // the last step's MFMAs cover the reads for X and for U = W X
@@ -484,10 +500,12 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
+      if constexpr (WRITE_O) {
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
+          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     // X = V - e^{G} (.) KS
@@ -546,7 +564,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
     float4 sq[4];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      if (s == 1) {
+      if (WRITE_O && s == 1) {
         // the last step's MFMAs cover the reads for the output product
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
@@ -571,6 +589,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb], St[nb][mc]);
     }
 
+    if constexpr (WRITE_O) {
     // O = scale e^{G} (.) QS + P U -> O tile
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi)
@@ -598,6 +617,7 @@ __global__ __launch_bounds__(512 / NB) void gdn_chunk_seq_kernel(const GdnPrefil
         orow[2 * PITCH128] = from_float<act_t>(QS[nb][mi][2]).bits;
         orow[3 * PITCH128] = from_float<act_t>(QS[nb][mi][3]).bits;
       }
+    }
   }
   __syncthreads();
   if (n_chunks > 0) flush_output(n_chunks - 1);
@@ -750,16 +770,21 @@ extern "C" int pla_gdn_prefill_launch(
         else hipLaunchKernelGGL(gdn_gram_solve_kernel<1>, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
       },
       [&](unsigned grid) {
-        if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2>), dim3(grid), dim3(256), 0, s, p);
-        else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3(grid), dim3(256), 0, s, p);
+        if (p.pass == 1) {        // first sweep over segments: no output
+          if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
+          else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
+        } else {
+          if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, true>), dim3(grid), dim3(256), 0, s, p);
+          else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, true>), dim3(grid), dim3(256), 0, s, p);
+        }
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+    if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, true>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, true>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
   }
   return check_launch("gdn prefill launch");
 }
