@@ -556,9 +556,8 @@ static inline SideStream* side_stream() {
 // Number of stages for a call of whole sequences: enough chains to fill the chip and 16 chunks per
 // sequence on average.  (Segmented calls already keep every CU busy with sweeps - staging them was measured
 // for GDN: 0.57 -> 0.66 ms for one sequence of 16 384 tokens, 0.99 -> 1.06 ms for 32 768 -; and staging only pays
-// where a preparation workgroup fits into a CU next to a sweep workgroup, which holds for GDN - 115 KB
-// + 18 or 33 KB of LDS - and not for KDA - 149 KB + 69 KB -, where it was measured to double the sweep
-// times.)
+// where the preparation is bound by memory latency and leaves the sweeps their issue slots, which holds for
+// GDN and not for KDA, whose preparation is instruction bound: the KDA path does not call this.)
 inline int pick_stages(int T, int N, int heads, int seg_chunks) {
   if (seg_chunks > 0) return 0;
   // (the stage map keeps (stages + 1) counters per sequence in LDS: at most 2048 sequences)

@@ -627,7 +627,10 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
     L.identity = take(16384 * 4);
   }
   // pipeline the preparation with the sweeps in stages where that pays
-  L.stages = 0;                                      // see pick_stages: the KDA kernels do not fit a CU together
+  // Not staged: a sweep (104 KB of LDS) and a preparation workgroup (51 KB) fit a CU together and the staged call
+  // is correct (bit-identical per sequence), but the instruction-bound preparation slows the sweeps more than its
+  // overlap saves: 8 x 2048 tokens, 32 heads 0.50 -> 0.57 ms, 18 x 1100 tokens, 12 heads 0.24 -> 0.31 ms.
+  L.stages = 0;
   if (L.stages > 0) {
     L.order = take((size_t)L.NC_max * 4);
     L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);

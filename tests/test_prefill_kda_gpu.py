@@ -305,3 +305,36 @@ def test_kda_prefill_split_sequences_match_oracle(lengths, pad, H):
                 assert torch.equal(final[n, head].cpu(), S0[n, head])   # an empty sequence publishes its incoming state
             else:
                 assert rel_l2(final[n, head], exp_final[n, head]) <= 1e-3, (n, head)
+
+
+def test_kda_prefill_many_chains_match_oracle_and_single_sequence_bits():
+    """128 chains of ragged lengths (an empty sequence, sequences of one token and of one chunk) in one call, against
+    the oracle; the short sequences run alone give the same bits.  (The shape is the one a pipelined call of
+    preparation and sweep would take: that variant passes this test too and is switched off for its speed.)"""
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    lengths = [3000, 0, 70, 1500, 64, 2100, 1, 1500]
+    H = 16
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=91, pad=5)
+    exp_o, exp_final = _oracle(q, k, v, raw, beta, A_log, dt_bias, offs, S0, fast=True)
+    dev = "cuda"
+    args = [t.to(dev) for t in (q, k, v, raw, beta, A_log, dt_bias)]
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    out = torch.full((q.shape[0], H, 128), 7.0, dtype=torch.bfloat16, device=dev)
+    final = torch.empty_like(S0, device=dev)
+    flashkda_fwd(*args, out, initial_state=S0.to(dev), final_state=final, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out[:offs[-1]].float().cpu(), exp_o[:offs[-1]].float(), atol=2e-2, rtol=2e-2)
+    assert torch.count_nonzero(out[offs[-1]:]) == 0
+    worst = max(rel_l2(final[n].cpu(), exp_final[n]) for n in range(len(lengths)))
+    assert worst <= 1e-3, worst
+    for n, length in enumerate(lengths):
+        if length == 0 or length >= 2048:
+            continue
+        lo, hi = offs[n], offs[n + 1]
+        one = torch.empty(hi - lo, H, 128, dtype=torch.bfloat16, device=dev)
+        fin1 = torch.empty(1, H, 128, 128, device=dev)
+        flashkda_fwd(*[t[lo:hi] for t in args[:5]], args[5], args[6], one, initial_state=S0[n:n + 1].to(dev),
+                     final_state=fin1, cu_seqlens=torch.tensor([0, hi - lo], dtype=torch.int32, device=dev))
+        torch.cuda.synchronize()
+        assert torch.equal(one, out[lo:hi]), n
+        assert torch.equal(fin1[0], final[n]), n
