@@ -336,6 +336,28 @@ int pla_gdn_prefill_launch(
     float* gcum_out, float* beta_out,
     int H, int HV, int K, int V, int act_dtype, void* stream);
 
+/*
+ * pla_gdn_prefill_launch for callers that cannot allocate (code under hipGraph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments without the workspace pair, same results bit
+ * for bit.  No counterpart in the reference.  The workspace is an array inside the library, one per GPU
+ * (PLA_GDN_PREFILL_STATIC_BYTES, held until the process ends); the call allocates nothing, creates no
+ * stream or event, and runs every kernel on `stream`.  Accepted: every shape whose
+ * pla_gdn_prefill_workspace_bytes(T, N, H, HV) is within PLA_GDN_PREFILL_STATIC_BYTES (about 3 500 tokens
+ * at H = 16, HV = 32); larger calls are rejected before any launch.  All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race and must be
+ * serialised by the caller.
+ */
+#define PLA_GDN_PREFILL_STATIC_BYTES (64ll << 20)
+int pla_gdn_prefill_launch_static(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream);
+
 /* Workspace bytes (256-byte aligned) needed by pla_kda_prefill_launch. */
 int64_t pla_kda_prefill_workspace_bytes(int T, int N, int H);
 

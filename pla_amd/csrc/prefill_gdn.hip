@@ -639,7 +639,7 @@ struct GdnWorkspaceLayout {
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
 };
-static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
+static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_stages = true) {
   GdnWorkspaceLayout L;
   L.NC_max = T / CHUNK + N;
   size_t off = 0;
@@ -667,7 +667,7 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
     L.identity = take(16384 * 4);
   }
   // pipeline the preparation with the sweeps in stages where that pays
-  L.stages = pick_stages(T, N, HV, L.seg_chunks);
+  L.stages = allow_stages ? pick_stages(T, N, HV, L.seg_chunks) : 0;
   if (L.stages > 0) {
     L.order = take((size_t)L.NC_max * 4);
     L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);
@@ -675,6 +675,25 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV) {
   }
   L.total = off;
   return L;
+}
+
+
+// Workspace of pla_gdn_prefill_launch_static: one array per GPU, held until the process ends.  In host code the
+// array's name is only a handle for the runtime, not a device address; the address on the current device comes from
+// hipGetSymbolAddress, is looked up once per device and is what kernels and launches receive.
+static __device__ __align__(256) unsigned char scratch[PLA_GDN_PREFILL_STATIC_BYTES];
+static void* static_scratch_address() {
+  static void* address[64] = {};
+  static std::mutex guard;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  std::lock_guard<std::mutex> lock(guard);
+  if (address[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    address[dev] = ptr;
+  }
+  return address[dev];
 }
 
 }  // namespace pla
@@ -686,14 +705,16 @@ extern "C" int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV) 
   return (int64_t)gdn_layout(T, N, H, HV).total;
 }
 
-extern "C" int pla_gdn_prefill_launch(
+// Checks and launches shared by the entry points below.  static_scratch: the workspace is the library's own
+// array (sized by the unstaged layout, which needs no side stream), else the caller's buffer.
+static int gdn_prefill_run(
     const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
     const void* a, const void* b, int64_t stride_a, int64_t stride_b,
     const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
     const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
     const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
     float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
-    void* o, void* workspace, int64_t workspace_bytes,
+    void* o, void* workspace, int64_t workspace_bytes, bool static_scratch,
     float* gcum_out, float* beta_out,
     int H, int HV, int K, int V, int act_dtype, void* stream) {
   PLA_REQUIRE(K == 128 && V == 128, "GDN prefill requires head_dim K == V == 128, got K=%d, V=%d", K, V);
@@ -701,15 +722,24 @@ extern "C" int pla_gdn_prefill_launch(
   PLA_REQUIRE(H > 0 && HV >= H && HV % H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", H, HV);
   PLA_REQUIRE(act_dtype == PLA_BF16 || act_dtype == PLA_F16, "GDN prefill takes bf16 or fp16 activations");
   const bool half_act = act_dtype == PLA_F16;
-  PLA_REQUIRE(q && k && v && o && cu_seqlens && workspace, "null tensor pointer");
+  PLA_REQUIRE(q && k && v && o && cu_seqlens, "null tensor pointer");
   PLA_REQUIRE((g_in != nullptr) == (beta_in != nullptr), "g and beta must be given together");
   PLA_REQUIRE(g_in != nullptr || (a && b && A_log && dt_bias), "raw gating needs a, b, A_log and dt_bias");
   PLA_REQUIRE(((uintptr_t)q % 4 == 0) && ((uintptr_t)k % 4 == 0) && stride_q % 2 == 0 && stride_k % 2 == 0,
               "q/k rows require 4-byte alignment");
   PLA_REQUIRE((uintptr_t)v % 16 == 0 && stride_v % 8 == 0, "v rows require 16-byte alignment (they are copied to LDS in 16-byte pieces)");
   PLA_REQUIRE((uintptr_t)o % 16 == 0, "o requires 16-byte alignment");
-  const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV);
-  PLA_REQUIRE(workspace_bytes >= (int64_t)L.total, "workspace too small: need %zu bytes", L.total);
+  const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV, !static_scratch);
+  if (static_scratch) {
+    PLA_REQUIRE((int64_t)L.total <= PLA_GDN_PREFILL_STATIC_BYTES,
+                "call too large for the built-in scratch array: it needs %zu bytes of workspace, the array holds %lld "
+                "(use pla_gdn_prefill_launch with a caller workspace)", L.total, (long long)PLA_GDN_PREFILL_STATIC_BYTES);
+    workspace = static_scratch_address();
+    PLA_REQUIRE(workspace != nullptr, "hipGetSymbolAddress failed for the built-in scratch array");
+  } else {
+    PLA_REQUIRE(workspace != nullptr, "null tensor pointer");
+    PLA_REQUIRE(workspace_bytes >= (int64_t)L.total, "workspace too small: need %zu bytes", L.total);
+  }
   PLA_REQUIRE((uintptr_t)workspace % 256 == 0, "workspace requires 256-byte alignment");
   if (h0) PLA_REQUIRE((uintptr_t)h0 % 16 == 0 && h0_slot_stride % 4 == 0, "state requires 16-byte alignment");
   if (ht) PLA_REQUIRE((uintptr_t)ht % 16 == 0 && ht_slot_stride % 4 == 0, "state requires 16-byte alignment");
@@ -787,4 +817,34 @@ extern "C" int pla_gdn_prefill_launch(
     else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, true>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
   }
   return check_launch("gdn prefill launch");
+}
+
+extern "C" int pla_gdn_prefill_launch(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream) {
+  return gdn_prefill_run(q, k, v, stride_q, stride_k, stride_v, a, b, stride_a, stride_b, A_log, dt_bias, g_in, beta_in,
+                         cu_seqlens, N, T, scale, normalize_qk, h0, h0_indices, h0_slot_stride, ht, ht_indices,
+                         ht_slot_stride, o, workspace, workspace_bytes, false, gcum_out, beta_out, H, HV, K, V, act_dtype,
+                         stream);
+}
+
+extern "C" int pla_gdn_prefill_launch_static(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream) {
+  return gdn_prefill_run(q, k, v, stride_q, stride_k, stride_v, a, b, stride_a, stride_b, A_log, dt_bias, g_in, beta_in,
+                         cu_seqlens, N, T, scale, normalize_qk, h0, h0_indices, h0_slot_stride, ht, ht_indices,
+                         ht_slot_stride, o, nullptr, 0, true, gcum_out, beta_out, H, HV, K, V, act_dtype, stream);
 }
