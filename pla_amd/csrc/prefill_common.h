@@ -55,6 +55,9 @@ __device__ __forceinline__ f32x4_t mfma_hilo(const HiLo& a, const HiLo& b, f32x4
   return mfma16(a.hi, b.hi, c);
 }
 
+// PAIR: W leaves as two fp16 tiles, hi at W and lo at W + 4096 (W = hi + lo to about 22 bits), else as one tile
+// rounded to nearest.
+template <bool PAIR>
 __device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const float* beta, int lane, uint16_t* W) {
   const int r16 = lane & 15, kb = lane >> 4;
   const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
@@ -132,11 +135,15 @@ __device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const floa
     const int i = 8 * pass + (lane >> 3);
     const float4 lo = *reinterpret_cast<const float4*>(&L[i][c8]), hi = *reinterpret_cast<const float4*>(&L[i][c8 + 4]);
     const float w[8] = {lo.x * b0.x, lo.y * b0.y, lo.z * b0.z, lo.w * b0.w, hi.x * b1.x, hi.y * b1.y, hi.z * b1.z, hi.w * b1.w};
-    uint32_t packed[4];
+    uint32_t packed[4], rest[4];
 #pragma unroll
-    for (int e = 0; e < 4; ++e)
-      packed[e] = pack2<f16_t>(c8 + 2 * e <= i ? w[2 * e] : 0.f, c8 + 2 * e + 1 <= i ? w[2 * e + 1] : 0.f);
+    for (int e = 0; e < 4; ++e) {
+      const float w0 = c8 + 2 * e <= i ? w[2 * e] : 0.f, w1 = c8 + 2 * e + 1 <= i ? w[2 * e + 1] : 0.f;
+      if constexpr (PAIR) pack2_pair(w0, w1, packed[e], rest[e]);
+      else packed[e] = pack2<f16_t>(w0, w1);
+    }
     *reinterpret_cast<uint4*>(W + i * 64 + c8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+    if constexpr (PAIR) *reinterpret_cast<uint4*>(W + 4096 + i * 64 + c8) = make_uint4(rest[0], rest[1], rest[2], rest[3]);
   }
 }
 

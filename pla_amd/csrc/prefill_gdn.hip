@@ -56,7 +56,8 @@ struct GdnPrefillParams {
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
   uint16_t* qn; uint16_t* kn;
   float* gcum; float* beta;
-  uint16_t* W; uint16_t* P;                           // fp16 [chunk, HV, 64, 64]
+  uint16_t* W;                                        // fp16 [chunk, HV, 2, 64, 64]: W = hi + lo
+  uint16_t* P;                                        // fp16 [chunk, HV, 64, 64]
   float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
   SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
   StageTable stg;        // pipelined preparation and sweep (stg.stages > 0)
@@ -150,10 +151,10 @@ __global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p)
     }
     if (j < len) {
       const int64_t t = t0 + j;
-      // rounded to the activation dtype (the reference's operand), then held as fp16
+      // rounded to the activation dtype (the reference's operand), then held as fp16 (exact; saturating beyond its range)
       const uint32_t qa = pack2<act_t>(q0, q1), ka = pack2<act_t>(k0, k1);
-      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2<f16_t>(lo16<act_t>(qa), hi16<act_t>(qa));
-      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2<f16_t>(lo16<act_t>(ka), hi16<act_t>(ka));
+      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2_rtz(lo16<act_t>(qa), hi16<act_t>(qa));
+      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2_rtz(lo16<act_t>(ka), hi16<act_t>(ka));
     }
   }
 }
@@ -249,13 +250,13 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPre
         const int i = 16 * mi + 4 * kb + r;
         pv[r] = i >= j ? p.scale * qk[r] * __expf(Gs[i] - Gj) : 0.f;
       }
-      Ppk[mi * (mi + 1) / 2 + ni][0] = pack2<f16_t>(pv[0], pv[1]);
-      Ppk[mi * (mi + 1) / 2 + ni][1] = pack2<f16_t>(pv[2], pv[3]);
+      Ppk[mi * (mi + 1) / 2 + ni][0] = pack2_rtz(pv[0], pv[1]);
+      Ppk[mi * (mi + 1) / 2 + ni][1] = pack2_rtz(pv[2], pv[3]);
     }
   }
 
   // W = (I + L)^-1 diag(beta): 16 x 16 blocks, the off-diagonal ones on MFMA
-  block_inverse_store_w(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * 4096);
+  block_inverse_store_w<true>(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * 8192);
   __syncthreads();
 
   // P leaves through the released tile in 16-byte pieces; blocks above the diagonal are never written and read as zero
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
   __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
-  __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tW[2][CHUNK * PITCH64];      // hi and lo parts
   __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
   // decay factors by chunk parity: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
@@ -374,7 +375,7 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
   const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 8192;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
   const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
   const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
 
@@ -406,7 +407,10 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
       }
     }
   };
-  auto issue_w = [&](int c) { plan_w.issue(tW, w_b + (int64_t)c * p.HV * 8192, wave); };
+  auto issue_w = [&](int c) {
+    plan_w.issue(tW[0], w_b + (int64_t)c * p.HV * 16384, wave);
+    plan_w.issue(tW[1], w_b + (int64_t)c * p.HV * 16384 + 8192, wave);
+  };
   auto issue_p = [&](int c) {
     if constexpr (WRITE_O) plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave);
   };
@@ -461,10 +465,10 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
     float4 eg[4];
     uint16_t vraw[NB][16];
-    bf16x8_t wa[2][4];
+    bf16x8_t wa[2][4], wl[2][4];
     bf16x8_t sb[2][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8(St[nb][0], St[nb][1]);
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
@@ -488,13 +492,16 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) wa[s2][mi] = operand_from(&tW[(16 * mi + r16) * PITCH64], s2, kb);
+          for (int mi = 0; mi < 4; ++mi) {
+            wa[s2][mi] = operand_from(&tW[0][(16 * mi + r16) * PITCH64], s2, kb);
+            wl[s2][mi] = operand_from(&tW[1][(16 * mi + r16) * PITCH64], s2, kb);
+          }
       }
       __builtin_amdgcn_sched_barrier(0);
       // the next step's state slice is rounded underneath this step's MFMAs
       if (s < 3) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -529,7 +536,11 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
     for (int s = 0; s < 2; ++s) {
       bf16x8_t xb[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8(X[nb][2 * s], X[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -574,19 +585,23 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
         for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
         __builtin_amdgcn_sched_barrier(0);
       }
-      bf16x8_t ub[NB];
+      HalfPair ub[NB];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) {
         const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
                             U[nb][2 * s][3] * dg[s][0].w};
         const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
                             U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
-        ub[nb] = half8(u0, u1);
+        ub[nb] = half8_pair(u0, u1);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb], St[nb][mc]);
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
     }
 
     if constexpr (WRITE_O) {
@@ -601,7 +616,7 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
     for (int s = 0; s < 2; ++s) {
       bf16x8_t ur[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -653,7 +668,7 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_sta
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
   L.gtile = take((size_t)L.NC_max * HV * 256 * 4);
-  L.W = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.W = take((size_t)L.NC_max * HV * 8192 * 2);
   L.P = take((size_t)L.NC_max * HV * 4096 * 2);
   L.seg_chunks = pick_segment_chunks(T, N, HV);
   L.max_segments = max_segments(T, N, L.seg_chunks);

@@ -42,8 +42,10 @@ struct KdaPrefillParams {
   void* o;
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
   // operand tiles of the sweeps, fp16 (every factor lies in (0, 1]; values below 6e-8 vanish)
-  uint16_t* Kg; uint16_t* Qg; uint16_t* Kt;        // [chunk, H, 64, 128]: k e^{G}, scale q e^{G}, k e^{G_last - G}
-  uint16_t* W; uint16_t* P;                        // [chunk, H, 64, 64]
+  uint16_t* Kg; uint16_t* Qg;                      // [chunk, H, 64, 128]: k e^{G}, scale q e^{G}
+  uint16_t* Kt;                                    // [chunk, H, 2, 64, 128]: k e^{G_last - G} as an fp16 hi + lo pair
+  uint16_t* W;                                     // [chunk, H, 2, 64, 64]: W = hi + lo
+  uint16_t* P;                                     // [chunk, H, 64, 64]
   float* eGlast;                                   // [chunk, H, 128]: e^{G_last}
   SegmentTable seg;                                // split long sequences (seg.seg_chunks > 0)
   StageTable stg;                                  // pipelined preparation and sweep (stg.stages > 0)
@@ -194,7 +196,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       const int j = (tid >> 4) + 16 * u, c0 = 8 * (tid & 15);   // the rows and channels this thread normalised
       const uint32_t* const kwv = kn[u];
       const uint32_t* const qwv = qn[u];
-      uint32_t kg[4], qg[4], kt[4];
+      uint32_t kg[4], qg[4], kt[4], ktl[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float g0 = sh.G[j][c0 + 2 * e], g1 = sh.G[j][c0 + 2 * e + 1];
@@ -202,12 +204,14 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
         const float k0 = lo16<bf16_t>(kwv[e]), k1 = hi16<bf16_t>(kwv[e]);
         kg[e] = pack2<f16_t>(k0 * e0, k1 * e1);
         qg[e] = pack2<f16_t>(p.scale * lo16<bf16_t>(qwv[e]) * e0, p.scale * hi16<bf16_t>(qwv[e]) * e1);
-        kt[e] = pack2<f16_t>(k0 * __expf(glast[c0 + 2 * e] - g0), k1 * __expf(glast[c0 + 2 * e + 1] - g1));
+        pack2_pair(k0 * __expf(glast[c0 + 2 * e] - g0), k1 * __expf(glast[c0 + 2 * e + 1] - g1), kt[e], ktl[e]);
       }
       const int64_t off = tile * 8192 + (int64_t)j * 128 + c0;
       *reinterpret_cast<uint4*>(p.Kg + off) = make_uint4(kg[0], kg[1], kg[2], kg[3]);
       *reinterpret_cast<uint4*>(p.Qg + off) = make_uint4(qg[0], qg[1], qg[2], qg[3]);
-      *reinterpret_cast<uint4*>(p.Kt + off) = make_uint4(kt[0], kt[1], kt[2], kt[3]);
+      const int64_t off2 = tile * 16384 + (int64_t)j * 128 + c0;
+      *reinterpret_cast<uint4*>(p.Kt + off2) = make_uint4(kt[0], kt[1], kt[2], kt[3]);
+      *reinterpret_cast<uint4*>(p.Kt + off2 + 8192) = make_uint4(ktl[0], ktl[1], ktl[2], ktl[3]);
     }
   }
 
@@ -283,7 +287,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 
   // ---- phase 4: W = L^-1 diag(beta) by blocks on one wavefront (which one rotates with the workgroup, so
   // that co-resident workgroups keep different SIMDs busy) -----------------------------------------
-  if (wave == (int)(blockIdx.x & 3)) block_inverse_store_w(sh.L, sh.B, lane, p.W + tile * 4096);
+  if (wave == (int)(blockIdx.x & 3)) block_inverse_store_w<true>(sh.L, sh.B, lane, p.W + tile * 8192);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 // WRITE_O = false is the first sweep over segments (affine summaries only): without the query, output and
 // P tiles the workgroup holds 60 KB of LDS and at most 256 registers per lane, so two of them share a CU.
 template <bool WRITE_O>
-__global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
+__global__ __launch_bounds__(256, 1) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2, WAVES = 4;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
@@ -338,8 +342,8 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
   __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
-  __shared__ __align__(16) uint16_t tKt[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tW[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];      // hi and lo parts
+  __shared__ __align__(16) uint16_t tW[2][CHUNK * PITCH64];        // hi and lo parts
   __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
   __shared__ __align__(16) float tE[128];            // e^{G_last} of the chunk
 
@@ -374,8 +378,8 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
   const int64_t tile0 = (int64_t)c_begin * p.H + h;                       // chunk tiles are [chunk, H, ...]
   const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
   const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
-  const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 16384;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 8192;
+  const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
   const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
   const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
@@ -401,10 +405,12 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
         tail_v.issue(tV, vs, wave);
       }
     }
-    plan_w.issue(tW, w_b + c * small_step, wave);
+    plan_w.issue(tW[0], w_b + c * 2 * small_step, wave);
+    plan_w.issue(tW[1], w_b + c * 2 * small_step + 8192, wave);
   };
   auto issue_second = [&](int c) {                   // K e^{G_last-G}, P, e^{G_last}
-    plan_k.issue(tKt, kt_b + c * big_step, wave);
+    plan_k.issue(tKt[0], kt_b + c * 2 * big_step, wave);
+    plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, wave);
     if constexpr (WRITE_O) plan_w.issue(tP, pp_b + c * small_step, wave);
     if (wave == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
   };
@@ -446,10 +452,10 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
     uint16_t vraw[NB][16];
-    bf16x8_t wa[2][4];
+    bf16x8_t wa[2][4], wl[2][4];
     bf16x8_t sb[2][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8(St[nb][0], St[nb][1]);
+    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
       if (s < 3) {
@@ -471,13 +477,16 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) wa[s2][mi] = operand_from(&tW[(16 * mi + r16) * PITCH64], s2, kb);
+          for (int mi = 0; mi < 4; ++mi) {
+            wa[s2][mi] = operand_from(&tW[0][(16 * mi + r16) * PITCH64], s2, kb);
+            wl[s2][mi] = operand_from(&tW[1][(16 * mi + r16) * PITCH64], s2, kb);
+          }
       }
       __builtin_amdgcn_sched_barrier(0);
       // the next step's state slice is rounded underneath this step's MFMAs
       if (s < 3) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
       }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -509,7 +518,11 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
     for (int s = 0; s < 2; ++s) {
       bf16x8_t xb[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8(X[nb][2 * s], X[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -519,11 +532,13 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
     // barrier B
     wait_vmcnt<0>();
     __syncthreads();
-    bf16x8_t kt[2][8];
+    bf16x8_t kt[2][8], ktl[8];
 #pragma unroll
     for (int s = 0; s < 2; ++s)
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tKt, s, mc, kb, r16);
+      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tKt[0], s, mc, kb, r16);
+#pragma unroll
+    for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
     float4 eg[8];
 #pragma unroll
     for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
@@ -547,13 +562,26 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
           for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
         __builtin_amdgcn_sched_barrier(0);
       }
-      bf16x8_t ub[NB];
+      HalfPair ub[NB];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ub[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
+      for (int nb = 0; nb < NB; ++nb) ub[nb] = half8_pair(U[nb][2 * s], U[nb][2 * s + 1]);
+      // hi . lo and lo . hi first, the large term last
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb], St[nb][mc]);
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
+      if (s == 0) {
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
       __builtin_amdgcn_sched_barrier(0);
     }
 
@@ -563,7 +591,7 @@ __global__ __launch_bounds__(256, WRITE_O ? 1 : 2) void kda_chunk_seq_kernel(con
       for (int s = 0; s < 2; ++s) {
         bf16x8_t ur[NB];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) ur[nb] = half8(U[nb][2 * s], U[nb][2 * s + 1]);
+        for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -612,8 +640,8 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   L.chunk_tok = take((size_t)L.NC_max * 4);
   L.chunk_len = take((size_t)L.NC_max * 4);
   const size_t big = (size_t)L.NC_max * H * 8192 * 2, small = (size_t)L.NC_max * H * 4096 * 2;
-  L.Kg = take(big); L.Qg = take(big); L.Kt = take(big);
-  L.W = take(small); L.P = take(small);
+  L.Kg = take(big); L.Qg = take(big); L.Kt = take(2 * big);
+  L.W = take(2 * small); L.P = take(small);
   L.eGlast = take((size_t)L.NC_max * H * 128 * 4);
   L.seg_chunks = pick_segment_chunks(T, N, H);
   L.max_segments = max_segments(T, N, L.seg_chunks);

@@ -338,3 +338,32 @@ def test_kda_prefill_many_chains_match_oracle_and_single_sequence_bits():
         torch.cuda.synchronize()
         assert torch.equal(one, out[lo:hi]), n
         assert torch.equal(fin1[0], final[n]), n
+
+
+@pytest.mark.parametrize("lengths,noise", [([200, 131], 0.1), ([1000, 700], 0.1), ([640], 0.03)])
+def test_kda_prefill_correlated_keys_dense_triangular_system(lengths, noise):
+    """The correlated-key stress of the GDN prefill on the KDA path: keys = one direction per head plus `noise` x
+    N(0, 1), beta = 0.982, a per-channel log-decay of -1.7e-3 per token.  Every entry of the chunk's triangular
+    system is of order one, U = W X cancels heavily and the final state is the work of the last few tokens, so
+    operand roundings show unaveraged; the bounds are the usual ones."""
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    H = 2
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=41 + len(lengths))
+    g = torch.Generator().manual_seed(5)
+    k = (torch.randn(1, H, 128, generator=g) + noise * torch.randn(q.shape[0], H, 128, generator=g)).bfloat16()
+    beta = torch.full_like(beta, 4.0)
+    raw = torch.full_like(raw, -8.0)
+    A_log = torch.zeros_like(A_log)
+    dt_bias = torch.zeros_like(dt_bias)
+    exp_o, exp_final = _oracle(q, k, v, raw, beta, A_log, dt_bias, offs, S0, fast=sum(lengths) > 600)
+    dev = "cuda"
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    out = torch.empty(q.shape[0], H, 128, dtype=torch.bfloat16, device=dev)
+    final = torch.empty(len(lengths), H, 128, 128, device=dev)
+    flashkda_fwd(*[t.to(dev) for t in (q, k, v, raw, beta, A_log, dt_bias)], out, initial_state=S0.to(dev),
+                 final_state=final, cu_seqlens=cu)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
+    worst = max(rel_l2(final[n], exp_final[n]) for n in range(len(lengths)))
+    print("KDA correlated keys", lengths, noise, "state rel-L2 %.3e" % worst)
+    assert worst <= 1e-3, worst

@@ -46,9 +46,9 @@ def test_static_scratch_prefill_equals_workspace_prefill_twice_then_rejects_over
     from pla_amd import _lib
     from pla_amd.workloads import gdn_prefill_packed
     size = _lib.load().pla_gdn_prefill_workspace_bytes
-    # first call: staged in the workspace form (128 chains, 16 chunks per sequence), unstaged in the array;
+    # first call: 64 chains of up to 18 chunks;
     # second call: smaller, ragged, with an empty sequence and a padded tail
-    cases = [dict(lengths=[1100, 1030], H=16, HV=64, tail_pad=0, seed=11),
+    cases = [dict(lengths=[1100, 700], H=16, HV=32, tail_pad=0, seed=11),
              dict(lengths=[200, 0, 33, 450], H=2, HV=4, tail_pad=5, seed=12)]
     for case in cases:
         lengths = case["lengths"]
