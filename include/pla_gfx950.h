@@ -269,8 +269,9 @@ int pla_kda_replay_verify_native_launch(
  * requests).  Replaces launch_commit_plan (src/decode/kda_replayssm_vllm/commit_plan.h:7-14, kernels
  * commit_plan.cu:19-117).  Index vectors are dense int32 or int64 (is_int64 flags): sampled [sampler_rows],
  * source [batch], offsets [batch+1], mapping [batch] or NULL, computed [>= sampler rows] and blocks
- * [block_rows, block_cols] (strides in elements) or both NULL with block_size 0.  candidate and plan:
- * int32 [4, capacity], distinct buffers.
+ * [block_rows, block_cols] (strides in elements) or both NULL with block_size 0.  plan: int32 [4, capacity];
+ * candidate: int32 scratch of the same size, a distinct buffer (it holds the requests' slot claims when the
+ * capacity exceeds the 4096 requests whose claims fit into LDS).
  */
 int pla_kda_commit_plan_launch(
     const void* sampled, int sampled_wide, const void* source, int source_wide, const void* offsets, int offsets_wide,

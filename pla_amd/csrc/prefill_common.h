@@ -534,31 +534,65 @@ inline void launch_tables(hipStream_t s, const int32_t* cu_seqlens, int N, int T
 
 inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-// One side stream (default priority, non-blocking) and its events per device, created on first use and
-// kept for the life of the process (creation is serialised; the calls themselves are expected from one
-// host thread at a time per device, as the events are shared).
+// Side streams (default priority, non-blocking), each with its own fork / ready events.  A call takes one from
+// its device's pool for the time it enqueues its launches and puts it back before it returns, so calls that
+// are enqueued concurrently (host threads launching on different streams) never share a stream or an event,
+// while consecutive calls reuse the same few objects: an event wait binds to the record that precedes it in
+// the calling thread, and work queued on a reused side stream simply runs after the previous call's.  A side
+// stream that is part of an unfinished graph capture is passed over.  Streams and events are created on first
+// need and kept for the life of the process.
 struct SideStream {
   hipStream_t stream;
   hipEvent_t fork;
   hipEvent_t ready[MAX_STAGES];
+  bool busy;
 };
-static inline SideStream* side_stream() {
-  static SideStream table[16];
-  static bool made[16] = {};
-  static std::mutex guard;
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
-  std::lock_guard<std::mutex> lock(guard);
-  if (!made[dev]) {
-    SideStream& t = table[dev];
-    if (hipStreamCreateWithFlags(&t.stream, hipStreamNonBlocking) != hipSuccess) return nullptr;
-    if (hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
-    for (int i = 0; i < MAX_STAGES; ++i)
-      if (hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) != hipSuccess) return nullptr;
-    made[dev] = true;
+class SideStreamLease {
+ public:
+  SideStreamLease() : taken_(nullptr) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return;
+    std::lock_guard<std::mutex> lock(guard());
+    SideStream* const pool = pools()[dev];
+    for (int i = 0; i < POOL; ++i)
+      if (pool[i].stream != nullptr && !pool[i].busy && !capturing(pool[i].stream)) { taken_ = &pool[i]; break; }
+    if (taken_ == nullptr)
+      for (int i = 0; i < POOL; ++i)
+        if (pool[i].stream == nullptr) {
+          if (create(pool[i])) taken_ = &pool[i];
+          break;
+        }
+    if (taken_ != nullptr) taken_->busy = true;
   }
-  return &table[dev];
-}
+  ~SideStreamLease() {
+    if (taken_ == nullptr) return;
+    std::lock_guard<std::mutex> lock(guard());
+    taken_->busy = false;
+  }
+  SideStreamLease(const SideStreamLease&) = delete;
+  SideStreamLease& operator=(const SideStreamLease&) = delete;
+  SideStream* get() const { return taken_; }     // nullptr: none could be created, or more than POOL calls at once
+
+ private:
+  static constexpr int MAX_DEVICES = 64, POOL = 16;
+  static std::mutex& guard() { static std::mutex m; return m; }
+  static SideStream (*pools())[POOL] { static SideStream table[MAX_DEVICES][POOL] = {}; return table; }
+  // a side stream that joined a graph capture stays part of it until the capture ends: leave it to that capture
+  static bool capturing(hipStream_t stream) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    return hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+  }
+  static bool create(SideStream& t) {
+    hipStream_t stream = nullptr;
+    if (hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) != hipSuccess) return false;
+    bool ok = hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) == hipSuccess;
+    for (int i = 0; i < MAX_STAGES && ok; ++i) ok = hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) == hipSuccess;
+    if (!ok) return false;
+    t.stream = stream;
+    return true;
+  }
+  SideStream* taken_;
+};
 
 // Number of stages for a call of whole sequences: enough chains to fill the chip and 16 chunks per
 // sequence on average.  (Segmented calls already keep every CU busy with sweeps - staging them was measured
@@ -586,7 +620,8 @@ inline bool launch_pipeline(hipStream_t s, int stages, bool segmented, unsigned 
     sweep(grid);
     return true;
   }
-  SideStream* side = side_stream();
+  const SideStreamLease lease;
+  SideStream* const side = lease.get();
   if (side == nullptr) return false;
   bool ok = true;
   for (int st = 0; st < stages; ++st) {

@@ -350,3 +350,46 @@ def test_gdn_prefill_operands_beyond_the_fp16_range_stay_finite():
     assert float(o[0, offs[0]:offs[1]].float().abs().max()) <= 64 * big and float(final[0].abs().max()) <= 64 * big
     torch.testing.assert_close(o[0, offs[1]:offs[2]].cpu().float(), exp_o[offs[1]:offs[2]].float(), atol=2e-2, rtol=2e-2)
     assert rel_l2(final[1], exp_final[1]) <= 1e-3
+
+
+def test_gdn_prefill_staged_calls_from_two_threads_on_two_streams():
+    """Two host threads, each on a stream of its own, enqueue staged calls (fork to a side stream, join again) at
+    the same time: every call takes a side stream and events of its own for the time it enqueues, so neither waits
+    on the other's events nor reads workspace tiles that are not prepared yet.  Each thread's results equal, bit
+    for bit, what the same call gives when it runs alone."""
+    import threading
+    from pla_amd.workloads import gdn_prefill_packed
+    works = [gdn_prefill_packed([1500, 2100, 900, 1500, 1300, 1100, 700, 1200], H=4, HV=16, pool_slots=10, seed=31),
+             gdn_prefill_packed([2300, 1700, 1100, 1900, 1600, 1250, 1800, 1400], H=4, HV=16, pool_slots=10, seed=32)]
+    pools = [w["initial_state"].clone() for w in works]
+    alone = []
+    for w in works:
+        _, _, o, _, _ = _run_workload(w, output_final_state=False)
+        torch.cuda.synchronize()
+        alone.append((o.clone(), w["initial_state"].clone()))
+    rounds = 6
+    errors = []
+    start = threading.Barrier(2)
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            w, pool0 = works[i], pools[i]
+            with torch.cuda.stream(stream):
+                start.wait()
+                for _ in range(rounds):
+                    w["initial_state"].copy_(pool0)
+                    _, _, o, _, _ = _run_workload(w, output_final_state=False)
+                    stream.synchronize()
+                    if not (torch.equal(o, alone[i][0]) and torch.equal(w["initial_state"], alone[i][1])):
+                        errors.append(i)
+        except Exception as exc:          # surfaced in the main thread
+            errors.append(repr(exc))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors

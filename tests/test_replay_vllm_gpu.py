@@ -348,3 +348,42 @@ def test_replay_commit_context_checks_and_graph_replay():
             for b, s in enumerate(slots):
                 changed = not torch.equal(layer.state[s], old[s])
                 assert changed == (want[b] > 0)
+
+
+@pytest.mark.parametrize("capacity", [384, 5000])
+@pytest.mark.parametrize("align", [False, True])
+def test_commit_plan_random_requests_match_the_oracle(capacity, align):
+    """The plan kernel alone, through the C ABI, on 300 random requests with few slots (so that destinations
+    clash), invalid sources, empty and oversized intervals and a sampler mapping; a capacity of 5000 keeps the
+    requests' claims in the caller's scratch rows instead of LDS."""
+    from pla_amd import _lib
+    gen = torch.Generator().manual_seed(capacity + int(align))
+    batch, slots, q, rows = 300, 900, 4, 320
+    block_size, cols = 8, 5
+    ri = lambda lo, hi, n: torch.randint(lo, hi, (n,), generator=gen)
+    lengths = ri(0, q + 2, batch)
+    offsets = [0] + lengths.cumsum(0).tolist()
+    token_capacity = offsets[-1] - 3                       # the last intervals end beyond the capacity
+    source = ri(-2, slots + 3, batch).tolist()
+    sampled = ri(-1, q + 2, rows).tolist()
+    mapping = ri(-1, rows + 2, batch).tolist()
+    computed = ri(-1, block_size * (cols + 1), rows).tolist()
+    table = ri(-1, slots + 2, rows * cols).reshape(rows, cols).tolist()
+    want = replay_commit_plan_reference(
+        sampled, source, offsets, slots=slots, Q=q, token_capacity=token_capacity, null_block_id=0,
+        request_indices=mapping, block_table=table if align else None, num_computed_tokens=computed if align else None,
+        block_size=block_size if align else None, capacity=capacity)
+    dev = "cuda"
+    t = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    d_sampled, d_source, d_offsets, d_mapping, d_computed, d_table = (t(x) for x in (sampled, source, offsets, mapping,
+                                                                                      computed, table))
+    scratch = torch.full((4, capacity), -9, dtype=torch.int32, device=dev)
+    plan = torch.full((4, capacity), -9, dtype=torch.int32, device=dev)
+    _lib.call("pla_kda_commit_plan_launch", d_sampled.data_ptr(), 0, d_source.data_ptr(), 0, d_offsets.data_ptr(), 0,
+              d_mapping.data_ptr(), 0, d_computed.data_ptr() if align else None, 0, d_table.data_ptr() if align else None, 0,
+              batch, capacity, rows, rows if align else 0, cols if align else 0, slots, q, 0, token_capacity,
+              cols if align else 0, 1 if align else 0, block_size if align else 0,
+              scratch.data_ptr(), plan.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert plan.cpu().tolist() == want
+    assert sum(1 for n in want[0] if n) >= 20 and sum(1 for n in want[0][:batch] if not n) >= 20
