@@ -61,6 +61,46 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+BINDING_SRC = os.path.join(CSRC, "decode_binding.cpp")
+
+
+def binding_path():
+    import sysconfig
+    return os.path.join(HERE, "decode", "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+
+
+def build_binding(verbose=True):
+    """Compile pla_amd/decode/_C (pybind11 over the C ABI; host code only, g++) against this interpreter's torch.
+
+    The module links libpla_gfx950.so by a path relative to itself; torch's libraries are found because importing
+    torch precedes importing the module (the reference's extension relies on the same order).
+    """
+    import sysconfig
+    import torch
+    from torch.utils import cpp_extension
+    cxx = shutil.which("g++") or shutil.which("c++")
+    if cxx is None:
+        raise RuntimeError("g++ not found; pla_amd.decode._C cannot be built")
+    out = binding_path()
+    tmp = out + ".tmp"
+    incs = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include"]
+    libdirs = cpp_extension.library_paths() + [LIB_DIR]
+    cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-attributes",
+           "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H", "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           *["-I" + p for p in incs], BINDING_SRC, "-o", tmp,
+           *["-L" + p for p in libdirs], "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
+           "-lpla_gfx950", "-Wl,-rpath,$ORIGIN/../lib"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building pla_amd.decode._C failed:\n%s\n%s" % (proc.stdout, proc.stderr[-4000:]))
+    os.replace(tmp, out)
+    if verbose:
+        print("built", out)
+    return out
+
+
 if __name__ == "__main__":
     build_library()
+    build_binding()
     sys.exit(0)

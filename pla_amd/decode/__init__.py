@@ -25,6 +25,38 @@ __all__ = [
 
 _BYPASS = os.environ.get("PLA_BYPASS_EXEC", "0") == "1"   # read once, like src/bypass_exec.h:44-50
 
+# The compiled host layer (pybind11 over the same C ABI; pla_amd/csrc/decode_binding.cpp): the two public entry
+# points go through it, as the reference's facade goes through pla.decode._C.  It is imported on first use.  The
+# Python implementations below are the same checks and the same launches through ctypes; they serve the
+# PLA_SANITY_CHECK diagnostics (value checks that read tensors back), the tunable entry points' callers that
+# pass a tile, and a tree in which only the library has been built (`python -m pla_amd.build` builds both).
+_native = None
+
+
+def _compiled():
+    global _native
+    if _native is None:
+        try:
+            # importlib, not `from . import _C`: the latter falls back to this module's __getattr__ when the
+            # import fails and would recurse
+            import importlib
+            module = importlib.import_module("._C", __name__)
+        except ModuleNotFoundError as exc:
+            if exc.name is None or not exc.name.endswith("_C"):
+                raise
+            module = False
+        _native = module
+    return _native
+
+
+def __getattr__(name):
+    if name == "_C":
+        module = _compiled()
+        if module is False:
+            raise ImportError("pla.decode._C is not built: run `python -m pla_amd.build`")
+        return module
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
+
 
 def _check(cond, msg):
     if not cond:
@@ -131,6 +163,11 @@ def fused_sigmoid_gating_delta_rule_forward_k_last_packed(
     otherwise) yields zeros and touches no state; a request of length zero
     touches nothing.
     """
+    native = _compiled()
+    if native and not _sanity_enabled():
+        return native.fused_sigmoid_gating_delta_rule_forward_k_last_packed(
+            mixed_qkv, a, b, A_log, dt_bias, softplus_beta, softplus_threshold, scale, initial_state_source,
+            initial_state_indices, out, use_qk_l2norm_in_kernel, cu_seqlens, is_kda, is_sglang)
     return _packed_impl(mixed_qkv, a, b, A_log, dt_bias, softplus_beta, softplus_threshold, scale,
                         initial_state_source, initial_state_indices, out, use_qk_l2norm_in_kernel,
                         cu_seqlens, is_kda, is_sglang, None)
@@ -323,6 +360,13 @@ def fused_sigmoid_gating_delta_rule_forward_k_last(
     ``retrieve_parent_token`` adds the eagle-tree parent reload;
     ``disable_state_update`` suppresses the final write-back.
     """
+    native = _compiled()
+    if native and not _sanity_enabled():
+        return native.fused_sigmoid_gating_delta_rule_forward_k_last(
+            A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, b, initial_state_source,
+            initial_state_indices, scale, use_qk_l2norm_in_kernel, cu_seqlens, is_kda, disable_state_update,
+            intermediate_states_buffer, intermediate_state_indices, cache_steps_or_num_accept, retrieve_parent_token,
+            lower_bound, is_sglang, out)
     return _k_last_impl(A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, b,
                         initial_state_source, initial_state_indices, scale, use_qk_l2norm_in_kernel,
                         cu_seqlens, is_kda, disable_state_update, intermediate_states_buffer,
