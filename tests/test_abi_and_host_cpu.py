@@ -83,7 +83,9 @@ def test_facade_validation_raises_before_native_code():
                torch.zeros(HV), torch.zeros(HV, dtype=torch.bfloat16), 1.0, 20.0, None, state,
                torch.zeros(2, dtype=torch.int32), torch.zeros(2, 1, HV, 128, dtype=torch.bfloat16), True, None, False)
     with pytest.raises(RuntimeError, match="initial_state_source is required"):
-        packed(mixed, None, None, None, None, 1.0, 20.0, None, None, None, None, True, None, False)
+        packed(mixed, torch.zeros(2, HV, dtype=torch.bfloat16), torch.zeros(2, HV, dtype=torch.bfloat16),
+               torch.zeros(HV), torch.zeros(HV, dtype=torch.bfloat16), 1.0, 20.0, None, None, None,
+               torch.zeros(2, 1, HV, 128, dtype=torch.bfloat16), True, None, False)
     with pytest.raises(ValueError, match="CUDA tensor"):
         gdn_prefill_packed_qkv_fwd(torch.zeros(4, 1024, dtype=torch.bfloat16), None, None, None, None, None,
                                    num_qk_heads=2, num_v_heads=4)
