@@ -123,7 +123,31 @@ GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 2691000000
 KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 10636000000
 
 
-def bench_prefill(steps, warmup, device):
+def cpu_baseline_prefill(w):
+    """The CPU oracle's token recurrence (FP32, vectorised over heads) over ALL tokens of config 3, one pass, all
+    host cores: tokens/s beside the GPU figure."""
+    import torch
+    from oracle import gdn_prefill_reference
+    m = w["_meta"]
+    T, H, HV = m["T"], m["H"], m["HV"]
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    packed = w["packed_qkv"].cpu()
+    q = packed[:, : H * 128].reshape(T, H, 128)
+    k = packed[:, H * 128: 2 * H * 128].reshape(T, H, 128)
+    v = packed[:, 2 * H * 128:].reshape(T, HV, 128)
+    S0 = w["initial_state"][w["initial_state_indices"].long()].cpu()
+    args = (q, k, v, w["raw_gate_a"].cpu(), w["raw_beta_b"].cpu(), w["A_log"].cpu(), w["dt_bias"].cpu(), m["offsets"], S0)
+    t0 = time.perf_counter()
+    gdn_prefill_reference(*args, scale=w["scale"])
+    t = time.perf_counter() - t0
+    tokens = m["offsets"][-1]
+    return dict(value=round(tokens / t, 1), unit="tokens/s", cores=threads, kind="port",
+                sample="all %d tokens of the 8 sequences, one pass of the token recurrence (%.1f s)" % (tokens, t),
+                threads_torch=torch.get_num_threads())
+
+
+def bench_prefill(steps, warmup, device, cpu_leg=False):
     """Config 3: GDN chunk-64 prefill, 8 ragged sequences (about 32K tokens), indexed FP32 pool."""
     import torch
     from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
@@ -149,7 +173,8 @@ def bench_prefill(steps, warmup, device):
     ms = start.elapsed_time(end) / steps
     T = sum(lengths)
     tflops = GDN_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
-    return dict(tokens=T, lengths=lengths, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
+    extra = dict(cpu_baseline=cpu_baseline_prefill(w)) if cpu_leg else {}
+    return dict(tokens=T, lengths=lengths, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1), **extra,
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
                               frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=GDN_PREFILL_TRAFFIC_BYTES_PER_CALL,
                               hbm_GBps=round(GDN_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
@@ -414,34 +439,36 @@ def bench_replay_paged(device, steps=100, N=64, H=32, Q=4, layout="SD"):
             "commit_us": round(us_commit, 2), "commit_state_GBps": round(touched * H * 131072 / us_commit / 1e3, 1)}
 
 
-def cpu_baseline_decode(w, sample_requests=32, reps=5):
-    """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on a bounded
-    sample: the first `sample_requests` requests of the same workload, one step, all host cores."""
+def cpu_baseline_decode(w, reps=20):
+    """The CPU oracle (a PyTorch restatement of the reference recurrence) timed on the whole workload: all 256
+    requests (the padded ones are skipped, as on the GPU), one step, median of `reps` steps, all host cores."""
     import torch
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
     from oracle import k_last_reference
     meta = w["_meta"]
-    H, HV = meta["H"], meta["HV"]
-    n = sample_requests
+    B, H, HV = meta["B"], meta["H"], meta["HV"]
     threads = os.cpu_count() or 1
     torch.set_num_threads(threads)
-    mixed = w["mixed_qkv"][:n].cpu()
-    q = mixed[:, : H * 128].reshape(n, H, 128)
-    k = mixed[:, H * 128: 2 * H * 128].reshape(n, H, 128)
-    v = mixed[:, 2 * H * 128:].reshape(n, HV, 128)
-    a, b = w["a"][:n].cpu(), w["b"][:n].cpu()
-    state = w["initial_state_source"][:n].cpu()
-    idx = list(range(n))
+    idx = w["initial_state_indices"].cpu().tolist()
+    active = [s for s in idx if s >= 0]
+    remap = {s: i for i, s in enumerate(active)}
+    state = w["initial_state_source"][torch.tensor(active, device=w["initial_state_source"].device)].cpu()
+    mixed = w["mixed_qkv"].cpu()
+    q = mixed[:, : H * 128].reshape(B, H, 128)
+    k = mixed[:, H * 128: 2 * H * 128].reshape(B, H, 128)
+    v = mixed[:, 2 * H * 128:].reshape(B, HV, 128)
+    a, b = w["a"].cpu(), w["b"].cpu()
+    slots = [remap.get(s, -1) for s in idx]
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
-        k_last_reference(q, k, v, a, b, w["A_log"].cpu(), w["dt_bias"].cpu(), state, idx, [1] * n,
+        k_last_reference(q, k, v, a, b, w["A_log"].cpu(), w["dt_bias"].cpu(), state, slots, [1] * B,
                          scale=w["scale"], use_qk_l2norm=True, is_kda=False)
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
+    n = len(active)
     return dict(value=n * HV * 131072 / t / 1e9, unit="GB/s", cores=threads, kind="port",
-                sample="first %d of the 256 requests, one step, median of %d runs (%.1f ms/step for the "
-                       "sample; %.0f us per request)" % (n, reps, t * 1e3, t / n * 1e6),
+                sample="all 256 requests (%d active), one step, median of %d steps (%.1f ms/step; %.0f us per "
+                       "active request)" % (n, reps, t * 1e3, t / n * 1e6),
                 threads_torch=torch.get_num_threads())
 
 
@@ -492,6 +519,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(d["achieved_gbps"], 1), "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": round(d["achieved_gbps"] / HBM_PEAK_GBPS, 4),
                      "traffic": DECODE_TRAFFIC_BYTES_PER_LAUNCH,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per launch, scaled by a 1 GiB device copy "
+                                       "(profiles/k_last_decode_kernel_gdn_b256.txt); a constant here, not measured in this run",
                      "kernel": "k_last_decode_kernel<bf16,GDN,rows_per_wave=32>",
                      "bytes_per_launch": d["bytes_state"], "launch_us_avg": round(d["kernel_us_avg"], 2)},
     }
@@ -507,7 +536,7 @@ def main():
         result["replay_verify"] = bench_replay_verify(device)
         result["replay_paged"] = bench_replay_paged(device)
         torch.cuda.empty_cache()
-        result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device)
+        result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
         result["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 20, 5), device)
         result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
