@@ -648,6 +648,308 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Sequential kernel with output (whole sequences, and the second sweep over segments): one workgroup per
+// (sequence, value head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
+// memory only to store their output rows; wavefront 4 moves data: it issues every global -> LDS copy of the
+// workgroup (an LDS copy instruction occupies its issuer for tens of cycles, about 2 k cycles per chunk in all,
+// which the computing wavefronts no longer pay).  Every tile is double buffered by chunk parity, so there is
+// ONE barrier per chunk: at the barrier that opens chunk c the tiles of c have landed (the copying wavefront
+// waited for them) and the buffers of chunk c - 1 are free, so it fills them with chunk c + 1 while the others
+// compute chunk c.  Per chunk and computing wavefront, nothing crossing wavefronts:
+//     KS = K S^T,  X = V - e^G (.) KS,  U = W X                  (W as an fp16 hi + lo pair)
+//     O^T = scale e^G (.) (S Q^T) + U^T P^T  -> rows of o         (the output product is formed transposed: a lane
+//                                                                  then holds four adjacent V columns of one token
+//                                                                  and stores them as 8 bytes, no LDS tile)
+//     S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)          (U as an fp16 hi + lo pair)
+// The query product is formed after U, so its accumulators and those of K S^T never live together and a
+// computing wavefront stays within 256 registers (five wavefronts put two on one SIMD).
+template <typename act_t>
+__global__ __launch_bounds__(320, 1) void gdn_sweep_kernel(const GdnPrefillParams p) {
+  constexpr int NB = 2;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
+  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
+  if (!role.active) return;
+  const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
+  const int h = hv / (p.HV / p.H);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
+  const int n_chunks = c_end - c_begin;
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];     // [parity][hi, lo]
+  __shared__ __align__(16) uint16_t tP[2][CHUNK * PITCH64];
+  // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
+  __shared__ __align__(16) float tG[2][256];
+
+  if (wave == 4) {
+    // ---- the copying wavefront -------------------------------------------------------------
+    const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
+    const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
+    const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
+    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
+    const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
+    const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
+    const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
+    CopyWide plan_kq, plan_v;
+    CopyNarrow plan_w;
+    plan_kq.plan((uint32_t)tok_pitch_b, CHUNK - 1, 0, lane);
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, 0, lane);
+    plan_w.plan(128, CHUNK - 1, 0, lane);
+    auto issue = [&](int c) {
+      const int par = c & 1;
+      const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
+      const char* qs = qn_b + (int64_t)c * CHUNK * tok_pitch_b;
+      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+      const int len = chunk_len(c);
+      dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[par][0]));
+      if (len == CHUNK) {
+        plan_kq.issue(tK[par], ks, 0);
+        plan_v.issue(tV[par], vs, 0);
+      } else {                                       // rows past the sequence end re-read its last row
+        CopyWide tail;
+        tail.plan((uint32_t)tok_pitch_b, len - 1, 0, lane);
+        tail.issue(tK[par], ks, 0);
+        tail.issue(tQ[par], qs, 0);
+        tail.plan((uint32_t)(p.stride_v * 2), len - 1, 0, lane);
+        tail.issue(tV[par], vs, 0);
+      }
+      plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, 0);
+      plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, 0);
+      if (len == CHUNK) plan_kq.issue(tQ[par], qs, 0);
+      plan_w.issue(tP[par], pp_b + (int64_t)c * p.HV * 8192, 0);
+    };
+    if (n_chunks > 0) issue(0);
+    for (int ci = 0; ci < n_chunks; ++ci) {
+      wait_vmcnt<0>();                               // chunk ci has landed
+      __syncthreads();                               // ... and chunk ci - 1 is finished: its buffers are free
+      if (ci + 1 < n_chunks) issue(ci + 1);
+    }
+    return;
+  }
+
+  // ---- the computing wavefronts ------------------------------------------------------------
+  const int vbase = 32 * wave;                       // this wavefront's V columns: vbase .. vbase + 31
+  const int vcol = vbase + r16;                      // state / KS / U layout: the lane's column (second block: + 16)
+  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
+  f32x4_t St[NB][8];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+    if (role.init != nullptr) {
+      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+      }
+    } else {
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  if (role.keep_init != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+  // output rows: in the transposed product a lane holds V columns vbase + 16 nb + 4 kb .. + 3 of token 16 ni + r16
+  uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.HV + hv) * 128 + vbase + 4 * kb;
+  const bool write_o = role.write_o;
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int par = ci & 1;
+    __syncthreads();
+    const uint16_t* const K = tK[par];
+    const uint16_t* const Q = tQ[par];
+    const uint16_t* const V = tV[par];
+    const float* const G = tG[par];
+
+    // ---- KS = K S^T ----
+    f32x4_t KS[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    {
+      bf16x8_t ka[2][4], sb[2][NB];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) {
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
+      }
+    }
+    // ---- X = V - e^G (.) KS,  U = W X ----
+    f32x4_t U[NB][4];
+    {
+      bf16x8_t wa[2][4], wl[2][4];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+          wa[s2][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], s2, kb);
+          wl[s2][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], s2, kb);
+        }
+      f32x4_t X[NB][4];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        const float4 eg = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+          X[nb][mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[nb][mi][0];
+          X[nb][mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[nb][mi][1];
+          X[nb][mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[nb][mi][2];
+          X[nb][mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[nb][mi][3];
+        }
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t xb[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+      }
+    }
+    // ---- O^T = scale e^G (.) (S Q^T) + U^T P^T -> o ----
+    {
+      f32x4_t OT[NB][4];                             // OT[nb][ni][r] = o[token 16 ni + r16][v = vbase + 16 nb + 4 kb + r]
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      bf16x8_t qa[2][4], sb[2][NB];
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], 0, kb);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) {
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], s + 1, kb);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(sb[s & 1][nb], qa[s & 1][ni], OT[nb][ni]);
+      }
+      bf16x8_t pa[2][4];
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[par][(16 * ni + r16) * PITCH64], s2, kb);
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) {
+        const float sq = G[16 * ni + r16];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) OT[nb][ni] *= sq;
+      }
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t ur[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(ur[nb], pa[s][ni], OT[nb][ni]);
+      }
+      if (write_o) {
+        const int len = chunk_len(ci);
+        uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.HV * 128;
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni)
+          if (16 * ni + r16 < len) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint2 packed = make_uint2(pack2<act_t>(OT[nb][ni][0], OT[nb][ni][1]), pack2<act_t>(OT[nb][ni][2], OT[nb][ni][3]));
+              *reinterpret_cast<uint2*>(dst + (int64_t)16 * ni * p.HV * 128 + 16 * nb) = packed;
+            }
+          }
+      }
+    }
+    // ---- S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U) ----
+    {
+      const float egl = G[192];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t kt[8];
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(K, s, mc, kb, r16);
+        const float4 d0 = *reinterpret_cast<const float4*>(&G[128 + 32 * s + 4 * kb]);
+        const float4 d1 = *reinterpret_cast<const float4*>(&G[128 + 32 * s + 16 + 4 * kb]);
+        HalfPair ub[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const f32x4_t u0 = {U[nb][2 * s][0] * d0.x, U[nb][2 * s][1] * d0.y, U[nb][2 * s][2] * d0.z, U[nb][2 * s][3] * d0.w};
+          const f32x4_t u1 = {U[nb][2 * s + 1][0] * d1.x, U[nb][2 * s + 1][1] * d1.y, U[nb][2 * s + 1][2] * d1.z,
+                              U[nb][2 * s + 1][3] * d1.w};
+          ub[nb] = half8_pair(u0, u1);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
+      }
+    }
+  }
+
+  if (role.fin != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+}
+
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, W, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
@@ -819,8 +1121,8 @@ static int gdn_prefill_run(
           if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
           else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
         } else {
-          if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, true>), dim3(grid), dim3(256), 0, s, p);
-          else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, true>), dim3(grid), dim3(256), 0, s, p);
+          if (half_act) hipLaunchKernelGGL(gdn_sweep_kernel<f16_t>, dim3(grid), dim3(320), 0, s, p);
+          else hipLaunchKernelGGL(gdn_sweep_kernel<bf16_t>, dim3(grid), dim3(320), 0, s, p);
         }
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
@@ -828,8 +1130,8 @@ static int gdn_prefill_run(
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, true>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
-    else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, true>), dim3((unsigned)L.max_segments * HV), dim3(256), 0, s, p);
+    if (half_act) hipLaunchKernelGGL(gdn_sweep_kernel<f16_t>, dim3((unsigned)L.max_segments * HV), dim3(320), 0, s, p);
+    else hipLaunchKernelGGL(gdn_sweep_kernel<bf16_t>, dim3((unsigned)L.max_segments * HV), dim3(320), 0, s, p);
   }
   return check_launch("gdn prefill launch");
 }
