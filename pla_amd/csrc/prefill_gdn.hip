@@ -664,9 +664,9 @@ __global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kerne
 //     S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)          (U as an fp16 hi + lo pair)
 // The query product is formed after U, so its accumulators and those of K S^T never live together and a
 // computing wavefront stays within 256 registers (five wavefronts put two on one SIMD).
-template <typename act_t>
-__global__ __launch_bounds__(320, 1) void gdn_sweep_kernel(const GdnPrefillParams p) {
-  constexpr int NB = 2;
+template <typename act_t, int NB>
+__global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const GdnPrefillParams p) {
+  constexpr int CW = 8 / NB;                                  // computing wavefronts, NB 16-column blocks of V each
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
@@ -691,7 +691,7 @@ __global__ __launch_bounds__(320, 1) void gdn_sweep_kernel(const GdnPrefillParam
   // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
 
-  if (wave == 4) {
+  if (wave == CW) {
     // ---- the copying wavefront -------------------------------------------------------------
     const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
     const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
@@ -738,7 +738,7 @@ __global__ __launch_bounds__(320, 1) void gdn_sweep_kernel(const GdnPrefillParam
   }
 
   // ---- the computing wavefronts ------------------------------------------------------------
-  const int vbase = 32 * wave;                       // this wavefront's V columns: vbase .. vbase + 31
+  const int vbase = 16 * NB * wave;                  // this wavefront's V columns: vbase .. vbase + 16 NB - 1
   const int vcol = vbase + r16;                      // state / KS / U layout: the lane's column (second block: + 16)
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
   f32x4_t St[NB][8];
@@ -950,6 +950,9 @@ __global__ __launch_bounds__(320, 1) void gdn_sweep_kernel(const GdnPrefillParam
   }
 }
 
+// 16-column V blocks per computing wavefront of gdn_sweep_kernel: 2 = four computing wavefronts (one per SIMD); 1 =
+// eight (two per SIMD, twice the LDS operand traffic) measures the same on config 3 (0.767 against 0.765 ms)
+constexpr int SWEEP_NB = 2;
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, W, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
@@ -1121,8 +1124,8 @@ static int gdn_prefill_run(
           if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
           else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
         } else {
-          if (half_act) hipLaunchKernelGGL(gdn_sweep_kernel<f16_t>, dim3(grid), dim3(320), 0, s, p);
-          else hipLaunchKernelGGL(gdn_sweep_kernel<bf16_t>, dim3(grid), dim3(320), 0, s, p);
+          if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(grid), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+          else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(grid), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
         }
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
@@ -1130,8 +1133,8 @@ static int gdn_prefill_run(
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    if (half_act) hipLaunchKernelGGL(gdn_sweep_kernel<f16_t>, dim3((unsigned)L.max_segments * HV), dim3(320), 0, s, p);
-    else hipLaunchKernelGGL(gdn_sweep_kernel<bf16_t>, dim3((unsigned)L.max_segments * HV), dim3(320), 0, s, p);
+    if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+    else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
   }
   return check_launch("gdn prefill launch");
 }
