@@ -768,6 +768,9 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
   uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.HV + hv) * 128 + vbase + 4 * kb;
   const bool write_o = role.write_o;
 
+  // Software pipeline of a chunk: the LDS operands of a product are requested one contraction step ahead, and the
+  // first operands of the next product under the last MFMAs of the current one.  The scheduling fences below pin
+  // memory operations only: arithmetic may move across them freely.
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
     __syncthreads();
@@ -778,14 +781,18 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
 
     // ---- KS = K S^T ----
     f32x4_t KS[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    bf16x8_t wa[2][4], wl[2][4];
+    float4 eg[4];
+    uint16_t vraw[NB][16];
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
 #pragma unroll
@@ -793,6 +800,26 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
         if (s < 3) {
 #pragma unroll
           for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+        } else {
+          // under the last step: V, e^G and the first half of W
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            eg[mi] = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+            }
+          }
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
+            wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+        if (s < 3) {
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
         }
@@ -804,28 +831,24 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
     }
     // ---- X = V - e^G (.) KS,  U = W X ----
     f32x4_t U[NB][4];
+    bf16x8_t qa[2][4];
     {
-      bf16x8_t wa[2][4], wl[2][4];
-#pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          wa[s2][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], s2, kb);
-          wl[s2][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], s2, kb);
-        }
-      f32x4_t X[NB][4];
 #pragma unroll
       for (int mi = 0; mi < 4; ++mi) {
-        const float4 eg = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-          X[nb][mi][0] = to_float(act_t{vr[0]}) - eg.x * KS[nb][mi][0];
-          X[nb][mi][1] = to_float(act_t{vr[PITCH128]}) - eg.y * KS[nb][mi][1];
-          X[nb][mi][2] = to_float(act_t{vr[2 * PITCH128]}) - eg.z * KS[nb][mi][2];
-          X[nb][mi][3] = to_float(act_t{vr[3 * PITCH128]}) - eg.w * KS[nb][mi][3];
-        }
+        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
+        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
       }
+      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+      f32x4_t X[NB][4];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+          X[nb][mi][0] = to_float(act_t{vraw[nb][4 * mi + 0]}) - eg[mi].x * KS[nb][mi][0];
+          X[nb][mi][1] = to_float(act_t{vraw[nb][4 * mi + 1]}) - eg[mi].y * KS[nb][mi][1];
+          X[nb][mi][2] = to_float(act_t{vraw[nb][4 * mi + 2]}) - eg[mi].z * KS[nb][mi][2];
+          X[nb][mi][3] = to_float(act_t{vraw[nb][4 * mi + 3]}) - eg[mi].w * KS[nb][mi][3];
+        }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -835,6 +858,12 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
         bf16x8_t xb[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+        if (s == 1) {
+          // under the last step: the first query operands
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], 0, kb);
+          __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -846,15 +875,17 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
       }
     }
     // ---- O^T = scale e^G (.) (S Q^T) + U^T P^T -> o ----
+    bf16x8_t kt[2][8];
+    float4 dg[2][2];
+    float egl;
     {
       f32x4_t OT[NB][4];                             // OT[nb][ni][r] = o[token 16 ni + r16][v = vbase + 16 nb + 4 kb + r]
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      bf16x8_t qa[2][4], sb[2][NB];
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], 0, kb);
+      bf16x8_t sb[2][NB], pa[2][4];
+      float sq[4];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
 #pragma unroll
@@ -862,6 +893,16 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
         if (s < 3) {
 #pragma unroll
           for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], s + 1, kb);
+        } else {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[par][(16 * ni + r16) * PITCH64], s2, kb);
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) sq[ni] = G[16 * ni + r16];
+        }
+        __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+        if (s < 3) {
 #pragma unroll
           for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
         }
@@ -870,22 +911,27 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
 #pragma unroll
           for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(sb[s & 1][nb], qa[s & 1][ni], OT[nb][ni]);
       }
-      bf16x8_t pa[2][4];
 #pragma unroll
-      for (int s2 = 0; s2 < 2; ++s2)
+      for (int ni = 0; ni < 4; ++ni)
 #pragma unroll
-        for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[par][(16 * ni + r16) * PITCH64], s2, kb);
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni) {
-        const float sq = G[16 * ni + r16];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) OT[nb][ni] *= sq;
-      }
+        for (int nb = 0; nb < NB; ++nb) OT[nb][ni] *= sq[ni];
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         bf16x8_t ur[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
+        if (s == 1) {
+          // under the last step: the transposed key operands and the decay factors of the state update
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) kt[0][mc] = operand_transposed(K, 0, mc, kb, r16);
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2) {
+            dg[s2][0] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 4 * kb]);
+            dg[s2][1] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 16 + 4 * kb]);
+          }
+          egl = G[192];
+          __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -907,34 +953,32 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
     }
     // ---- S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U) ----
     {
-      const float egl = G[192];
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) kt[1][mc] = operand_transposed(K, 1, mc, kb, r16);
+      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
-        bf16x8_t kt[8];
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(K, s, mc, kb, r16);
-        const float4 d0 = *reinterpret_cast<const float4*>(&G[128 + 32 * s + 4 * kb]);
-        const float4 d1 = *reinterpret_cast<const float4*>(&G[128 + 32 * s + 16 + 4 * kb]);
         HalfPair ub[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
-          const f32x4_t u0 = {U[nb][2 * s][0] * d0.x, U[nb][2 * s][1] * d0.y, U[nb][2 * s][2] * d0.z, U[nb][2 * s][3] * d0.w};
-          const f32x4_t u1 = {U[nb][2 * s + 1][0] * d1.x, U[nb][2 * s + 1][1] * d1.y, U[nb][2 * s + 1][2] * d1.z,
-                              U[nb][2 * s + 1][3] * d1.w};
+          const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
+                              U[nb][2 * s][3] * dg[s][0].w};
+          const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
+                              U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
           ub[nb] = half8_pair(u0, u1);
         }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].lo, St[nb][mc]);
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
       }
     }
   }
