@@ -319,6 +319,23 @@ __device__ __forceinline__ int staged_chunk(const StageTable& t, int stage, int 
   return begin + index < end ? t.order[begin + index] : -1;
 }
 
+// Workgroups are handed to the eight XCDs (each with an L2 of its own) round robin by index.  Workgroups that read
+// the same tiles at the same time - the `group` value heads of one q/k head sweep the same K and Q - fetch them
+// from memory once if they share an L2: this maps the hardware index onto a logical one such that the members
+// of a group get indices that are equal modulo 8.  The grid must be xcd_grouped_grid(total, group); indices
+// beyond `total` come back as -1.
+constexpr int XCDS = 8;
+inline unsigned xcd_grouped_grid(unsigned total, unsigned group) {
+  const unsigned groups = (total + group - 1) / group;
+  return (groups + XCDS - 1) / XCDS * XCDS * group;
+}
+__device__ __forceinline__ int xcd_grouped_index(int hw_index, int group, int total) {
+  const int xcd = hw_index % XCDS, t = hw_index / XCDS;
+  const int member = t % group, g = (t / group) * XCDS + xcd;
+  const int logical = g * group + member;
+  return logical < total ? logical : -1;
+}
+
 // What one workgroup of a sequential kernel sweeps: a whole sequence (pass 0, blockIdx = (sequence,
 // head)) or one segment in one of the roles above (pass 1: blockIdx = (segment, head, from-identity
 // flag); pass 2: (segment, head)); with stages (passes 0 and 1) only the part of it that belongs to
@@ -334,7 +351,8 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
                                                   const SegmentTable& seg, const StageTable& stg, int stage,
                                                   const float* h0, const int32_t* h0_indices,
                                                   int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
-                                                  int64_t ht_slot_stride, bool resweep_first = false) {
+                                                  int64_t ht_slot_stride, bool resweep_first = false, int block = -1) {
+  // block: the logical workgroup index when the caller remaps blockIdx (see xcd_grouped_index), else blockIdx.x
   // resweep_first: the first sweep publishes no output at all (first segments keep a copy of their start
   // state and only deliver the state they end in), the second sweep runs every segment with output.
   SweepRole r{};
@@ -349,8 +367,9 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
   };
   float* carry = nullptr;
   if (pass == 0) {
-    r.n = blockIdx.x / heads;
-    r.head = blockIdx.x - r.n * heads;
+    const int logical = block >= 0 ? block : (int)blockIdx.x;
+    r.n = logical / heads;
+    r.head = logical - r.n * heads;
     r.c_begin = seq_chunk_off[r.n];
     r.c_end = seq_chunk_off[r.n + 1];
     if (r.c_begin >= r.c_end) return r;              // empty sequence: state untouched, no output
@@ -358,8 +377,9 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     r.fin = state_out(r.n, r.head);
     if (stg.stages > 0) carry = stg.carry + ((int64_t)r.n * heads + r.head) * 16384;
   } else {
-    const int item = pass == 1 ? (int)(blockIdx.x >> 1) : (int)blockIdx.x;
-    const bool from_identity = pass == 1 && (blockIdx.x & 1);
+    const int logical = block >= 0 ? block : (int)blockIdx.x;
+    const int item = pass == 1 ? (logical >> 1) : logical;
+    const bool from_identity = pass == 1 && (logical & 1);
     const int s = item / heads;
     r.head = item - s * heads;
     if (s >= seg.seq_seg_off[N]) return r;

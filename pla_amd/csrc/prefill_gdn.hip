@@ -15,24 +15,24 @@
 // row or column scaling of a GEMM result, and every factor lies in (0, 1].  All MFMA operands are
 // fp16 (v_mfma_f32_16x16x32_f16, the rate of the bf16 instruction): normalised q / k (rounded to the
 // activation dtype first, as the reference does, which fp16 then holds exactly) and the FP32
-// quantities S, X, W, U, P rounded once to fp16 (11 significant bits; accumulation and the state stay
-// FP32).  A float64 simulation of these rounding points over 8192 tokens gives a final-state rel-L2
-// of 3.7e-4 .. 4.8e-4 from strong decay to none at all (bound 1e-3), against 2.3e-3 .. 3.8e-3 for single
-// bf16 operands, which therefore need hi + lo pairs (1.75 x the MFMAs and six VALU operations per
-// element pair instead of one).  Operands beyond the fp16 range (|x| > 65504) are not supported.
+// quantities S, X, W, U, P rounded to fp16 (11 significant bits; accumulation and the state stay
+// FP32).  W and the U of the state update travel as hi + lo pairs: when keys nearly repeat and beta is
+// near 1, U = W X cancels heavily and the state is the work of the last few tokens, so a single rounding of
+// those two shows unaveraged (final-state rel-L2 1e-3 .. 3.5e-3 in a float64 simulation of the rounding
+// points, 2.5e-4 .. 2.7e-4 with the pairs; random keys: 3.7e-4 .. 4.8e-4 single, bound 1e-3).  Every rounding
+// saturates at +-65504, the fp16 range, instead of producing infinities.
 //
 // Kernels:
 //   prefill_tables_kernel    chunk / segment / stage tables from cu_seqlens (device side, graph-capturable)
-//   gdn_prep_kernel          gate, beta, chunk-local cumsum and per-chunk decay-factor tiles, q/k L2
-//                            norm (rounded to the activation dtype, stored as fp16)
-//   gdn_gram_solve_kernel    one wavefront per (chunk, value head): K K^T, Q K^T on MFMA, the inverse of
-//                            I + L by 16 x 16 blocks in LDS, W and P (fp16) to the workspace
-//   gdn_chunk_seq_kernel     one workgroup per (sequence, value head), four wavefronts each owning a
-//                            32-wide V slice of S^T in MFMA accumulator layout; the chain
-//                            K S^T -> X -> U -> O, S^T runs on v_mfma_f32_16x16x32_f16 with every
-//                            intermediate staying in registers (an accumulator tile is already a
-//                            valid B operand of the next product); A operands come from LDS tiles
-//                            filled by asynchronous global -> LDS copies one chunk ahead.
+//   gdn_prepare_kernel       one wavefront per (chunk, value head): gate, beta and their chunk-local cumsum, the
+//                            decay-factor tile, q/k L2 norm (rounded to the activation dtype, stored as fp16),
+//                            K K^T and Q K^T on MFMA, the inverse of I + L by 16 x 16 blocks, W (hi, lo) and P
+//   gdn_sweep_kernel         sequential kernel with output: one workgroup per (sequence, value head) of four
+//                            computing wavefronts (32 V columns of S^T each, in MFMA accumulator layout, the
+//                            chain K S^T -> X -> U -> S^T in registers) and one wavefront that issues every
+//                            global -> LDS copy; all tiles double buffered, one barrier per chunk
+//   gdn_chunk_seq_kernel     sequential kernel of the first sweep over segments (no output): four wavefronts
+//                            that issue their own copies, single-buffered tiles, two workgroups per CU
 
 #include "prefill_common.h"
 
@@ -67,109 +67,28 @@ struct GdnPrefillParams {
 };
 
 // ---------------------------------------------------------------------------------------------
-// grid (chunk, 1 + H), 256 threads.  blockIdx.y == 0: gate, beta and the chunk-local cumulative log-decay
-// (the longest workgroups, so they are dispatched first); blockIdx.y - 1 = head: L2 norm of q and k of
-// that head for the chunk's 64 tokens (each wavefront owns 16 rows and requests all of them before reducing).
-template <typename act_t>
-__global__ __launch_bounds__(256) void gdn_prep_kernel(const GdnPrefillParams p) {
-  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x, p.seq_chunk_off[p.N]);
-  if (cb < 0) return;
-  const int t0 = p.chunk_tok[cb];
-  const int len = p.chunk_len[cb];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  __shared__ struct {
-    float g[CHUNK][129];              // per-token log-decay of up to 128 value heads
-  } sh;
-
-  if (blockIdx.y == 0) {
-    for (int hv0 = 0; hv0 < p.HV; hv0 += 128) {
-      const int nh = min(128, p.HV - hv0);
-      for (int idx = threadIdx.x; idx < CHUNK * nh; idx += 256) {
-        const int j = idx / nh, hv = hv0 + idx - j * nh;
-        float g = 0.f;
-        if (j < len) {
-          const int64_t t = t0 + j;
-          float bt;
-          if (p.g_in) {
-            g = p.g_in[t * p.HV + hv];
-            bt = p.beta_in[t * p.HV + hv];
-          } else {
-            const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
-            const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
-            g = -expf(p.A_log[hv]) * sp;
-            const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
-            bt = 1.0f / (1.0f + expf(-braw));
-          }
-          p.beta[t * p.HV + hv] = bt;
-        }
-        sh.g[j][hv - hv0] = g;
-      }
-      __syncthreads();
-      if ((int)threadIdx.x < nh) {
-        float cum = 0.f;
-        for (int j = 0; j < len; ++j) {
-          cum += sh.g[j][threadIdx.x];
-          sh.g[j][threadIdx.x] = cum;
-          p.gcum[(int64_t)(t0 + j) * p.HV + hv0 + threadIdx.x] = cum;
-        }
-      }
-      __syncthreads();
-      // per-chunk decay factors, one 1 KiB tile per value head (rows past the chunk repeat its last row)
-      for (int idx = threadIdx.x; idx < CHUNK * nh; idx += 256) {
-        const int hl = idx >> 6, j = idx & 63;
-        const float g = sh.g[min(j, len - 1)][hl], glast = sh.g[len - 1][hl];
-        float* gt = p.gtile + ((int64_t)cb * p.HV + hv0 + hl) * 256;
-        const float e = __expf(g);
-        gt[j] = p.scale * e;
-        gt[64 + j] = e;
-        gt[128 + j] = __expf(glast - g);
-        gt[192 + j] = __expf(glast);
-      }
-      __syncthreads();
-    }
-    return;
-  }
-
-  const int h = (int)blockIdx.y - 1;
-  uint32_t qw[16], kw[16];
-#pragma unroll
-  for (int x = 0; x < 16; ++x) {
-    const int j = 16 * wave + x;
-    const int64_t t = t0 + (j < len ? j : 0);
-    qw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.q) + t * p.stride_q + h * 128 + 2 * lane);
-    kw[x] = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const act_t*>(p.k) + t * p.stride_k + h * 128 + 2 * lane);
-  }
-#pragma unroll
-  for (int x = 0; x < 16; ++x) {
-    const int j = 16 * wave + x;
-    float q0 = lo16<act_t>(qw[x]), q1 = hi16<act_t>(qw[x]), k0 = lo16<act_t>(kw[x]), k1 = hi16<act_t>(kw[x]);
-    if (p.normalize_qk) {
-      const float qs = wave64_allreduce(q0 * q0 + q1 * q1);
-      const float ks = wave64_allreduce(k0 * k0 + k1 * k1);
-      const float qi = rsqrtf(qs + 1e-6f), ki = rsqrtf(ks + 1e-6f);
-      q0 *= qi; q1 *= qi; k0 *= ki; k1 *= ki;
-    }
-    if (j < len) {
-      const int64_t t = t0 + j;
-      // rounded to the activation dtype (the reference's operand), then held as fp16 (exact; saturating beyond its range)
-      const uint32_t qa = pack2<act_t>(q0, q1), ka = pack2<act_t>(k0, k1);
-      *reinterpret_cast<uint32_t*>(p.qn + (t * p.H + h) * 128 + 2 * lane) = pack2_rtz(lo16<act_t>(qa), hi16<act_t>(qa));
-      *reinterpret_cast<uint32_t*>(p.kn + (t * p.H + h) * 128 + 2 * lane) = pack2_rtz(lo16<act_t>(ka), hi16<act_t>(ka));
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// One wavefront per (chunk, value head); the WAVES wavefronts of a workgroup take consecutive value heads
-// of one q/k head, so their K and Q rows meet in the CU's cache instead of crossing HBM once per value head.
-template <int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPrefillParams p) {
+// Preparation of a chunk, everything that does not depend on the state, in one kernel: one wavefront per
+// (chunk, value head); the WAVES wavefronts of a workgroup take consecutive value heads of one q/k head, so the
+// raw K and Q rows they all read meet in the CU's cache.  Per wavefront:
+//   gate      lane j = token j: g_j = -exp(A_log) softplus(a_j + dt_bias) and beta_j = sigmoid(b_j) (or the
+//             caller's g / beta), the chunk-local cumulative log-decay G by a scan over the lanes, the copies the
+//             call returns (g_cum, beta) and the chunk's tile of decay factors for the sequential kernel
+//   q, k      the raw rows are loaded directly in MFMA operand layout (lane (r, kb) holds 32 values of a row; the
+//             four lanes of a row meet through two lane swaps), L2-normalised, rounded to the activation dtype
+//             (the reference's operand) and held as fp16, which represents those values exactly; one wavefront of
+//             the q/k head stores the normalised K rows for the sequential kernel, another the Q rows
+//   products  K K^T and Q K^T on MFMA, L = strict_tril(beta_i (k_i.k_j) e^{G_i - G_j}), W = (I + L)^-1 diag(beta)
+//             by 16 x 16 blocks (an fp16 hi + lo pair), P = scale tril(q_i.k_j e^{G_i - G_j}) (fp16)
+template <typename act_t, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefillParams p) {
   const int groups = p.HV / WAVES;
   const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
   if (cb < 0) return;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int hv = (blockIdx.x % groups) * WAVES + wave;
-  const int h = hv / (p.HV / p.H);
+  const int hv0 = (blockIdx.x % groups) * WAVES;           // first value head of this workgroup
+  const int hv = hv0 + wave;
+  const int ratio = p.HV / p.H;
+  const int h = hv / ratio;
   const int t0 = p.chunk_tok[cb];
   const int len = p.chunk_len[cb];
   const int lane = threadIdx.x & 63;
@@ -182,36 +101,131 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_gram_solve_kernel(const GdnPre
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
-  // K and Q operands: 4 row blocks x 4 contraction steps (rows beyond the chunk are zero).  All 32 loads of a
-  // lane are requested before the first use: the LDS tile limits a SIMD to two wavefronts, which hide no
-  // memory latency, and leaves them 256 registers each.
-  const uint4 zero4 = make_uint4(0, 0, 0, 0);
-  bf16x8_t Kop[4][4], Qop[4][4];
+  // raw K and Q operands: 4 row blocks x 4 contraction steps, two 8-byte pieces each; all 64 loads of a lane are
+  // requested before the first use (the LDS tile limits a SIMD to two wavefronts, which hide no latency)
+  uint2 kraw[4][4][2], qraw[4][4][2];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
     const int row = 16 * mb + r16;
-    const bool ok = row < len;
-    const uint16_t* kr = p.kn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
-    const uint16_t* qr = p.qn + ((int64_t)(t0 + (ok ? row : 0)) * p.H + h) * 128;
+    const int64_t t = t0 + (row < len ? row : 0);
+    const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128;
+    const uint16_t* qr = reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128;
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const bf16x8_t kz = operand_from(kr, s, kb);
-      Kop[mb][s] = ok ? kz : __builtin_bit_cast(bf16x8_t, zero4);
+      kraw[mb][s][0] = *reinterpret_cast<const uint2*>(kr + 32 * s + 4 * kb);
+      kraw[mb][s][1] = *reinterpret_cast<const uint2*>(kr + 32 * s + 16 + 4 * kb);
     }
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      const bf16x8_t qz = operand_from(qr, s, kb);
-      Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
+      qraw[mb][s][0] = *reinterpret_cast<const uint2*>(qr + 32 * s + 4 * kb);
+      qraw[mb][s][1] = *reinterpret_cast<const uint2*>(qr + 32 * s + 16 + 4 * kb);
     }
   }
+
+  // ---- gate: lane = token ----
   {
-    // rows beyond the chunk repeat its last log-decay (their K rows are zero) and have beta = 0; requested
-    // after the operands and in the same round trip
-    const int64_t at = (int64_t)(t0 + min(lane, len - 1)) * p.HV + hv;
-    const float gl = p.gcum[at], bl = p.beta[at];
-    __builtin_amdgcn_sched_barrier(0);
-    Gs[lane] = gl;
-    Bs[lane] = lane < len ? bl : 0.f;
+    float g = 0.f, bt = 0.f;
+    if (lane < len) {
+      const int64_t t = t0 + lane;
+      if (p.g_in) {
+        g = p.g_in[t * p.HV + hv];
+        bt = p.beta_in[t * p.HV + hv];
+      } else {
+        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
+        const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
+        g = -expf(p.A_log[hv]) * sp;
+        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
+        bt = 1.0f / (1.0f + expf(-braw));
+      }
+    }
+    // inclusive scan over the 64 lanes (rows beyond the chunk have g = 0 and so repeat G_last)
+    float cum = g;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float up = __shfl_up(cum, d, 64);
+      if (lane >= d) cum += up;
+    }
+    const float glast = __shfl(cum, 63, 64);
+    if (lane < len) {
+      const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;
+      p.gcum[at] = cum;
+      p.beta[at] = bt;
+    }
+    Gs[lane] = cum;
+    Bs[lane] = bt;
+    // decay factors of the sequential kernel, one 1 KiB tile per (chunk, value head)
+    float* gt = p.gtile + ((int64_t)cb * p.HV + hv) * 256;
+    const float e = __expf(cum);
+    gt[lane] = p.scale * e;
+    gt[64 + lane] = e;
+    gt[128 + lane] = __expf(glast - cum);
+    gt[192 + lane] = __expf(glast);
+  }
+
+  // ---- q / k: normalise, round to the activation dtype, hold as fp16 (exact; saturating beyond its range) ----
+  bf16x8_t Kop[4][4], Qop[4][4];
+  {
+    auto row_scale = [&](const uint2 (&raw)[4][2]) {
+      float ss = 0.f;
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int hlf = 0; hlf < 2; ++hlf) {
+          const float a0 = lo16<act_t>(raw[s][hlf].x), a1 = hi16<act_t>(raw[s][hlf].x);
+          const float a2 = lo16<act_t>(raw[s][hlf].y), a3 = hi16<act_t>(raw[s][hlf].y);
+          ss += a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3;
+        }
+      const LanePair r1 = swap_rows16(ss);               // the four lanes of a row are 16 lanes apart
+      const LanePair r2 = swap_halves(r1.lo + r1.hi);
+      return rsqrtf(r2.lo + r2.hi + 1e-6f);
+    };
+    auto normalised = [&](const uint2 (&raw)[2], float inv) {
+      uint32_t w[4];
+#pragma unroll
+      for (int hlf = 0; hlf < 2; ++hlf) {
+        const uint32_t a = pack2<act_t>(lo16<act_t>(raw[hlf].x) * inv, hi16<act_t>(raw[hlf].x) * inv);
+        const uint32_t b = pack2<act_t>(lo16<act_t>(raw[hlf].y) * inv, hi16<act_t>(raw[hlf].y) * inv);
+        w[2 * hlf] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
+        w[2 * hlf + 1] = pack2_rtz(lo16<act_t>(b), hi16<act_t>(b));
+      }
+      return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
+    };
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    // the normalised rows go to the sequential kernel from one wavefront of the q/k head each (K from the first,
+    // Q from the second, or both from the only one)
+    const bool first_group = hv0 % ratio == 0;
+    const bool store_k = first_group && wave == 0, store_q = first_group && wave == (WAVES > 1 ? 1 : 0);
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const int row = 16 * mb + r16;
+      const bool ok = row < len;
+      const float ki = p.normalize_qk ? row_scale(kraw[mb]) : 1.f;
+      const float qi = p.normalize_qk ? row_scale(qraw[mb]) : 1.f;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const bf16x8_t kz = normalised(kraw[mb][s], ki), qz = normalised(qraw[mb][s], qi);
+        Kop[mb][s] = ok ? kz : __builtin_bit_cast(bf16x8_t, zero4);
+        Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
+      }
+      if (ok && (store_k || store_q)) {
+        uint16_t* dst = (store_k ? p.kn : p.qn) + ((int64_t)(t0 + row) * p.H + h) * 128;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint4 w = __builtin_bit_cast(uint4, store_k ? Kop[mb][s] : Qop[mb][s]);
+          *reinterpret_cast<uint2*>(dst + 32 * s + 4 * kb) = make_uint2(w.x, w.y);
+          *reinterpret_cast<uint2*>(dst + 32 * s + 16 + 4 * kb) = make_uint2(w.z, w.w);
+        }
+        if (store_k && store_q) {                      // one wavefront per q/k head: it stores both
+          uint16_t* dq = p.qn + ((int64_t)(t0 + row) * p.H + h) * 128;
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const uint4 w = __builtin_bit_cast(uint4, Qop[mb][s]);
+            *reinterpret_cast<uint2*>(dq + 32 * s + 4 * kb) = make_uint2(w.x, w.y);
+            *reinterpret_cast<uint2*>(dq + 32 * s + 16 + 4 * kb) = make_uint2(w.z, w.w);
+          }
+        }
+      }
+    }
   }
   __syncthreads();
 
@@ -669,8 +683,11 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
   constexpr int CW = 8 / NB;                                  // computing wavefronts, NB 16-column blocks of V each
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
+  // whole sequences: the value heads of a q/k head run on one XCD, so that K and Q reach its L2 once
+  const int block = p.pass == 0 ? xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV) : (int)blockIdx.x;
+  if (block < 0) return;
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int h = hv / (p.HV / p.H);
@@ -773,7 +790,11 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
   // memory operations only: arithmetic may move across them freely.
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
-    __syncthreads();
+    // A bare barrier: the tiles were written by the copying wavefront's LDS copies, which it waited for before it
+    // arrived, and this wavefront's own LDS reads of the previous chunk are complete (their MFMAs have issued).  A
+    // full workgroup fence would also wait for this wavefront's output stores, which nobody in the workgroup reads.
+    __builtin_amdgcn_s_waitcnt(0xc07f);              // lgkmcnt(0) only
+    __builtin_amdgcn_s_barrier();
     const uint16_t* const K = tK[par];
     const uint16_t* const Q = tQ[par];
     const uint16_t* const V = tV[par];
@@ -1156,20 +1177,27 @@ static int gdn_prefill_run(
   const bool ok = launch_pipeline(
       s, L.stages, segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
       [&](hipStream_t ps) {
-        if (half_act) hipLaunchKernelGGL(gdn_prep_kernel<f16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
-        else hipLaunchKernelGGL(gdn_prep_kernel<bf16_t>, dim3(L.NC_max, H + 1), dim3(256), 0, ps, p);
         const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
-        if (ratio % 4 == 0) hipLaunchKernelGGL(gdn_gram_solve_kernel<4>, dim3((unsigned)L.NC_max * (HV / 4)), dim3(256), 0, ps, p);
-        else if (ratio % 2 == 0) hipLaunchKernelGGL(gdn_gram_solve_kernel<2>, dim3((unsigned)L.NC_max * (HV / 2)), dim3(128), 0, ps, p);
-        else hipLaunchKernelGGL(gdn_gram_solve_kernel<1>, dim3((unsigned)L.NC_max * HV), dim3(64), 0, ps, p);
+        const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
+        const dim3 grid((unsigned)L.NC_max * (HV / waves)), block(64 * waves);
+        if (half_act) {
+          if (waves == 4) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 4>), grid, block, 0, ps, p);
+          else if (waves == 2) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 2>), grid, block, 0, ps, p);
+          else hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 1>), grid, block, 0, ps, p);
+        } else {
+          if (waves == 4) hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 4>), grid, block, 0, ps, p);
+          else if (waves == 2) hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 2>), grid, block, 0, ps, p);
+          else hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 1>), grid, block, 0, ps, p);
+        }
       },
       [&](unsigned grid) {
         if (p.pass == 1) {        // first sweep over segments: no output
           if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
           else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
         } else {
-          if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(grid), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
-          else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(grid), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+          const unsigned g = xcd_grouped_grid(grid, (unsigned)(HV / H));
+          if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+          else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
         }
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
