@@ -624,6 +624,285 @@ __global__ __launch_bounds__(256, 1) void kda_chunk_seq_kernel(const KdaPrefillP
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// First sweep over segments, both roles in one workgroup.  A later segment is swept twice without output - from a
+// zero state (its B summary) and from the identity with v = 0 (its transition matrix M) - and both sweeps multiply
+// the same operand tiles.  One workgroup of eight wavefronts per (segment, head) therefore runs them side by side:
+// wavefronts 0-3 carry the B columns (32 each), wavefronts 4-7 the M columns and, having no values to subtract,
+// also issue every global -> LDS copy, so each tile crosses memory and LDS once for the two sweeps and two
+// wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
+// from its real start state (of which they keep a copy for the second sweep).
+//
+// The tiles of a chunk's first half (K e^G, V, W hi / lo) are double buffered by chunk parity, the hi / lo pair of
+// K e^{G_last - G} and e^{G_last} single (142 KB of LDS), with two barriers per chunk:
+//   barrier A   first-half tiles of chunk c landed, chunk c - 1 finished    copy K e^{G_last-G} (hi, lo), e^{G_last} of c,
+//               KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X             then the first-half tiles of chunk c + 1
+//   barrier B   the pair of c landed
+//               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U              (pairs: hi.lo + lo.hi + hi.hi)
+__global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefillParams p) {
+  constexpr int NB = 2;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, kb = lane >> 4;
+  const bool m_side = wave >= 4;                               // wavefronts 4-7: transition-matrix columns + copies
+  const int cw = wave & 3;                                     // position among the four wavefronts of a role
+  const int vcol = 32 * cw + r16;
+
+  // the two roles of this (segment, head): logical workgroups 2 i (zero state / real state) and 2 i + 1 (identity)
+  const SweepRole lead = select_sweep(1, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, 0, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x);
+  if (!lead.active) return;
+  const SweepRole mrole = select_sweep(1, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, 0, p.h0, p.h0_indices, p.h0_slot_stride,
+                                       p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x + 1);
+  const SweepRole& role = m_side ? mrole : lead;
+  const bool computing = role.active;                          // wave-uniform; false: wavefronts 4-7 of a first segment
+  const int n = lead.n, h = lead.head, c_begin = lead.c_begin, c_end = lead.c_end;
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
+  const int n_chunks = c_end - c_begin;
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
+  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
+  __shared__ __align__(16) float tE[128];
+
+  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
+  f32x4_t St[NB][8];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+    if (computing && role.init != nullptr) {
+      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+      }
+    } else {
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  if (computing && role.keep_init != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+  const bool use_v = computing && !role.zero_v;                // the identity sweep runs with v = 0
+
+  // ---- copies (wavefronts 4-7) ----
+  const int64_t tile0 = (int64_t)c_begin * p.H + h;
+  const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
+  const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
+  const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
+  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
+  const int64_t big_step = (int64_t)p.H * 16384, e_step = (int64_t)p.H * 512;
+  CopyWide plan_k, plan_v;
+  CopyNarrow plan_w;
+  if (m_side) {
+    plan_k.plan(256, CHUNK - 1, cw, lane);
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
+    plan_w.plan(128, CHUNK - 1, cw, lane);
+  }
+  auto issue_first = [&](int c) {                    // K e^G, V, W (hi, lo) into the buffers of c's parity
+    const int par = c & 1;
+    plan_k.issue(tK[par], kg_b + c * big_step, cw);
+    const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+    const int len = chunk_len(c);
+    if (len == CHUNK) {
+      plan_v.issue(tV[par], vs, cw);
+    } else {                                         // rows past the sequence re-read its last row
+      CopyWide tail_v;
+      tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
+      tail_v.issue(tV[par], vs, cw);
+    }
+    plan_w.issue(tW[par][0], w_b + c * big_step, cw);
+    plan_w.issue(tW[par][1], w_b + c * big_step + 8192, cw);
+  };
+  auto issue_second = [&](int c) {                   // K e^{G_last-G} (hi, lo), e^{G_last}
+    plan_k.issue(tKt[0], kt_b + c * 2 * big_step, cw);
+    plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, cw);
+    if (cw == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
+  };
+  // copies one wavefront issues in issue_first (constant: a tail plan has the same piece counts)
+  constexpr int FIRST_REST = 2 * (CopyWide::FIRST) + 2 * (CopyNarrow::FIRST);      // wavefront 4
+  constexpr int EACH_REST = 2 * (CopyWide::EACH) + 2 * (CopyNarrow::EACH);         // wavefronts 5-7
+
+  if (m_side && n_chunks > 0) issue_first(0);
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int par = ci & 1;
+    const bool more = ci + 1 < n_chunks;
+    // barrier A
+    if (m_side) wait_vmcnt<0>();
+    __syncthreads();
+    if (m_side) {
+      issue_second(ci);
+      if (more) issue_first(ci + 1);
+    }
+    f32x4_t U[NB][4];
+    if (computing) {
+      const uint16_t* const K = tK[par];
+      const uint16_t* const V = tV[par];
+      // ---- KS = (K e^G) S^T ----
+      f32x4_t KS[NB][4];
+      bf16x8_t wa[2][4], wl[2][4];
+      uint16_t vraw[NB][16];
+      {
+        bf16x8_t ka[2][4], sb[2][NB];
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+        __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          if (s < 3) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+          } else {
+            // under the last step: V and the first half of W
+            if (use_v) {
+#pragma unroll
+              for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                  const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+                }
+            }
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) {
+              wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
+              wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0x000F);
+          if (s < 3) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+          }
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
+        }
+      }
+      // ---- X = V - KS,  U = W X ----
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) {
+        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
+        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
+      }
+      __builtin_amdgcn_sched_barrier(0x000F);
+      f32x4_t X[NB][4];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            X[nb][mi][r] = (use_v ? to_float(bf16_t{vraw[nb][4 * mi + r]}) : 0.f) - KS[nb][mi][r];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t xb[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+      }
+    }
+    // barrier B: the pair of this chunk has landed (copies issued after it may still be in flight)
+    if (m_side) {
+      if (!more) wait_vmcnt<0>();
+      else if (cw == 0) wait_vmcnt<FIRST_REST>();
+      else wait_vmcnt<EACH_REST>();
+    }
+    __syncthreads();
+    if (computing) {
+      // ---- S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U ----
+      bf16x8_t kt[8], ktl[8];
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        kt[mc] = operand_transposed(tKt[0], 0, mc, kb, r16);
+        ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
+      }
+      float4 eg[8];
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
+      __builtin_amdgcn_sched_barrier(0x000F);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc)
+          St[nb][mc] = f32x4_t{St[nb][mc][0] * eg[mc].x, St[nb][mc][1] * eg[mc].y, St[nb][mc][2] * eg[mc].z,
+                               St[nb][mc][3] * eg[mc].w};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        HalfPair ub[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) ub[nb] = half8_pair(U[nb][2 * s], U[nb][2 * s + 1]);
+        // hi . lo and lo . hi first, the large term last
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
+        if (s == 0) {
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+          __builtin_amdgcn_sched_barrier(0x000F);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
+        if (s == 0) {
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(tKt[0], 1, mc, kb, r16);
+          __builtin_amdgcn_sched_barrier(0x000F);
+        }
+      }
+    }
+  }
+
+  if (computing && role.fin != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+}
+
 struct KdaWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, Kg, Qg, Kt, W, P, eGlast;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
@@ -750,7 +1029,8 @@ extern "C" int pla_kda_prefill_launch(
       [&](hipStream_t ps) { hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, ps, p); },
       [&](unsigned grid) {
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
-        if (p.pass == 1) hipLaunchKernelGGL(kda_chunk_seq_kernel<false>, dim3(grid), dim3(256), 0, s, p);
+        // the first sweep over segments publishes no output: both of its roles in one workgroup per (segment, head)
+        if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
         else hipLaunchKernelGGL(kda_chunk_seq_kernel<true>, dim3(grid), dim3(256), 0, s, p);
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
