@@ -31,8 +31,8 @@
 //                            computing wavefronts (32 V columns of S^T each, in MFMA accumulator layout, the
 //                            chain K S^T -> X -> U -> S^T in registers) and one wavefront that issues every
 //                            global -> LDS copy; all tiles double buffered, one barrier per chunk
-//   gdn_chunk_seq_kernel     sequential kernel of the first sweep over segments (no output): four wavefronts
-//                            that issue their own copies, single-buffered tiles, two workgroups per CU
+//   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
+//                            segment side by side in one workgroup of eight wavefronts that share every tile
 
 #include "prefill_common.h"
 
@@ -297,368 +297,6 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
       else if (c8 + 2 * e + 1 > i) we[e] &= 0xffffu;
     }
     *reinterpret_cast<uint4*>(Pt + i * 64 + c8) = w;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
-// Sequential kernel: one workgroup per (sequence, value head), 8 / NB wavefronts, each owning NB
-// 16-column blocks of V that share every A operand (NB = 2: four wavefronts, one per SIMD; every
-// wavefront reads every A tile once per chunk, so fewer, wider wavefronts halve the LDS traffic,
-// which is what bounds this kernel).  S^T stays in MFMA
-// accumulator layout (an accumulator tile pair is already a valid B operand of the next product),
-// A operands come from LDS tiles that are filled by asynchronous global -> LDS copies.  There are two
-// barriers per chunk; a tile's next version is requested at the barrier after its last use and has
-// half a chunk of compute time to land.  The K tile is used in both halves (as K for K S^T, and
-// transposed by ds_read_b64_tr_b16 for the state update), so it alone is double buffered by chunk
-// parity; no K^T copy exists in memory:
-//
-//   barrier A   K, Q, V, W, decay factors of chunk c landed   flush O(c-1); issue P(c), factors of c+1
-//               KS = K S^T, QS = Q S^T, X = V - e^G (.) KS, U = W X
-//   barrier B   P of chunk c landed                           issue K, Q, V, W of chunk c+1
-//               S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U),  O = scale e^G (.) QS + P U -> O tile
-//
-// Every wait is for all outstanding copies (s_waitcnt vmcnt(0)): whatever is in flight at a barrier is
-// exactly what the next half needs.
-//
-// WRITE_O = false is the first sweep over segments (affine summaries only): without the query, output and P
-// tiles (62 KB of LDS) two workgroups share a CU and every chain of that sweep is resident at once.  First
-// segments then keep a copy of their start state and are swept again, with output, in the second sweep.
-template <typename act_t, int NB, bool WRITE_O>
-__global__ __launch_bounds__(512 / NB, WRITE_O ? 1 : 2) void gdn_chunk_seq_kernel(const GdnPrefillParams p) {
-  constexpr int WAVES = 8 / NB;                            // NB 16-column blocks of V per wavefront
-  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
-  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
-  if (!role.active) return;
-  const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
-  const bool zero_v = role.zero_v, write_o = WRITE_O && role.write_o;
-  const int h = hv / (p.HV / p.H);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r16 = lane & 15, kb = lane >> 4;
-  const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the others: +16 each)
-  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
-  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
-  const int n_chunks = c_end - c_begin;
-
-  // distinct LDS objects: the compiler tracks outstanding direct-to-LDS loads per object
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];      // by chunk parity: the state update reads it last
-  __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
-  __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
-  __shared__ __align__(16) uint16_t tW[2][CHUNK * PITCH64];      // hi and lo parts
-  __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
-  // decay factors by chunk parity: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
-  __shared__ __align__(16) float tG[2][256];
-
-  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
-  f32x4_t St[NB][8];
-  {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-      if (role.init != nullptr) {
-        const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) {
-          const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
-          St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
-        }
-      } else {
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      }
-  }
-
-  if (role.keep_init != nullptr) {                   // a first segment that is swept again later: keep its start state
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
-    }
-  }
-
-  if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
-    for (int i = tid; i < CHUNK * PITCH128 / 2; i += 256 * 2 / NB) reinterpret_cast<uint32_t*>(tV)[i] = 0u;
-  }
-
-  const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
-  const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
-  const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
-  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
-  const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
-  const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
-
-  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
-  // Copy plans.  K and Q share one (same pitch); the last chunk of a sequence gets plans of its own
-  // that keep rows past the sequence end inside it.
-  CopyWide plan_kq, plan_v;
-  CopyNarrow plan_w;
-  plan_kq.plan((uint32_t)tok_pitch_b, CHUNK - 1, wave, lane);
-  plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
-  plan_w.plan(128, CHUNK - 1, wave, lane);
-  auto issue_kqv = [&](int c) {
-    const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
-    const char* qs = qn_b + (int64_t)c * CHUNK * tok_pitch_b;
-    const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
-    const int len = chunk_len(c);
-    if (len == CHUNK) {
-      plan_kq.issue(tK[c & 1], ks, wave);
-      if constexpr (WRITE_O) plan_kq.issue(tQ, qs, wave);
-      if (!zero_v) plan_v.issue(tV, vs, wave);
-    } else {
-      CopyWide tail_kq, tail_v;
-      tail_kq.plan((uint32_t)tok_pitch_b, len - 1, wave, lane);
-      tail_kq.issue(tK[c & 1], ks, wave);
-      if constexpr (WRITE_O) tail_kq.issue(tQ, qs, wave);
-      if (!zero_v) {
-        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
-        tail_v.issue(tV, vs, wave);
-      }
-    }
-  };
-  auto issue_w = [&](int c) {
-    plan_w.issue(tW[0], w_b + (int64_t)c * p.HV * 16384, wave);
-    plan_w.issue(tW[1], w_b + (int64_t)c * p.HV * 16384 + 8192, wave);
-  };
-  auto issue_p = [&](int c) {
-    if constexpr (WRITE_O) plan_w.issue(tP, pp_b + (int64_t)c * p.HV * 8192, wave);
-  };
-  auto issue_gates = [&](int c) {                            // one 1 KiB piece, wavefront 0
-    if (wave == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[c & 1][0]));
-  };
-  // coalesced write of a finished output tile
-  constexpr int FLUSH_ROWS = 32 / NB;                       // rows covered by one pass of the workgroup
-  const int krow = tid >> 4, kcv = tid & 15;
-  uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.HV + hv) * 128 + 8 * kcv;
-  auto flush_output = [&](int c) {
-    if (!WRITE_O || !write_o) return;
-    const int len = chunk_len(c);
-    uint16_t* dst = o_b + (int64_t)c * CHUNK * p.HV * 128;
-#pragma unroll
-    for (int i = 0; i < CHUNK / FLUSH_ROWS; ++i)
-      if (krow + FLUSH_ROWS * i < len)
-        *reinterpret_cast<uint4*>(dst + (int64_t)FLUSH_ROWS * i * p.HV * 128) =
-            *reinterpret_cast<const uint4*>(&tO[(krow + FLUSH_ROWS * i) * PITCH128 + 8 * kcv]);
-  };
-
-  if (n_chunks > 0) {                                // a stage of a short sequence may hold no chunk
-    issue_gates(0);
-    issue_kqv(0);
-    issue_w(0);
-  }
-
-  for (int ci = 0; ci < n_chunks; ++ci) {
-    const int par = ci & 1;
-    const bool more = ci + 1 < n_chunks;
-    // Within a half the LDS operands are requested ahead of the MFMAs that use them (scheduling
-    // fences keep that order), so a wavefront waits for LDS once per product, not once per MFMA.
-
-    // barrier A: K, Q, V, W and the decay factors of this chunk have landed (nothing younger is in flight)
-    wait_vmcnt<0>();
-    __syncthreads();
-    bf16x8_t ka[2][4], qa[2][4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      ka[0][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], 0, kb);
-      if constexpr (WRITE_O) qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (ci > 0) flush_output(ci - 1);
-    issue_p(ci);
-    if (more) issue_gates(ci + 1);
-
-    f32x4_t KS[NB][4], QS[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
-    float4 eg[4];
-    uint16_t vraw[NB][16];
-    bf16x8_t wa[2][4], wl[2][4];
-    bf16x8_t sb[2][NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (s < 3) {
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          ka[(s + 1) & 1][mi] = operand_from(&tK[par][(16 * mi + r16) * PITCH128], s + 1, kb);
-          if constexpr (WRITE_O) qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
-        }
-      } else {
-        // the last step's MFMAs cover the reads for X and for U = W X
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          eg[mi] = *reinterpret_cast<const float4*>(&tG[par][64 + 16 * mi + 4 * kb]);
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
-          }
-        }
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wa[s2][mi] = operand_from(&tW[0][(16 * mi + r16) * PITCH64], s2, kb);
-            wl[s2][mi] = operand_from(&tW[1][(16 * mi + r16) * PITCH64], s2, kb);
-          }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // the next step's state slice is rounded underneath this step's MFMAs
-      if (s < 3) {
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
-      if constexpr (WRITE_O) {
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // X = V - e^{G} (.) KS
-    f32x4_t X[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        X[nb][mi][0] = to_float(act_t{vraw[nb][4 * mi + 0]}) - eg[mi].x * KS[nb][mi][0];
-        X[nb][mi][1] = to_float(act_t{vraw[nb][4 * mi + 1]}) - eg[mi].y * KS[nb][mi][1];
-        X[nb][mi][2] = to_float(act_t{vraw[nb][4 * mi + 2]}) - eg[mi].z * KS[nb][mi][2];
-        X[nb][mi][3] = to_float(act_t{vraw[nb][4 * mi + 3]}) - eg[mi].w * KS[nb][mi][3];
-      }
-    // U = W X
-    f32x4_t U[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      bf16x8_t xb[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
-    }
-
-    // barrier B: P of this chunk has landed; Q, V, W and the other K tile are free for the next chunk
-    wait_vmcnt<0>();
-    __syncthreads();
-    bf16x8_t kt[2][8];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tK[par], s, mc, kb, r16);
-    float4 dg[2][2];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      dg[s][0] = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 4 * kb]);
-      dg[s][1] = *reinterpret_cast<const float4*>(&tG[par][128 + 32 * s + 16 + 4 * kb]);
-    }
-    const float egl = tG[par][192];
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) {
-      issue_kqv(ci + 1);
-      issue_w(ci + 1);
-    }
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
-    bf16x8_t pa[2][4];
-    float4 sq[4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      if (WRITE_O && s == 1) {
-        // the last step's MFMAs cover the reads for the output product
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) sq[mi] = *reinterpret_cast<const float4*>(&tG[par][16 * mi + 4 * kb]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      HalfPair ub[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
-                            U[nb][2 * s][3] * dg[s][0].w};
-        const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
-                            U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
-        ub[nb] = half8_pair(u0, u1);
-      }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
-    }
-
-    if constexpr (WRITE_O) {
-    // O = scale e^{G} (.) QS + P U -> O tile
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        QS[nb][mi][0] *= sq[mi].x; QS[nb][mi][1] *= sq[mi].y; QS[nb][mi][2] *= sq[mi].z; QS[nb][mi][3] *= sq[mi].w;
-      }
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      bf16x8_t ur[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
-    }
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-        orow[0] = from_float<act_t>(QS[nb][mi][0]).bits;
-        orow[PITCH128] = from_float<act_t>(QS[nb][mi][1]).bits;
-        orow[2 * PITCH128] = from_float<act_t>(QS[nb][mi][2]).bits;
-        orow[3 * PITCH128] = from_float<act_t>(QS[nb][mi][3]).bits;
-      }
-    }
-  }
-  __syncthreads();
-  if (n_chunks > 0) flush_output(n_chunks - 1);
-
-  if (role.fin != nullptr) {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
-    }
   }
 }
 
@@ -1015,6 +653,258 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// First sweep over segments, both roles in one workgroup.  A later segment is swept twice without output - from a
+// zero state (its B summary) and from the identity with v = 0 (its transition matrix M) - and both sweeps multiply
+// the same K and W tiles.  One workgroup of eight wavefronts per (segment, value head) runs them side by side:
+// wavefronts 0-3 carry the B columns (32 each), wavefronts 4-7 the M columns and, having no values to subtract,
+// also issue every global -> LDS copy, so each tile crosses memory and LDS once for the two sweeps and two
+// wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
+// from its real start state (of which they keep a copy for the second sweep).  All tiles are double buffered by
+// chunk parity (109 KB of LDS) and there is one barrier per chunk, as in gdn_sweep_kernel.
+template <typename act_t>
+__global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefillParams p) {
+  constexpr int NB = 2;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, kb = lane >> 4;
+  const bool m_side = wave >= 4;                               // wavefronts 4-7: transition-matrix columns + copies
+  const int cw = wave & 3;                                     // position among the four wavefronts of a role
+  const int vcol = 32 * cw + r16;
+
+  // the two roles of this (segment, head): logical workgroups 2 i (zero state / real state) and 2 i + 1 (identity)
+  const SweepRole lead = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x);
+  if (!lead.active) return;
+  const SweepRole mrole = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
+                                       p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x + 1);
+  const SweepRole& role = m_side ? mrole : lead;
+  const bool computing = role.active;                          // wave-uniform; false: wavefronts 4-7 of a first segment
+  const int n = lead.n, hv = lead.head, c_begin = lead.c_begin, c_end = lead.c_end;
+  const int h = hv / (p.HV / p.H);
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
+  const int n_chunks = c_end - c_begin;
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
+  // decay factors: [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
+  __shared__ __align__(16) float tG[2][256];
+
+  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
+  f32x4_t St[NB][8];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+    if (computing && role.init != nullptr) {
+      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+      }
+    } else {
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  if (computing && role.keep_init != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+  const bool use_v = computing && !role.zero_v;                // the identity sweep runs with v = 0
+
+  // ---- copies (wavefronts 4-7) ----
+  const int64_t tok_pitch_b = (int64_t)p.H * 256;              // bytes between tokens of kn
+  const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
+  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
+  const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
+  CopyWide plan_k, plan_v;
+  CopyNarrow plan_w;
+  if (m_side) {
+    plan_k.plan((uint32_t)tok_pitch_b, CHUNK - 1, cw, lane);
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
+    plan_w.plan(128, CHUNK - 1, cw, lane);
+  }
+  auto issue = [&](int c) {
+    const int par = c & 1;
+    const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
+    const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+    const int len = chunk_len(c);
+    if (cw == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[par][0]));
+    if (len == CHUNK) {
+      plan_k.issue(tK[par], ks, cw);
+      plan_v.issue(tV[par], vs, cw);
+    } else {                                         // rows past the sequence end re-read its last row
+      CopyWide tail;
+      tail.plan((uint32_t)tok_pitch_b, len - 1, cw, lane);
+      tail.issue(tK[par], ks, cw);
+      tail.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
+      tail.issue(tV[par], vs, cw);
+    }
+    plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, cw);
+    plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, cw);
+  };
+  if (m_side && n_chunks > 0) issue(0);
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int par = ci & 1;
+    if (m_side) wait_vmcnt<0>();                     // chunk ci has landed
+    __syncthreads();                                 // ... and chunk ci - 1 is finished: its buffers are free
+    if (m_side && ci + 1 < n_chunks) issue(ci + 1);
+    if (!computing) continue;
+    const uint16_t* const K = tK[par];
+    const uint16_t* const V = tV[par];
+    const float* const G = tG[par];
+    // ---- KS = K S^T ----
+    f32x4_t KS[NB][4];
+    bf16x8_t wa[2][4], wl[2][4];
+    float4 eg[4];
+    uint16_t vraw[NB][16];
+    {
+      bf16x8_t ka[2][4], sb[2][NB];
+#pragma unroll
+      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+      __builtin_amdgcn_sched_barrier(0x000F);        // LDS requests stay above this line; ALU and MFMA work may cross it
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) {
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+        } else {
+          // under the last step: V and e^G
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            eg[mi] = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
+            if (use_v) {
+#pragma unroll
+              for (int nb = 0; nb < NB; ++nb) {
+                const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+              }
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0x000F);
+        if (s < 3) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
+      }
+    }
+    // ---- X = V - e^G (.) KS,  U = W X ----
+    f32x4_t U[NB][4];
+    bf16x8_t kt[2][8];
+    float4 dg[2][2];
+    float egl;
+    {
+      // W is requested here: the arithmetic of X covers the LDS latency
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+          wa[s2][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], s2, kb);
+          wl[s2][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], s2, kb);
+        }
+      __builtin_amdgcn_sched_barrier(0x000F);
+      f32x4_t X[NB][4];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) {
+          X[nb][mi][0] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 0]}) : 0.f) - eg[mi].x * KS[nb][mi][0];
+          X[nb][mi][1] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 1]}) : 0.f) - eg[mi].y * KS[nb][mi][1];
+          X[nb][mi][2] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 2]}) : 0.f) - eg[mi].z * KS[nb][mi][2];
+          X[nb][mi][3] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 3]}) : 0.f) - eg[mi].w * KS[nb][mi][3];
+        }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t xb[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+      }
+    }
+    // ---- S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U) ----
+    {
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) kt[s2][mc] = operand_transposed(K, s2, mc, kb, r16);
+        dg[s2][0] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 4 * kb]);
+        dg[s2][1] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 16 + 4 * kb]);
+      }
+      egl = G[192];
+      __builtin_amdgcn_sched_barrier(0x000F);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        HalfPair ub[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
+                              U[nb][2 * s][3] * dg[s][0].w};
+          const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
+                              U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
+          ub[nb] = half8_pair(u0, u1);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
+      }
+    }
+  }
+
+  if (computing && role.fin != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+}
+
 // 16-column V blocks per computing wavefront of gdn_sweep_kernel: 2 = four computing wavefronts (one per SIMD); 1 =
 // eight (two per SIMD, twice the LDS operand traffic) measures the same on config 3 (0.767 against 0.765 ms)
 constexpr int SWEEP_NB = 2;
@@ -1191,9 +1081,9 @@ static int gdn_prefill_run(
         }
       },
       [&](unsigned grid) {
-        if (p.pass == 1) {        // first sweep over segments: no output
-          if (half_act) hipLaunchKernelGGL((gdn_chunk_seq_kernel<f16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
-          else hipLaunchKernelGGL((gdn_chunk_seq_kernel<bf16_t, 2, false>), dim3(grid), dim3(256), 0, s, p);
+        if (p.pass == 1) {        // first sweep over segments: no output, both roles in one workgroup per (segment, head)
+          if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(grid / 2), dim3(512), 0, s, p);
+          else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
         } else {
           const unsigned g = xcd_grouped_grid(grid, (unsigned)(HV / H));
           if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
