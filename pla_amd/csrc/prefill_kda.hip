@@ -23,9 +23,16 @@
 //   kda_prep_solve_kernel   one workgroup per (chunk, head): q/k L2 norm (rounded to bf16), lower-bound
 //                           gate, cumulative decay, decayed operand tiles (fp16), M / P on MFMA, the
 //                           inverse of I + L by 16 x 16 blocks, W and P (fp16)
-//   kda_chunk_seq_kernel    one workgroup per (sequence, head) or segment sweep, four wavefronts x 32 V
-//                           columns, same register-chained MFMA pipeline and asynchronous LDS tile
-//                           copies as the GDN kernel
+//   kda_sweep_kernel        one workgroup per (sequence, head) or second segment sweep: four computing
+//                           wavefronts x 32 V columns with a register-chained MFMA pipeline, one wavefront
+//                           that issues the asynchronous global -> LDS tile copies; writes o
+//   kda_lean_sweep_kernel   first sweep over segments: the zero-state sweep and the transition-matrix
+//                           sweep of two segments in one workgroup of eight wavefronts, no output
+// The operands of every sweep product are fp16 (v_mfma_f32_16x16x32_f16): the decayed tiles hold factors in
+// (0, 1].  W, K e^{G_last-G} and the U of the state update are hi + lo pairs; a float64 simulation of these
+// rounding points gives a final-state rel-L2 below 5e-4 from strong to weak decay (bound 1e-3); the pairs are
+// what keeps keys that repeat within a chunk inside the same bound.  The K e^{G_last-G} tile is stored row major like the others; its transposed
+// operands come from ds_read_b64_tr_b16.
 
 #include "prefill_common.h"
 
@@ -291,68 +298,115 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sequential kernel: one workgroup per (sequence, head) or per segment sweep, four wavefronts (one per
-// SIMD), each owning two 16-column blocks of V that share every A operand.  S^T stays in MFMA
-// accumulator layout (an accumulator tile pair is already a valid B operand of the next product); the
-// A operands come from LDS tiles filled by asynchronous global -> LDS copies.  Every tile is single
-// buffered (104 KB of LDS) and there are two barriers per chunk; a tile's next version is requested at
-// the barrier after its last use and has half a chunk of compute time to land.  Every operand is fp16
-// (v_mfma_f32_16x16x32_f16), rounded once: the decayed tiles hold factors in (0, 1], and a float64
-// simulation of these rounding points gives a final-state rel-L2 of 2.5e-4 .. 4.8e-4 from strong to weak
-// decay (bound 1e-3; 2.6e-3 .. 3.8e-3 with single bf16 operands, which therefore needed hi + lo pairs):
-//
-//   barrier A   K e^G, scale Q e^G, V, W of chunk c landed
-//               flush O(c-1); issue K e^{G_last-G}, P, e^{G_last} of chunk c
-//               KS = (K e^G) S^T, QS = (scale Q e^G) S^T, X = V - KS, U = W X
-//   barrier B   the tiles issued at A landed; issue the first group for chunk c+1
-//               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U,  O = QS + P U -> O tile
-// The K e^{G_last-G} tile is stored row major like the others; its transposed operands come from
-// ds_read_b64_tr_b16.
-//
-// Every wait is for all outstanding copies: what is in flight at a barrier is what the next half needs.
-//
-// WRITE_O = false is the first sweep over segments (affine summaries only): without the query, output and
-// P tiles the workgroup holds 60 KB of LDS and at most 256 registers per lane, so two of them share a CU.
-template <bool WRITE_O>
-__global__ __launch_bounds__(256, 1) void kda_chunk_seq_kernel(const KdaPrefillParams p) {
-  constexpr int NB = 2, WAVES = 4;
-  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, WAVES>;     // 64 x 128 tile
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, WAVES>;    // 64 x 64 tile
+// Sequential kernel with output (whole sequences, and the second sweep over segments): one workgroup per
+// (sequence or segment, head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
+// memory only to store their output rows; wavefront 4 issues every global -> LDS copy of the workgroup (an LDS
+// copy occupies its issuer for tens of cycles, about 2.5 k cycles per chunk in all).  S^T stays in MFMA
+// accumulator layout (an accumulator tile pair is already a valid operand of the next product); the output product
+// is formed transposed, so that a lane holds four adjacent V columns of one token and stores them as 8 bytes.
+// 151 KB of LDS: K e^G and W (hi, lo) are double buffered by chunk parity, everything else is single, with two
+// barriers per chunk:
+//   barrier A   K e^G, W, V of chunk c landed; chunk c - 1 finished     copy scale Q e^G, P, K e^{G_last-G} (hi, lo),
+//               KS = (K e^G) S^T,  X = V - KS,  U = W X                 e^{G_last} of c, then K e^G and W of c + 1
+//   barrier B   the tiles requested at A landed; V is free              copy V of c + 1
+//               O^T = S (scale Q e^G)^T + U^T P^T -> rows of o
+//               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U         (pairs: hi.lo + lo.hi + hi.hi)
+__global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParams p) {
+  constexpr int NB = 2;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
+  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int vcol = 16 * NB * wave + r16;             // first of this lane's V columns (the other: +16)
-
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride, true);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
-  const float* const init = role.init;
-  float* const fin = role.fin;
-  const bool zero_v = role.zero_v, write_o = WRITE_O && role.write_o;
-  const int chunk_in_seq = c_begin - p.seq_chunk_off[n];
-  const int seq_start = p.cu_seqlens[n] + chunk_in_seq * CHUNK;
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
   const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
-
   const int n_chunks = c_end - c_begin;
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  // distinct LDS objects, 16-byte aligned, filled in 1 KiB pieces
-  __shared__ __align__(16) uint16_t tK[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tQ[WRITE_O ? CHUNK * PITCH128 : 8];
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tO[WRITE_O ? CHUNK * PITCH128 : 8];
-  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];      // hi and lo parts
-  __shared__ __align__(16) uint16_t tW[2][CHUNK * PITCH64];        // hi and lo parts
-  __shared__ __align__(16) uint16_t tP[WRITE_O ? CHUNK * PITCH64 : 8];
-  __shared__ __align__(16) float tE[128];            // e^{G_last} of the chunk
+  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
+  __shared__ __align__(16) float tE[128];
 
+  if (wave == 4) {
+    // ---- the copying wavefront -------------------------------------------------------------
+    const int64_t tile0 = (int64_t)c_begin * p.H + h;
+    const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
+    const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
+    const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
+    const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
+    const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
+    const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
+    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
+    const int64_t big_step = (int64_t)p.H * 16384, small_step = (int64_t)p.H * 8192, e_step = (int64_t)p.H * 512;
+    CopyWide plan_k, plan_v;
+    CopyNarrow plan_w;
+    plan_k.plan(256, CHUNK - 1, 0, lane);
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, 0, lane);
+    plan_w.plan(128, CHUNK - 1, 0, lane);
+    auto issue_kw = [&](int c) {                     // K e^G and W (hi, lo) into the buffers of c's parity
+      const int par = c & 1;
+      plan_k.issue(tK[par], kg_b + c * big_step, 0);
+      plan_w.issue(tW[par][0], w_b + c * big_step, 0);
+      plan_w.issue(tW[par][1], w_b + c * big_step + 8192, 0);
+    };
+    auto issue_v = [&](int c) {
+      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+      const int len = chunk_len(c);
+      if (len == CHUNK) {
+        plan_v.issue(tV, vs, 0);
+      } else {                                       // rows past the sequence re-read its last row
+        CopyWide tail_v;
+        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, 0, lane);
+        tail_v.issue(tV, vs, 0);
+      }
+    };
+    auto issue_second = [&](int c) {                 // scale Q e^G, P, K e^{G_last-G} (hi, lo), e^{G_last}
+      plan_k.issue(tQ, qg_b + c * big_step, 0);
+      plan_w.issue(tP, pp_b + c * small_step, 0);
+      plan_k.issue(tKt[0], kt_b + c * 2 * big_step, 0);
+      plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, 0);
+      if (lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
+    };
+    constexpr int KW_COPIES = CopyWide::FIRST + 2 * CopyNarrow::FIRST;       // copies of one issue_kw
+    if (n_chunks > 0) {
+      issue_kw(0);
+      issue_v(0);
+    }
+    for (int ci = 0; ci < n_chunks; ++ci) {
+      const bool more = ci + 1 < n_chunks;
+      wait_vmcnt<0>();                               // K e^G, W, V of chunk ci have landed
+      __syncthreads();                               // barrier A: ... and chunk ci - 1 is finished
+      issue_second(ci);
+      if (more) {
+        issue_kw(ci + 1);
+        wait_vmcnt<KW_COPIES>();                     // the second-half tiles of ci have landed (what follows may be in flight)
+      } else {
+        wait_vmcnt<0>();
+      }
+      __syncthreads();                               // barrier B: ... and V is free
+      if (more) issue_v(ci + 1);
+    }
+    return;
+  }
+
+  // ---- the computing wavefronts ------------------------------------------------------------
+  const int vbase = 32 * wave;
+  const int vcol = vbase + r16;                      // state / KS / U layout: the lane's column (second block: + 16)
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
   f32x4_t St[NB][8];
 #pragma unroll
   for (int nb = 0; nb < NB; ++nb)
-    if (init != nullptr) {
-      const float* src = init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+    if (role.init != nullptr) {
+      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
         const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
@@ -362,7 +416,7 @@ __global__ __launch_bounds__(256, 1) void kda_chunk_seq_kernel(const KdaPrefillP
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     }
-  if (role.keep_init != nullptr) {                   // a first segment that is swept again later: keep its start state
+  if (role.keep_init != nullptr) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
       float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
@@ -371,252 +425,217 @@ __global__ __launch_bounds__(256, 1) void kda_chunk_seq_kernel(const KdaPrefillP
         *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
     }
   }
-  if (zero_v) {                                      // the identity sweep runs with v = 0: no V copies
-    for (int i = tid; i < CHUNK * PITCH128 / 2; i += 256) reinterpret_cast<uint32_t*>(tV)[i] = 0u;
-  }
-
-  const int64_t tile0 = (int64_t)c_begin * p.H + h;                       // chunk tiles are [chunk, H, ...]
-  const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
-  const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
-  const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
-  const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
-  const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
-  const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
-  const int64_t big_step = (int64_t)p.H * 16384, small_step = (int64_t)p.H * 8192, e_step = (int64_t)p.H * 512;
-
-  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
-  CopyWide plan_k, plan_v;
-  CopyNarrow plan_w;
-  plan_k.plan(256, CHUNK - 1, wave, lane);
-  plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, wave, lane);
-  plan_w.plan(128, CHUNK - 1, wave, lane);
-  auto issue_first = [&](int c) {                    // K e^G, scale Q e^G, V, W
-    plan_k.issue(tK, kg_b + c * big_step, wave);
-    if constexpr (WRITE_O) plan_k.issue(tQ, qg_b + c * big_step, wave);
-    if (!zero_v) {
-      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
-      const int len = chunk_len(c);
-      if (len == CHUNK) {
-        plan_v.issue(tV, vs, wave);
-      } else {                                       // rows past the sequence re-read its last row
-        CopyWide tail_v;
-        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, wave, lane);
-        tail_v.issue(tV, vs, wave);
-      }
-    }
-    plan_w.issue(tW[0], w_b + c * 2 * small_step, wave);
-    plan_w.issue(tW[1], w_b + c * 2 * small_step + 8192, wave);
-  };
-  auto issue_second = [&](int c) {                   // K e^{G_last-G}, P, e^{G_last}
-    plan_k.issue(tKt[0], kt_b + c * 2 * big_step, wave);
-    plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, wave);
-    if constexpr (WRITE_O) plan_w.issue(tP, pp_b + c * small_step, wave);
-    if (wave == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
-  };
-  // coalesced write of a finished output tile
-  const int krow = tid >> 4, kcv = tid & 15;
-  uint16_t* const o_b = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + krow) * p.H + h) * 128 + 8 * kcv;
-  auto flush_output = [&](int c) {
-    if (!write_o) return;
-    const int len = chunk_len(c);
-    uint16_t* dst = o_b + (int64_t)c * CHUNK * p.H * 128;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (krow + 16 * i < len)
-        *reinterpret_cast<uint4*>(dst + (int64_t)16 * i * p.H * 128) =
-            *reinterpret_cast<const uint4*>(&tO[(krow + 16 * i) * PITCH128 + 8 * kcv]);
-  };
-
-  if (n_chunks > 0) issue_first(0);                  // a stage of a short sequence may hold no chunk
+  // output rows: in the transposed product a lane holds V columns vbase + 16 nb + 4 kb .. + 3 of token 16 ni + r16
+  uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.H + h) * 128 + vbase + 4 * kb;
+  const bool write_o = role.write_o;
 
   for (int ci = 0; ci < n_chunks; ++ci) {
-    const bool more = ci + 1 < n_chunks;
-
-    // barrier A
-    wait_vmcnt<0>();
-    __syncthreads();
-    bf16x8_t ka[2][4], qa[2][4];
-#pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
-      ka[0][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], 0, kb);
-      if constexpr (WRITE_O) qa[0][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], 0, kb);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    if (ci > 0) flush_output(ci - 1);
-    issue_second(ci);
-
-    f32x4_t KS[NB][4], QS[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) { KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f}; QS[nb][mi] = KS[nb][mi]; }
-    uint16_t vraw[NB][16];
+    const int par = ci & 1;
+    // barrier A (bare: the tiles come from the copying wavefront's LDS copies, which it waited for)
+    __builtin_amdgcn_s_waitcnt(0xc07f);              // lgkmcnt(0) only
+    __builtin_amdgcn_s_barrier();
+    const uint16_t* const K = tK[par];
+    // ---- KS = (K e^G) S^T ----
+    f32x4_t KS[NB][4];
     bf16x8_t wa[2][4], wl[2][4];
-    bf16x8_t sb[2][NB];
+    uint16_t vraw[NB][16];
+    {
+      bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (s < 3) {
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          ka[(s + 1) & 1][mi] = operand_from(&tK[(16 * mi + r16) * PITCH128], s + 1, kb);
-          if constexpr (WRITE_O) qa[(s + 1) & 1][mi] = operand_from(&tQ[(16 * mi + r16) * PITCH128], s + 1, kb);
-        }
-      } else {
-        // the last step's MFMAs cover the reads for X and for U = W X
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) {
-            const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
-          }
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wa[s2][mi] = operand_from(&tW[0][(16 * mi + r16) * PITCH64], s2, kb);
-            wl[s2][mi] = operand_from(&tW[1][(16 * mi + r16) * PITCH64], s2, kb);
-          }
-      }
-      __builtin_amdgcn_sched_barrier(0);
-      // the next step's state slice is rounded underneath this step's MFMAs
-      if (s < 3) {
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
-      }
+      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+      __builtin_amdgcn_sched_barrier(0x000F);        // LDS requests stay above this line; ALU and MFMA work may cross it
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
-      if constexpr (WRITE_O) {
+        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) {
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+        } else {
+          // under the last step: V and the first half of W
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+            }
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) {
+            wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
+            wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0x000F);
+        if (s < 3) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(qa[s & 1][mi], sb[s & 1][nb], QS[nb][mi]);
+          for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
       }
-      __builtin_amdgcn_sched_barrier(0);
     }
-    // X = V - KS
-    f32x4_t X[NB][4];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) X[nb][mi][r] = to_float(bf16_t{vraw[nb][4 * mi + r]}) - KS[nb][mi][r];
-    // U = W X
+    // ---- X = V - KS,  U = W X ----
     f32x4_t U[NB][4];
+    {
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      bf16x8_t xb[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
-    }
-
-    // barrier B
-    wait_vmcnt<0>();
-    __syncthreads();
-    bf16x8_t kt[2][8], ktl[8];
-#pragma unroll
-    for (int s = 0; s < 2; ++s)
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) kt[s][mc] = operand_transposed(tKt[0], s, mc, kb, r16);
-#pragma unroll
-    for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
-    float4 eg[8];
-#pragma unroll
-    for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
-    __builtin_amdgcn_sched_barrier(0);
-    if (more) issue_first(ci + 1);
-    // S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        St[nb][mc] = f32x4_t{St[nb][mc][0] * eg[mc].x, St[nb][mc][1] * eg[mc].y, St[nb][mc][2] * eg[mc].z,
-                             St[nb][mc][3] * eg[mc].w};
-    bf16x8_t pa[2][4];
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      if (WRITE_O && s == 1) {
-        // the last step's MFMAs cover the reads for the output product
-#pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) pa[s2][mi] = operand_from(&tP[(16 * mi + r16) * PITCH64], s2, kb);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int mi = 0; mi < 4; ++mi) {
+        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
+        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
       }
-      HalfPair ub[NB];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) ub[nb] = half8_pair(U[nb][2 * s], U[nb][2 * s + 1]);
-      // hi . lo and lo . hi first, the large term last
+      __builtin_amdgcn_sched_barrier(0x000F);
+      f32x4_t X[NB][4];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
-      if (s == 0) {
+        for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+          for (int r = 0; r < 4; ++r) X[nb][mi][r] = to_float(bf16_t{vraw[nb][4 * mi + r]}) - KS[nb][mi][r];
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        bf16x8_t xb[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
       }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
-      __builtin_amdgcn_sched_barrier(0);
     }
-
-    if constexpr (WRITE_O) {
-      // O = QS + P U -> O tile
+    // barrier B: Q, P, the K e^{G_last-G} pair and e^{G_last} of this chunk have landed
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    // ---- O^T = S (scale Q e^G)^T + U^T P^T -> o ----
+    bf16x8_t kt[8], ktl[8];
+    {
+      f32x4_t OT[NB][4];                             // OT[nb][ni][r] = o[token 16 ni + r16][v = vbase + 16 nb + 4 kb + r]
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      bf16x8_t qa[2][4], sb[2][NB], pa[2][4];
+#pragma unroll
+      for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], 0, kb);
+      __builtin_amdgcn_sched_barrier(0x000F);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) {
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], s + 1, kb);
+        } else {
+#pragma unroll
+          for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+            for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[(16 * ni + r16) * PITCH64], s2, kb);
+        }
+        __builtin_amdgcn_sched_barrier(0x000F);
+        if (s < 3) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
+        }
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(sb[s & 1][nb], qa[s & 1][ni], OT[nb][ni]);
+      }
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         bf16x8_t ur[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
+        if (s == 1) {
+          // under the last step: the first transposed key operands of the state update
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) {
+            kt[mc] = operand_transposed(tKt[0], 0, mc, kb, r16);
+            ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
+          }
+          __builtin_amdgcn_sched_barrier(0x000F);
+        }
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) QS[nb][mi] = mfma16h(pa[s][mi], ur[nb], QS[nb][mi]);
+          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(ur[nb], pa[s][ni], OT[nb][ni]);
       }
+      if (write_o) {
+        const int len = chunk_len(ci);
+        uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.H * 128;
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi)
+        for (int ni = 0; ni < 4; ++ni)
+          if (16 * ni + r16 < len) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          uint16_t* orow = &tO[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-          orow[0] = from_float<bf16_t>(QS[nb][mi][0]).bits;
-          orow[PITCH128] = from_float<bf16_t>(QS[nb][mi][1]).bits;
-          orow[2 * PITCH128] = from_float<bf16_t>(QS[nb][mi][2]).bits;
-          orow[3 * PITCH128] = from_float<bf16_t>(QS[nb][mi][3]).bits;
+            for (int nb = 0; nb < NB; ++nb) {
+              const uint2 packed = make_uint2(pack2<bf16_t>(OT[nb][ni][0], OT[nb][ni][1]), pack2<bf16_t>(OT[nb][ni][2], OT[nb][ni][3]));
+              *reinterpret_cast<uint2*>(dst + (int64_t)16 * ni * p.H * 128 + 16 * nb) = packed;
+            }
+          }
+      }
+    }
+    // ---- S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U ----
+    {
+      float4 eg[8];
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
+      __builtin_amdgcn_sched_barrier(0x000F);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int mc = 0; mc < 8; ++mc)
+          St[nb][mc] = f32x4_t{St[nb][mc][0] * eg[mc].x, St[nb][mc][1] * eg[mc].y, St[nb][mc][2] * eg[mc].z,
+                               St[nb][mc][3] * eg[mc].w};
+#pragma unroll
+      for (int s = 0; s < 2; ++s) {
+        HalfPair ub[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) ub[nb] = half8_pair(U[nb][2 * s], U[nb][2 * s + 1]);
+        // hi . lo and lo . hi first, the large term last
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
+        if (s == 0) {
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+          __builtin_amdgcn_sched_barrier(0x000F);
         }
-  
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].lo, St[nb][mc]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
+        if (s == 0) {
+#pragma unroll
+          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(tKt[0], 1, mc, kb, r16);
+          __builtin_amdgcn_sched_barrier(0x000F);
+        }
+      }
     }
   }
-  __syncthreads();
-  if (n_chunks > 0) flush_output(n_chunks - 1);
 
-  if (fin != nullptr) {
+  if (role.fin != nullptr) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      float* dst = fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc)
         *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
@@ -1031,14 +1050,14 @@ extern "C" int pla_kda_prefill_launch(
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
         // the first sweep over segments publishes no output: both of its roles in one workgroup per (segment, head)
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(kda_chunk_seq_kernel<true>, dim3(grid), dim3(256), 0, s, p);
+        else hipLaunchKernelGGL(kda_sweep_kernel, dim3(grid), dim3(320), 0, s, p);
       });
   PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_chunk_seq_kernel<true>, dim3((unsigned)L.max_segments * H), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(kda_sweep_kernel, dim3((unsigned)L.max_segments * H), dim3(320), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
