@@ -64,6 +64,7 @@ struct GdnPrefillParams {
   int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments
   int stage;             // stage handled by this launch (per-chunk kernels and pass 3)
   int H, HV, NC_max;
+  int qk_rows_16;        // q and k rows start on 16-byte boundaries (else on 4-byte ones)
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -101,24 +102,31 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
-  // raw K and Q operands: 4 row blocks x 4 contraction steps, two 8-byte pieces each; all 64 loads of a lane are
-  // requested before the first use (the LDS tile limits a SIMD to two wavefronts, which hide no latency)
-  uint2 kraw[4][4][2], qraw[4][4][2];
+  // raw K and Q operands: 4 row blocks x 4 contraction steps of 16 bytes (lane (r, kb) takes elements 32 s + 8 kb .. + 7
+  // of its row; the contraction index may be assigned to operand slots in any order as long as both operands of a
+  // product agree); all 32 loads of a lane are requested before the first use (a SIMD holds two wavefronts, which
+  // hide no latency)
+  uint4 kraw[4][4], qraw[4][4];
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb) {
     const int row = 16 * mb + r16;
     const int64_t t = t0 + (row < len ? row : 0);
-    const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128;
-    const uint16_t* qr = reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128;
+    const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + 8 * kb;
+    const uint16_t* qr = reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128 + 8 * kb;
+    if (p.qk_rows_16) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      kraw[mb][s][0] = *reinterpret_cast<const uint2*>(kr + 32 * s + 4 * kb);
-      kraw[mb][s][1] = *reinterpret_cast<const uint2*>(kr + 32 * s + 16 + 4 * kb);
-    }
+      for (int s = 0; s < 4; ++s) kraw[mb][s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      qraw[mb][s][0] = *reinterpret_cast<const uint2*>(qr + 32 * s + 4 * kb);
-      qraw[mb][s][1] = *reinterpret_cast<const uint2*>(qr + 32 * s + 16 + 4 * kb);
+      for (int s = 0; s < 4; ++s) qraw[mb][s] = *reinterpret_cast<const uint4*>(qr + 32 * s);
+    } else {                                             // rows aligned to 4 bytes only
+      auto four_words = [](const uint16_t* at) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(at);
+        return make_uint4(w[0], w[1], w[2], w[3]);
+      };
+#pragma unroll
+      for (int s = 0; s < 4; ++s) kraw[mb][s] = four_words(kr + 32 * s);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) qraw[mb][s] = four_words(qr + 32 * s);
     }
   }
 
@@ -165,28 +173,28 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
   // ---- q / k: normalise, round to the activation dtype, hold as fp16 (exact; saturating beyond its range) ----
   bf16x8_t Kop[4][4], Qop[4][4];
   {
-    auto row_scale = [&](const uint2 (&raw)[4][2]) {
+    auto row_scale = [&](const uint4 (&raw)[4]) {
       float ss = 0.f;
 #pragma unroll
-      for (int s = 0; s < 4; ++s)
+      for (int s = 0; s < 4; ++s) {
+        const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
 #pragma unroll
-        for (int hlf = 0; hlf < 2; ++hlf) {
-          const float a0 = lo16<act_t>(raw[s][hlf].x), a1 = hi16<act_t>(raw[s][hlf].x);
-          const float a2 = lo16<act_t>(raw[s][hlf].y), a3 = hi16<act_t>(raw[s][hlf].y);
-          ss += a0 * a0 + a1 * a1 + a2 * a2 + a3 * a3;
+        for (int e = 0; e < 4; ++e) {
+          const float a0 = lo16<act_t>(w[e]), a1 = hi16<act_t>(w[e]);
+          ss += a0 * a0 + a1 * a1;
         }
+      }
       const LanePair r1 = swap_rows16(ss);               // the four lanes of a row are 16 lanes apart
       const LanePair r2 = swap_halves(r1.lo + r1.hi);
       return rsqrtf(r2.lo + r2.hi + 1e-6f);
     };
-    auto normalised = [&](const uint2 (&raw)[2], float inv) {
+    auto normalised = [&](const uint4& raw, float inv) {
+      const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
       uint32_t w[4];
 #pragma unroll
-      for (int hlf = 0; hlf < 2; ++hlf) {
-        const uint32_t a = pack2<act_t>(lo16<act_t>(raw[hlf].x) * inv, hi16<act_t>(raw[hlf].x) * inv);
-        const uint32_t b = pack2<act_t>(lo16<act_t>(raw[hlf].y) * inv, hi16<act_t>(raw[hlf].y) * inv);
-        w[2 * hlf] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
-        w[2 * hlf + 1] = pack2_rtz(lo16<act_t>(b), hi16<act_t>(b));
+      for (int e = 0; e < 4; ++e) {
+        const uint32_t a = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
+        w[e] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
       }
       return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
     };
@@ -208,21 +216,14 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
         Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
       }
       if (ok && (store_k || store_q)) {
-        uint16_t* dst = (store_k ? p.kn : p.qn) + ((int64_t)(t0 + row) * p.H + h) * 128;
+        uint16_t* dst = (store_k ? p.kn : p.qn) + ((int64_t)(t0 + row) * p.H + h) * 128 + 8 * kb;
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          const uint4 w = __builtin_bit_cast(uint4, store_k ? Kop[mb][s] : Qop[mb][s]);
-          *reinterpret_cast<uint2*>(dst + 32 * s + 4 * kb) = make_uint2(w.x, w.y);
-          *reinterpret_cast<uint2*>(dst + 32 * s + 16 + 4 * kb) = make_uint2(w.z, w.w);
-        }
+        for (int s = 0; s < 4; ++s)
+          *reinterpret_cast<uint4*>(dst + 32 * s) = __builtin_bit_cast(uint4, store_k ? Kop[mb][s] : Qop[mb][s]);
         if (store_k && store_q) {                      // one wavefront per q/k head: it stores both
-          uint16_t* dq = p.qn + ((int64_t)(t0 + row) * p.H + h) * 128;
+          uint16_t* dq = p.qn + ((int64_t)(t0 + row) * p.H + h) * 128 + 8 * kb;
 #pragma unroll
-          for (int s = 0; s < 4; ++s) {
-            const uint4 w = __builtin_bit_cast(uint4, Qop[mb][s]);
-            *reinterpret_cast<uint2*>(dq + 32 * s + 4 * kb) = make_uint2(w.x, w.y);
-            *reinterpret_cast<uint2*>(dq + 32 * s + 16 + 4 * kb) = make_uint2(w.z, w.w);
-          }
+          for (int s = 0; s < 4; ++s) *reinterpret_cast<uint4*>(dq + 32 * s) = __builtin_bit_cast(uint4, Qop[mb][s]);
         }
       }
     }
@@ -1040,6 +1041,7 @@ static int gdn_prefill_run(
   p.W = reinterpret_cast<uint16_t*>(ws + L.W);
   p.P = reinterpret_cast<uint16_t*>(ws + L.P);
   p.H = H; p.HV = HV; p.NC_max = L.NC_max;
+  p.qk_rows_16 = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && stride_q % 8 == 0 && stride_k % 8 == 0;
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool segmented = L.seg_chunks > 0;
