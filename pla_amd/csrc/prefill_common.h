@@ -35,6 +35,13 @@ __device__ __forceinline__ bf16x8_t operand_transposed(const uint16_t* tile, int
   return __builtin_bit_cast(bf16x8_t, u);
 }
 
+// One transposing read: lane i of a group of 16 receives column i of the four rows the group addresses (lane t
+// addresses columns 4 (t % 4) .. + 3 of row t / 4), packed as 16-bit (row 0, row 1), (row 2, row 3).
+__device__ __forceinline__ uint2 read_tr4(const uint16_t* at) {
+  const i16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)at);
+  return __builtin_bit_cast(uint2, v);
+}
+
 // LDS tile pitches (bf16 elements): rows stay 16-byte aligned and consecutive rows start 4 (128-wide)
 // or 36 (64-wide) banks apart, which keeps the 8-byte operand reads of a wavefront conflict free.
 constexpr int PITCH128 = 136;
@@ -55,10 +62,9 @@ __device__ __forceinline__ f32x4_t mfma_hilo(const HiLo& a, const HiLo& b, f32x4
   return mfma16(a.hi, b.hi, c);
 }
 
-// PAIR: W leaves as two fp16 tiles, hi at W and lo at W + 4096 (W = hi + lo to about 22 bits), else as one tile
-// rounded to nearest.
-template <bool PAIR>
-__device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const float* beta, int lane, uint16_t* W) {
+// block_inverse_inplace leaves N = (I + L)^-1 in the lower triangle of L (the blocks above the diagonal hold
+// scratch); the two functions after it scale by beta and store W in one of two layouts.
+__device__ __forceinline__ void block_inverse_inplace(float (*L)[68], int lane) {
   const int r16 = lane & 15, kb = lane >> 4;
   const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
   {
@@ -127,6 +133,13 @@ __device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const floa
   put(1, 0, X10); put(2, 1, X21); put(3, 2, X32); put(2, 0, X20); put(3, 1, X31); put(3, 0, X30);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
+}
+
+// Row-major store.  PAIR: W leaves as two fp16 tiles, hi at W and lo at W + 4096 (W = hi + lo to about 22 bits),
+// else as one tile rounded to nearest.
+template <bool PAIR>
+__device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const float* beta, int lane, uint16_t* W) {
+  block_inverse_inplace(L, lane);
   // W[i][j] = N[i][j] beta_j for j <= i, zero above: lane -> row 8 pass + lane / 8, columns 8 (lane % 8) ..
   const int c8 = 8 * (lane & 7);
   const float4 b0 = *reinterpret_cast<const float4*>(&beta[c8]), b1 = *reinterpret_cast<const float4*>(&beta[c8 + 4]);
@@ -144,6 +157,37 @@ __device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const floa
     }
     *reinterpret_cast<uint4*>(W + i * 64 + c8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
     if constexpr (PAIR) *reinterpret_cast<uint4*>(W + 4096 + i * 64 + c8) = make_uint4(rest[0], rest[1], rest[2], rest[3]);
+  }
+}
+
+// A lower triangular 64 x 64 tile as the A (or B) operands of the products that contract over its columns: only six
+// of the eight 16 x 32 operand blocks hold anything (row block m, column half s: s = 0 for every m, s = 1 for
+// m = 2, 3).  Block b is 1 KiB: lane (r, kb) owns 16 bytes, columns 32 s + 4 kb .. + 3 and 32 s + 16 + 4 kb .. + 3 of
+// row 16 m + r, which is the contraction order in which a pair of accumulator tiles presents its rows.  A consumer
+// copies the blocks to LDS as they are and reads an operand with one 16-byte access per lane.
+constexpr int TRI_BLOCKS = 6;
+__device__ __forceinline__ constexpr int tri_block_m(int b) { return b < 4 ? b : b - 2; }
+__device__ __forceinline__ constexpr int tri_block_s(int b) { return b < 4 ? 0 : 1; }
+// W = N diag(beta) from the tile block_inverse_inplace leaves, as an fp16 hi + lo pair in that layout: hi blocks at
+// W, lo blocks at W + TRI_BLOCKS * 512 (halves).
+__device__ __forceinline__ void store_w_operand_blocks(float (*L)[68], const float* beta, int lane, uint16_t* W) {
+  const int r16 = lane & 15, kb = lane >> 4;
+#pragma unroll
+  for (int b = 0; b < TRI_BLOCKS; ++b) {
+    const int i = 16 * tri_block_m(b) + r16;
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int j0 = 32 * tri_block_s(b) + 16 * half + 4 * kb;
+      const float4 n4 = *reinterpret_cast<const float4*>(&L[i][j0]);
+      const float4 b4 = *reinterpret_cast<const float4*>(&beta[j0]);
+      const float w0 = j0 <= i ? n4.x * b4.x : 0.f, w1 = j0 + 1 <= i ? n4.y * b4.y : 0.f;
+      const float w2 = j0 + 2 <= i ? n4.z * b4.z : 0.f, w3 = j0 + 3 <= i ? n4.w * b4.w : 0.f;
+      pack2_pair(w0, w1, hi[2 * half], lo[2 * half]);
+      pack2_pair(w2, w3, hi[2 * half + 1], lo[2 * half + 1]);
+    }
+    *reinterpret_cast<uint4*>(W + b * 512 + lane * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    *reinterpret_cast<uint4*>(W + (TRI_BLOCKS + b) * 512 + lane * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
   }
 }
 

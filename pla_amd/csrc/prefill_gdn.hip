@@ -34,9 +34,14 @@
 //   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
 //                            segment side by side in one workgroup of eight wavefronts that share every tile
 
+#include <type_traits>
+
 #include "prefill_common.h"
 
 namespace pla {
+
+// Floats per (chunk, value head) tile of decay factors: scale e^G | e^G | e^{G_last - G} | e^{G_last} (x 64) | G
+constexpr int GTILE_FLOATS = 320;
 
 struct GdnPrefillParams {
   // inputs
@@ -55,6 +60,7 @@ struct GdnPrefillParams {
   // workspace
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
   uint16_t* qn; uint16_t* kn;
+  float* kinv;                                        // [T, H] 1 / |k| per row (fused sweep)
   float* gcum; float* beta;
   uint16_t* W;                                        // fp16 [chunk, HV, 2, 64, 64]: W = hi + lo
   uint16_t* P;                                        // fp16 [chunk, HV, 64, 64]
@@ -299,6 +305,144 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
     }
     *reinterpret_cast<uint4*>(Pt + i * 64 + c8) = w;
   }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Preparation for the fused sweep (gdn_fused_sweep_kernel), which normalises q and k and forms P itself: only what
+// needs the triangular solve leaves this kernel.  One wavefront per (chunk, value head) as above, the key side only:
+// gate, beta and their cumulative sum (g_cum and beta as the call returns them, the chunk's tile of decay factors
+// with the raw cumulative log-decay appended for the sweep's P), normalised K in registers, K K^T on MFMA, the
+// inverse of I + L by 16 x 16 blocks, and W = (I + L)^-1 diag(beta) as an fp16 hi + lo pair in the six-block
+// operand layout (12 KiB per (chunk, value head) instead of 16 KiB row-major + 8 KiB of P + the normalised rows).
+template <typename act_t, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefillParams p) {
+  const int groups = p.HV / WAVES;
+  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
+  if (cb < 0) return;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int hv = (blockIdx.x % groups) * WAVES + wave;
+  const int h = hv / (p.HV / p.H);
+  const int t0 = p.chunk_tok[cb];
+  const int len = p.chunk_len[cb];
+  const int lane = threadIdx.x & 63;
+  const int r16 = lane & 15, kb = lane >> 4;
+
+  __shared__ __align__(16) float Lm_all[WAVES][CHUNK][68];
+  __shared__ __align__(16) float Gs_all[WAVES][CHUNK];
+  __shared__ __align__(16) float Bs_all[WAVES][CHUNK];
+  float (*const Lm)[68] = Lm_all[wave];
+  float* const Gs = Gs_all[wave];
+  float* const Bs = Bs_all[wave];
+
+  // raw K operands, all 16 loads of a lane requested before the first use (rows are 16-byte aligned on this path)
+  uint4 kraw[4][4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb) {
+    const int row = 16 * mb + r16;
+    const int64_t t = t0 + (row < len ? row : 0);
+    const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + 8 * kb;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) kraw[mb][s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
+  }
+
+  // ---- gate: lane = token ----
+  {
+    float g = 0.f, bt = 0.f;
+    if (lane < len) {
+      const int64_t t = t0 + lane;
+      if (p.g_in) {
+        g = p.g_in[t * p.HV + hv];
+        bt = p.beta_in[t * p.HV + hv];
+      } else {
+        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
+        const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
+        g = -expf(p.A_log[hv]) * sp;
+        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
+        bt = 1.0f / (1.0f + expf(-braw));
+      }
+    }
+    float cum = g;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const float up = __shfl_up(cum, d, 64);
+      if (lane >= d) cum += up;
+    }
+    const float glast = __shfl(cum, 63, 64);
+    if (lane < len) {
+      const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;
+      p.gcum[at] = cum;
+      p.beta[at] = bt;
+    }
+    Gs[lane] = cum;
+    Bs[lane] = bt;
+    float* gt = p.gtile + ((int64_t)cb * p.HV + hv) * GTILE_FLOATS;
+    const float e = __expf(cum);
+    gt[lane] = p.scale * e;
+    gt[64 + lane] = e;
+    gt[128 + lane] = __expf(glast - cum);
+    gt[192 + lane] = __expf(glast);
+    gt[256 + lane] = cum;
+  }
+
+  // ---- k: normalise, round to the activation dtype, hold as fp16 ----
+  bf16x8_t Kop[4][4];
+  {
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const bool ok = 16 * mb + r16 < len;
+      float inv = 1.f;
+      if (p.normalize_qk) {
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          const uint32_t w[4] = {kraw[mb][s].x, kraw[mb][s].y, kraw[mb][s].z, kraw[mb][s].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float a0 = lo16<act_t>(w[e]), a1 = hi16<act_t>(w[e]);
+            ss += a0 * a0 + a1 * a1;
+          }
+        }
+        const LanePair r1 = swap_rows16(ss);
+        const LanePair r2 = swap_halves(r1.lo + r1.hi);
+        inv = rsqrtf(r2.lo + r2.hi + 1e-6f);
+        // the sweep scales the raw rows by the same factor, so both kernels hold the same rounded keys
+        if (ok && kb == 0 && hv % (p.HV / p.H) == 0) p.kinv[(int64_t)(t0 + 16 * mb + r16) * p.H + h] = inv;
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const uint32_t in[4] = {kraw[mb][s].x, kraw[mb][s].y, kraw[mb][s].z, kraw[mb][s].w};
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t a = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
+          w[e] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
+        }
+        Kop[mb][s] = ok ? __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3])) : __builtin_bit_cast(bf16x8_t, zero4);
+      }
+    }
+  }
+  __syncthreads();
+
+  // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
+#pragma unroll
+  for (int mi = 0; mi < 4; ++mi) {
+#pragma unroll
+    for (int ni = 0; ni <= mi; ++ni) {
+      f32x4_t kk = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < 4; ++s) kk = mfma16h(Kop[mi][s], Kop[ni][s], kk);
+      const int j = 16 * ni + r16;
+      const float Gj = Gs[j];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int i = 16 * mi + 4 * kb + r;
+        Lm[i][j] = i > j ? Bs[i] * kk[r] * __expf(Gs[i] - Gj) : 0.f;
+      }
+    }
+  }
+  block_inverse_inplace(Lm, lane);
+  store_w_operand_blocks(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * (2 * TRI_BLOCKS * 512));
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -906,11 +1050,479 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fused sweep for whole sequences: one workgroup of EIGHT wavefronts per (sequence, value head).  Wavefronts 0-3
+// compute as in gdn_sweep_kernel (32 V columns of S^T each, the chain K S^T -> X -> U -> S^T in registers).
+// Wavefronts 4-7 feed them, so that neither the normalised rows nor P cross memory:
+//   rows   wavefronts 4, 5 take the raw K rows of the next chunk (32 rows each), 6, 7 the raw Q rows: loaded one
+//          chunk ahead into registers (16 lanes per row, 16 bytes per lane), scaled by the row's 1 / |k| (from the
+//          preparation kernel, so that both kernels round the very same normalised keys) or 1 / |q| (summed here),
+//          rounded to the activation dtype, and written to the LDS tiles as fp16
+//   P      scale tril(q_i . k_j e^{G_i - G_j}) of the current chunk from those tiles: the products are formed
+//          transposed (A = K rows, B = Q rows), which leaves a lane with four consecutive j of one token i, i.e. with
+//          8 of the 16 bytes it owns in the six-block operand layout (prefill_common.h) that phase 3 reads
+//   copies V, W (12 KiB, six-block layout, hi then lo) and the decay-factor tile by global -> LDS copies
+// Two barriers per chunk: A opens the chunk (all tiles of it are complete, those of the chunk before are free),
+// B follows the query product (P is complete).  The computing wavefronts run a hand-ordered schedule: every LDS
+// operand is requested a fixed number of steps before the MFMA that uses it and the VALU work (conversions, X, the
+// hi / lo split of U, the decay of S) is placed under the MFMAs; scheduling barriers keep that order.
+#define SB() __builtin_amdgcn_sched_barrier(0)
+template <typename act_t>
+__global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefillParams p) {
+  constexpr int NB = 2, CW = 4, AUX = 4;
+  using CopyV = TileCopy<CHUNK, 2 * PITCH128, 256, AUX>;
+  const int block = xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV);
+  if (block < 0) return;
+  const SweepRole role = select_sweep(0, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block);
+  if (!role.active) return;
+  const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
+  const int h = hv / (p.HV / p.H);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r16 = lane & 15, kb = lane >> 4;
+  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
+  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
+  const int n_chunks = c_end - c_begin;
+  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
+
+  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tQ[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  __shared__ __align__(16) uint16_t tW[2][2 * TRI_BLOCKS * 512];    // [parity][hi blocks, lo blocks]
+  __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
+  // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}, [256,320) G
+  __shared__ __align__(16) float tG[2][512];
+
+  if (wave >= CW) {
+    // ---- the feeding wavefronts ----
+    const int a = wave - CW;
+    const bool q_side = a >= 2;
+    const int row0 = 32 * (a & 1);                      // this wavefront's rows of a chunk: row0 .. row0 + 31
+    const int lr = lane >> 4, lc = lane & 15;           // piece j: row row0 + 4 j + lr, columns 8 lc .. 8 lc + 7
+    const int64_t row_pitch = q_side ? p.stride_q : p.stride_k;
+    const uint16_t* const rows = reinterpret_cast<const uint16_t*>(q_side ? p.q : p.k) + (int64_t)seq_start * row_pitch + h * 128 + 8 * lc;
+    const float* const kinv = p.kinv + (int64_t)seq_start * p.H + h;
+    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
+    const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * (2 * TRI_BLOCKS * 1024);
+    const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * (GTILE_FLOATS * 4);
+    CopyV plan_v;
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, a, lane);
+
+    // global -> LDS copies of chunk c (its buffers are free): V, W and the decay-factor tile
+    auto issue_copies = [&](int c) {
+      const int par = c & 1;
+      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+      const int len = chunk_len(c);
+      if (len == CHUNK) plan_v.issue(tV[par], vs, a);
+      else {                                           // rows past the sequence end re-read its last row
+        CopyV tail;
+        tail.plan((uint32_t)(p.stride_v * 2), len - 1, a, lane);
+        tail.issue(tV[par], vs, a);
+      }
+      const char* ws = w_b + (int64_t)c * p.HV * (2 * TRI_BLOCKS * 1024);
+#pragma unroll
+      for (int j = 0; j < 2 * TRI_BLOCKS / AUX; ++j)
+        dma16(ws, 1024u * (AUX * j + a) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (AUX * j + a));
+      const char* gs = gt_b + (int64_t)c * p.HV * (GTILE_FLOATS * 4);
+      if (a == 1) dma16(gs, 16u * lane, lds_address(&tG[par][0]));
+      if (a == 2) dma16(gs, 1024u + 16u * (lane & 15), lds_address(&tG[par][256]));     // 64 floats; lanes 16-63 repeat them
+    };
+    // raw rows of chunk c into registers (rows past the end of the sequence part re-read its last row)
+    auto load_rows = [&](int c, uint4 (&raw)[8], float (&inv)[8]) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int t = min(c * CHUNK + row0 + 4 * j + lr, seq_len - 1);
+        raw[j] = *reinterpret_cast<const uint4*>(rows + (int64_t)t * row_pitch);
+        inv[j] = q_side ? 0.f : kinv[(int64_t)t * p.H];
+      }
+    };
+    // normalise, round to the activation dtype, write as fp16 into the tile of chunk c
+    auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
+      uint16_t* const T = q_side ? tQ[c & 1] : tK[c & 1];
+      const int len = chunk_len(c);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row = row0 + 4 * j + lr;
+        const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+        float inv = inv_in[j];
+        if (q_side) {
+          float ss = 0.f;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float a0 = lo16<act_t>(in[e]), a1 = hi16<act_t>(in[e]);
+            ss += a0 * a0 + a1 * a1;
+          }
+          inv = rsqrtf(row16_allreduce(ss) + 1e-6f);
+        }
+        if (!p.normalize_qk) inv = 1.f;
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
+          w[e] = row < len ? pack2_rtz(lo16<act_t>(r), hi16<act_t>(r)) : 0u;
+        }
+        *reinterpret_cast<uint4*>(T + row * PITCH128 + 8 * lc) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    };
+    // P of chunk c from its K and Q tiles: this wavefront's blocks of the six
+    auto form_p = [&](int c) {
+      const uint16_t* const K = tK[c & 1];
+      const uint16_t* const Q = tQ[c & 1];
+      const float* const G = &tG[c & 1][256];
+      auto block = [&](int b) {
+        const int ni = tri_block_m(b), s = tri_block_s(b);
+        bf16x8_t qb[4];
+#pragma unroll
+        for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_from(Q + (16 * ni + r16) * PITCH128, s2, kb);
+        const float Gi = G[16 * ni + r16];
+        const int i = 16 * ni + r16;
+        uint32_t w[4];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int nj = 2 * s + half;
+          if (nj > ni) { w[2 * half] = 0u; w[2 * half + 1] = 0u; continue; }
+          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s2 = 0; s2 < 4; ++s2) acc = mfma16h(operand_from(K + (16 * nj + r16) * PITCH128, s2, kb), qb[s2], acc);
+          const float4 Gj = *reinterpret_cast<const float4*>(&G[16 * nj + 4 * kb]);
+          const int j0 = 16 * nj + 4 * kb;
+          const float p0 = j0 <= i ? p.scale * acc[0] * __expf(Gi - Gj.x) : 0.f;
+          const float p1 = j0 + 1 <= i ? p.scale * acc[1] * __expf(Gi - Gj.y) : 0.f;
+          const float p2 = j0 + 2 <= i ? p.scale * acc[2] * __expf(Gi - Gj.z) : 0.f;
+          const float p3 = j0 + 3 <= i ? p.scale * acc[3] * __expf(Gi - Gj.w) : 0.f;
+          w[2 * half] = pack2_rtz(p0, p1);
+          w[2 * half + 1] = pack2_rtz(p2, p3);
+        }
+        *reinterpret_cast<uint4*>(tP + b * 512 + lane * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+      };
+      if (a == 0) { block(0); block(3); }
+      else if (a == 1) block(1);
+      else if (a == 2) { block(2); block(4); }
+      else block(5);
+    };
+
+    uint4 raw[8], raw_next[8];
+    float inv[8], inv_next[8];
+    if (n_chunks > 0) {
+      issue_copies(0);
+      load_rows(0, raw, inv);
+      if (n_chunks > 1) load_rows(1, raw_next, inv_next);
+      write_rows(0, raw, inv);
+    }
+    for (int ci = 0; ci < n_chunks; ++ci) {
+      wait_vmcnt<0>();                               // this wavefront's copies for chunk ci have landed
+      __syncthreads();                               // barrier A
+      if (ci + 1 < n_chunks) issue_copies(ci + 1);
+      form_p(ci);
+      __syncthreads();                               // barrier B
+      if (ci + 1 < n_chunks) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { raw[j] = raw_next[j]; inv[j] = inv_next[j]; }
+        if (ci + 2 < n_chunks) load_rows(ci + 2, raw_next, inv_next);
+        write_rows(ci + 1, raw, inv);
+      }
+    }
+    return;
+  }
+
+  // ---- the computing wavefronts ----
+  const int vbase = 32 * wave;
+  const int vcol = vbase + r16;
+  f32x4_t St[NB][8];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb)
+    if (role.init != nullptr) {
+      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) {
+        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
+        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
+      }
+    } else {
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  if (role.keep_init != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+  uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.HV + hv) * 128 + vbase + 4 * kb;
+  const int rowA128 = r16 * PITCH128, rowA64 = r16 * PITCH64;
+  const int trV = (4 * kb + (r16 >> 2)) * PITCH128 + vbase + 4 * (r16 & 3);
+  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+
+  auto pk = [](float x, float y) { return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x, y)); };
+  auto pk_sat = [](float x, float y) {
+    const f32x2_t c = {__builtin_amdgcn_fmed3f(x, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(y, -65504.f, 65504.f)};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(c, f16x2_t));
+  };
+  // hi = nearest after a clamp, lo = the rest toward zero
+  auto pk_pair = [](float x, float y) {
+    const f32x2_t c = {__builtin_amdgcn_fmed3f(x, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(y, -65504.f, 65504.f)};
+    const f16x2_t hh = __builtin_convertvector(c, f16x2_t);
+    return make_uint2(__builtin_bit_cast(uint32_t, hh),
+                      __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x - (float)hh[0], y - (float)hh[1])));
+  };
+  auto op = [](u32x4_t w) { return __builtin_bit_cast(bf16x8_t, w); };
+
+  // One chunk.  FULL: all 64 rows are tokens (no store masks).
+  auto chunk = [&](int ci, auto full_tag) __attribute__((always_inline)) {
+    constexpr bool FULL = decltype(full_tag)::value;
+    const int par = ci & 1;
+    const uint16_t* const K = tK[par];
+    const uint16_t* const Q = tQ[par];
+    const uint16_t* const V = tV[par];
+    const uint16_t* const Wt = tW[par];
+    const uint16_t* const Pt = tP;
+    const float* const G = tG[par];
+    auto ldK = [&](int j) { return operand_from(K + 16 * (j & 3) * PITCH128 + rowA128, j >> 2, kb); };
+    auto ldQ = [&](int j) { return operand_from(Q + 16 * (j & 3) * PITCH128 + rowA128, j >> 2, kb); };
+    // W operands in the order they are used: 0-3 lo (s 0, m 0..3), 4-7 hi (s 0), 8-9 lo (s 1, m 2, 3), 10-11 hi (s 1);
+    // block b = m for s 0, 4 and 5 for s 1 (tri_block_m / tri_block_s), hi blocks first in the tile, then lo
+    auto w_blk = [](int w) { return w < 8 ? (w & 3) : 4 + (w & 1); };
+    auto w_mi = [](int w) { return tri_block_m(w < 8 ? (w & 3) : 4 + (w & 1)); };
+    auto w_s = [](int w) { return w < 8 ? 0 : 1; };
+    auto ldW = [&](int w) {
+      const bool lo = (w < 4) || (w == 8) || (w == 9);
+      return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(Wt + ((lo ? TRI_BLOCKS : 0) + w_blk(w)) * 512 + lane * 8));
+    };
+    // P operands: block i (token rows tri_block_m(i), contraction half tri_block_s(i))
+    auto p_ni = [](int i) { return tri_block_m(i); };
+    auto p_s = [](int i) { return tri_block_s(i); };
+    auto ldP = [&](int i) { return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(Pt + i * 512 + lane * 8)); };
+
+    // ================= phase 1: KS = K S^T =================
+    bf16x8_t ka[16];
+    u32x4_t sb[4][NB];
+#pragma unroll
+    for (int j = 0; j < 6; ++j) ka[j] = ldK(j);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      sb[0][nb] = u32x4_t{pk(St[nb][0][0], St[nb][0][1]), pk(St[nb][0][2], St[nb][0][3]), pk(St[nb][1][0], St[nb][1][1]),
+                          pk(St[nb][1][2], St[nb][1][3])};
+    SB();
+    f32x4_t KS[NB][4];
+    uint2 vraw[4][NB];
+    float4 eg[4];
+    float sq[4], egl;
+    bf16x8_t qa[16];
+    u32x4_t sq_[4][NB];          // the state operands again for the query product
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int s = j >> 2, mi = j & 3;
+      if (j + 6 < 16) ka[j + 6] = ldK(j + 6);
+      else if (j == 10) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) { vraw[0][nb] = read_tr4(V + trV + 16 * nb); vraw[1][nb] = read_tr4(V + trV + 16 * PITCH128 + 16 * nb); }
+      } else if (j == 11) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) { vraw[2][nb] = read_tr4(V + trV + 32 * PITCH128 + 16 * nb); vraw[3][nb] = read_tr4(V + trV + 48 * PITCH128 + 16 * nb); }
+      } else if (j == 12) {
+#pragma unroll
+        for (int m2 = 0; m2 < 4; ++m2) eg[m2] = *reinterpret_cast<const float4*>(&G[64 + 16 * m2 + 4 * kb]);
+#pragma unroll
+        for (int ni = 0; ni < 4; ++ni) sq[ni] = G[16 * ni + r16];
+        egl = G[192];
+      } else {
+        qa[2 * (j - 13)] = ldQ(2 * (j - 13));
+        qa[2 * (j - 13) + 1] = ldQ(2 * (j - 13) + 1);
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        KS[nb][mi] = mfma16h(ka[j], op(sb[s][nb]), s == 0 ? zero4 : KS[nb][mi]);
+      if (s < 3) {
+        // dword mi of the next step's state operands
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const f32x4_t src = St[nb][2 * s + 2 + (mi >> 1)];
+          sb[s + 1][nb][mi] = (mi & 1) ? pk(src[2], src[3]) : pk(src[0], src[1]);
+        }
+      } else {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const f32x4_t src = St[nb][mi >> 1];
+          sq_[0][nb][mi] = (mi & 1) ? pk(src[2], src[3]) : pk(src[0], src[1]);
+        }
+      }
+      SB();
+    }
+
+    // ================= phase 2a: O^T = S Q^T (query product) under X = V - e^G (.) KS =================
+    f32x4_t OT[NB][4];
+    bf16x8_t wq[12];
+    u32x4_t xb[2][NB];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int s = j >> 2, ni = j & 3;
+      if (j + 6 < 16) qa[j + 6] = ldQ(j + 6);
+      else wq[j - 10] = ldW(j - 10);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        OT[nb][ni] = mfma16h(op(sq_[s][nb]), qa[j], s == 0 ? zero4 : OT[nb][ni]);
+      if (s < 3) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const f32x4_t src = St[nb][2 * s + 2 + (ni >> 1)];
+          sq_[s + 1][nb][ni] = (ni & 1) ? pk(src[2], src[3]) : pk(src[0], src[1]);
+        }
+      }
+      {
+        // half an X tile: tile t = (mi, nb), elements 2 h, 2 h + 1
+        const int t = j >> 1, mi = t >> 1, nb = t & 1, hh = j & 1;
+        const uint32_t w = hh ? vraw[mi][nb].y : vraw[mi][nb].x;
+        const float v0 = lo16<act_t>(w), v1 = hi16<act_t>(w);
+        const float e0 = hh ? eg[mi].z : eg[mi].x, e1 = hh ? eg[mi].w : eg[mi].y;
+        const float x0 = v0 - e0 * KS[nb][mi][2 * hh], x1 = v1 - e1 * KS[nb][mi][2 * hh + 1];
+        xb[mi >> 1][nb][2 * (mi & 1) + hh] = pk_sat(x0, x1);
+      }
+      SB();
+    }
+
+    // P of this chunk is complete (the other four wavefronts formed it while phases 1 and 2a ran)
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    SB();
+    // ================= phase 2b: U = W X (lower triangular W: 6 of the 8 operand blocks) =================
+    f32x4_t U[NB][4];
+    bf16x8_t pa[6];
+    float4 dg[2][2];
+#pragma unroll
+    for (int w = 0; w < 12; ++w) {
+      const int s = w_s(w), mi = w_mi(w);
+      if (w + 6 < 12) wq[w + 6] = ldW(w + 6);
+      else if (w == 6) { pa[0] = ldP(0); pa[1] = ldP(1); }
+      else if (w == 7) { pa[2] = ldP(2); pa[3] = ldP(3); }
+      else if (w == 8) { pa[4] = ldP(4); pa[5] = ldP(5); }
+      else if (w == 9) {
+        dg[0][0] = *reinterpret_cast<const float4*>(&G[128 + 4 * kb]);
+        dg[0][1] = *reinterpret_cast<const float4*>(&G[128 + 16 + 4 * kb]);
+        dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
+        dg[1][1] = *reinterpret_cast<const float4*>(&G[128 + 48 + 4 * kb]);
+      }
+      const bool first = w < 4;        // first product into this accumulator (lo, s 0)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        U[nb][mi] = mfma16h(wq[w], op(xb[s][nb]), first ? zero4 : U[nb][mi]);
+      // VALU underneath: the query product scaled by scale e^G (w 0..5), then the decay of the first half of S
+      if (w < 4) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) OT[nb][w] *= sq[w];
+      } else {
+        const int mc = (w - 4) >> 1, nb = (w - 4) & 1;      // (mc, nb) for w = 4..11 -> mc 0..3
+        St[nb][mc] *= egl;
+      }
+      SB();
+    }
+
+    // ================= phase 3: O^T += U^T P^T (6 operand blocks), under the hi/lo split of e^{G_last - G} (.) U =================
+    u32x4_t ur[2][NB];
+    u32x4_t ubh[2][NB], ubl[2][NB];
+    bf16x8_t kt[16];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      ur[0][nb] = u32x4_t{pk(U[nb][0][0], U[nb][0][1]), pk(U[nb][0][2], U[nb][0][3]), pk(U[nb][1][0], U[nb][1][1]), pk(U[nb][1][2], U[nb][1][3])};
+      ur[1][nb] = u32x4_t{pk(U[nb][2][0], U[nb][2][1]), pk(U[nb][2][2], U[nb][2][3]), pk(U[nb][3][0], U[nb][3][1]), pk(U[nb][3][2], U[nb][3][3])};
+    }
+    SB();
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+      const int s = p_s(i), ni = p_ni(i);
+      if (i >= 2) kt[i - 2] = operand_transposed(K, 0, i - 2, kb, r16);       // kt[0..3]: (s 0, mc 0..3)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) OT[nb][ni] = mfma16h(op(ur[s][nb]), pa[i], OT[nb][ni]);
+      if (i < 4) {
+        // ub[0][nb] dword i: from U tile (i >> 1), elements 2 (i & 1), +1
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int tl = i >> 1, e = 2 * (i & 1);
+          const float4 d = dg[0][tl];
+          const float d0 = e ? d.z : d.x, d1 = e ? d.w : d.y;
+          const uint2 hl = pk_pair(U[nb][tl][e] * d0, U[nb][tl][e + 1] * d1);
+          ubh[0][nb][i] = hl.x; ubl[0][nb][i] = hl.y;
+        }
+      } else {
+        // the decay of S, rows mc 4, 5 (both nb) under the last two steps
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) St[nb][i] *= egl;
+      }
+      SB();
+    }
+
+    // ================= phase 4: S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U), output under it =================
+    const int len = FULL ? CHUNK : chunk_len(ci);
+    uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.HV * 128;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int s = k >> 3, mc = k & 7;
+      if (k + 4 < 16) kt[k + 4] = operand_transposed(K, (k + 4) >> 3, (k + 4) & 7, kb, r16);
+      if (k == 0) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) St[nb][6] *= egl;
+      } else if (k == 1) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) St[nb][7] *= egl;
+      }
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) St[nb][mc] = mfma16h(kt[k], op(ubl[s][nb]), St[nb][mc]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) St[nb][mc] = mfma16h(kt[k], op(ubh[s][nb]), St[nb][mc]);
+      if (k >= 2 && k < 6) {
+        // ub[1][nb] dword (k - 2)
+        const int i = k - 2;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const int tl = i >> 1, e = 2 * (i & 1);
+          const float4 d = dg[1][tl];
+          const float d0 = e ? d.z : d.x, d1 = e ? d.w : d.y;
+          const uint2 hl = pk_pair(U[nb][2 + tl][e] * d0, U[nb][2 + tl][e + 1] * d1);
+          ubh[1][nb][i] = hl.x; ubl[1][nb][i] = hl.y;
+        }
+      } else if (k >= 8 && k < 12) {
+        // output rows of token block ni = k - 8
+        const int ni = k - 8;
+        if (FULL || 16 * ni + r16 < len) {
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            const uint2 packed = make_uint2(pack2<act_t>(OT[nb][ni][0], OT[nb][ni][1]), pack2<act_t>(OT[nb][ni][2], OT[nb][ni][3]));
+            *reinterpret_cast<uint2*>(dst + (int64_t)16 * ni * p.HV * 128 + 16 * nb) = packed;
+          }
+        }
+      }
+      SB();
+    }
+  };
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    __builtin_amdgcn_s_waitcnt(0xc07f);              // lgkmcnt(0) only: output stores may stay in flight
+    __builtin_amdgcn_s_barrier();                    // barrier A: the tiles of chunk ci are complete
+    if (ci + 1 < n_chunks || seq_len - ci * CHUNK == CHUNK) chunk(ci, std::true_type{});
+    else chunk(ci, std::false_type{});
+  }
+
+  if (role.fin != nullptr) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
+#pragma unroll
+      for (int mc = 0; mc < 8; ++mc)
+        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
+    }
+  }
+}
+#undef SB
+
 // 16-column V blocks per computing wavefront of gdn_sweep_kernel: 2 = four computing wavefronts (one per SIMD); 1 =
 // eight (two per SIMD, twice the LDS operand traffic) measures the same on config 3 (0.767 against 0.765 ms)
 constexpr int SWEEP_NB = 2;
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, gcum, beta, gtile, W, P;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, kinv, gcum, beta, gtile, W, P;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -926,9 +1538,10 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_sta
   L.chunk_len = take((size_t)L.NC_max * 4);
   L.qn = take((size_t)T * H * 128 * 2);
   L.kn = take((size_t)T * H * 128 * 2);
+  L.kinv = take((size_t)T * H * 4);
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
-  L.gtile = take((size_t)L.NC_max * HV * 256 * 4);
+  L.gtile = take((size_t)L.NC_max * HV * GTILE_FLOATS * 4);
   L.W = take((size_t)L.NC_max * HV * 8192 * 2);
   L.P = take((size_t)L.NC_max * HV * 4096 * 2);
   L.seg_chunks = pick_segment_chunks(T, N, HV);
@@ -1035,6 +1648,7 @@ static int gdn_prefill_run(
   p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
   p.qn = reinterpret_cast<uint16_t*>(ws + L.qn);
   p.kn = reinterpret_cast<uint16_t*>(ws + L.kn);
+  p.kinv = reinterpret_cast<float*>(ws + L.kinv);
   p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
   p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
   p.gtile = reinterpret_cast<float*>(ws + L.gtile);
@@ -1045,6 +1659,8 @@ static int gdn_prefill_run(
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool segmented = L.seg_chunks > 0;
+  // whole sequences with 16-byte aligned q / k rows take the fused sweep (rows normalised and P formed inside it)
+  const bool fused = !segmented && p.qk_rows_16;
   if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
@@ -1072,7 +1688,17 @@ static int gdn_prefill_run(
         const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
         const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
         const dim3 grid((unsigned)L.NC_max * (HV / waves)), block(64 * waves);
-        if (half_act) {
+        if (fused) {
+          if (half_act) {
+            if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 4>), grid, block, 0, ps, p);
+            else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 2>), grid, block, 0, ps, p);
+            else hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 1>), grid, block, 0, ps, p);
+          } else {
+            if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 4>), grid, block, 0, ps, p);
+            else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 2>), grid, block, 0, ps, p);
+            else hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 1>), grid, block, 0, ps, p);
+          }
+        } else if (half_act) {
           if (waves == 4) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 4>), grid, block, 0, ps, p);
           else if (waves == 2) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 2>), grid, block, 0, ps, p);
           else hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 1>), grid, block, 0, ps, p);
@@ -1088,7 +1714,10 @@ static int gdn_prefill_run(
           else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
         } else {
           const unsigned g = xcd_grouped_grid(grid, (unsigned)(HV / H));
-          if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+          if (fused) {
+            if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+            else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
+          } else if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
           else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
         }
       });
