@@ -211,6 +211,12 @@ __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
+// Workgroup barrier that orders LDS traffic only: this wavefront's LDS operations are complete before it arrives
+// and the compiler moves no memory access across it, but vector memory operations (copies, loads, stores that
+// nobody in the workgroup waits for) stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
 __device__ __forceinline__ uint32_t lds_address(const void* ptr) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)ptr;
 }

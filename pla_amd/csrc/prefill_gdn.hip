@@ -1157,11 +1157,12 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
           inv = rsqrtf(row16_allreduce(ss) + 1e-6f);
         }
         if (!p.normalize_qk) inv = 1.f;
+        if (row >= len) inv = 0.f;                   // rows past the end of the sequence are zero
         uint32_t w[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
-          w[e] = row < len ? pack2_rtz(lo16<act_t>(r), hi16<act_t>(r)) : 0u;
+          w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
         }
         *reinterpret_cast<uint4*>(T + row * PITCH128 + 8 * lc) = make_uint4(w[0], w[1], w[2], w[3]);
       }
@@ -1203,25 +1204,28 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       else block(5);
     };
 
-    uint4 raw[8], raw_next[8];
-    float inv[8], inv_next[8];
+    // `raw` holds the rows of the chunk that is written next; the rows after those are requested right after
+    // barrier A (behind the copies, so that the wait for the copies leaves them in flight) into `ahead` and
+    // change over at the end of the iteration.
+    uint4 raw[8], ahead[8];
+    float inv[8], inv_ahead[8];
     if (n_chunks > 0) {
       issue_copies(0);
       load_rows(0, raw, inv);
-      if (n_chunks > 1) load_rows(1, raw_next, inv_next);
       write_rows(0, raw, inv);
+      if (n_chunks > 1) load_rows(1, raw, inv);
     }
     for (int ci = 0; ci < n_chunks; ++ci) {
       wait_vmcnt<0>();                               // this wavefront's copies for chunk ci have landed
-      __syncthreads();                               // barrier A
+      lds_barrier();                                 // barrier A (the rows this wavefront wrote are in LDS)
       if (ci + 1 < n_chunks) issue_copies(ci + 1);
+      if (ci + 2 < n_chunks) load_rows(ci + 2, ahead, inv_ahead);
       form_p(ci);
-      __syncthreads();                               // barrier B
-      if (ci + 1 < n_chunks) {
+      lds_barrier();                                 // barrier B (P is in LDS; copies and loads stay in flight)
+      if (ci + 1 < n_chunks) write_rows(ci + 1, raw, inv);
+      if (ci + 2 < n_chunks) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { raw[j] = raw_next[j]; inv[j] = inv_next[j]; }
-        if (ci + 2 < n_chunks) load_rows(ci + 2, raw_next, inv_next);
-        write_rows(ci + 1, raw, inv);
+        for (int j = 0; j < 8; ++j) { raw[j] = ahead[j]; inv[j] = inv_ahead[j]; }
       }
     }
     return;
