@@ -1055,9 +1055,10 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 // compute as in gdn_sweep_kernel (32 V columns of S^T each, the chain K S^T -> X -> U -> S^T in registers).
 // Wavefronts 4-7 feed them, so that neither the normalised rows nor P cross memory:
 //   rows   wavefronts 4, 5 take the raw K rows of the next chunk (32 rows each), 6, 7 the raw Q rows: loaded one
-//          chunk ahead into registers (16 lanes per row, 16 bytes per lane), scaled by the row's 1 / |k| (from the
-//          preparation kernel, so that both kernels round the very same normalised keys) or 1 / |q| (summed here),
-//          rounded to the activation dtype, and written to the LDS tiles as fp16
+//          chunk ahead into registers (16 lanes per row, 16 bytes per lane).  K rows are scaled by the row's 1 / |k|
+//          (from the preparation kernel, so that both kernels round the very same normalised keys), rounded to the
+//          activation dtype and written to the LDS tile as fp16.  Q only enters the output, so its rows are written
+//          unscaled and 1 / |q| (summed here) joins the row factors of the output and of P instead
 //   P      scale tril(q_i . k_j e^{G_i - G_j}) of the current chunk from those tiles: the products are formed
 //          transposed (A = K rows, B = Q rows), which leaves a lane with four consecutive j of one token i, i.e. with
 //          8 of the 16 bytes it owns in the six-block operand layout (prefill_common.h) that phase 3 reads
@@ -1094,6 +1095,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
   // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}, [256,320) G
   __shared__ __align__(16) float tG[2][512];
+  __shared__ __align__(16) float tRq[2][CHUNK];        // 1 / |q| per row of the Q tile
 
   if (wave >= CW) {
     // ---- the feeding wavefronts ----
@@ -1138,7 +1140,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
         inv[j] = q_side ? 0.f : kinv[(int64_t)t * p.H];
       }
     };
-    // normalise, round to the activation dtype, write as fp16 into the tile of chunk c
+    // K rows: scaled by 1 / |k|, rounded to the activation dtype (the operand of the reference), written as fp16,
+    // which holds those values exactly; rows past the end of the sequence are zero.  Q rows feed the output only:
+    // they are written as they are (fp16 of the raw value) and 1 / |q| goes to tRq, from where it enters the
+    // output through the row factor scale e^G and P through its row factor.
     auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
       uint16_t* const T = q_side ? tQ[c & 1] : tK[c & 1];
       const int len = chunk_len(c);
@@ -1146,23 +1151,25 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       for (int j = 0; j < 8; ++j) {
         const int row = row0 + 4 * j + lr;
         const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-        float inv = inv_in[j];
+        uint32_t w[4];
         if (q_side) {
           float ss = 0.f;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float a0 = lo16<act_t>(in[e]), a1 = hi16<act_t>(in[e]);
             ss += a0 * a0 + a1 * a1;
+            w[e] = pack2_rtz(a0, a1);
           }
-          inv = rsqrtf(row16_allreduce(ss) + 1e-6f);
-        }
-        if (!p.normalize_qk) inv = 1.f;
-        if (row >= len) inv = 0.f;                   // rows past the end of the sequence are zero
-        uint32_t w[4];
+          const float rq = p.normalize_qk ? rsqrtf(row16_allreduce(ss) + 1e-6f) : 1.f;
+          if (lc == 0) tRq[c & 1][row] = rq;
+        } else {
+          float inv = p.normalize_qk ? inv_in[j] : 1.f;
+          if (row >= len) inv = 0.f;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
-          w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
+            w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
+          }
         }
         *reinterpret_cast<uint4*>(T + row * PITCH128 + 8 * lc) = make_uint4(w[0], w[1], w[2], w[3]);
       }
@@ -1179,6 +1186,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
         for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_from(Q + (16 * ni + r16) * PITCH128, s2, kb);
         const float Gi = G[16 * ni + r16];
         const int i = 16 * ni + r16;
+        const float pre = p.scale * tRq[c & 1][i];
         uint32_t w[4];
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -1189,19 +1197,20 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
           for (int s2 = 0; s2 < 4; ++s2) acc = mfma16h(operand_from(K + (16 * nj + r16) * PITCH128, s2, kb), qb[s2], acc);
           const float4 Gj = *reinterpret_cast<const float4*>(&G[16 * nj + 4 * kb]);
           const int j0 = 16 * nj + 4 * kb;
-          const float p0 = j0 <= i ? p.scale * acc[0] * __expf(Gi - Gj.x) : 0.f;
-          const float p1 = j0 + 1 <= i ? p.scale * acc[1] * __expf(Gi - Gj.y) : 0.f;
-          const float p2 = j0 + 2 <= i ? p.scale * acc[2] * __expf(Gi - Gj.z) : 0.f;
-          const float p3 = j0 + 3 <= i ? p.scale * acc[3] * __expf(Gi - Gj.w) : 0.f;
+          const float p0 = j0 <= i ? pre * acc[0] * __expf(Gi - Gj.x) : 0.f;
+          const float p1 = j0 + 1 <= i ? pre * acc[1] * __expf(Gi - Gj.y) : 0.f;
+          const float p2 = j0 + 2 <= i ? pre * acc[2] * __expf(Gi - Gj.z) : 0.f;
+          const float p3 = j0 + 3 <= i ? pre * acc[3] * __expf(Gi - Gj.w) : 0.f;
           w[2 * half] = pack2_rtz(p0, p1);
           w[2 * half + 1] = pack2_rtz(p2, p3);
         }
         *reinterpret_cast<uint4*>(tP + b * 512 + lane * 8) = make_uint4(w[0], w[1], w[2], w[3]);
       };
-      if (a == 0) { block(0); block(3); }
-      else if (a == 1) block(1);
-      else if (a == 2) { block(2); block(4); }
-      else block(5);
+      // three (nj, ni) products on each wavefront of the Q side, two on each of the K side (whose rows cost more)
+      if (a == 0) block(1);
+      else if (a == 1) block(5);
+      else if (a == 2) { block(0); block(3); }
+      else { block(2); block(4); }
     };
 
     // `raw` holds the rows of the chunk that is written next; the rows after those are requested right after
@@ -1331,9 +1340,6 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       } else if (j == 12) {
 #pragma unroll
         for (int m2 = 0; m2 < 4; ++m2) eg[m2] = *reinterpret_cast<const float4*>(&G[64 + 16 * m2 + 4 * kb]);
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni) sq[ni] = G[16 * ni + r16];
-        egl = G[192];
       } else {
         qa[2 * (j - 13)] = ldQ(2 * (j - 13));
         qa[2 * (j - 13) + 1] = ldQ(2 * (j - 13) + 1);
@@ -1367,6 +1373,11 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       const int s = j >> 2, ni = j & 3;
       if (j + 6 < 16) qa[j + 6] = ldQ(j + 6);
       else wq[j - 10] = ldW(j - 10);
+      if (j == 8) {
+#pragma unroll
+        for (int n2 = 0; n2 < 4; ++n2) sq[n2] = G[16 * n2 + r16] * tRq[par][16 * n2 + r16];
+        egl = G[192];
+      }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
         OT[nb][ni] = mfma16h(op(sq_[s][nb]), qa[j], s == 0 ? zero4 : OT[nb][ni]);
@@ -1407,8 +1418,6 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       else if (w == 9) {
         dg[0][0] = *reinterpret_cast<const float4*>(&G[128 + 4 * kb]);
         dg[0][1] = *reinterpret_cast<const float4*>(&G[128 + 16 + 4 * kb]);
-        dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
-        dg[1][1] = *reinterpret_cast<const float4*>(&G[128 + 48 + 4 * kb]);
       }
       const bool first = w < 4;        // first product into this accumulator (lo, s 0)
 #pragma unroll
@@ -1467,6 +1476,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       const int s = k >> 3, mc = k & 7;
       if (k + 4 < 16) kt[k + 4] = operand_transposed(K, (k + 4) >> 3, (k + 4) & 7, kb, r16);
       if (k == 0) {
+        dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
+        dg[1][1] = *reinterpret_cast<const float4*>(&G[128 + 48 + 4 * kb]);
+      }
+      if (k == 0) {
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) St[nb][6] *= egl;
       } else if (k == 1) {
@@ -1503,6 +1516,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     }
   };
 
+  wait_vmcnt<0>();                                   // the start state has arrived: no wait for it inside the loop
   for (int ci = 0; ci < n_chunks; ++ci) {
     __builtin_amdgcn_s_waitcnt(0xc07f);              // lgkmcnt(0) only: output stores may stay in flight
     __builtin_amdgcn_s_barrier();                    // barrier A: the tiles of chunk ci are complete
