@@ -1098,145 +1098,179 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   __shared__ __align__(16) float tRq[2][CHUNK];        // 1 / |q| per row of the Q tile
 
   if (wave >= CW) {
-    // ---- the feeding wavefronts ----
-    const int a = wave - CW;
-    const bool q_side = a >= 2;
-    const int row0 = 32 * (a & 1);                      // this wavefront's rows of a chunk: row0 .. row0 + 31
-    const int lr = lane >> 4, lc = lane & 15;           // piece j: row row0 + 4 j + lr, columns 8 lc .. 8 lc + 7
-    const int64_t row_pitch = q_side ? p.stride_q : p.stride_k;
-    const uint16_t* const rows = reinterpret_cast<const uint16_t*>(q_side ? p.q : p.k) + (int64_t)seq_start * row_pitch + h * 128 + 8 * lc;
-    const float* const kinv = p.kinv + (int64_t)seq_start * p.H + h;
-    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-    const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * (2 * TRI_BLOCKS * 1024);
-    const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * (GTILE_FLOATS * 4);
-    CopyV plan_v;
-    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, a, lane);
+    // ---- the feeding wavefronts: one instance of this code per wavefront (its role is a compile-time constant) ----
+    auto feed = [&](auto role_tag) __attribute__((always_inline)) {
+      constexpr int a = decltype(role_tag)::value;
+      constexpr bool q_side = a >= 2;
+      constexpr int row0 = 32 * (a & 1);                  // this wavefront's rows of a chunk: row0 .. row0 + 31
+      const int lr = lane >> 4, lc = lane & 15;           // piece j: row row0 + 4 j + lr, columns 8 lc .. 8 lc + 7
+      const int64_t row_pitch = q_side ? p.stride_q : p.stride_k;
+      // bases of the sequence part (wave-uniform, 64-bit) and offsets inside a chunk (per lane, 32-bit)
+      const char* const rows_b = reinterpret_cast<const char*>(q_side ? p.q : p.k) + ((int64_t)seq_start * row_pitch + h * 128) * 2;
+      const char* const kinv_b = reinterpret_cast<const char*>(p.kinv + (int64_t)seq_start * p.H + h);
+      const int64_t chunk_pitch_b = (int64_t)CHUNK * row_pitch * 2;
+      const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
+      const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * (2 * TRI_BLOCKS * 1024);
+      const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * (GTILE_FLOATS * 4);
+      CopyV plan_v;
+      plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, a, lane);
 
-    // global -> LDS copies of chunk c (its buffers are free): V, W and the decay-factor tile
-    auto issue_copies = [&](int c) {
-      const int par = c & 1;
-      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
-      const int len = chunk_len(c);
-      if (len == CHUNK) plan_v.issue(tV[par], vs, a);
-      else {                                           // rows past the sequence end re-read its last row
-        CopyV tail;
-        tail.plan((uint32_t)(p.stride_v * 2), len - 1, a, lane);
-        tail.issue(tV[par], vs, a);
-      }
-      const char* ws = w_b + (int64_t)c * p.HV * (2 * TRI_BLOCKS * 1024);
-#pragma unroll
-      for (int j = 0; j < 2 * TRI_BLOCKS / AUX; ++j)
-        dma16(ws, 1024u * (AUX * j + a) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (AUX * j + a));
-      const char* gs = gt_b + (int64_t)c * p.HV * (GTILE_FLOATS * 4);
-      if (a == 1) dma16(gs, 16u * lane, lds_address(&tG[par][0]));
-      if (a == 2) dma16(gs, 1024u + 16u * (lane & 15), lds_address(&tG[par][256]));     // 64 floats; lanes 16-63 repeat them
-    };
-    // raw rows of chunk c into registers (rows past the end of the sequence part re-read its last row)
-    auto load_rows = [&](int c, uint4 (&raw)[8], float (&inv)[8]) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int t = min(c * CHUNK + row0 + 4 * j + lr, seq_len - 1);
-        raw[j] = *reinterpret_cast<const uint4*>(rows + (int64_t)t * row_pitch);
-        inv[j] = q_side ? 0.f : kinv[(int64_t)t * p.H];
-      }
-    };
-    // K rows: scaled by 1 / |k|, rounded to the activation dtype (the operand of the reference), written as fp16,
-    // which holds those values exactly; rows past the end of the sequence are zero.  Q rows feed the output only:
-    // they are written as they are (fp16 of the raw value) and 1 / |q| goes to tRq, from where it enters the
-    // output through the row factor scale e^G and P through its row factor.
-    auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
-      uint16_t* const T = q_side ? tQ[c & 1] : tK[c & 1];
-      const int len = chunk_len(c);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int row = row0 + 4 * j + lr;
-        const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-        uint32_t w[4];
-        if (q_side) {
-          float ss = 0.f;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float a0 = lo16<act_t>(in[e]), a1 = hi16<act_t>(in[e]);
-            ss += a0 * a0 + a1 * a1;
-            w[e] = pack2_rtz(a0, a1);
-          }
-          const float rq = p.normalize_qk ? rsqrtf(row16_allreduce(ss) + 1e-6f) : 1.f;
-          if (lc == 0) tRq[c & 1][row] = rq;
-        } else {
-          float inv = p.normalize_qk ? inv_in[j] : 1.f;
-          if (row >= len) inv = 0.f;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
-            w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
-          }
+      // global -> LDS copies of chunk c (its buffers are free): V, W and the decay-factor tile
+      auto issue_copies = [&](int c) {
+        const int par = c & 1;
+        const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+        const int len = chunk_len(c);
+        if (len == CHUNK) plan_v.issue(tV[par], vs, a);
+        else {                                           // rows past the sequence end re-read its last row
+          CopyV tail;
+          tail.plan((uint32_t)(p.stride_v * 2), len - 1, a, lane);
+          tail.issue(tV[par], vs, a);
         }
-        *reinterpret_cast<uint4*>(T + row * PITCH128 + 8 * lc) = make_uint4(w[0], w[1], w[2], w[3]);
-      }
-    };
-    // P of chunk c from its K and Q tiles: this wavefront's blocks of the six
-    auto form_p = [&](int c) {
-      const uint16_t* const K = tK[c & 1];
-      const uint16_t* const Q = tQ[c & 1];
-      const float* const G = &tG[c & 1][256];
-      auto block = [&](int b) {
-        const int ni = tri_block_m(b), s = tri_block_s(b);
-        bf16x8_t qb[4];
+        const char* ws = w_b + (int64_t)c * p.HV * (2 * TRI_BLOCKS * 1024);
 #pragma unroll
-        for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_from(Q + (16 * ni + r16) * PITCH128, s2, kb);
-        const float Gi = G[16 * ni + r16];
-        const int i = 16 * ni + r16;
-        const float pre = p.scale * tRq[c & 1][i];
-        uint32_t w[4];
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int nj = 2 * s + half;
-          if (nj > ni) { w[2 * half] = 0u; w[2 * half + 1] = 0u; continue; }
-          f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-          for (int s2 = 0; s2 < 4; ++s2) acc = mfma16h(operand_from(K + (16 * nj + r16) * PITCH128, s2, kb), qb[s2], acc);
-          const float4 Gj = *reinterpret_cast<const float4*>(&G[16 * nj + 4 * kb]);
-          const int j0 = 16 * nj + 4 * kb;
-          const float p0 = j0 <= i ? pre * acc[0] * __expf(Gi - Gj.x) : 0.f;
-          const float p1 = j0 + 1 <= i ? pre * acc[1] * __expf(Gi - Gj.y) : 0.f;
-          const float p2 = j0 + 2 <= i ? pre * acc[2] * __expf(Gi - Gj.z) : 0.f;
-          const float p3 = j0 + 3 <= i ? pre * acc[3] * __expf(Gi - Gj.w) : 0.f;
-          w[2 * half] = pack2_rtz(p0, p1);
-          w[2 * half + 1] = pack2_rtz(p2, p3);
-        }
-        *reinterpret_cast<uint4*>(tP + b * 512 + lane * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+        for (int j = 0; j < 2 * TRI_BLOCKS / AUX; ++j)
+          dma16(ws, 1024u * (AUX * j + a) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (AUX * j + a));
+        const char* gs = gt_b + (int64_t)c * p.HV * (GTILE_FLOATS * 4);
+        if (a == 1) dma16(gs, 16u * lane, lds_address(&tG[par][0]));
+        if (a == 2) dma16(gs, 1024u + 16u * (lane & 15), lds_address(&tG[par][256]));   // 64 floats; lanes 16-63 repeat them
       };
-      // three (nj, ni) products on each wavefront of the Q side, two on each of the K side (whose rows cost more)
-      if (a == 0) block(1);
-      else if (a == 1) block(5);
-      else if (a == 2) { block(0); block(3); }
-      else { block(2); block(4); }
-    };
-
-    // `raw` holds the rows of the chunk that is written next; the rows after those are requested right after
-    // barrier A (behind the copies, so that the wait for the copies leaves them in flight) into `ahead` and
-    // change over at the end of the iteration.
-    uint4 raw[8], ahead[8];
-    float inv[8], inv_ahead[8];
-    if (n_chunks > 0) {
-      issue_copies(0);
-      load_rows(0, raw, inv);
-      write_rows(0, raw, inv);
-      if (n_chunks > 1) load_rows(1, raw, inv);
-    }
-    for (int ci = 0; ci < n_chunks; ++ci) {
-      wait_vmcnt<0>();                               // this wavefront's copies for chunk ci have landed
-      lds_barrier();                                 // barrier A (the rows this wavefront wrote are in LDS)
-      if (ci + 1 < n_chunks) issue_copies(ci + 1);
-      if (ci + 2 < n_chunks) load_rows(ci + 2, ahead, inv_ahead);
-      form_p(ci);
-      lds_barrier();                                 // barrier B (P is in LDS; copies and loads stay in flight)
-      if (ci + 1 < n_chunks) write_rows(ci + 1, raw, inv);
-      if (ci + 2 < n_chunks) {
+      // raw rows of chunk c into registers (rows past the end of the sequence part re-read its last row)
+      auto load_rows = [&](int c, uint4 (&raw)[8], float (&inv)[8]) {
+        const char* const cb = rows_b + (int64_t)c * chunk_pitch_b;
+        const char* const ib = kinv_b + (int64_t)c * CHUNK * p.H * 4;
+        const int last = seq_len - 1 - c * CHUNK;          // last valid row of this chunk (>= 63 for a full one)
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { raw[j] = ahead[j]; inv[j] = inv_ahead[j]; }
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t row = (uint32_t)min(row0 + 4 * j + lr, last);
+          raw[j] = *reinterpret_cast<const uint4*>(cb + row * (uint32_t)(row_pitch * 2) + 16u * lc);
+          inv[j] = q_side ? 0.f : *reinterpret_cast<const float*>(ib + row * (uint32_t)(p.H * 4));
+        }
+      };
+      // K rows: scaled by 1 / |k|, rounded to the activation dtype (the operand of the reference), written as fp16,
+      // which holds those values exactly; rows past the end of the sequence are zero.  Q rows feed the output only:
+      // they are written as they are (fp16 of the raw value) and 1 / |q| goes to tRq, from where it enters the
+      // output through the row factor scale e^G and P through its row factor.
+      auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
+        uint16_t* const T = (q_side ? tQ[c & 1] : tK[c & 1]) + (row0 + lr) * PITCH128 + 8 * lc;
+        const int len = chunk_len(c);
+        const float on = p.normalize_qk ? 1.f : 0.f;
+        if constexpr (q_side) {
+          float ss[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+            uint32_t w[4];
+            float acc = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float a0 = lo16<act_t>(in[e]), a1 = hi16<act_t>(in[e]);
+              acc += a0 * a0 + a1 * a1;
+              w[e] = pack2_rtz(a0, a1);
+            }
+            ss[j] = acc;
+            *reinterpret_cast<uint4*>(T + 4 * j * PITCH128) = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ss[j] = row16_allreduce(ss[j]);
+          float* const rq = &tRq[c & 1][row0 + lr];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const float r = rsqrtf(ss[j] + 1e-6f);
+            if (lc == 0) rq[4 * j] = on * r + (1.f - on);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+            float inv = on * inv_in[j] + (1.f - on);
+            inv = row0 + 4 * j + lr < len ? inv : 0.f;
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
+              w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
+            }
+            *reinterpret_cast<uint4*>(T + 4 * j * PITCH128) = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+        }
+      };
+      // P of chunk c from its K and Q tiles: this wavefront's blocks of the six
+      auto form_p = [&](int c) {
+        const uint16_t* const K = tK[c & 1];
+        const uint16_t* const Q = tQ[c & 1];
+        const float* const G = &tG[c & 1][256];
+        auto block = [&](auto b_tag) {
+          constexpr int b = decltype(b_tag)::value;
+          constexpr int ni = tri_block_m(b), s = tri_block_s(b);
+          constexpr int halves = 2 * s + 1 > ni ? 1 : 2;        // (nj, ni) products of this block that are not all zero
+          bf16x8_t qb[4], kb_op[halves][4];
+#pragma unroll
+          for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_from(Q + (16 * ni + r16) * PITCH128, s2, kb);
+#pragma unroll
+          for (int half = 0; half < halves; ++half)
+#pragma unroll
+            for (int s2 = 0; s2 < 4; ++s2) kb_op[half][s2] = operand_from(K + (16 * (2 * s + half) + r16) * PITCH128, s2, kb);
+          const int i = 16 * ni + r16;
+          const float Gi = G[i];
+          const float pre = p.scale * tRq[c & 1][i];
+          float4 Gj[halves];
+#pragma unroll
+          for (int half = 0; half < halves; ++half) Gj[half] = *reinterpret_cast<const float4*>(&G[16 * (2 * s + half) + 4 * kb]);
+          f32x4_t acc[halves];
+#pragma unroll
+          for (int half = 0; half < halves; ++half) acc[half] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s2 = 0; s2 < 4; ++s2)
+#pragma unroll
+            for (int half = 0; half < halves; ++half) acc[half] = mfma16h(kb_op[half][s2], qb[s2], acc[half]);
+          uint32_t w[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+          for (int half = 0; half < halves; ++half) {
+            const int j0 = 16 * (2 * s + half) + 4 * kb;
+            const float p0 = j0 <= i ? pre * acc[half][0] * __expf(Gi - Gj[half].x) : 0.f;
+            const float p1 = j0 + 1 <= i ? pre * acc[half][1] * __expf(Gi - Gj[half].y) : 0.f;
+            const float p2 = j0 + 2 <= i ? pre * acc[half][2] * __expf(Gi - Gj[half].z) : 0.f;
+            const float p3 = j0 + 3 <= i ? pre * acc[half][3] * __expf(Gi - Gj[half].w) : 0.f;
+            w[2 * half] = pack2_rtz(p0, p1);
+            w[2 * half + 1] = pack2_rtz(p2, p3);
+          }
+          *reinterpret_cast<uint4*>(tP + b * 512 + lane * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+        };
+        // three (nj, ni) products on each wavefront of the Q side, two on each of the K side (whose rows cost more)
+        if constexpr (a == 0) block(std::integral_constant<int, 1>{});
+        else if constexpr (a == 1) block(std::integral_constant<int, 5>{});
+        else if constexpr (a == 2) { block(std::integral_constant<int, 0>{}); block(std::integral_constant<int, 3>{}); }
+        else { block(std::integral_constant<int, 2>{}); block(std::integral_constant<int, 4>{}); }
+      };
+
+      // `raw` holds the rows of the chunk that is written next; the rows after those are requested right after
+      // barrier A (behind the copies) into `ahead` and change over at the end of the iteration.
+      uint4 raw[8], ahead[8];
+      float inv[8], inv_ahead[8];
+      if (n_chunks > 0) {
+        issue_copies(0);
+        load_rows(0, raw, inv);
+        write_rows(0, raw, inv);
+        if (n_chunks > 1) load_rows(1, raw, inv);
       }
-    }
+      for (int ci = 0; ci < n_chunks; ++ci) {
+        wait_vmcnt<0>();                               // this wavefront's copies for chunk ci have landed
+        lds_barrier();                                 // barrier A (the rows this wavefront wrote are in LDS)
+        if (ci + 1 < n_chunks) issue_copies(ci + 1);
+        if (ci + 2 < n_chunks) load_rows(ci + 2, ahead, inv_ahead);
+        form_p(ci);
+        lds_barrier();                                 // barrier B (P is in LDS; copies and loads stay in flight)
+        if (ci + 1 < n_chunks) write_rows(ci + 1, raw, inv);
+        if (ci + 2 < n_chunks) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) { raw[j] = ahead[j]; inv[j] = inv_ahead[j]; }
+        }
+      }
+    };
+    if (wave == CW) feed(std::integral_constant<int, 0>{});
+    else if (wave == CW + 1) feed(std::integral_constant<int, 1>{});
+    else if (wave == CW + 2) feed(std::integral_constant<int, 2>{});
+    else feed(std::integral_constant<int, 3>{});
     return;
   }
 
