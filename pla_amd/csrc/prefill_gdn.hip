@@ -1064,7 +1064,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 //          8 of the 16 bytes it owns in the six-block operand layout (prefill_common.h) that phase 3 reads
 //   copies V, W (12 KiB, six-block layout, hi then lo) and the decay-factor tile by global -> LDS copies
 // Two barriers per chunk: A opens the chunk (all tiles of it are complete, those of the chunk before are free),
-// B follows the query product (P is complete).  The computing wavefronts run a hand-ordered schedule: every LDS
+// B precedes the product with P (P is complete).  The computing wavefronts run a hand-ordered schedule: every LDS
 // operand is requested a fixed number of steps before the MFMA that uses it and the VALU work (conversions, X, the
 // hi / lo split of U, the decay of S) is placed under the MFMAs; scheduling barriers keep that order.
 #define SB() __builtin_amdgcn_sched_barrier(0)
@@ -1434,10 +1434,6 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       SB();
     }
 
-    // P of this chunk is complete (the other four wavefronts formed it while phases 1 and 2a ran)
-    __builtin_amdgcn_s_waitcnt(0xc07f);
-    __builtin_amdgcn_s_barrier();
-    SB();
     // ================= phase 2b: U = W X (lower triangular W: 6 of the 8 operand blocks) =================
     f32x4_t U[NB][4];
     bf16x8_t pa[6];
@@ -1446,9 +1442,6 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     for (int w = 0; w < 12; ++w) {
       const int s = w_s(w), mi = w_mi(w);
       if (w + 6 < 12) wq[w + 6] = ldW(w + 6);
-      else if (w == 6) { pa[0] = ldP(0); pa[1] = ldP(1); }
-      else if (w == 7) { pa[2] = ldP(2); pa[3] = ldP(3); }
-      else if (w == 8) { pa[4] = ldP(4); pa[5] = ldP(5); }
       else if (w == 9) {
         dg[0][0] = *reinterpret_cast<const float4*>(&G[128 + 4 * kb]);
         dg[0][1] = *reinterpret_cast<const float4*>(&G[128 + 16 + 4 * kb]);
@@ -1469,6 +1462,14 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     }
 
     // ================= phase 3: O^T += U^T P^T (6 operand blocks), under the hi/lo split of e^{G_last - G} (.) U =================
+    // Barrier B: P of this chunk is complete (the other four wavefronts formed it while phases 1 to 2b ran, which
+    // take them about as long); its operands are requested at once and arrive under the conversions of U.
+    __builtin_amdgcn_s_waitcnt(0xc07f);
+    __builtin_amdgcn_s_barrier();
+    SB();
+#pragma unroll
+    for (int i = 0; i < TRI_BLOCKS; ++i) pa[i] = ldP(i);
+    SB();
     u32x4_t ur[2][NB];
     u32x4_t ubh[2][NB], ubl[2][NB];
     bf16x8_t kt[16];
@@ -1505,10 +1506,17 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     // ================= phase 4: S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U), output under it =================
     const int len = FULL ? CHUNK : chunk_len(ci);
     uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.HV * 128;
+    // The K^T operands go through in pairs: the lo products of both, then the hi products, so that two products into
+    // the same accumulator are four MFMAs apart (the accumulator changes registers between them, which makes the
+    // second wait for the first to retire).  Step k handles pair k / 2: even k the lo products, odd k the hi ones.
 #pragma unroll
     for (int k = 0; k < 16; ++k) {
-      const int s = k >> 3, mc = k & 7;
-      if (k + 4 < 16) kt[k + 4] = operand_transposed(K, (k + 4) >> 3, (k + 4) & 7, kb, r16);
+      const int pair = k >> 1, s = pair >> 2, mc0 = 2 * (pair & 3);
+      const bool hi_part = k & 1;
+      if (!hi_part && 2 * pair + 4 < 16) {
+        kt[2 * pair + 4] = operand_transposed(K, (2 * pair + 4) >> 3, (2 * pair + 4) & 7, kb, r16);
+        kt[2 * pair + 5] = operand_transposed(K, (2 * pair + 5) >> 3, (2 * pair + 5) & 7, kb, r16);
+      }
       if (k == 0) {
         dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
         dg[1][1] = *reinterpret_cast<const float4*>(&G[128 + 48 + 4 * kb]);
@@ -1521,9 +1529,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
         for (int nb = 0; nb < NB; ++nb) St[nb][7] *= egl;
       }
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) St[nb][mc] = mfma16h(kt[k], op(ubl[s][nb]), St[nb][mc]);
+      for (int m2 = 0; m2 < 2; ++m2)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) St[nb][mc] = mfma16h(kt[k], op(ubh[s][nb]), St[nb][mc]);
+        for (int nb = 0; nb < NB; ++nb)
+          St[nb][mc0 + m2] = mfma16h(kt[2 * pair + m2], op(hi_part ? ubh[s][nb] : ubl[s][nb]), St[nb][mc0 + m2]);
       if (k >= 2 && k < 6) {
         // ub[1][nb] dword (k - 2)
         const int i = k - 2;
