@@ -1310,10 +1310,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     const f32x2_t c = {__builtin_amdgcn_fmed3f(x, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(y, -65504.f, 65504.f)};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(c, f16x2_t));
   };
-  // hi = nearest after a clamp, lo = the rest toward zero
+  // hi = x rounded toward zero (which saturates at the largest finite fp16 value by itself), lo = the rest,
+  // again toward zero: hi + lo carries x to about 21 bits
   auto pk_pair = [](float x, float y) {
-    const f32x2_t c = {__builtin_amdgcn_fmed3f(x, -65504.f, 65504.f), __builtin_amdgcn_fmed3f(y, -65504.f, 65504.f)};
-    const f16x2_t hh = __builtin_convertvector(c, f16x2_t);
+    const auto hh = __builtin_amdgcn_cvt_pkrtz(x, y);
     return make_uint2(__builtin_bit_cast(uint32_t, hh),
                       __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x - (float)hh[0], y - (float)hh[1])));
   };
