@@ -252,18 +252,24 @@ def main(argv=None):
     if not torch.cuda.is_available():
         print("a GPU is required to replay a caselist", file=sys.stderr)
         return 2
-    rows = []
-    for case in read_caselist(args.caselist, args.limit):
-        row = replay_case(case, reps=args.reps)
-        rows.append(row)
-        print(row, flush=True)
-        torch.cuda.empty_cache()
-    if args.csv:
-        keys = sorted({k for r in rows for k in r})
-        with open(args.csv, "w", newline="") as fh:
-            writer = csv.DictWriter(fh, fieldnames=keys)
-            writer.writeheader()
-            writer.writerows(rows)
+    # rows are written as they are measured, so that an interrupted replay keeps what it has
+    keys = ["family", "phase", "kind", "batch", "heads", "seqlen_q", "tokens", "us", "tokens_per_s", "state_GBps",
+            "status", "reason"]
+    fh = open(args.csv, "w", newline="") if args.csv else None
+    writer = csv.DictWriter(fh, fieldnames=keys) if fh else None
+    if writer:
+        writer.writeheader()
+    try:
+        for case in read_caselist(args.caselist, args.limit):
+            row = replay_case(case, reps=args.reps)
+            print(row, flush=True)
+            if writer:
+                writer.writerow(row)
+                fh.flush()
+            torch.cuda.empty_cache()
+    finally:
+        if fh:
+            fh.close()
     return 0
 
 
