@@ -44,8 +44,8 @@ def build_decode_sets(w, n_sets, pool_slots, B, pad_frac, seed, device):
     return sets, B - n_pad
 
 
-def bench_decode(steps, warmup, device):
-    import torch
+def prepare_decode(device):
+    """The headline workload (inputs resident in HBM) and the closure that runs one step on slot set i."""
     from pla_amd.decode import fused_sigmoid_gating_delta_rule_forward_k_last_packed as packed
     from pla_amd.workloads import gdn_decode_packed
 
@@ -53,33 +53,45 @@ def bench_decode(steps, warmup, device):
     w = gdn_decode_packed(B, H=H, HV=HV, pool_slots=slots, pad_frac=pad, seed=101, device=device)
     call = {k: v for k, v in w.items() if not k.startswith("_")}
     sets, n_active = build_decode_sets(w, slots // B, slots, B, pad, 11, device)
-    bytes_state = n_active * HV * 131072
 
     def step(i):
         call["initial_state_indices"] = sets[i % len(sets)]
         packed(**call)
 
+    return dict(workload=w, step=step, n_active=n_active, bytes_state=n_active * HV * 131072)
+
+
+def time_decode(prep, steps, warmup):
+    """W untimed warm-up steps, then exactly K timed steps bracketed by synchronisations."""
+    import torch
+    step, bytes_state = prep["step"], prep["bytes_state"]
+    filler = torch.empty(32 << 20, dtype=torch.float32, device=prep["workload"]["mixed_qkv"].device)
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     # The op launches on torch's current stream, so torch events bracket exactly these launches.
     # One event pair around the K back-to-back launches: their mean is the kernel's average
-    # launch duration (rocprofv3 --kernel-trace reports the same average within 2 %).
+    # launch duration (rocprofv3 --kernel-trace reports the same average within 2 %).  A 128 MB fill runs
+    # in front of the start event: while it runs the host enqueues the event and the first steps, so the event's
+    # time stamp is followed at once by the first kernel and the K steps are back to back from the first one on
+    # (with an idle stream the 10-20 us between enqueueing the event and the first launch would be counted, which
+    # is 0.5 % of a 20-step run).  The wall clock below includes the fill.
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    filler.zero_()
     start.record()
     for i in range(steps):
-        step(i)
+        step(warmup + i)
     end.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     avg_kernel_s = start.elapsed_time(end) * 1e-3 / steps
     return dict(
-        wall_s=wall, ms_per_step=wall / steps * 1e3, bytes_state=bytes_state, n_active=n_active,
+        wall_s=wall, ms_per_step=wall / steps * 1e3, bytes_state=bytes_state, n_active=prep["n_active"],
         kernel_us_avg=avg_kernel_s * 1e6,
         achieved_gbps=bytes_state / avg_kernel_s / 1e9,
-        value_gbps=bytes_state * steps / wall / 1e9, workload=w)
+        value_gbps=bytes_state * steps / wall / 1e9, workload=prep["workload"])
 
 
 def bench_decode_bf16_pool(w, steps, device):
@@ -502,7 +514,25 @@ def main():
             result["copy_calibration"] = copy_calibration(device)
         print(json.dumps(result))
         return
-    d = bench_decode(args.steps, args.warmup, device)
+    # Order of the run: the CPU legs and the secondary workloads first, the headline decode last.  The driver's
+    # short runs (5 warm-up steps are under a millisecond of GPU work) then measure the headline on a GPU that has
+    # been busy for a while, as it is in serving, instead of one that has just left idle clocks.
+    prep = prepare_decode(device)
+    cpu_leg = None if args.no_cpu_baseline else cpu_baseline_decode(prep["workload"])
+    extra = {}
+    if not args.decode_only:
+        extra["other_decode"] = bench_small_decode(device)
+        extra["other_decode"].update(bench_decode_bf16_pool(prep["workload"], args.steps, device))
+        extra["decode_mega"] = bench_decode_mega(device)
+        extra["replay_verify"] = bench_replay_verify(device)
+        extra["replay_paged"] = bench_replay_paged(device)
+        torch.cuda.empty_cache()
+        extra["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device, cpu_leg=not args.no_cpu_baseline)
+        torch.cuda.empty_cache()
+        extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 20, 5), device)
+        extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+        torch.cuda.empty_cache()
+    d = time_decode(prep, args.steps, args.warmup)
     result = {
         "metric": "gdn_packed_decode_state_hbm_GBps@B=256",
         "value": round(d["value_gbps"], 1),
@@ -523,23 +553,11 @@ def main():
                                        "(profiles/k_last_decode_kernel_gdn_b256.txt); a constant here, not measured in this run",
                      "kernel": "k_last_decode_kernel<bf16,GDN,rows_per_wave=32>",
                      "bytes_per_launch": d["bytes_state"], "launch_us_avg": round(d["kernel_us_avg"], 2)},
+        "run_order": "CPU baselines and the secondary workloads first, the headline steps last",
     }
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline_decode(d["workload"])
-    bf16_pool = None if args.decode_only else bench_decode_bf16_pool(d["workload"], args.steps, device)
-    del d
-    torch.cuda.empty_cache()
-    if not args.decode_only:
-        result["other_decode"] = bench_small_decode(device)
-        result["other_decode"].update(bf16_pool)
-        result["decode_mega"] = bench_decode_mega(device)
-        result["replay_verify"] = bench_replay_verify(device)
-        result["replay_paged"] = bench_replay_paged(device)
-        torch.cuda.empty_cache()
-        result["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device, cpu_leg=not args.no_cpu_baseline)
-        torch.cuda.empty_cache()
-        result["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 20, 5), device)
-        result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+    if cpu_leg is not None:
+        result["cpu_baseline"] = cpu_leg
+    result.update(extra)
     if args.copy_calibration:
         result["copy_calibration"] = copy_calibration(device)
     print(json.dumps(result))

@@ -264,14 +264,25 @@ struct TileCopy {
 // Single workgroup.  seq_chunk_off[n] = first chunk of sequence n (seq_chunk_off[N] = total).
 __device__ __forceinline__ void chunk_map(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,
                                           int32_t* chunk_seq, int32_t* chunk_tok, int32_t* chunk_len) {
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int n = 0; n < N; ++n) {
-      seq_chunk_off[n] = acc;
-      const int len = max(cu_seqlens[n + 1] - cu_seqlens[n], 0);
-      acc += (len + CHUNK - 1) / CHUNK;
+  // exclusive scan of the chunk counts by the first wavefront, 64 sequences per trip to memory (a serial loop
+  // over the sequences would pay one memory latency per sequence)
+  if (threadIdx.x < 64) {
+    const int lane0 = threadIdx.x;
+    int carry = 0;
+    for (int base = 0; base < N; base += 64) {
+      const int n = base + lane0;
+      int nc = 0;
+      if (n < N) nc = (max(cu_seqlens[n + 1] - cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+      int incl = nc;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane0 >= d) incl += up;
+      }
+      if (n < N) seq_chunk_off[n] = carry + incl - nc;
+      carry += __shfl(incl, 63, 64);
     }
-    seq_chunk_off[N] = acc;
+    if (lane0 == 0) seq_chunk_off[N] = carry;
   }
   __syncthreads();
   // one wavefront per sequence, its lanes stride over the chunks
@@ -469,14 +480,23 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
 
 // Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map.
 __device__ __forceinline__ void segment_map(const int32_t* seq_chunk_off, int N, SegmentTable t) {
-  if (threadIdx.x == 0) {
-    int acc = 0;
-    for (int n = 0; n < N; ++n) {
-      t.seq_seg_off[n] = acc;
-      const int nc = seq_chunk_off[n + 1] - seq_chunk_off[n];
-      acc += (nc + t.seg_chunks - 1) / t.seg_chunks;
+  if (threadIdx.x < 64) {                     // exclusive scan of the segment counts, as in chunk_map
+    const int lane0 = threadIdx.x;
+    int carry = 0;
+    for (int base = 0; base < N; base += 64) {
+      const int n = base + lane0;
+      int ns = 0;
+      if (n < N) ns = (seq_chunk_off[n + 1] - seq_chunk_off[n] + t.seg_chunks - 1) / t.seg_chunks;
+      int incl = ns;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(incl, d, 64);
+        if (lane0 >= d) incl += up;
+      }
+      if (n < N) t.seq_seg_off[n] = carry + incl - ns;
+      carry += __shfl(incl, 63, 64);
     }
-    t.seq_seg_off[N] = acc;
+    if (lane0 == 0) t.seq_seg_off[N] = carry;
   }
   for (int i = threadIdx.x; i < 128 * 128; i += blockDim.x) t.identity[i] = (i >> 7) == (i & 127) ? 1.f : 0.f;
   __syncthreads();

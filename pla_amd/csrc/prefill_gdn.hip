@@ -24,13 +24,19 @@
 //
 // Kernels:
 //   prefill_tables_kernel    chunk / segment / stage tables from cu_seqlens (device side, graph-capturable)
-//   gdn_prepare_kernel       one wavefront per (chunk, value head): gate, beta and their chunk-local cumsum, the
-//                            decay-factor tile, q/k L2 norm (rounded to the activation dtype, stored as fp16),
-//                            K K^T and Q K^T on MFMA, the inverse of I + L by 16 x 16 blocks, W (hi, lo) and P
-//   gdn_sweep_kernel         sequential kernel with output: one workgroup per (sequence, value head) of four
-//                            computing wavefronts (32 V columns of S^T each, in MFMA accumulator layout, the
-//                            chain K S^T -> X -> U -> S^T in registers) and one wavefront that issues every
-//                            global -> LDS copy; all tiles double buffered, one barrier per chunk
+//   gdn_wsolve_kernel        preparation for the fused sweep, one wavefront per (chunk, value head): gate, beta and
+//                            their chunk-local cumsum, the decay-factor tile, normalised K, K K^T on MFMA, the
+//                            inverse of I + L by 16 x 16 blocks, W (hi, lo) in the six-block operand layout
+//   gdn_fused_sweep_kernel   whole sequences with 16-byte aligned q / k rows: one workgroup per (sequence, value
+//                            head) of four computing wavefronts (32 V columns of S^T each, in MFMA accumulator
+//                            layout, the chain K S^T -> X -> U -> S^T in registers) and four feeding wavefronts
+//                            that normalise the raw q / k rows into LDS tiles, form P and issue the global -> LDS
+//                            copies of V, W and the decay factors; two barriers per chunk
+//   gdn_prepare_kernel       preparation for the two kernels below: as gdn_wsolve_kernel, plus the normalised q / k
+//                            rows, Q K^T and P, W row-major (any 4-byte aligned q / k rows)
+//   gdn_sweep_kernel         sequential kernel with output for calls split into segments (second sweep) and for
+//                            q / k rows that are only 4-byte aligned: four computing wavefronts and one that issues
+//                            every global -> LDS copy; all tiles double buffered, one barrier per chunk
 //   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
 //                            segment side by side in one workgroup of eight wavefronts that share every tile
 

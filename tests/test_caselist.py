@@ -8,7 +8,10 @@ import torch
 
 from pla_amd import caselist
 
-SAMPLE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "caselist_sample.list")
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+SAMPLE = os.path.join(GOLDEN, "caselist_sample.list")
+DECODE_HEAD_SHAPES = os.path.join(GOLDEN, "caselist_decode_head_shapes.list")
+PREFILL_EVERY50 = os.path.join(GOLDEN, "caselist_prefill_every50.list")
 
 
 def test_parse_sample_lines():
@@ -28,6 +31,25 @@ def test_parse_sample_lines():
     with pytest.raises(ValueError):
         caselist.parse_case("gdn_attn:seqlen_q:1")
     assert caselist.read_caselist(SAMPLE, limit=3) == cases[:3]
+
+
+def test_full_caselist_fixtures_parse_and_are_served():
+    """The head shapes of every decode caselist and the sampled prefill caselists: every GDN / KDA line parses,
+    and the only decode shapes without an operator here are one-token KDA head counts the fused step does not build."""
+    decode = caselist.read_caselist(DECODE_HEAD_SHAPES)
+    assert len(decode) == 114 and all(c["phase"] == "D" for c in decode)
+    heads = {(c["family"], c["num_heads_qk"], c["num_heads_v"]) for c in decode}
+    assert len([h for h in heads if h[0] == "GDN"]) == 16 and len([h for h in heads if h[0] == "KDA"]) == 11
+    assert {c["seqlen_q"] for c in decode} == {1, 3, 4, 5, 8}
+    unserved = {(c["num_heads_qk"], c["seqlen_q"]) for c in decode if caselist.unsupported_reason(c)}
+    assert unserved == {(3, 1), (32, 1)}
+    from pla_amd.autotune import shapes_from_caselists
+    assert len(shapes_from_caselists([DECODE_HEAD_SHAPES])) == 27
+    prefill = caselist.read_caselist(PREFILL_EVERY50)
+    assert len(prefill) == 943 and all(c["phase"] == "P" for c in prefill)
+    assert all(caselist.unsupported_reason(c) is None for c in prefill)
+    assert all(c["cu_seqlens_q"][0] == 0 and len(c["cu_seqlens_q"]) == c["batch_size"] + 1 for c in prefill)
+    assert max(c["cu_seqlens_q"][-1] for c in prefill) == 32768
 
 
 @pytest.mark.gpu
