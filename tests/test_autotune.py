@@ -100,7 +100,7 @@ def test_library_lookup_matches_the_table():
             assert lib.pla_tuned_rows_per_wave(*key, B) == _nearest(rows, B)
     # a shape the table does not hold: thresholds on B * HV
     for B, want in ((1, 8), (2, 8), (3, 16), (7, 16), (8, 32), (100, 32)):
-        assert lib.pla_tuned_rows_per_wave(1, 0, 1, 0, 8, 64, B) == want
+        assert lib.pla_tuned_rows_per_wave(1, 0, 1, 0, 32, 64, B) == want
     assert lib.pla_tuned_rows_per_wave(7, 0, 1, 0, 16, 32, 8) == 0
     assert lib.pla_tuned_rows_per_wave(1, 0, 1, 0, 16, 32, 0) == 0
 
