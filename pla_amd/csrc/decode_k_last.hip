@@ -42,13 +42,13 @@ struct KLastParams {
   int tuned_kernel;         // host only: which rows of the tuned table apply (TunedKernel)
 };
 
-// READONCE (verify of up to four draft tokens that writes no state, no snapshots and follows no tree):
-// the recurrence is unrolled algebraically instead of being stepped through the state (readonce_verify.h):
-// wavefront t of the workgroup works out the effective query w_t and the coefficients c_{.,t} of token t
-// from K-vectors and publishes them in LDS; the state tile is then used once, as the MFMA A operand of
-// S_0 [w_0 .. w_3].  One workgroup covers a whole tile: RPW is 32 and wavefront w owns rows
+// READONCE > 0 (verify of up to READONCE = 4 or 8 draft tokens that writes no state, no snapshots and follows no
+// tree): the recurrence is unrolled algebraically instead of being stepped through the state (readonce_verify.h):
+// wavefront w of the workgroup works out the effective queries w_t and the coefficients c_{.,t} of tokens w and
+// w + 4 from K-vectors and publishes them in LDS; the state tile is then used once, as the MFMA A operand of
+// S_0 [w_0 .. w_{T-1}].  One workgroup covers a whole tile: RPW is 32 and wavefront w owns rows
 // 32 w .. 32 w + 31 as two 16-row MFMA tiles.
-template <typename act_t, bool IS_KDA, bool MTP, int RPW, bool READONCE = false, typename state_t = float>
+template <typename act_t, bool IS_KDA, bool MTP, int RPW, int READONCE = 0, typename state_t = float>
 __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   state_t* const pool = reinterpret_cast<state_t*>(p.h0);
   state_t* const snapshots = reinterpret_cast<state_t*>(p.cache);
@@ -143,33 +143,38 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       in.a1 = fetch_scalar(p.a, log_decay, tok * p.stride_a + i_hv);
     }
     in.b1 = fetch_scalar(p.b, beta_wide, tok * p.stride_b + i_hv);
-    if constexpr (!READONCE) load_row_words<RPW>(vp + tok * p.stride_v, in.vw);
+    if constexpr (READONCE == 0) load_row_words<RPW>(vp + tok * p.stride_v, in.vw);
     return in;
   };
 
   TokenIn cur = fetch(0);
   // read-once verify: every token is requested ahead of the state tile, so that the K-vector algebra runs
   // while the tile is in flight (memory returns in issue order)
-  TokenIn ahead[3] = {cur, cur, cur};
-  if constexpr (READONCE) {
+  constexpr int TM = READONCE > 0 ? READONCE : 1;      // draft tokens the read-once verify is built for
+  TokenIn ahead[TM > 1 ? TM - 1 : 1];
+  if constexpr (READONCE > 0) {
 #pragma unroll
-    for (int t = 1; t < 4; ++t)
-      if (t < T) ahead[t - 1] = fetch(t);
+    for (int t = 1; t < TM; ++t) ahead[t - 1] = t < T ? fetch(t) : cur;
   }
   float s[R][4];
-  // read-once verify: the tile in MFMA A-operand layout, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
+  // read-once verify: the tile in MFMA A-operand layout, lane (r16, kb) holds eight elements of row 32 w + 16 m + r16
+  // per contraction step ks
   const int r16 = lane & 15, kb = lane >> 4;
   constexpr bool POOL_BF16 = sizeof(state_t) == 2;      // a bf16 tile is an MFMA operand as it is
   f32x4_t sa[2][4][2];
   bf16x8_t sb16[2][4];
-  uint2 vq[2][4];
-  if constexpr (READONCE) {
-    static_assert(!READONCE || RPW == 32, "the read-once verify covers a whole tile per workgroup");
+  uint2 vq[2][TM];
+  if constexpr (READONCE > 0) {
+    static_assert(READONCE == 0 || RPW == 32, "the read-once verify covers a whole tile per workgroup");
+    static_assert(READONCE == 0 || READONCE == 4 || READONCE == 8, "the read-once verify is built for 4 or 8 draft tokens");
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * (int)sizeof(state_t);
+        // bf16 pool: the lane's eight elements 32 ks + 8 kb .. + 7 are 16 contiguous bytes.  FP32 pool: two loads of
+        // 16 bytes, elements 32 ks + 4 kb .. + 3 and 32 ks + 16 + 4 kb .. + 3, so that the four lanes of a row read 64
+        // contiguous bytes per instruction
+        const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + (POOL_BF16 ? 8 : 4) * kb) * (int)sizeof(state_t);
         if constexpr (POOL_BF16) {
           const v4i_t zero = {0, 0, 0, 0};
           sb16[m][ks] = __builtin_bit_cast(bf16x8_t, have_state ? __builtin_bit_cast(v4i_t, __builtin_amdgcn_raw_buffer_load_b128(
@@ -178,7 +183,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
 #pragma unroll
           for (int hf = 0; hf < 2; ++hf)
             sa[m][ks][hf] = have_state ? __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                             h_tile.rsrc, at + 16 * hf, 0, kLoadPolicy))
+                                             h_tile.rsrc, at + 64 * hf, 0, kLoadPolicy))
                                        : f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
       }
@@ -186,7 +191,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
 #pragma unroll
     for (int m = 0; m < 2; ++m)
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < TM; ++t)
         vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
                                                    ((int64_t)bos + min(t, T - 1)) * p.stride_v);
   } else if (have_state) {
@@ -204,14 +209,13 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   if constexpr (IS_KDA) decode_k4<act_t>(dt_raw_k4, dt_wide || log_decay, dt);
   else dt_scalar = decode_scalar_act<act_t>(dt_raw, dt_wide || log_decay);
 
-  if constexpr (READONCE) {
-    const TokenIn tok[4] = {cur, ahead[0], ahead[1], ahead[2]};        // absent tokens repeat token 0, never stored
-    __shared__ __align__(16) float sW[4][128];     // effective queries w_t
-    __shared__ __align__(16) float sC[4][4];       // sC[t][j] = c_{j,t}
-    float kv[4][4], dec[4][4], beta[4];
+  if constexpr (READONCE > 0) {
+    __shared__ __align__(16) float sW[TM][128];    // effective queries w_t
+    __shared__ __align__(16) float sC[TM][TM];     // sC[t][j] = c_{j,t}
+    float kv[TM][4], dec[TM][4], beta[TM];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const TokenIn& in = tok[t];
+    for (int t = 0; t < TM; ++t) {
+      const TokenIn& in = t == 0 ? cur : ahead[t > 0 ? t - 1 : 0];      // absent tokens repeat token 0, never stored
       const float k4[4] = {lo16<act_t>(in.kw.x), hi16<act_t>(in.kw.x), lo16<act_t>(in.kw.y), hi16<act_t>(in.kw.y)};
       float kn = 1.f;
       if (p.use_qk_l2norm) {
@@ -237,11 +241,11 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       const float b_in = decode_scalar_act<act_t>(in.b1, beta_wide);
       beta[t] = beta_wide ? b_in : fast_sigmoid(b_in);
     }
-    // wavefront t: effective query w_t and bias coefficients c_{j,t} of token t
+    // wavefront w: effective queries w_t and bias coefficients c_{j,t} of tokens t = w and t = w + 4
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      if (wave != t) continue;
-      const TokenIn& in = tok[t];
+    for (int t = 0; t < TM; ++t) {
+      if (wave != (t & 3)) continue;
+      const TokenIn& in = t == 0 ? cur : ahead[t > 0 ? t - 1 : 0];
       const float q4[4] = {lo16<act_t>(in.qw.x), hi16<act_t>(in.qw.x), lo16<act_t>(in.qw.y), hi16<act_t>(in.qw.y)};
       float qn = p.scale;
       if (p.use_qk_l2norm) {
@@ -251,41 +255,73 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
       }
       float w[4] = {q4[0] * qn, q4[1] * qn, q4[2] * qn, q4[3] * qn};
-      float cf[4];
-      effective_query<4>(t, w, kv, dec, beta, cf);
+      float cf[TM];
+      effective_query<TM>(t, w, kv, dec, beta, cf);
       if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
-      if (lane == 0) *reinterpret_cast<float4*>(&sC[t][0]) = make_float4(cf[0], cf[1], cf[2], cf[3]);
+      if (lane == 0) {
+#pragma unroll
+        for (int j4 = 0; j4 < TM; j4 += 4)
+          *reinterpret_cast<float4*>(&sC[t][j4]) = make_float4(cf[j4], cf[j4 + 1], cf[j4 + 2], cf[j4 + 3]);
+      }
     }
     __syncthreads();
-    // B operands: column r16 of [w_0 .. w_3 0 .. 0], contraction elements 32 ks + 8 kb .. + 7
-    const int tcol = min(r16, 3);
-    const float keep = r16 < 4 ? 1.f : 0.f;
-    HiLo wb[4];
-    query_operands(sW, tcol, keep, kb, wb);
-    const float4 cmine = *reinterpret_cast<const float4*>(&sC[tcol][0]);
-    const float cs[4] = {cmine.x, cmine.y, cmine.z, cmine.w};
+    // B operands: column r16 of [w_0 .. w_{TM-1} 0 .. 0]
+    const int tcol = min(r16, TM - 1);
+    const float keep = r16 < TM ? 1.f : 0.f;
+    float cs[TM];
 #pragma unroll
-    for (int m = 0; m < 2; ++m) {
-      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-      if constexpr (POOL_BF16) {
+    for (int j4 = 0; j4 < TM; j4 += 4) {
+      const float4 cmine = *reinterpret_cast<const float4*>(&sC[tcol][j4]);
+      cs[j4] = cmine.x; cs[j4 + 1] = cmine.y; cs[j4 + 2] = cmine.z; cs[j4 + 3] = cmine.w;
+    }
+    f32x4_t accs[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    if constexpr (POOL_BF16) {
+      HiLo wb[4];
+      query_operands(sW, tcol, keep, kb, wb);
+#pragma unroll
+      for (int m = 0; m < 2; ++m)
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-          acc = mfma16(sb16[m][ks], wb[ks].hi, acc);
-          acc = mfma16(sb16[m][ks], wb[ks].lo, acc);
+          accs[m] = mfma16(sb16[m][ks], wb[ks].hi, accs[m]);
+          accs[m] = mfma16(sb16[m][ks], wb[ks].lo, accs[m]);
         }
-      } else {
-        acc = rows_times_queries(sa[m], wb);
+    } else {
+      // An FP32 tile goes through the FP32 MFMA as it is (v_mfma_f32_16x16x4_f32: lane (r16, kb) supplies one
+      // element of row r16 for contraction slot kb, here its own element 32 ks + 16 hf + 4 kb + e), so neither the
+      // tile nor the queries are split into 16-bit pairs: 64 matrix instructions per wavefront instead of 24, but
+      // about 300 vector instructions fewer, and the products are exact.  The two row blocks alternate, so that
+      // consecutive instructions never wait for the same accumulator.
+      float wq[4][8];
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 4 * kb]);
+        const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 16 + 4 * kb]);
+        wq[ks][0] = w0.x * keep; wq[ks][1] = w0.y * keep; wq[ks][2] = w0.z * keep; wq[ks][3] = w0.w * keep;
+        wq[ks][4] = w1.x * keep; wq[ks][5] = w1.y * keep; wq[ks][6] = w1.z * keep; wq[ks][7] = w1.w * keep;
       }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+              accs[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[m][ks][hf][e], wq[ks][4 * hf + e], accs[m], 0, 0, 0);
+    }
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const f32x4_t acc = accs[m];
       // lane (r16 = token, kb): rows 16 m + 4 kb .. + 3 of S_0 w_token; add the bias terms
       float o[4] = {acc[0], acc[1], acc[2], acc[3]};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < TM; ++j) {
         o[0] = fmaf(cs[j], lo16<act_t>(vq[m][j].x), o[0]);
         o[1] = fmaf(cs[j], hi16<act_t>(vq[m][j].x), o[1]);
         o[2] = fmaf(cs[j], lo16<act_t>(vq[m][j].y), o[2]);
         o[3] = fmaf(cs[j], hi16<act_t>(vq[m][j].y), o[3]);
       }
-      if (r16 < 4 && r16 < T)
+      if (r16 < TM && r16 < T)
         *reinterpret_cast<uint2*>(o_base + (int64_t)r16 * p.HV * 128 + 16 * m + 4 * kb) =
             make_uint2(pack2<act_t>(o[0], o[1]), pack2<act_t>(o[2], o[3]));
     }
@@ -566,17 +602,18 @@ static int launch_rpw(const KLastParams& p, int rpw, hipStream_t stream) {
   const unsigned tiles = (unsigned)p.B * (unsigned)p.HV;
   if constexpr (MTP) {
     // a verify that leaves no trace in memory but o: the state is read once and used once
-    const bool read_once = p.disable_state_update && p.T_max <= 4 && p.cache == nullptr && p.cache_indices == nullptr &&
+    const bool read_once = p.disable_state_update && p.T_max <= 8 && p.cache == nullptr && p.cache_indices == nullptr &&
                            p.parents == nullptr && p.stride_h0_indices_seq == 0;
     if (read_once) {
-      hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, true, state_t>), dim3(tiles, 1), block, 0, stream, p);
+      if (p.T_max <= 4) hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, 4, state_t>), dim3(tiles, 1), block, 0, stream, p);
+      else hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, true, 32, 8, state_t>), dim3(tiles, 1), block, 0, stream, p);
       return check_launch("k_last_kernel launch");
     }
   }
   switch (rpw) {
-    case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 32, false, state_t>), dim3(tiles, 1), block, 0, stream, p); break;
-    case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 16, false, state_t>), dim3(tiles, 2), block, 0, stream, p); break;
-    case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 8, false, state_t>),  dim3(tiles, 4), block, 0, stream, p); break;
+    case 32: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 32, 0, state_t>), dim3(tiles, 1), block, 0, stream, p); break;
+    case 16: hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 16, 0, state_t>), dim3(tiles, 2), block, 0, stream, p); break;
+    case 8:  hipLaunchKernelGGL((k_last_kernel<act_t, IS_KDA, MTP, 8, 0, state_t>),  dim3(tiles, 4), block, 0, stream, p); break;
     default: return fail("rows_per_wave must be 0, 8, 16 or 32, got %d", rpw);
   }
   return check_launch("k_last_kernel launch");

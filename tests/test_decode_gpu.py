@@ -199,13 +199,14 @@ def test_mtp_lengths(T, mode, lower_bound):
 
 
 @pytest.mark.parametrize("is_kda,lower_bound", [(False, None), (True, None), (True, -5.0)])
-@pytest.mark.parametrize("T", [1, 2, 3, 4])
+@pytest.mark.parametrize("T", [1, 2, 3, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("H,HV", [(4, 8), (6, 6)])
 @pytest.mark.parametrize("act_dtype,state_dtype", [(torch.bfloat16, torch.float32), (torch.float16, torch.float32),
                                                    (torch.bfloat16, torch.bfloat16)])
 def test_read_once_verify(is_kda, lower_bound, T, H, HV, act_dtype, state_dtype):
-    """A verify that writes neither state nor snapshots (up to four draft tokens, [B, T, ...] inputs, no
-    cache) takes the read-once kernel: outputs equal the stepped recurrence, the pool stays bit-identical."""
+    """A verify that writes neither state nor snapshots (up to eight draft tokens, [B, T, ...] inputs, no
+    cache) takes the read-once kernel (built for four tokens, and for eight): outputs equal the stepped
+    recurrence, the pool stays bit-identical."""
     forward = _ops()[0]
     args, backing, lengths, state_ids, _ = make_k_last_case(is_kda, "verify", H=H, HV=HV, T=T, act_dtype=act_dtype,
                                                             state_dtype=state_dtype)
@@ -229,12 +230,14 @@ def test_read_once_verify(is_kda, lower_bound, T, H, HV, act_dtype, state_dtype)
     assert pad and all(torch.count_nonzero(out[n]) == 0 for n in pad)
 
 
-def test_read_once_verify_ragged_requests():
-    """Requests of 4, 2, 0, 3 and 1 draft tokens in one launch, a padded request among them."""
+@pytest.mark.parametrize("lengths,max_tokens", [([4, 2, 0, 3, 1, 4], 4), ([8, 5, 0, 3, 1, 7], 8)])
+def test_read_once_verify_ragged_requests(lengths, max_tokens):
+    """Requests of different numbers of draft tokens (one of them none) in one launch, a padded request among them;
+    windows of up to four and of up to eight tokens."""
     from pla_amd.decode.kda_replayssm_sglang import kda_mtp_verify
     from oracle import k_last_reference
     g = torch.Generator().manual_seed(77)
-    lengths, slots = [4, 2, 0, 3, 1, 4], [5, 0, 3, -1, 2, 6]
+    slots = [5, 0, 3, -1, 2, 6]
     nt, H, D = sum(lengths), 6, 128
     rnd = lambda *shape: torch.randn(*shape, generator=g)
     q, k, v = (rnd(1, nt, H, D).to(torch.bfloat16) for _ in range(3))
@@ -247,11 +250,12 @@ def test_read_once_verify_ragged_requests():
     pool_d = pool.cuda()
     before = pool_d.clone()
     out = kda_mtp_verify(q.cuda(), k.cuda(), v.cuda(), log_decay.cuda(), beta.cuda(), pool_d,
-                         torch.tensor(slots, dtype=torch.int32, device="cuda"), cu.cuda(), max_tokens=4)
+                         torch.tensor(slots, dtype=torch.int32, device="cuda"), cu.cuda(), max_tokens=max_tokens)
     torch.cuda.synchronize()
     torch.testing.assert_close(out[0].cpu().float(), want.float(), atol=1e-3, rtol=1.6e-2)
     assert torch.equal(pool_d, before)
-    assert torch.count_nonzero(out[0, 6:9]) == 0                                      # the padded request's three tokens
+    first = sum(lengths[:3])
+    assert torch.count_nonzero(out[0, first:first + 3]) == 0                          # the padded request's three tokens
 
 
 @pytest.mark.parametrize("layout", ["heads3", "strided_heads3", "flat2", "flat3", "batch4"])
