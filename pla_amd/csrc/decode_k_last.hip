@@ -148,13 +148,15 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   };
 
   TokenIn cur = fetch(0);
-  // read-once verify: every token is requested ahead of the state tile, so that the K-vector algebra runs
-  // while the tile is in flight (memory returns in issue order)
+  // read-once verify: wavefront w takes tokens w and w + 4; they are requested ahead of the state tile, so that
+  // the K-vector algebra runs while the tile is in flight (memory returns in issue order).  Tokens the request
+  // does not have repeat its last one (their results are never stored).
   constexpr int TM = READONCE > 0 ? READONCE : 1;      // draft tokens the read-once verify is built for
-  TokenIn ahead[TM > 1 ? TM - 1 : 1];
+  constexpr int NT = TM > 4 ? TM / 4 : 1;              // tokens per wavefront
+  TokenIn mine[NT];
   if constexpr (READONCE > 0) {
 #pragma unroll
-    for (int t = 1; t < TM; ++t) ahead[t - 1] = t < T ? fetch(t) : cur;
+    for (int u = 0; u < NT; ++u) mine[u] = fetch(min(wave + 4 * u, T - 1));
   }
   float s[R][4];
   // read-once verify: the tile in MFMA A-operand layout, lane (r16, kb) holds eight elements of row 32 w + 16 m + r16
@@ -212,10 +214,15 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   if constexpr (READONCE > 0) {
     __shared__ __align__(16) float sW[TM][128];    // effective queries w_t
     __shared__ __align__(16) float sC[TM][TM];     // sC[t][j] = c_{j,t}
-    float kv[TM][4], dec[TM][4], beta[TM];
+    __shared__ __align__(16) float sK[TM][128];    // normalised keys
+    __shared__ __align__(16) float sD[TM][128];    // decays exp(g)
+    __shared__ float sB[TM];                       // activated beta
+    // each wavefront prepares the K-vectors of its own tokens once and shares them through LDS (every wavefront
+    // working them out for every token cost four times the instructions)
 #pragma unroll
-    for (int t = 0; t < TM; ++t) {
-      const TokenIn& in = t == 0 ? cur : ahead[t > 0 ? t - 1 : 0];      // absent tokens repeat token 0, never stored
+    for (int u = 0; u < NT; ++u) {
+      const int t = wave + 4 * u;
+      const TokenIn& in = mine[u];
       const float k4[4] = {lo16<act_t>(in.kw.x), hi16<act_t>(in.kw.x), lo16<act_t>(in.kw.y), hi16<act_t>(in.kw.y)};
       float kn = 1.f;
       if (p.use_qk_l2norm) {
@@ -224,28 +231,32 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         for (int e = 0; e < 4; ++e) ks = fmaf(k4[e], k4[e], ks);
         kn = fast_rsqrt(row32_allreduce(ks) + 1e-6f);
       }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) kv[t][e] = k4[e] * kn;
+      float d4[4];
       if constexpr (IS_KDA) {
         float av[4];
         decode_k4<act_t>(in.a4, log_decay, av);
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          dec[t][e] = gate_decay(av[e], dt[e], eA, p.gate_p0, p.softplus_threshold, p.gate_mode);
+          d4[e] = gate_decay(av[e], dt[e], eA, p.gate_p0, p.softplus_threshold, p.gate_mode);
       } else {
         const float d1 = gate_decay(decode_scalar_act<act_t>(in.a1, log_decay), dt_scalar, eA, p.gate_p0,
                                     p.softplus_threshold, p.gate_mode);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dec[t][e] = d1;
+        for (int e = 0; e < 4; ++e) d4[e] = d1;
       }
       const float b_in = decode_scalar_act<act_t>(in.b1, beta_wide);
-      beta[t] = beta_wide ? b_in : fast_sigmoid(b_in);
+      if (half == 0) {
+        *reinterpret_cast<float4*>(&sK[t][4 * c]) = make_float4(k4[0] * kn, k4[1] * kn, k4[2] * kn, k4[3] * kn);
+        *reinterpret_cast<float4*>(&sD[t][4 * c]) = make_float4(d4[0], d4[1], d4[2], d4[3]);
+      }
+      if (lane == 0) sB[t] = beta_wide ? b_in : fast_sigmoid(b_in);
     }
+    __syncthreads();
     // wavefront w: effective queries w_t and bias coefficients c_{j,t} of tokens t = w and t = w + 4
 #pragma unroll
     for (int t = 0; t < TM; ++t) {
       if (wave != (t & 3)) continue;
-      const TokenIn& in = t == 0 ? cur : ahead[t > 0 ? t - 1 : 0];
+      const TokenIn& in = mine[t >> 2];
       const float q4[4] = {lo16<act_t>(in.qw.x), hi16<act_t>(in.qw.x), lo16<act_t>(in.qw.y), hi16<act_t>(in.qw.y)};
       float qn = p.scale;
       if (p.use_qk_l2norm) {
@@ -255,6 +266,16 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
       }
       float w[4] = {q4[0] * qn, q4[1] * qn, q4[2] * qn, q4[3] * qn};
+      float kv[TM][4], dec[TM][4], beta[TM];
+#pragma unroll
+      for (int j = 0; j < TM; ++j) {
+        // tokens after t do not enter w_t; the request's tokens before t are all present
+        const float4 k4 = j <= t ? *reinterpret_cast<const float4*>(&sK[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
+        const float4 d4 = j <= t ? *reinterpret_cast<const float4*>(&sD[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
+        kv[j][0] = k4.x; kv[j][1] = k4.y; kv[j][2] = k4.z; kv[j][3] = k4.w;
+        dec[j][0] = d4.x; dec[j][1] = d4.y; dec[j][2] = d4.z; dec[j][3] = d4.w;
+        beta[j] = j <= t ? sB[j] : 0.f;
+      }
       float cf[TM];
       effective_query<TM>(t, w, kv, dec, beta, cf);
       if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
