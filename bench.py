@@ -131,8 +131,8 @@ GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64
 KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00), summed over the kernels of
 # one call (profiles/gdn_prefill_kernels_32k.txt, profiles/kda_prefill_kernels_64k.txt)
-GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 2691000000
-KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 10636000000
+GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 1687000000
+KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11896000000
 
 
 def cpu_baseline_prefill(w):
@@ -193,7 +193,8 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
                               flop_per_token=GDN_FLOP_PER_TOKEN,
                               note="algorithmic flops (dense) over the whole call; fp16 operands, FP32 accumulation "
                                    "(v_mfma_f32_16x16x32_f16, the rate of the bf16 instruction): "
-                                   "chunk map + prep + gram/solve + sequential kernels"))
+                                   "table kernel + key-side preparation + fused sweeps, four pipelined stages; "
+                                   "traffic is a constant from rocprofv3 --pmc runs (profiles/gdn_prefill_kernels_32k.txt)"))
 
 
 # GDN prefill shapes the reference publishes timings for (reports/prefill_bench_20260911.json, family gdn,
