@@ -513,9 +513,13 @@ __device__ __forceinline__ void segment_map(const int32_t* seq_chunk_off, int N,
 }
 
 // Eight workgroups of 256 threads per (sequence, head), each owning 16 rows of the state (rows transform
-// independently): walks the sequence's segments, stores the state entering each later segment and the
-// final state.  Thread (row, tk) owns columns 8 tk .. 8 tk + 7 of its row; the row slice of S lives in
-// LDS between steps, M and B are streamed from global memory.
+// independently): walks the sequence's segments, stores the state entering every later segment and the final
+// state.  A step S <- S M + B is a 16 x 128 x 128 product per workgroup on the FP32 MFMA
+// (v_mfma_f32_16x16x4_f32, exact products, FP32 accumulation): wavefront w owns columns 32 w .. 32 w + 31 as two
+// accumulator tiles that start from B; the A operand is the workgroup's 16 rows of S from LDS (lane (r, kb) takes
+// S[r][16 s + 4 kb + e] for step (s, e)), the B operand the matching row of M straight from memory (lane (c, kb):
+// M[16 s + 4 kb + e][column c], 64 contiguous bytes per group of 16 lanes), all 64 loads of a step requested before
+// the first product.
 constexpr int COMBINE_SPLIT = 8;
 static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads, float* ht,
                                                                      const int32_t* ht_indices, int64_t ht_slot_stride) {
@@ -524,45 +528,66 @@ static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTabl
   const int n = chain / heads, h = chain - n * heads;
   const int first = t.seq_seg_off[n], end = t.seq_seg_off[n + 1];
   if (end - first < 2) return;                 // a single segment wrote its final state itself
-  __shared__ float S[16][132];
-  const int row = threadIdx.x >> 4, tk = threadIdx.x & 15;
-  const int64_t at = (int64_t)(16 * part + row) * 128 + 8 * tk;      // this thread's place in a [128, 128] tile
-  float acc[8];
+  __shared__ __align__(16) float S[16][132];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, kb = lane >> 4;
+  const int col0 = 32 * wave + c;              // this lane's column of accumulator tile 0 (tile 1: + 16)
+  // place of accumulator element (tile cb, row v) inside a [128, 128] tile
+  auto at = [&](int cb, int v) { return (int64_t)(16 * part + 4 * kb + v) * 128 + col0 + 16 * cb; };
+  f32x4_t acc[2];
   {
-    const float* src = t.B + ((int64_t)first * heads + h) * 16384 + at;
-    const float4 b0 = *reinterpret_cast<const float4*>(src), b1 = *reinterpret_cast<const float4*>(src + 4);
-    acc[0] = b0.x; acc[1] = b0.y; acc[2] = b0.z; acc[3] = b0.w; acc[4] = b1.x; acc[5] = b1.y; acc[6] = b1.z; acc[7] = b1.w;
+    const float* src = t.B + ((int64_t)first * heads + h) * 16384;
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[cb][v] = src[at(cb, v)];
   }
   for (int seg = first + 1; seg < end; ++seg) {
     const int64_t tile = ((int64_t)seg * heads + h) * 16384;
-    *reinterpret_cast<float4*>(&S[row][8 * tk]) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    *reinterpret_cast<float4*>(&S[row][8 * tk + 4]) = make_float4(acc[4], acc[5], acc[6], acc[7]);
-    *reinterpret_cast<float4*>(t.S + tile + at) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    *reinterpret_cast<float4*>(t.S + tile + at + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    // the state entering this segment: to memory for the second sweep, to LDS as the A operand of this step
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        t.S[tile + at(cb, v)] = acc[cb][v];
+        S[4 * kb + v][col0 + 16 * cb] = acc[cb][v];
+      }
+    // M rows and the B tile of this segment, requested before the barrier
+    const float* Mt = t.M + tile;
+    float m[2][32];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) m[cb][4 * s8 + e] = Mt[(int64_t)(16 * s8 + 4 * kb + e) * 128 + col0 + 16 * cb];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[cb][v] = t.B[tile + at(cb, v)];
     __syncthreads();
-    const float* Mt = t.M + tile + 8 * tk;
-    {
-      const float4 b0 = *reinterpret_cast<const float4*>(t.B + tile + at);
-      const float4 b1 = *reinterpret_cast<const float4*>(t.B + tile + at + 4);
-      acc[0] = b0.x; acc[1] = b0.y; acc[2] = b0.z; acc[3] = b0.w; acc[4] = b1.x; acc[5] = b1.y; acc[6] = b1.z; acc[7] = b1.w;
-    }
-#pragma unroll 8
-    for (int j = 0; j < 128; ++j) {
-      const float4 m0 = *reinterpret_cast<const float4*>(Mt + j * 128);
-      const float4 m1 = *reinterpret_cast<const float4*>(Mt + j * 128 + 4);
-      const float sv = S[row][j];
-      acc[0] = fmaf(sv, m0.x, acc[0]); acc[1] = fmaf(sv, m0.y, acc[1]); acc[2] = fmaf(sv, m0.z, acc[2]);
-      acc[3] = fmaf(sv, m0.w, acc[3]); acc[4] = fmaf(sv, m1.x, acc[4]); acc[5] = fmaf(sv, m1.y, acc[5]);
-      acc[6] = fmaf(sv, m1.z, acc[6]); acc[7] = fmaf(sv, m1.w, acc[7]);
-    }
-    __syncthreads();
+    float4 a[8];
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8) a[s8] = *reinterpret_cast<const float4*>(&S[c][16 * s8 + 4 * kb]);
+#pragma unroll
+    for (int s8 = 0; s8 < 8; ++s8)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float av = e == 0 ? a[s8].x : e == 1 ? a[s8].y : e == 2 ? a[s8].z : a[s8].w;
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, m[cb][4 * s8 + e], acc[cb], 0, 0, 0);
+      }
+    __syncthreads();                           // every wavefront has read S before the next step overwrites it
   }
   if (ht != nullptr) {
     const int slot = ht_indices ? ht_indices[n] : n;
     if (slot >= 0) {
-      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384 + at;
-      *reinterpret_cast<float4*>(dst) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-      *reinterpret_cast<float4*>(dst + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384;
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) dst[at(cb, v)] = acc[cb][v];
     }
   }
 }
