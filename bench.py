@@ -159,6 +159,30 @@ def cpu_baseline_prefill(w):
                 threads_torch=torch.get_num_threads())
 
 
+def time_calls(run, steps, warmup, device):
+    """Mean milliseconds of `steps` back-to-back calls of `run` after `warmup` untimed ones.
+
+    A prefill call is a Python wrapper around several kernel launches: on an idle stream the time between
+    enqueueing the start event and the first kernel of the first call (allocations, argument checks, the first
+    launches: a few hundred microseconds) would be counted, which is a tenth of a five-call run.  A 2 GiB fill runs in
+    front of the start event instead: while it runs the host enqueues the event and the first calls, so the event's
+    time stamp is followed at once by the first kernel and the calls are back to back from the first one on."""
+    import torch
+    filler = torch.empty(512 << 20, dtype=torch.float32, device=device)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    filler.zero_()
+    start.record()
+    for _ in range(steps):
+        run()
+    end.record()
+    torch.cuda.synchronize()
+    del filler
+    return start.elapsed_time(end) / steps
+
+
 def bench_prefill(steps, warmup, device, cpu_leg=False):
     """Config 3: GDN chunk-64 prefill, 8 ragged sequences (about 32K tokens), indexed FP32 pool."""
     import torch
@@ -173,16 +197,7 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
     def run():
         return gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, output_final_state=False, **call)
 
-    for _ in range(warmup):
-        run()
-    torch.cuda.synchronize()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        run()
-    end.record()
-    torch.cuda.synchronize()
-    ms = start.elapsed_time(end) / steps
+    ms = time_calls(run, steps, warmup, device)
     T = sum(lengths)
     tflops = GDN_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     extra = dict(cpu_baseline=cpu_baseline_prefill(w)) if cpu_leg else {}
@@ -193,7 +208,8 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
                               flop_per_token=GDN_FLOP_PER_TOKEN,
                               note="algorithmic flops (dense) over the whole call; fp16 operands, FP32 accumulation "
                                    "(v_mfma_f32_16x16x32_f16, the rate of the bf16 instruction): "
-                                   "table kernel + key-side preparation + fused sweeps, four pipelined stages; "
+                                   "table kernel + key-side preparation + fused sweeps, two pipelined stages, steady state after "
+                                   "%d warm-up calls; " % warmup +
                                    "traffic is a constant from rocprofv3 --pmc runs (profiles/gdn_prefill_kernels_32k.txt)"))
 
 
@@ -215,16 +231,7 @@ def bench_prefill_reference_shapes(steps, device):
         packed = call.pop("packed_qkv")
         a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
         run = lambda: gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, **call)
-        for _ in range(3):
-            run()
-        torch.cuda.synchronize()
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
-        for _ in range(steps):
-            run()
-        end.record()
-        torch.cuda.synchronize()
-        ms = start.elapsed_time(end) / steps
+        ms = time_calls(run, steps, 20, device)
         rows.append({"shape": "%d x %d tokens" % (len(lengths), lengths[0]), "ms_per_call": round(ms, 4),
                      "tokens_per_s": round(sum(lengths) / ms * 1e3, 1), "reference_ppu_ms": published_ms,
                      "reference_ms_over_ours": round(published_ms / ms, 2)})
@@ -246,16 +253,7 @@ def bench_prefill_kda(steps, device):
                      lower_bound=c["lower_bound"], initial_state=c["initial_state"], final_state=c["final_state"],
                      cu_seqlens=c["cu_seqlens"])
 
-    for _ in range(2):
-        run()
-    torch.cuda.synchronize()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record()
-    for _ in range(steps):
-        run()
-    end.record()
-    torch.cuda.synchronize()
-    ms = start.elapsed_time(end) / steps
+    ms = time_calls(run, steps, 3, device)
     tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     return dict(tokens=T, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
@@ -508,9 +506,9 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     if args.prefill_only:
-        result = {"prefill": bench_prefill(max(args.steps // 10, 5), 3, device)}
+        result = {"prefill": bench_prefill(max(args.steps, 50), 50, device)}
         torch.cuda.empty_cache()
-        result["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+        result["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device)
         if args.copy_calibration:
             result["copy_calibration"] = copy_calibration(device)
         print(json.dumps(result))
@@ -528,10 +526,10 @@ def main():
         extra["replay_verify"] = bench_replay_verify(device)
         extra["replay_paged"] = bench_replay_paged(device)
         torch.cuda.empty_cache()
-        extra["prefill"] = bench_prefill(max(args.steps // 10, 5), 3, device, cpu_leg=not args.no_cpu_baseline)
+        extra["prefill"] = bench_prefill(max(args.steps, 50), 50, device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
-        extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 20, 5), device)
-        extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 40, 3), device)
+        extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 2, 10), device)
+        extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device)
         torch.cuda.empty_cache()
     d = time_decode(prep, args.steps, args.warmup)
     result = {

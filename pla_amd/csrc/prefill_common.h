@@ -331,13 +331,14 @@ struct SegmentTable {
 // carried from stage to stage through one [V, K] tile per chain.
 struct StageTable {
   int32_t* order;         // [chunks] global chunk ids, all of stage 0 first, then stage 1, ...
-  int32_t* stage_begin;   // [stages + 1] offsets into `order`
+  int32_t* stage_begin;   // [MAX_STAGES + 2]: offsets into `order` per stage, then (last word) the number of stages in effect
   float* carry;           // [N, heads, V, K] (whole sequences; segments carry in their own tiles)
   int stages;             // 0: not staged
 };
-constexpr int MAX_STAGES = 4;
-// Chunks [lo, hi) of an item of `nc` chunks that belong to stage s of S.
-__device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((int64_t)nc * s / S); }
+constexpr int MAX_STAGES = 2;
+// Chunks [stage_cut(nc, s, S), stage_cut(nc, s + 1, S)) of an item of `nc` chunks belong to stage s of the S stages in
+// effect (stages beyond S are empty).
+__device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((int64_t)nc * min(s, S) / S); }
 
 // Single workgroup of 256 threads with (stages + 1) * n_items_max + 1 words of LDS at `pair_begin`.  The items are sequences (`counts` null: item i holds chunks
 // starts[i] .. starts[i + 1]) or segments (chunks starts[i] .. starts[i] + counts[i]); `n_items` is read
@@ -349,25 +350,38 @@ __device__ __forceinline__ void stage_map(const int32_t* starts, const int32_t* 
   const int S = t.stages;
   const int n_items = n_items_ptr ? min(*n_items_ptr, n_items_max) : n_items_max;
   int32_t* const count = pair_begin + S * n_items_max + 1;
+  __shared__ int stages_in_effect;
   for (int i = threadIdx.x; i < n_items; i += blockDim.x) count[i] = counts ? counts[i] : starts[i + 1] - starts[i];
   __syncthreads();
   auto count_of = [&](int i) { return count[i]; };
   if (threadIdx.x == 0) {
+    // The stages pay where chains of unequal length leave CUs idle for the later preparation to run on: with
+    // chains of (nearly) equal length the chip stays full to the end of a sweep, the preparation of the next stage
+    // runs after it either way, and the second pair of launches is pure overhead (measured on 8 x 2048 tokens:
+    // 0.24 ms in one stage, 0.27 ms in two; on eight ragged sequences of 32 810 tokens 0.50 against 0.48 ms).
+    // One stage then takes everything, the others stay empty.
+    int64_t total = 0;
+    int longest = 0;
+    for (int i = 0; i < n_items; ++i) { total += count_of(i); longest = max(longest, count_of(i)); }
+    const int E = 5 * total < 4 * (int64_t)n_items * longest ? S : 1;      // idle share of the chains' rectangle above 20 %
+    stages_in_effect = E;
+    t.stage_begin[MAX_STAGES + 1] = E;
     int k = 0;
     for (int s = 0; s < S; ++s) {
       t.stage_begin[s] = k;
       for (int i = 0; i < n_items; ++i) {
         const int nc = count_of(i);
         pair_begin[s * n_items + i] = k;
-        k += stage_cut(nc, s + 1, S) - stage_cut(nc, s, S);
+        k += stage_cut(nc, s + 1, E) - stage_cut(nc, s, E);
       }
     }
     t.stage_begin[S] = k;
   }
   __syncthreads();
+  const int E = stages_in_effect;
   for (int pair = threadIdx.x >> 3; pair < S * n_items; pair += blockDim.x >> 3) {      // eight threads per pair
     const int s = pair / n_items, i = pair - s * n_items;
-    const int nc = count_of(i), lo = stage_cut(nc, s, S), hi = stage_cut(nc, s + 1, S);
+    const int nc = count_of(i), lo = stage_cut(nc, s, E), hi = stage_cut(nc, s + 1, E);
     const int base = pair_begin[pair];
     for (int cc = lo + (threadIdx.x & 7); cc < hi; cc += 8)
       if (base + cc - lo < NC_max) t.order[base + cc - lo] = starts[i] + cc;
@@ -468,11 +482,13 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     }
   }
   if (carry != nullptr && stg.stages > 0) {
+    const int E = stg.stage_begin[MAX_STAGES + 1];                 // stages in effect (the table kernel's choice)
+    if (stage >= E) return r;                                      // an empty stage: the one before it delivered the state
     const int nc = r.c_end - r.c_begin, c0 = r.c_begin;
-    r.c_begin = c0 + stage_cut(nc, stage, stg.stages);
-    r.c_end = c0 + stage_cut(nc, stage + 1, stg.stages);
+    r.c_begin = c0 + stage_cut(nc, stage, E);
+    r.c_end = c0 + stage_cut(nc, stage + 1, E);
     if (stage > 0) { r.init = carry; r.keep_init = nullptr; }      // the start state is kept by stage 0 only
-    if (stage < stg.stages - 1) r.fin = carry;
+    if (stage < E - 1) r.fin = carry;
   }
   r.active = true;
   return r;
@@ -709,11 +725,15 @@ class SideStreamLease {
   SideStream* taken_;
 };
 
-// Number of stages for a call of whole sequences: enough chains to fill the chip and 16 chunks per
-// sequence on average.  (Segmented calls already keep every CU busy with sweeps - staging them was measured
-// for GDN: 0.57 -> 0.66 ms for one sequence of 16 384 tokens, 0.99 -> 1.06 ms for 32 768 -; and staging only pays
-// where the preparation is bound by memory latency and leaves the sweeps their issue slots, which holds for
-// GDN and not for KDA, whose preparation is instruction bound: the KDA path does not call this.)
+// Stages for a call of whole sequences: two, where there are enough chains to fill the chip and 16 chunks per
+// sequence on average; the table kernel then keeps both only for chains of unequal length (stage_map).  Measured on
+// GDN, eight ragged sequences of 32 810 tokens: 0.50 ms in one stage, 0.48 in two, 0.52 in four - every further stage
+// costs about 25 us (two more launches, an event between two streams, the state through memory, a pipeline that
+// fills again), and the preparation only hides under a sweep on CUs that chains which ended early have left.
+// (Segmented calls already keep every CU busy with sweeps - staging them was measured for GDN: 0.57 -> 0.66 ms for
+// one sequence of 16 384 tokens -; and staging only pays where the preparation is bound by memory latency and leaves
+// the sweeps their issue slots, which holds for GDN and not for KDA, whose preparation is instruction bound: the KDA
+// path does not call this.)
 inline int pick_stages(int T, int N, int heads, int seg_chunks) {
   if (seg_chunks > 0) return 0;
   // (the stage map keeps (stages + 1) counters per sequence in LDS: at most 2048 sequences)

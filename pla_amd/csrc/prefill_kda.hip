@@ -959,7 +959,7 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   L.stages = 0;
   if (L.stages > 0) {
     L.order = take((size_t)L.NC_max * 4);
-    L.stage_begin = take((size_t)(MAX_STAGES + 1) * 4);
+    L.stage_begin = take((size_t)(MAX_STAGES + 2) * 4);
     L.carry = L.seg_chunks > 0 ? 0 : take((size_t)N * H * 16384 * 4);
   }
   L.total = off;

@@ -233,6 +233,16 @@ def test_gdn_prefill_staged_pipeline_matches_oracle_and_unstaged_bits():
         assert torch.equal(w["initial_state"][slot], pool_staged[slot]), n
 
 
+def test_gdn_prefill_equal_lengths_collapse_the_stages():
+    """Chains of (nearly) equal length leave no idle CUs for a later preparation to hide on: the table kernel then
+    puts every chunk into the first stage and the launches of the second find nothing to do.  Against the oracle,
+    with initial states and final states through the pool (which the first stage now writes itself)."""
+    from pla_amd.workloads import gdn_prefill_packed
+    for lengths in ([1100] * 8, [1100, 1090, 1150, 1100, 1024, 1100, 1120, 1100]):
+        w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 3, seed=4242, tail_pad=3)
+        _check(w, fast=True)
+
+
 def test_gdn_prefill_staged_pipeline_in_a_graph():
     """The staged call forks to a side stream and joins again, so it can be captured: three replays with
     eager work and synchronisation in between reproduce the eager result bit for bit."""
