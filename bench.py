@@ -201,7 +201,8 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
     T = sum(lengths)
     tflops = GDN_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     extra = dict(cpu_baseline=cpu_baseline_prefill(w)) if cpu_leg else {}
-    return dict(tokens=T, lengths=lengths, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1), **extra,
+    return dict(tokens=T, lengths=lengths, steps=steps, warmup=warmup, ms_per_call=round(ms, 4),
+                tokens_per_s=round(T / ms * 1e3, 1), **extra,
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
                               frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=GDN_PREFILL_TRAFFIC_BYTES_PER_CALL,
                               hbm_GBps=round(GDN_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
@@ -255,7 +256,7 @@ def bench_prefill_kda(steps, device):
 
     ms = time_calls(run, steps, 3, device)
     tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
-    return dict(tokens=T, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
+    return dict(tokens=T, steps=steps, warmup=3, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
                               frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=KDA_PREFILL_TRAFFIC_BYTES_PER_CALL,
                               hbm_GBps=round(KDA_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
