@@ -241,6 +241,13 @@ def test_gdn_prefill_equal_lengths_collapse_the_stages():
     for lengths in ([1100] * 8, [1100, 1090, 1150, 1100, 1024, 1100, 1120, 1100]):
         w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 3, seed=4242, tail_pad=3)
         _check(w, fast=True)
+    # either side of the rule (one stage when the chunks fill at least 80 % of sequences x longest chain):
+    # 154 of 8 x 24 chunks -> one stage, 153 -> two
+    for lengths in ([1530, 1536, 1530, 1536, 955, 960, 890, 896], [1530, 1536, 1530, 1536, 955, 896, 890, 896]):
+        chunks = sum((n + 63) // 64 for n in lengths)
+        assert (5 * chunks < 4 * 8 * 24) == (chunks == 153)
+        w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 3, seed=chunks)
+        _check(w, fast=True)
 
 
 def test_gdn_prefill_staged_pipeline_in_a_graph():
