@@ -340,6 +340,21 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
+  // gate inputs of the lane's token, requested ahead of the K rows: memory returns in issue order, so the gate math
+  // below starts as soon as these few words are here and runs while the rows are still in flight
+  float gate_in = 0.f, beta_raw = 0.f, dt_b = 0.f, a_log = 0.f;
+  if (lane < len) {
+    const int64_t t = t0 + lane;
+    if (p.g_in) {
+      gate_in = p.g_in[t * p.HV + hv];
+      beta_raw = p.beta_in[t * p.HV + hv];
+    } else {
+      gate_in = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]);
+      beta_raw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
+      dt_b = p.dt_bias[hv];
+      a_log = p.A_log[hv];
+    }
+  }
   // raw K operands, all 16 loads of a lane requested before the first use (rows are 16-byte aligned on this path)
   uint4 kraw[4][4];
 #pragma unroll
@@ -355,16 +370,14 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   {
     float g = 0.f, bt = 0.f;
     if (lane < len) {
-      const int64_t t = t0 + lane;
       if (p.g_in) {
-        g = p.g_in[t * p.HV + hv];
-        bt = p.beta_in[t * p.HV + hv];
+        g = gate_in;
+        bt = beta_raw;
       } else {
-        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
+        const float x = gate_in + dt_b;
         const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
-        g = -expf(p.A_log[hv]) * sp;
-        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
-        bt = 1.0f / (1.0f + expf(-braw));
+        g = -expf(a_log) * sp;
+        bt = 1.0f / (1.0f + expf(-beta_raw));
       }
     }
     float cum = g;
