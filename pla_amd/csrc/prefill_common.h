@@ -670,8 +670,11 @@ inline size_t align_up256(size_t x) { return (x + 255) & ~(size_t)255; }
 // are enqueued concurrently (host threads launching on different streams) never share a stream or an event,
 // while consecutive calls reuse the same few objects: an event wait binds to the record that precedes it in
 // the calling thread, and work queued on a reused side stream simply runs after the previous call's.  A side
-// stream that is part of an unfinished graph capture is passed over.  Streams and events are created on first
-// need and kept for the life of the process.
+// stream that has joined a graph capture stays part of it until the capture ends: only calls of that same
+// capture may take it again (every staged call of one capture then shares one side stream), any other call
+// passes it over.  Streams and events are created on first need and kept for the life of the process.  A call
+// that finds no side stream (the pool is exhausted, or creation failed) is not staged: the lease is taken
+// before the first launch, so nothing has been enqueued by then.
 struct SideStream {
   hipStream_t stream;
   hipEvent_t fork;
@@ -680,13 +683,22 @@ struct SideStream {
 };
 class SideStreamLease {
  public:
-  SideStreamLease() : taken_(nullptr) {
+  // caller: the stream the call launches on; wanted: false leaves the lease empty
+  SideStreamLease(hipStream_t caller, bool wanted) : taken_(nullptr) {
     int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return;
+    if (!wanted || hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return;
+    unsigned long long caller_capture = 0;
+    const bool caller_capturing = capture_of(caller, &caller_capture);
     std::lock_guard<std::mutex> lock(guard());
     SideStream* const pool = pools()[dev];
-    for (int i = 0; i < POOL; ++i)
-      if (pool[i].stream != nullptr && !pool[i].busy && !capturing(pool[i].stream)) { taken_ = &pool[i]; break; }
+    SideStream* idle = nullptr;
+    for (int i = 0; i < POOL && taken_ == nullptr; ++i) {
+      if (pool[i].stream == nullptr || pool[i].busy) continue;
+      unsigned long long id = 0;
+      if (!capture_of(pool[i].stream, &id)) { if (idle == nullptr) idle = &pool[i]; }
+      else if (caller_capturing && id == caller_capture) taken_ = &pool[i];      // already part of the caller's capture
+    }
+    if (taken_ == nullptr) taken_ = idle;
     if (taken_ == nullptr)
       for (int i = 0; i < POOL; ++i)
         if (pool[i].stream == nullptr) {
@@ -702,24 +714,32 @@ class SideStreamLease {
   }
   SideStreamLease(const SideStreamLease&) = delete;
   SideStreamLease& operator=(const SideStreamLease&) = delete;
-  SideStream* get() const { return taken_; }     // nullptr: none could be created, or more than POOL calls at once
+  SideStream* get() const { return taken_; }     // nullptr: not wanted, none could be created, or the pool is in use
 
  private:
   static constexpr int MAX_DEVICES = 64, POOL = 16;
   static std::mutex& guard() { static std::mutex m; return m; }
   static SideStream (*pools())[POOL] { static SideStream table[MAX_DEVICES][POOL] = {}; return table; }
-  // a side stream that joined a graph capture stays part of it until the capture ends: leave it to that capture
-  static bool capturing(hipStream_t stream) {
+  // true (and the capture's id) while the stream is part of an unfinished graph capture; a stream whose state
+  // cannot be read counts as capturing with an id no caller has
+  static bool capture_of(hipStream_t stream, unsigned long long* id) {
     hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-    return hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone;
+    if (hipStreamGetCaptureInfo(stream, &status, id) != hipSuccess) { *id = ~0ull; return true; }
+    return status != hipStreamCaptureStatusNone;
   }
   static bool create(SideStream& t) {
-    hipStream_t stream = nullptr;
-    if (hipStreamCreateWithFlags(&stream, hipStreamNonBlocking) != hipSuccess) return false;
-    bool ok = hipEventCreateWithFlags(&t.fork, hipEventDisableTiming) == hipSuccess;
-    for (int i = 0; i < MAX_STAGES && ok; ++i) ok = hipEventCreateWithFlags(&t.ready[i], hipEventDisableTiming) == hipSuccess;
-    if (!ok) return false;
-    t.stream = stream;
+    SideStream made{};
+    if (hipStreamCreateWithFlags(&made.stream, hipStreamNonBlocking) != hipSuccess) return false;
+    bool ok = hipEventCreateWithFlags(&made.fork, hipEventDisableTiming) == hipSuccess;
+    for (int i = 0; i < MAX_STAGES && ok; ++i) ok = hipEventCreateWithFlags(&made.ready[i], hipEventDisableTiming) == hipSuccess;
+    if (!ok) {                                   // give back what was created
+      for (int i = 0; i < MAX_STAGES; ++i)
+        if (made.ready[i] != nullptr) (void)hipEventDestroy(made.ready[i]);
+      if (made.fork != nullptr) (void)hipEventDestroy(made.fork);
+      (void)hipStreamDestroy(made.stream);
+      return false;
+    }
+    t = made;
     return true;
   }
   SideStream* taken_;
@@ -742,11 +762,11 @@ inline int pick_stages(int T, int N, int heads, int seg_chunks) {
 
 // Launch order of a prefill call, shared by both paths.  `prepare(stream)` launches the per-chunk
 // kernels of stage *stage_field, `sweep(grid)` the sequential kernel for (*pass_field, *stage_field).
-// Stage 0 is prepared on the caller's stream, alone; the side stream prepares the other stages
-// underneath the sweeps and is joined before the last sweep starts.
+// Stage 0 is prepared on the caller's stream, alone; the side stream (a SideStreamLease the caller holds for the
+// time of the call) prepares the other stages underneath the sweeps and is joined before the last sweep starts.
 template <typename Prepare, typename Sweep>
-inline bool launch_pipeline(hipStream_t s, int stages, bool segmented, unsigned grid_whole, unsigned grid_segments,
-                            int* pass_field, int* stage_field, Prepare prepare, Sweep sweep) {
+inline bool launch_pipeline(hipStream_t s, int stages, SideStream* side, bool segmented, unsigned grid_whole,
+                            unsigned grid_segments, int* pass_field, int* stage_field, Prepare prepare, Sweep sweep) {
   *pass_field = segmented ? 1 : 0;
   const unsigned grid = segmented ? 2 * grid_segments : grid_whole;
   if (stages == 0) {
@@ -755,9 +775,7 @@ inline bool launch_pipeline(hipStream_t s, int stages, bool segmented, unsigned 
     sweep(grid);
     return true;
   }
-  const SideStreamLease lease;
-  SideStream* const side = lease.get();
-  if (side == nullptr) return false;
+  if (side == nullptr) return false;             // (callers stage a call only with a side stream in hand)
   bool ok = true;
   for (int st = 0; st < stages; ++st) {
     *stage_field = st;

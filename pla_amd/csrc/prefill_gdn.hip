@@ -1162,7 +1162,8 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
         for (int j = 0; j < 8; ++j) {
           const uint32_t row = (uint32_t)min(row0 + 4 * j + lr, last);
           raw[j] = *reinterpret_cast<const uint4*>(cb + row * (uint32_t)(row_pitch * 2) + 16u * lc);
-          inv[j] = q_side ? 0.f : *reinterpret_cast<const float*>(ib + row * (uint32_t)(p.H * 4));
+          // without normalisation the preparation never writes 1 / |k|: the workspace words are not read at all
+          inv[j] = (q_side || !p.normalize_qk) ? 1.f : *reinterpret_cast<const float*>(ib + row * (uint32_t)(p.H * 4));
         }
       };
       // K rows: scaled by 1 / |k|, rounded to the activation dtype (the operand of the reference), written as fp16,
@@ -1172,7 +1173,6 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
         uint16_t* const T = (q_side ? tQ[c & 1] : tK[c & 1]) + (row0 + lr) * PITCH128 + 8 * lc;
         const int len = chunk_len(c);
-        const float on = p.normalize_qk ? 1.f : 0.f;
         if constexpr (q_side) {
           float ss[8];
 #pragma unroll
@@ -1195,14 +1195,13 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const float r = rsqrtf(ss[j] + 1e-6f);
-            if (lc == 0) rq[4 * j] = on * r + (1.f - on);
+            if (lc == 0) rq[4 * j] = p.normalize_qk ? r : 1.f;
           }
         } else {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const uint32_t in[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
-            float inv = on * inv_in[j] + (1.f - on);
-            inv = row0 + 4 * j + lr < len ? inv : 0.f;
+            const float inv = row0 + 4 * j + lr < len ? inv_in[j] : 0.f;
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -1754,16 +1753,20 @@ static int gdn_prefill_run(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
   }
-  if (L.stages > 0) {
+  // the staged pipeline needs a side stream: without one (pool exhausted) the call runs unstaged, decided before
+  // anything is launched
+  const SideStreamLease lease(s, L.stages > 0);
+  const int stages = lease.get() != nullptr ? L.stages : 0;
+  if (stages > 0) {
     p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
     p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
-    p.stg.stages = L.stages;
+    p.stg.stages = stages;
   }
   launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
                 segmented ? L.max_segments : N, o, HV);
   const bool ok = launch_pipeline(
-      s, L.stages, segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
+      s, stages, lease.get(), segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
       [&](hipStream_t ps) {
         const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
         const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
@@ -1801,7 +1804,7 @@ static int gdn_prefill_run(
           else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
         }
       });
-  PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
+  PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);

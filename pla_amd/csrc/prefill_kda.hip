@@ -1035,16 +1035,18 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
   }
-  if (L.stages > 0) {
+  const SideStreamLease lease(s, L.stages > 0);
+  const int stages = lease.get() != nullptr ? L.stages : 0;
+  if (stages > 0) {
     p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
     p.stg.stage_begin = reinterpret_cast<int32_t*>(ws + L.stage_begin);
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
-    p.stg.stages = L.stages;
+    p.stg.stages = stages;
   }
   launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
                 segmented ? L.max_segments : N, o, H);
   const bool ok = launch_pipeline(
-      s, L.stages, segmented, (unsigned)N * H, (unsigned)L.max_segments * H, &p.pass, &p.stage,
+      s, stages, lease.get(), segmented, (unsigned)N * H, (unsigned)L.max_segments * H, &p.pass, &p.stage,
       [&](hipStream_t ps) { hipLaunchKernelGGL(kda_prep_solve_kernel, dim3(L.NC_max, H), dim3(256), 0, ps, p); },
       [&](unsigned grid) {
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
@@ -1052,7 +1054,7 @@ extern "C" int pla_kda_prefill_launch(
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
         else hipLaunchKernelGGL(kda_sweep_kernel, dim3(grid), dim3(320), 0, s, p);
       });
-  PLA_REQUIRE(ok, "could not create the side stream for the staged prefill");
+  PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
                        ht_indices, ht_slot_stride);

@@ -33,6 +33,11 @@ def _token_rows(name, t, H, width):
     return t, t.stride(0)
 
 
+def _workspace(T, N, H, device):
+    nbytes = _lib.load().pla_kda_prefill_workspace_bytes(T, N, H)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
+
+
 def flashkda_fwd(
     q: torch.Tensor,                       # [total_tokens, H, DK] bf16
     k: torch.Tensor,                       # [total_tokens, H, DK] bf16
@@ -148,9 +153,7 @@ def flashkda_fwd(
             final_state[rows] = fin32.to(final_state.dtype)
         return None
 
-    lib = _lib.load()
-    nbytes = lib.pla_kda_prefill_workspace_bytes(T, N, H)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+    ws, nbytes = _workspace(T, N, H, q.device)
     if final_state is not None and not (initial_state is not None and final_state.data_ptr() == initial_state.data_ptr()):
         # sequences of length zero keep their incoming (or zero) state
         if initial_state is not None:

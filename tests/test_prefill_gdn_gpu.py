@@ -10,6 +10,20 @@ from oracle import gdn_prefill_reference, chunked_delta_rule_fp64, softplus_gate
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def poisoned_workspace(monkeypatch):
+    """Every call of this file gets a workspace whose bytes are all 0xFF (NaN as FP32 and as fp16): a kernel that
+    reads a workspace word no kernel of the same call has written turns its results into NaN.  (The workspace
+    comes from torch.empty, so recycled memory may hold anything.)"""
+    from pla_amd.prefill.flashqla import ops
+
+    def workspace(T, N, Hg, H, device):
+        from pla_amd import _lib
+        nbytes = _lib.load().pla_gdn_prefill_workspace_bytes(T, N, Hg, H)
+        return torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=device), nbytes
+    monkeypatch.setattr(ops, "_workspace", workspace)
+
+
 def _run_workload(w, output_final_state=True):
     from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
     call = {k: v for k, v in w.items() if not k.startswith("_")}
@@ -172,6 +186,32 @@ def test_gdn_prefill_split_inputs_and_compact_state():
     torch.testing.assert_close(g_cum[0].cpu(), want, rtol=1e-5, atol=1e-6)
 
 
+def test_gdn_prefill_without_normalisation_on_a_poisoned_workspace_fused_sweep():
+    """normalize_qk=False through the fused sweep (16-byte aligned rows, whole sequences, several chunks): the
+    preparation then writes no 1 / |k| factors, and the sweep must not read them (the workspace holds NaN)."""
+    from pla_amd.prefill.flashqla import chunk_gated_delta_rule_fwd
+    from oracle.prefill import token_recurrence
+    g = torch.Generator().manual_seed(11)
+    T, H, HV = 700, 2, 4
+    q = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
+    k = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
+    v = torch.randn(T, HV, 128, generator=g).bfloat16()
+    gate = -torch.rand(T, HV, generator=g) * 0.3
+    beta = torch.rand(T, HV, generator=g)
+    S0 = torch.randn(3, HV, 128, 128, generator=g) * 0.1
+    offs = [0, 130, 130, 700]
+    exp_o, exp_final = token_recurrence(q, k, v, gate, beta, offs, S0, scale=128 ** -0.5)
+    dev = "cuda"
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    _, _, o, _, final = chunk_gated_delta_rule_fwd(
+        q[None].to(dev), k[None].to(dev), v[None].to(dev), gate[None].to(dev), beta[None].to(dev),
+        initial_state=S0.to(dev), cu_seqlens=cu)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(final).all()
+    torch.testing.assert_close(o[0].cpu().float(), exp_o, atol=2e-2, rtol=2e-2)
+    assert max(rel_l2(final[n], exp_final[n]) for n in range(3)) <= 1e-3
+
+
 @pytest.mark.parametrize("seed,tokens", [(348, 32810), (303, 41582)])
 def test_config3_gdn_prefill_32k_varlen(seed, tokens):
     """Config 3 at full size.  Seed 348 is the workload bench.py times (32 810 tokens, its lengths sum closest to
@@ -280,6 +320,44 @@ def test_gdn_prefill_staged_pipeline_in_a_graph():
         assert scratch == scratch
         assert torch.equal(o_graph, o_eager), replay
         assert torch.equal(w["initial_state"], pool_eager), replay
+
+
+def test_gdn_prefill_twenty_staged_calls_in_one_graph():
+    """One capture holding more staged calls than the library keeps side streams (a model with twenty GDN layers):
+    a side stream that has joined a capture is taken again by the later calls of that capture.  The calls chain on
+    one pool, so every call's result depends on all calls before it; three replays reproduce the eager chain bit
+    for bit."""
+    from pla_amd.workloads import gdn_prefill_packed
+    lengths = [1500, 2100, 900, 1500, 1300, 1100, 700, 1200]
+    layers = 20
+    w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 2, seed=77)
+    pool0 = w["initial_state"].clone()
+    o_eager = [_run_workload(w, output_final_state=False)[2] for _ in range(layers)]
+    torch.cuda.synchronize()
+    pool_eager = w["initial_state"].clone()
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    w["initial_state"].copy_(pool0)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=stream):
+        o_graph = [_run_workload(w, output_final_state=False)[2] for _ in range(layers)]
+    for replay in range(3):
+        w["initial_state"].copy_(pool0)
+        for o in o_graph:
+            o.zero_()
+        scratch = torch.randn(1 << 20, device="cuda").sum().item()     # eager work and a sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert scratch == scratch
+        for layer in range(layers):
+            assert torch.equal(o_graph[layer], o_eager[layer]), (replay, layer)
+        assert torch.equal(w["initial_state"], pool_eager), replay
+    # an eager call afterwards finds a side stream again (the capture has ended)
+    w["initial_state"].copy_(pool0)
+    o_after = _run_workload(w, output_final_state=False)[2]
+    torch.cuda.synchronize()
+    assert torch.equal(o_after, o_eager[0])
 
 
 def test_gdn_prefill_rows_aligned_to_4_bytes_only():

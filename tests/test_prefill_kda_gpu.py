@@ -9,6 +9,19 @@ from oracle import kda_prefill_reference, chunked_delta_rule_fp64, lower_bound_g
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def poisoned_workspace(monkeypatch):
+    """Every call of this file gets a workspace of 0xFF bytes (NaN as FP32 and as fp16), so a kernel that reads a
+    workspace word no kernel of the same call has written turns its results into NaN."""
+    from pla_amd.prefill.flashkdapro import ops
+
+    def workspace(T, N, H, device):
+        from pla_amd import _lib
+        nbytes = _lib.load().pla_kda_prefill_workspace_bytes(T, N, H)
+        return torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=device), nbytes
+    monkeypatch.setattr(ops, "_workspace", workspace)
+
+
 def _inputs(lengths, H, seed, pad=0, gate_scale=1.0):
     g = torch.Generator().manual_seed(seed)
     T = sum(lengths) + pad
