@@ -260,6 +260,59 @@ struct TileCopy {
   }
 };
 
+// ---------------------------------------------------------------------------------------------
+// Unpadded, swizzled 64 x 128 tiles of 16-bit values (16 KiB).  A row is sixteen 16-byte granules; granule g of row i
+// lies at granule g ^ (2 (i & 7)) of that row's 256 bytes.  Measured on gfx950 with all eight wavefronts of a workgroup
+// reading: 16-byte operand reads (sixteen consecutive rows, one granule index) run at the LDS peak of 256 bytes per
+// cycle and the transposing 8-byte reads (four rows x four 8-byte pieces per group of sixteen lanes) at the 128 bytes
+// per cycle of 8-byte reads, where rows padded to 272 bytes give 85 (two 8-byte reads per operand) and 128.
+//
+// Operand tiles (K, Q) also permute the columns inside each group of 32 so that the eight contraction elements a lane
+// feeds to one MFMA step - columns 32 s + 4 kb .. + 3 and 32 s + 16 + 4 kb .. + 3, the order in which a pair of
+// accumulator tiles presents its rows - are the two halves of ONE granule, index 4 s + kb.
+constexpr int TILE128_HALVES = CHUNK * 128;
+__device__ __forceinline__ int swizzled_granule(int row, int g) { return g ^ (2 * (row & 7)); }
+// offset (in 16-bit elements) of granule g of row `row`
+__device__ __forceinline__ int tile_offset(int row, int g) { return row * 128 + 8 * swizzled_granule(row, g); }
+// A (or B) operand of contraction step s for row `row` of an operand tile: one 16-byte read
+__device__ __forceinline__ bf16x8_t operand_granule(const uint16_t* tile, int row, int s, int kb) {
+  return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(tile + tile_offset(row, 4 * s + kb)));
+}
+// The same operand from the TRANSPOSE of an operand tile: lane (r, kb) takes rows [32 s + 4 kb, + 4) and
+// [32 s + 16 + 4 kb, + 4) of original column 16 m + r.  Lane t of a group of 16 addresses the four columns
+// 16 m + 4 (t % 4) .. + 3 of row base + t / 4, which are half (m & 1) of granule 4 (m / 2) + t % 4.
+__device__ __forceinline__ bf16x8_t operand_granule_transposed(const uint16_t* tile, int s, int m, int kb, int r) {
+  const int row = 32 * s + 4 * kb + (r >> 2);                  // (row + 16) & 7 == row & 7: both reads share the swizzle
+  const uint16_t* at = tile + tile_offset(row, 4 * (m >> 1) + (r & 3)) + 4 * (m & 1);
+  const i16x4_t p0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)at);
+  const i16x4_t p1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(at + 16 * 128));
+  typedef short i16x8_t __attribute__((ext_vector_type(8)));
+  const i16x8_t u = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+  return __builtin_bit_cast(bf16x8_t, u);
+}
+// Copy plan for a swizzled 64 x 128 tile whose columns keep their order (V): a 1 KiB piece is four rows, lane i of
+// the issuing wavefront fills physical granule i % 16 of row 4 piece + i / 16, which holds granule
+// (i % 16) ^ swizzle of that row.  Rows beyond `last_row` re-read that row.
+template <int WAVES>
+struct SwizzledTileCopy {
+  static constexpr int PIECES = TILE128_HALVES * 2 / 1024;
+  static_assert(PIECES % WAVES == 0, "every wavefront issues the same number of copies");
+  static constexpr int EACH = PIECES / WAVES;
+  uint32_t off[EACH];
+  __device__ __forceinline__ void plan(uint32_t row_pitch_b, int last_row, int wave, int lane) {
+#pragma unroll
+    for (int j = 0; j < EACH; ++j) {
+      const int row = 4 * (WAVES * j + wave) + (lane >> 4);
+      off[j] = (uint32_t)min(row, last_row) * row_pitch_b + 16u * (uint32_t)swizzled_granule(row, lane & 15);
+    }
+  }
+  __device__ __forceinline__ void issue(const void* tile, const char* gbase, int wave) const {
+    const uint32_t base = lds_address(tile) + 1024u * wave;
+#pragma unroll
+    for (int j = 0; j < EACH; ++j) dma16(gbase, off[j], base + 1024u * WAVES * j);
+  }
+};
+
 // Chunk table from cu_seqlens, built on the device so that no call reads offsets back to the host.
 // Single workgroup.  seq_chunk_off[n] = first chunk of sequence n (seq_chunk_off[N] = total).
 __device__ __forceinline__ void chunk_map(const int32_t* cu_seqlens, int N, int NC_max, int32_t* seq_chunk_off,

@@ -1090,7 +1090,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 template <typename act_t>
 __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefillParams p) {
   constexpr int NB = 2, CW = 4, AUX = 4;
-  using CopyV = TileCopy<CHUNK, 2 * PITCH128, 256, AUX>;
+  using CopyV = SwizzledTileCopy<AUX>;
   const int block = xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV);
   if (block < 0) return;
   const SweepRole role = select_sweep(0, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
@@ -1107,9 +1107,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tQ[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  // K and Q: swizzled operand tiles (columns permuted inside groups of 32); V: swizzled, columns in order
+  __shared__ __align__(16) uint16_t tK[2][TILE128_HALVES];
+  __shared__ __align__(16) uint16_t tQ[2][TILE128_HALVES];
+  __shared__ __align__(16) uint16_t tV[2][TILE128_HALVES];
   __shared__ __align__(16) uint16_t tW[2][2 * TRI_BLOCKS * 512];    // [parity][hi blocks, lo blocks]
   __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
   // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}, [256,320) G
@@ -1171,7 +1172,18 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       // they are written as they are (fp16 of the raw value) and 1 / |q| goes to tRq, from where it enters the
       // output through the row factor scale e^G and P through its row factor.
       auto write_rows = [&](int c, const uint4 (&raw)[8], const float (&inv_in)[8]) {
-        uint16_t* const T = (q_side ? tQ[c & 1] : tK[c & 1]) + (row0 + lr) * PITCH128 + 8 * lc;
+        // The lane's 16 bytes are columns 8 lc .. 8 lc + 7 of row row0 + lr + 4 j: the first 8 bytes belong to granule
+        // 4 (lc / 4) + 2 (lc % 2), half (lc / 2) % 2, the other 8 to the granule after it (same half).  The row's swizzle
+        // 2 (row & 7) = 2 lr + 8 (j & 1) is even, so the second granule lies 16 bytes after the first.
+        uint16_t* const tile = q_side ? tQ[c & 1] : tK[c & 1];
+        const int g0 = 4 * (lc >> 2) + 2 * (lc & 1), half = (lc >> 1) & 1;
+        uint16_t* const T_even = tile + (row0 + lr) * 128 + 8 * (g0 ^ (2 * lr)) + 4 * half;        // j even
+        uint16_t* const T_odd = tile + (row0 + lr) * 128 + 8 * (g0 ^ (2 * lr + 8)) + 4 * half;     // j odd
+        auto put = [&](int j, uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+          uint16_t* const at = ((j & 1) ? T_odd : T_even) + 4 * j * 128;
+          *reinterpret_cast<uint2*>(at) = make_uint2(w0, w1);
+          *reinterpret_cast<uint2*>(at + 8) = make_uint2(w2, w3);
+        };
         const int len = chunk_len(c);
         if constexpr (q_side) {
           float ss[8];
@@ -1187,7 +1199,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
               w[e] = pack2_rtz(a0, a1);
             }
             ss[j] = acc;
-            *reinterpret_cast<uint4*>(T + 4 * j * PITCH128) = make_uint4(w[0], w[1], w[2], w[3]);
+            put(j, w[0], w[1], w[2], w[3]);
           }
 #pragma unroll
           for (int j = 0; j < 8; ++j) ss[j] = row16_allreduce(ss[j]);
@@ -1208,7 +1220,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
               const uint32_t r = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
               w[e] = pack2_rtz(lo16<act_t>(r), hi16<act_t>(r));
             }
-            *reinterpret_cast<uint4*>(T + 4 * j * PITCH128) = make_uint4(w[0], w[1], w[2], w[3]);
+            put(j, w[0], w[1], w[2], w[3]);
           }
         }
       };
@@ -1223,11 +1235,11 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
           constexpr int halves = 2 * s + 1 > ni ? 1 : 2;        // (nj, ni) products of this block that are not all zero
           bf16x8_t qb[4], kb_op[halves][4];
 #pragma unroll
-          for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_from(Q + (16 * ni + r16) * PITCH128, s2, kb);
+          for (int s2 = 0; s2 < 4; ++s2) qb[s2] = operand_granule(Q, 16 * ni + r16, s2, kb);
 #pragma unroll
           for (int half = 0; half < halves; ++half)
 #pragma unroll
-            for (int s2 = 0; s2 < 4; ++s2) kb_op[half][s2] = operand_from(K + (16 * (2 * s + half) + r16) * PITCH128, s2, kb);
+            for (int s2 = 0; s2 < 4; ++s2) kb_op[half][s2] = operand_granule(K, 16 * (2 * s + half) + r16, s2, kb);
           const int i = 16 * ni + r16;
           const float Gi = G[i];
           const float pre = p.scale * tRq[c & 1][i];
@@ -1319,8 +1331,11 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     }
   }
   uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.HV + hv) * 128 + vbase + 4 * kb;
-  const int rowA128 = r16 * PITCH128, rowA64 = r16 * PITCH64;
-  const int trV = (4 * kb + (r16 >> 2)) * PITCH128 + vbase + 4 * (r16 & 3);
+  // V through the transposing read: lane t of a group addresses columns vbase + 16 nb + 4 (t % 4) .. + 3 of row
+  // 16 mi + 4 kb + t / 4, i.e. half (t % 2) of granule 4 wave + 2 nb + (t % 4) / 2; the swizzle 8 (kb & 1) + 2 (t / 4)
+  // of that row does not depend on mi, and block nb = 1 differs from nb = 0 in one bit of the granule index
+  const int trV = (4 * kb + (r16 >> 2)) * 128 + 8 * ((4 * wave + ((r16 & 3) >> 1)) ^ (8 * (kb & 1) + 2 * (r16 >> 2))) + 4 * (r16 & 1);
+  auto v_at = [&](const uint16_t* V, int mi, int nb) { return V + ((trV + 16 * 128 * mi) ^ (16 * nb)); };
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
   auto pk = [](float x, float y) { return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x, y)); };
@@ -1347,8 +1362,8 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     const uint16_t* const Wt = tW[par];
     const uint16_t* const Pt = tP;
     const float* const G = tG[par];
-    auto ldK = [&](int j) { return operand_from(K + 16 * (j & 3) * PITCH128 + rowA128, j >> 2, kb); };
-    auto ldQ = [&](int j) { return operand_from(Q + 16 * (j & 3) * PITCH128 + rowA128, j >> 2, kb); };
+    auto ldK = [&](int j) { return operand_granule(K, 16 * (j & 3) + r16, j >> 2, kb); };
+    auto ldQ = [&](int j) { return operand_granule(Q, 16 * (j & 3) + r16, j >> 2, kb); };
     // W operands in the order they are used: 0-3 lo (s 0, m 0..3), 4-7 hi (s 0), 8-9 lo (s 1, m 2, 3), 10-11 hi (s 1);
     // block b = m for s 0, 4 and 5 for s 1 (tri_block_m / tri_block_s), hi blocks first in the tile, then lo
     auto w_blk = [](int w) { return w < 8 ? (w & 3) : 4 + (w & 1); };
@@ -1385,10 +1400,10 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       if (j + 6 < 16) ka[j + 6] = ldK(j + 6);
       else if (j == 10) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) { vraw[0][nb] = read_tr4(V + trV + 16 * nb); vraw[1][nb] = read_tr4(V + trV + 16 * PITCH128 + 16 * nb); }
+        for (int nb = 0; nb < NB; ++nb) { vraw[0][nb] = read_tr4(v_at(V, 0, nb)); vraw[1][nb] = read_tr4(v_at(V, 1, nb)); }
       } else if (j == 11) {
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) { vraw[2][nb] = read_tr4(V + trV + 32 * PITCH128 + 16 * nb); vraw[3][nb] = read_tr4(V + trV + 48 * PITCH128 + 16 * nb); }
+        for (int nb = 0; nb < NB; ++nb) { vraw[2][nb] = read_tr4(v_at(V, 2, nb)); vraw[3][nb] = read_tr4(v_at(V, 3, nb)); }
       } else if (j == 12) {
 #pragma unroll
         for (int m2 = 0; m2 < 4; ++m2) eg[m2] = *reinterpret_cast<const float4*>(&G[64 + 16 * m2 + 4 * kb]);
@@ -1500,7 +1515,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 #pragma unroll
     for (int i = 0; i < 6; ++i) {
       const int s = p_s(i), ni = p_ni(i);
-      if (i >= 2) kt[i - 2] = operand_transposed(K, 0, i - 2, kb, r16);       // kt[0..3]: (s 0, mc 0..3)
+      if (i >= 2) kt[i - 2] = operand_granule_transposed(K, 0, i - 2, kb, r16);       // kt[0..3]: (s 0, mc 0..3)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) OT[nb][ni] = mfma16h(op(ur[s][nb]), pa[i], OT[nb][ni]);
       if (i < 4) {
@@ -1532,8 +1547,8 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       const int pair = k >> 1, s = pair >> 2, mc0 = 2 * (pair & 3);
       const bool hi_part = k & 1;
       if (!hi_part && 2 * pair + 4 < 16) {
-        kt[2 * pair + 4] = operand_transposed(K, (2 * pair + 4) >> 3, (2 * pair + 4) & 7, kb, r16);
-        kt[2 * pair + 5] = operand_transposed(K, (2 * pair + 5) >> 3, (2 * pair + 5) & 7, kb, r16);
+        kt[2 * pair + 4] = operand_granule_transposed(K, (2 * pair + 4) >> 3, (2 * pair + 4) & 7, kb, r16);
+        kt[2 * pair + 5] = operand_granule_transposed(K, (2 * pair + 5) >> 3, (2 * pair + 5) & 7, kb, r16);
       }
       if (k == 0) {
         dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
