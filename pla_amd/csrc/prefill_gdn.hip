@@ -1107,15 +1107,24 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  // K and Q: swizzled operand tiles (columns permuted inside groups of 32); V: swizzled, columns in order
-  __shared__ __align__(16) uint16_t tK[2][TILE128_HALVES];
-  __shared__ __align__(16) uint16_t tQ[2][TILE128_HALVES];
-  __shared__ __align__(16) uint16_t tV[2][TILE128_HALVES];
-  __shared__ __align__(16) uint16_t tW[2][2 * TRI_BLOCKS * 512];    // [parity][hi blocks, lo blocks]
-  __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
+  // K and Q: swizzled operand tiles (columns permuted inside groups of 32); V: swizzled, columns in order.  All of the
+  // workgroup's LDS is ONE array with a fixed layout: what is read at many constant offsets from one per-lane address
+  // (the blocks of P and W, the decay factors) lies in the first 64 KiB, where those offsets fit the 16-bit offset
+  // field of an LDS instruction; above that every distinct offset would cost a register for its address.
+  constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;       // hi blocks, then lo blocks
+  constexpr int OFF_P = 0, OFF_G = OFF_P + TRI_BLOCKS * 1024, OFF_RQ = OFF_G + 2 * 2048;
+  constexpr int OFF_W = (OFF_RQ + 2 * CHUNK * 4 + 1023) / 1024 * 1024, OFF_Q = OFF_W + 2 * W_HALVES * 2;
+  constexpr int OFF_K = OFF_Q + 2 * TILE128_HALVES * 2, OFF_V = OFF_K + 2 * TILE128_HALVES * 2;
+  constexpr int LDS_BYTES = OFF_V + 2 * TILE128_HALVES * 2;
+  __shared__ __align__(1024) unsigned char lds_all[LDS_BYTES];
+  uint16_t* const tP = reinterpret_cast<uint16_t*>(lds_all + OFF_P);
   // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}, [256,320) G
-  __shared__ __align__(16) float tG[2][512];
-  __shared__ __align__(16) float tRq[2][CHUNK];        // 1 / |q| per row of the Q tile
+  float (*const tG)[512] = reinterpret_cast<float (*)[512]>(lds_all + OFF_G);                       // [2][512]
+  float (*const tRq)[CHUNK] = reinterpret_cast<float (*)[CHUNK]>(lds_all + OFF_RQ);                 // [2][64]: 1 / |q| per row of the Q tile
+  uint16_t (*const tW)[W_HALVES] = reinterpret_cast<uint16_t (*)[W_HALVES]>(lds_all + OFF_W);       // [parity][hi blocks, lo blocks]
+  uint16_t (*const tQ)[TILE128_HALVES] = reinterpret_cast<uint16_t (*)[TILE128_HALVES]>(lds_all + OFF_Q);
+  uint16_t (*const tK)[TILE128_HALVES] = reinterpret_cast<uint16_t (*)[TILE128_HALVES]>(lds_all + OFF_K);
+  uint16_t (*const tV)[TILE128_HALVES] = reinterpret_cast<uint16_t (*)[TILE128_HALVES]>(lds_all + OFF_V);
 
   if (wave >= CW) {
     // ---- the feeding wavefronts: one instance of this code per wavefront (its role is a compile-time constant) ----
@@ -1336,6 +1345,29 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   // of that row does not depend on mi, and block nb = 1 differs from nb = 0 in one bit of the granule index
   const int trV = (4 * kb + (r16 >> 2)) * 128 + 8 * ((4 * wave + ((r16 & 3) >> 1)) ^ (8 * (kb & 1) + 2 * (r16 >> 2))) + 4 * (r16 & 1);
   auto v_at = [&](const uint16_t* V, int mi, int nb) { return V + ((trV + 16 * 128 * mi) ^ (16 * nb)); };
+  // Byte offsets of this lane's operand reads inside an operand tile.  The granule index enters the address in bits 4-7
+  // and the swizzle is an exclusive or, so a step (or a group of 32 columns) further is one exclusive or of the WHOLE
+  // address with 64 s (tile bases are multiples of 256); row blocks and halves are constant offsets of the read.
+  // Only these two values are kept across chunks: a chunk derives its addresses from them behind an opaque
+  // statement, so that the compiler does not carry one register per (tile, step) through the whole loop.
+  const uint32_t offA0 = 2 * tile_offset(r16, kb);                          // row r16, granule kb (step 0)
+  const uint32_t offT0 = 2 * tile_offset(4 * kb + (r16 >> 2), r16 & 3);     // transposing reads: row 4 kb + r16 / 4, granule r16 % 4
+  typedef const __attribute__((address_space(3))) unsigned char* lds_bytes_t;
+  auto opaque = [](uint32_t x) { asm volatile("" : "+v"(x)); return x; };
+  auto read_operand = [](uint32_t base, int step, int byte_offset) {
+    const lds_bytes_t at = (lds_bytes_t)(uintptr_t)(base ^ (64u * step));
+    return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const __attribute__((address_space(3))) u32x4_t*>(at + byte_offset));
+  };
+  // K^T operand (contraction half s2, column block m) = two transposing reads 16 rows apart
+  auto read_transposed = [](uint32_t base, int s2, int m) {
+    const lds_bytes_t at = (lds_bytes_t)(uintptr_t)(base ^ (64u * (m >> 1)));
+    typedef __attribute__((address_space(3))) i16x4_t* tr_ptr_t;
+    const i16x4_t p0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(at + 8192 * s2 + 8 * (m & 1)));
+    const i16x4_t p1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_ptr_t)(at + 8192 * s2 + 8 * (m & 1) + 4096));
+    typedef short i16x8_t __attribute__((ext_vector_type(8)));
+    const i16x8_t u = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+    return __builtin_bit_cast(bf16x8_t, u);
+  };
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 
   auto pk = [](float x, float y) { return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(x, y)); };
@@ -1362,8 +1394,9 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     const uint16_t* const Wt = tW[par];
     const uint16_t* const Pt = tP;
     const float* const G = tG[par];
-    auto ldK = [&](int j) { return operand_granule(K, 16 * (j & 3) + r16, j >> 2, kb); };
-    auto ldQ = [&](int j) { return operand_granule(Q, 16 * (j & 3) + r16, j >> 2, kb); };
+    const uint32_t kA = opaque(lds_address(K) + offA0), qA = opaque(lds_address(Q) + offA0), kT = opaque(lds_address(K) + offT0);
+    auto ldK = [&](int j) { return read_operand(kA, j >> 2, 4096 * (j & 3)); };
+    auto ldQ = [&](int j) { return read_operand(qA, j >> 2, 4096 * (j & 3)); };
     // W operands in the order they are used: 0-3 lo (s 0, m 0..3), 4-7 hi (s 0), 8-9 lo (s 1, m 2, 3), 10-11 hi (s 1);
     // block b = m for s 0, 4 and 5 for s 1 (tri_block_m / tri_block_s), hi blocks first in the tile, then lo
     auto w_blk = [](int w) { return w < 8 ? (w & 3) : 4 + (w & 1); };
@@ -1515,7 +1548,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 #pragma unroll
     for (int i = 0; i < 6; ++i) {
       const int s = p_s(i), ni = p_ni(i);
-      if (i >= 2) kt[i - 2] = operand_granule_transposed(K, 0, i - 2, kb, r16);       // kt[0..3]: (s 0, mc 0..3)
+      if (i >= 2) kt[i - 2] = read_transposed(kT, 0, i - 2);       // kt[0..3]: (s 0, mc 0..3)
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) OT[nb][ni] = mfma16h(op(ur[s][nb]), pa[i], OT[nb][ni]);
       if (i < 4) {
@@ -1547,8 +1580,8 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       const int pair = k >> 1, s = pair >> 2, mc0 = 2 * (pair & 3);
       const bool hi_part = k & 1;
       if (!hi_part && 2 * pair + 4 < 16) {
-        kt[2 * pair + 4] = operand_granule_transposed(K, (2 * pair + 4) >> 3, (2 * pair + 4) & 7, kb, r16);
-        kt[2 * pair + 5] = operand_granule_transposed(K, (2 * pair + 5) >> 3, (2 * pair + 5) & 7, kb, r16);
+        kt[2 * pair + 4] = read_transposed(kT, (2 * pair + 4) >> 3, (2 * pair + 4) & 7);
+        kt[2 * pair + 5] = read_transposed(kT, (2 * pair + 5) >> 3, (2 * pair + 5) & 7);
       }
       if (k == 0) {
         dg[1][0] = *reinterpret_cast<const float4*>(&G[128 + 32 + 4 * kb]);
