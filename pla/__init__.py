@@ -21,14 +21,23 @@ __all__ = []
 
 
 class _AliasLoader(importlib.abc.Loader):
+    """Hands importlib the pla_amd module itself.  importlib then stamps the alias spec (and loader) on whatever
+    module a loader returns; ``exec_module`` puts the module's own ones back, so that ``pla_amd.X`` keeps
+    ``__spec__.name == "pla_amd.X"`` (relative imports inside it, ``importlib.reload`` and ``pkgutil`` go on
+    using the real spec) while ``sys.modules["pla.X"]`` is the same object."""
+
     def __init__(self, target):
         self._target = target
+        self._own = None
 
     def create_module(self, spec):
-        return importlib.import_module(self._target)      # the pla_amd module itself, not a copy
+        module = importlib.import_module(self._target)    # the pla_amd module itself, not a copy
+        self._own = (module.__spec__, getattr(module, "__loader__", None))
+        return module
 
     def exec_module(self, module):
-        pass
+        if self._own is not None:
+            module.__spec__, module.__loader__ = self._own
 
 
 class _AliasFinder(importlib.abc.MetaPathFinder):

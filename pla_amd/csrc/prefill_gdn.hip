@@ -1698,13 +1698,18 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_sta
 // array's name is only a handle for the runtime, not a device address; the address on the current device comes from
 // hipGetSymbolAddress, is looked up once per device and is what kernels and launches receive.
 static __device__ __align__(256) unsigned char scratch[PLA_GDN_PREFILL_STATIC_BYTES];
-static void* static_scratch_address() {
+// The first look-up on a device may load the code object, which must not happen while `stream` captures a graph: a
+// capturing caller that has not called the entry point on this device before gets CAPTURE_BEFORE_LOOKUP back.
+static void* const CAPTURE_BEFORE_LOOKUP = reinterpret_cast<void*>(1);
+static void* static_scratch_address(hipStream_t stream) {
   static void* address[64] = {};
   static std::mutex guard;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
   std::lock_guard<std::mutex> lock(guard);
   if (address[dev] == nullptr) {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &status) != hipSuccess || status != hipStreamCaptureStatusNone) return CAPTURE_BEFORE_LOOKUP;
     void* ptr = nullptr;
     if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
     address[dev] = ptr;
@@ -1750,7 +1755,10 @@ static int gdn_prefill_run(
     PLA_REQUIRE((int64_t)L.total <= PLA_GDN_PREFILL_STATIC_BYTES,
                 "call too large for the built-in scratch array: it needs %zu bytes of workspace, the array holds %lld "
                 "(use pla_gdn_prefill_launch with a caller workspace)", L.total, (long long)PLA_GDN_PREFILL_STATIC_BYTES);
-    workspace = static_scratch_address();
+    workspace = static_scratch_address(reinterpret_cast<hipStream_t>(stream));
+    PLA_REQUIRE(workspace != CAPTURE_BEFORE_LOOKUP,
+                "the first call of pla_gdn_prefill_launch_static on a device looks up the scratch array's address and must "
+                "not be captured: call it once on this device before capturing");
     PLA_REQUIRE(workspace != nullptr, "hipGetSymbolAddress failed for the built-in scratch array");
   } else {
     PLA_REQUIRE(workspace != nullptr, "null tensor pointer");

@@ -63,6 +63,21 @@ def _check(cond, msg):
         raise RuntimeError(msg)
 
 
+# Messages name dtypes and shapes the way the compiled host layer (and the reference's C++) prints them: the scalar
+# type's name ("Half", "Float", "BFloat16") and sizes in brackets.
+_CPP_DTYPE = {torch.float16: "Half", torch.bfloat16: "BFloat16", torch.float32: "Float", torch.float64: "Double",
+              torch.int32: "Int", torch.int64: "Long", torch.int16: "Short", torch.int8: "Char", torch.uint8: "Byte",
+              torch.bool: "Bool"}
+
+
+def _dt(dtype):
+    return _CPP_DTYPE.get(dtype, str(dtype))
+
+
+def _sizes(shape):
+    return "[" + ", ".join(str(int(n)) for n in shape) + "]"
+
+
 def _sanity_enabled():
     # Read on every call (src/sanity_check.h:50-53).
     return os.environ.get("PLA_SANITY_CHECK", "0") == "1"
@@ -122,7 +137,7 @@ def _packed_impl(mixed_qkv, a, b, A_log, dt_bias, softplus_beta, softplus_thresh
     _check(a.dtype == mixed_qkv.dtype and b.dtype == mixed_qkv.dtype and dt_bias.dtype == mixed_qkv.dtype
            and out.dtype == mixed_qkv.dtype, "a, b, dt_bias and out must have mixed_qkv's dtype")
     _check(state.dtype in (torch.float32, torch.bfloat16),
-           f"k-last state dtype must be float32 or bfloat16, got {state.dtype}")
+           f"k-last state dtype must be float32 or bfloat16, got {_dt(state.dtype)}")
     _check(mixed_qkv.stride(1) == 1 and state.stride(-1) == 1 and state.stride(-2) == K
            and state.stride(-3) == V * K, "mixed_qkv rows and state slots must be dense")
     _check(out.is_contiguous(), "out must be contiguous")
@@ -220,8 +235,8 @@ def _resolve_out(out, v):
     if out is None:
         return torch.empty(v.shape, dtype=v.dtype, device=v.device)
     _check(out.device == v.device, f"out must be on the same device as v, got {out.device} vs {v.device}")
-    _check(out.dtype == v.dtype, f"out dtype must match v ({v.dtype}), got {out.dtype}")
-    _check(out.shape == v.shape, f"out shape must match v {tuple(v.shape)}, got {tuple(out.shape)}")
+    _check(out.dtype == v.dtype, f"out dtype must match v ({_dt(v.dtype)}), got {_dt(out.dtype)}")
+    _check(out.shape == v.shape, f"out shape must match v {_sizes(v.shape)}, got {_sizes(out.shape)}")
     _check(out.is_contiguous(), "out must be contiguous")
     return out
 
@@ -261,7 +276,7 @@ def _k_last_impl(A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, 
     H, HV, K, V = _k_last_heads(q, k, v, a, b, A_log, dt_bias, state, cache, is_kda)
     state_dtype = state.dtype if state is not None else (cache.dtype if cache is not None else torch.float32)
     _check(state_dtype in (torch.float32, torch.bfloat16),
-           f"k-last state dtype must be float32 or bfloat16, got {state_dtype}")
+           f"k-last state dtype must be float32 or bfloat16, got {_dt(state_dtype)}")
     _check(cache is None or cache.dtype == state_dtype,
            "initial_state_source and intermediate_states_buffer must have the same dtype")
 
@@ -294,8 +309,8 @@ def _k_last_impl(A_log, a, dt_bias, softplus_beta, softplus_threshold, q, k, v, 
     mtp_verify = T_max > 1 or bool(disable_state_update) or target_verify
     want = torch.float32 if (is_kda and mtp_verify) else q.dtype
     _check(dt_bias.dtype == want,
-           f"dt_bias must be {want} here (is_kda={is_kda}, mtp_verify={mtp_verify}): only KDA MTP "
-           f"verify reads it as float32, every other path reads it as q's dtype. Got {dt_bias.dtype}")
+           f"dt_bias must be {_dt(want)} here (is_kda={int(bool(is_kda))}, mtp_verify={int(bool(mtp_verify))}): only KDA MTP "
+           f"verify reads it as float32, every other path reads it as q's dtype. Got {_dt(dt_bias.dtype)}")
 
     for name, t in (("cu_seqlens", cu_seqlens), ("initial_state_indices", idx)):
         if t is not None:

@@ -479,3 +479,96 @@ def test_sanity_mode_rejects_before_launch_and_bypass_flag(monkeypatch):
         packed(**kw)
     torch.cuda.synchronize()
     assert torch.equal(backing, before)
+
+
+def _reject_cases():
+    """(name, kernel, edit) for calls both host layers must refuse: `edit` changes the keyword arguments of a valid
+    T = 1 case (packed or not) in place."""
+    def sl(key, index):
+        def edit(kw):
+            kw[key] = kw[key][index].contiguous()
+        return edit
+
+    def put(key, value):
+        def edit(kw):
+            kw[key] = value(kw) if callable(value) else value
+        return edit
+
+    cases = [
+        ("no_state", "packed", put("initial_state_source", None)),
+        ("state_rank", "packed", put("initial_state_source", lambda kw: kw["initial_state_source"][0])),
+        ("head_dim", "packed", put("initial_state_source", lambda kw: kw["initial_state_source"][..., :64].contiguous())),
+        ("qkv_rank", "packed", put("mixed_qkv", lambda kw: kw["mixed_qkv"][None])),
+        ("qkv_width", "packed", sl("mixed_qkv", (slice(None), slice(0, -1)))),
+        ("head_ratio", "packed", put("mixed_qkv", lambda kw: kw["mixed_qkv"].new_zeros(3, (2 * 5 + 18) * 128))),
+        ("a_width", "packed", sl("a", (Ellipsis, slice(0, -1)))),
+        ("b_width", "packed", sl("b", (Ellipsis, slice(0, -1)))),
+        ("A_log", "packed", sl("A_log", (slice(0, -1),))),
+        ("dt_bias", "packed", sl("dt_bias", (Ellipsis, slice(0, -1)))),
+        ("out_shape", "packed", put("out", lambda kw: kw["out"][:, :, :-1].contiguous())),
+        ("cpu_qkv", "packed", put("mixed_qkv", lambda kw: kw["mixed_qkv"].cpu())),
+        ("act_dtype", "packed", put("mixed_qkv", lambda kw: kw["mixed_qkv"].float())),
+        ("mixed_dtypes", "packed", put("b", lambda kw: kw["b"].half())),
+        ("state_dtype", "packed", put("initial_state_source", lambda kw: kw["initial_state_source"].half())),
+        ("qkv_rows", "packed", put("mixed_qkv", lambda kw: kw["mixed_qkv"].t().contiguous().t())),
+        ("out_strided", "packed", put("out", lambda kw: torch.empty(*kw["out"].shape[:-1], 256, dtype=kw["out"].dtype, device="cuda")[..., ::2])),
+        ("cu_dtype", "packed", put("cu_seqlens", lambda kw: kw["cu_seqlens"].long())),
+        ("idx_dtype", "packed", put("initial_state_indices", lambda kw: kw["initial_state_indices"].long())),
+        ("lower_bound_gdn", "k_last_gdn", put("lower_bound", -5.0)),
+        ("accepted_dtype", "k_last", put("cache_steps_or_num_accept", lambda kw: torch.ones(3, dtype=torch.int64, device="cuda"))),
+        ("vllm_table_sglang", "k_last", put("initial_state_indices", lambda kw: kw["initial_state_indices"][:, None].contiguous())),
+        ("q_rank", "k_last", put("q", lambda kw: kw["q"][0])),
+        ("zero_heads", "k_last", lambda kw: kw.update(q=kw["q"][:, :, :0].contiguous(), k=kw["k"][:, :, :0].contiguous())),
+        ("head_ratio", "k_last", lambda kw: kw.update(q=kw["q"][:, :, :5].contiguous(), k=kw["k"][:, :, :5].contiguous())),
+        ("qk_shapes", "k_last", put("q", lambda kw: kw["q"][:, :, :3].contiguous())),
+        ("a_width", "k_last", sl("a", (Ellipsis, slice(0, -1)))),
+        ("b_width", "k_last", sl("b", (Ellipsis, slice(0, -1)))),
+        ("A_log", "k_last", sl("A_log", (slice(0, -1),))),
+        ("state_heads", "k_last", put("initial_state_source", lambda kw: kw["initial_state_source"][:, :-1].contiguous())),
+        ("state_dtype", "k_last", put("initial_state_source", lambda kw: kw["initial_state_source"].half())),
+        ("cpu_q", "k_last", put("q", lambda kw: kw["q"].cpu())),
+        ("act_dtype", "k_last", lambda kw: kw.update({n: kw[n].float() for n in ("q", "k", "v", "a", "b")})),
+        ("mixed_dtypes", "k_last", put("k", lambda kw: kw["k"].half())),
+        ("out_dtype", "k_last", put("out", lambda kw: torch.empty_like(kw["v"]).float())),
+        ("out_shape", "k_last", put("out", lambda kw: torch.empty_like(kw["v"])[:, :, :-1].contiguous())),
+        ("dt_bias_dtype", "k_last", put("dt_bias", lambda kw: kw["dt_bias"].float())),
+        ("cu_dtype", "k_last", put("cu_seqlens", lambda kw: kw["cu_seqlens"].long())),
+        ("idx_dtype", "k_last", put("initial_state_indices", lambda kw: kw["initial_state_indices"].long())),
+    ]
+    return cases
+
+
+@pytest.mark.parametrize("name,kernel,edit", _reject_cases(), ids=lambda v: v if isinstance(v, str) else "")
+def test_compiled_and_python_host_layers_reject_the_same_calls(name, kernel, edit):
+    """The decode checks exist twice: compiled (pla.decode._C, the path every call takes) and in Python (the
+    PLA_SANITY_CHECK diagnostics and the tunable entry points).  Every call one of them refuses the other refuses
+    too, with the same exception type and the same message, and neither touches the pool."""
+    import pla_amd.decode as dec
+    native = dec._compiled()
+    assert native, "pla_amd.decode._C is not importable"
+    args, backing, _, _, _ = make_k_last_case(kernel != "k_last_gdn", "decode", H=6, HV=18)
+    before = backing.clone()
+    caught = []
+    for layer in ("compiled", "python"):
+        kw = packed_from(args) if kernel == "packed" else dict(args, lower_bound=None, is_sglang=True, out=torch.empty_like(args["v"]))
+        edit(kw)
+        if kernel == "packed":
+            order = ["mixed_qkv", "a", "b", "A_log", "dt_bias", "softplus_beta", "softplus_threshold", "scale",
+                     "initial_state_source", "initial_state_indices", "out", "use_qk_l2norm_in_kernel", "cu_seqlens",
+                     "is_kda", "is_sglang"]
+            call = native.fused_sigmoid_gating_delta_rule_forward_k_last_packed if layer == "compiled" else \
+                (lambda *a: dec._packed_impl(*a, None))
+        else:
+            order = ["A_log", "a", "dt_bias", "softplus_beta", "softplus_threshold", "q", "k", "v", "b",
+                     "initial_state_source", "initial_state_indices", "scale", "use_qk_l2norm_in_kernel", "cu_seqlens",
+                     "is_kda", "disable_state_update", "intermediate_states_buffer", "intermediate_state_indices",
+                     "cache_steps_or_num_accept", "retrieve_parent_token", "lower_bound", "is_sglang", "out"]
+            call = native.fused_sigmoid_gating_delta_rule_forward_k_last if layer == "compiled" else \
+                (lambda *a: dec._k_last_impl(*a, None))
+        with pytest.raises(Exception) as info:
+            call(*[kw[n] for n in order])
+        caught.append((type(info.value), str(info.value).splitlines()[0]))
+    torch.cuda.synchronize()
+    assert caught[0] == caught[1], caught
+    assert caught[0][0] is RuntimeError
+    assert torch.equal(backing, before)

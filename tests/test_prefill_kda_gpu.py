@@ -243,8 +243,8 @@ def test_config4_kda_prefill_strong_and_weak_decay_prefix():
 
 
 def test_config4_kda_prefill_full_size():
-    """Config 4 at its full size (one sequence of 65536 tokens, 32 heads).  Three heads (strong
-    decay, first weak-decay head, last head) are checked against the float64 chunked oracle over
+    """Config 4 at its full size (one sequence of 65536 tokens, 32 heads).  Eight heads (four that decay
+    strongly, four that decay weakly) are checked against the float64 chunked oracle over
     the whole sequence; every head is checked through the chained-calls invariant: two calls
     that split the sequence at a chunk boundary and pass the state on give the same o and final
     state."""
@@ -279,7 +279,7 @@ def test_config4_kda_prefill_full_size():
     for head in range(H):
         assert rel_l2(fin[0, head], call["final_state"][0, head]) <= 5e-4, head
 
-    heads = [0, H // 2, H - 1]
+    heads = [0, 5, 10, 15, 16, 21, 26, 31]                  # four strongly and four weakly decaying heads
     cpu = {k: (v.cpu() if torch.is_tensor(v) else v) for k, v in call.items()}
     sel = lambda t: t[:, heads].contiguous()
     exp_o, exp_final = _oracle(sel(cpu["q"]), sel(cpu["k"]), sel(cpu["v"]), sel(cpu["g"]), sel(cpu["beta"]),
@@ -287,6 +287,48 @@ def test_config4_kda_prefill_full_size():
     torch.testing.assert_close(call["out"][:, heads].cpu().float(), exp_o.float(), atol=2e-2, rtol=2e-2)
     for i, head in enumerate(heads):
         assert rel_l2(call["final_state"][0, head], exp_final[0, i]) <= 1e-3, head
+
+
+@pytest.mark.parametrize("lengths,H", [([700, 0, 130, 64, 1], 24), ([4096, 40], 2)])
+def test_kda_prefill_in_a_graph(lengths, H):
+    """flashkda_fwd allocates (workspace) and launches only, so it can be captured: a call of whole sequences (more
+    than 64 chains) and a call that is split into segments (zero-state / identity sweeps, combine, second sweep),
+    each replayed three times with eager work and a synchronisation in between, reproduce the eager result bit for
+    bit (outputs and written-back states)."""
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=77 + H, pad=3)
+    dev = "cuda"
+    T, N = q.shape[0], len(lengths)
+    dq, dk, dv, dg, db = (t.to(dev) for t in (q, k, v, raw, beta))
+    dA, dD, dS = A_log.to(dev), dt_bias.to(dev), S0.to(dev)
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+
+    def run(out, final):
+        flashkda_fwd(dq, dk, dv, dg, db, dA, dD, out, initial_state=dS, final_state=final, cu_seqlens=cu)
+
+    o_eager = torch.empty(T, H, 128, dtype=torch.bfloat16, device=dev)
+    f_eager = torch.empty(N, H, 128, 128, device=dev)
+    run(o_eager, f_eager)
+    torch.cuda.synchronize()
+    o_graph, f_graph = torch.empty_like(o_eager), torch.empty_like(f_eager)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        run(o_graph, f_graph)                                  # warm-up on the capture stream
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        run(o_graph, f_graph)
+    for replay in range(3):
+        o_graph.fill_(float("nan"))
+        f_graph.fill_(float("nan"))
+        scratch = torch.randn(1 << 20, device=dev).sum().item()        # eager work and a sync between replays
+        graph.replay()
+        torch.cuda.synchronize()
+        assert scratch == scratch
+        assert torch.equal(o_graph.view(torch.int16), o_eager.view(torch.int16)), replay
+        assert torch.equal(f_graph.view(torch.int32), f_eager.view(torch.int32)), replay
 
 
 @pytest.mark.parametrize("lengths,pad,H", [([2500, 0, 1111, 40], 5, 2), ([4096], 0, 1), ([1030, 2049], 0, 3)])
