@@ -241,7 +241,7 @@ def bench_prefill_reference_shapes(steps, device):
     return rows
 
 
-def bench_prefill_kda(steps, device):
+def bench_prefill_kda(steps, device, cpu_leg=False):
     """Config 4: KDA chunk-64 prefill of one 65 536-token sequence, 32 heads (32 independent chains)."""
     import torch
     from pla_amd.prefill.flashkdapro import flashkda_fwd
@@ -256,11 +256,65 @@ def bench_prefill_kda(steps, device):
 
     ms = time_calls(run, steps, 3, device)
     tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
-    return dict(tokens=T, steps=steps, warmup=3, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1),
+    extra = {}
+    if cpu_leg:
+        # the CPU oracle's token recurrence over a prefix of the same sequence (the whole of it would take minutes)
+        import time as _time
+        from oracle import kda_prefill_reference
+        prefix = 8192
+        threads = os.cpu_count() or 1
+        torch.set_num_threads(threads)
+        cpu = {k: (v[:prefix].cpu() if k in ("q", "k", "v", "g", "beta") else v.cpu() if torch.is_tensor(v) else v)
+               for k, v in c.items()}
+        t0 = _time.perf_counter()
+        kda_prefill_reference(cpu["q"], cpu["k"], cpu["v"], cpu["g"], cpu["beta"], cpu["A_log"], cpu["dt_bias"],
+                              [0, prefix], cpu["initial_state"], scale=c["scale"], lower_bound=c["lower_bound"])
+        t = _time.perf_counter() - t0
+        extra["cpu_baseline"] = dict(value=round(prefix / t, 1), unit="tokens/s", cores=threads, kind="port",
+                                     sample="the first %d tokens of the 65 536-token sequence, all 32 heads, one pass of "
+                                            "the token recurrence (%.1f s)" % (prefix, t),
+                                     threads_torch=torch.get_num_threads())
+    return dict(tokens=T, steps=steps, warmup=3, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1), **extra,
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
                               frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=KDA_PREFILL_TRAFFIC_BYTES_PER_CALL,
                               hbm_GBps=round(KDA_PREFILL_TRAFFIC_BYTES_PER_CALL / ms / 1e6, 1),
                               flop_per_token=KDA_FLOP_PER_TOKEN))
+
+
+def bench_prefill_host_time(device, calls=200):
+    """Host time of one prefill call (argument checks, workspace from torch's allocator, launches; the stream is not
+    waited for): 8 x 2048-token GDN prefill and 1 x 2048-token KDA prefill, eager, best of three batches.  The GPU
+    needs longer than the host for these shapes, so the launch queue is drained between batches and the batch is
+    short enough not to fill it."""
+    import torch
+    from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from pla_amd.prefill.flashkdapro import flashkda_fwd
+    from pla_amd.workloads import gdn_prefill_packed, kda_prefill
+    out = {}
+    w = gdn_prefill_packed([2048] * 8, H=16, HV=32, pool_slots=10, seed=1, device=device)
+    call = {k: v for k, v in w.items() if not k.startswith("_")}
+    packed = call.pop("packed_qkv")
+    a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+    c = {k: v for k, v in kda_prefill(T=2048, H=32, seed=4, device=device).items() if not k.startswith("_")}
+    runs = {
+        "gdn_8x2048": lambda: gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, output_final_state=False, **call),
+        "kda_1x2048": lambda: flashkda_fwd(c["q"], c["k"], c["v"], c["g"], c["beta"], c["A_log"], c["dt_bias"], c["out"],
+                                           scale=c["scale"], lower_bound=c["lower_bound"], initial_state=c["initial_state"],
+                                           final_state=c["final_state"], cu_seqlens=c["cu_seqlens"]),
+    }
+    for name, run in runs.items():
+        for _ in range(20):
+            run()
+        best = 1e9
+        for _ in range(3):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(calls // 10):
+                run()
+            best = min(best, (time.perf_counter() - t0) / (calls // 10) * 1e6)
+        torch.cuda.synchronize()
+        out[name] = round(best, 1)
+    return out
 
 
 def copy_calibration(device, reps=5):
@@ -301,24 +355,37 @@ def bench_small_decode(device, steps=200):
     out["config0_gdn_decode_b8_us"] = round(us, 2)
     out["config0_state_GBps"] = round(8 * 32 * 131072 / us / 1e3, 1)
     v = make_verify(B=64, pool_slots=1024, seed=202, device=device)
-    us = timed(lambda: kda_mtp_verify(v["q"], v["k"], v["v"], v["log_decay"], v["beta"], v["state"], v["indices"],
+    # Consecutive steps take disjoint sets of 64 slots (16 sets cover the pool of 1024: 2.1 GB of state), so that no
+    # step finds its tiles in the 256 MB last-level cache, as the headline does.
+    B, slots = 64, 1024
+    perm = torch.randperm(slots, generator=torch.Generator().manual_seed(7)).to(device=device, dtype=torch.int32)
+    slot_sets = [perm[i * B:(i + 1) * B].contiguous() for i in range(slots // B)]
+    turn = [0]
+
+    def next_set():
+        turn[0] = (turn[0] + 1) % len(slot_sets)
+        return slot_sets[turn[0]]
+
+    us = timed(lambda: kda_mtp_verify(v["q"], v["k"], v["v"], v["log_decay"], v["beta"], v["state"], next_set(),
                                       v["cu_seqlens"], scale=v["scale"]))
     out["config2_kda_verify_t4_b64_us"] = round(us, 2)
     out["config2_verify_state_read_GBps"] = round(64 * 32 * 65536 / us / 1e3, 1)
+    out["config2_slot_sets"] = len(slot_sets)
     # accepted-prefix commit of the same window: per-slot records, num_accepted ~ U{0..4}
     from pla_amd.decode.kda_replayssm_sglang import fold_accepted_prefix
-    B, T, HV, slots = 64, 4, 32, 1024
-    idx = v["indices"].long()
+    T, HV = 4, 32
     rawk = torch.zeros(slots, HV, T, 128, dtype=torch.bfloat16, device=device)
     rawv = torch.zeros_like(rawk)
     gk = torch.zeros(slots, HV, T, 128, dtype=torch.float32, device=device)
     beta = torch.zeros(slots, HV, T, dtype=torch.float32, device=device)
-    rawk[idx] = v["k"][0].view(B, T, HV, 128).transpose(1, 2)
-    rawv[idx] = v["v"][0].view(B, T, HV, 128).transpose(1, 2)
-    gk[idx] = v["log_decay"].view(B, T, HV, 128).transpose(1, 2)
-    beta[idx] = v["beta"].view(B, T, HV).transpose(1, 2)
+    for ids in slot_sets:                             # every set of slots holds the records of the same draft window
+        idx = ids.long()
+        rawk[idx] = v["k"][0].view(B, T, HV, 128).transpose(1, 2)
+        rawv[idx] = v["v"][0].view(B, T, HV, 128).transpose(1, 2)
+        gk[idx] = v["log_decay"].view(B, T, HV, 128).transpose(1, 2)
+        beta[idx] = v["beta"].view(B, T, HV).transpose(1, 2)
     us = timed(lambda: fold_accepted_prefix(v["state"][None], rawv[None], rawk[None], gk[None], beta[None],
-                                            v["indices"], v["num_accepted"], null_block_id=-1))
+                                            next_set(), v["num_accepted"], null_block_id=-1))
     touched = int((v["num_accepted"] > 0).sum().item())
     out["config2_kda_commit_b64_us"] = round(us, 2)
     out["config2_commit_state_GBps"] = round(touched * 32 * 2 * 65536 / us / 1e3, 1)     # tiles read and written
@@ -478,7 +545,19 @@ def cpu_baseline_decode(w, reps=20):
         times.append(time.perf_counter() - t0)
     t = statistics.median(times)
     n = len(active)
-    return dict(value=n * HV * 131072 / t / 1e9, unit="GB/s", cores=threads, kind="port",
+    # the same oracle on one thread, on the first 32 requests (a bounded sample: the whole batch takes seconds per step)
+    sub = 32
+    sub_slots = slots[:sub]
+    n_sub = sum(1 for x in sub_slots if x >= 0)
+    torch.set_num_threads(1)
+    t0 = time.perf_counter()
+    k_last_reference(q[:sub], k[:sub], v[:sub], a[:sub], b[:sub], w["A_log"].cpu(), w["dt_bias"].cpu(), state, sub_slots,
+                     [1] * sub, scale=w["scale"], use_qk_l2norm=True, is_kda=False)
+    t1 = time.perf_counter() - t0
+    torch.set_num_threads(threads)
+    single = dict(value=round(n_sub * HV * 131072 / t1 / 1e9, 2), unit="GB/s", cores=1,
+                  sample="the first %d requests (%d active), one step (%.1f ms)" % (sub, n_sub, t1 * 1e3))
+    return dict(value=n * HV * 131072 / t / 1e9, unit="GB/s", cores=threads, kind="port", single_thread=single,
                 sample="all 256 requests (%d active), one step, median of %d steps (%.1f ms/step; %.0f us per "
                        "active request)" % (n, reps, t * 1e3, t / n * 1e6),
                 threads_torch=torch.get_num_threads())
@@ -530,7 +609,9 @@ def main():
         extra["prefill"] = bench_prefill(max(args.steps, 50), 50, device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
         extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 2, 10), device)
-        extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device)
+        extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device, cpu_leg=not args.no_cpu_baseline)
+        torch.cuda.empty_cache()
+        extra["prefill_host_us"] = bench_prefill_host_time(device)
         torch.cuda.empty_cache()
     d = time_decode(prep, args.steps, args.warmup)
     result = {

@@ -62,45 +62,61 @@ def build_library(verbose=True):
 
 
 BINDING_SRC = os.path.join(CSRC, "decode_binding.cpp")
+PREFILL_BINDING_SRC = os.path.join(CSRC, "prefill_binding.cpp")
+
+# compiled host modules: package directory (relative to pla_amd) -> (source, extra defines)
+BINDINGS = {
+    "decode": (BINDING_SRC, []),
+    os.path.join("prefill", "flashqla"): (PREFILL_BINDING_SRC, ["-DPLA_BIND_FLASHQLA"]),
+    os.path.join("prefill", "flashkdapro"): (PREFILL_BINDING_SRC, ["-DPLA_BIND_FLASHKDAPRO"]),
+}
 
 
-def binding_path():
+def binding_path(package="decode"):
     import sysconfig
-    return os.path.join(HERE, "decode", "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
+    return os.path.join(HERE, package, "_C" + sysconfig.get_config_var("EXT_SUFFIX"))
 
 
-def build_binding(verbose=True):
-    """Compile pla_amd/decode/_C (pybind11 over the C ABI; host code only, g++) against this interpreter's torch.
+def build_binding(verbose=True, package="decode"):
+    """Compile pla_amd/<package>/_C (pybind11 over the C ABI; host code only, g++) against this interpreter's torch.
 
     The module links libpla_gfx950.so by a path relative to itself; torch's libraries are found because importing
-    torch precedes importing the module (the reference's extension relies on the same order).
+    torch precedes importing the module (the reference's extensions rely on the same order).
     """
     import sysconfig
     import torch
     from torch.utils import cpp_extension
     cxx = shutil.which("g++") or shutil.which("c++")
     if cxx is None:
-        raise RuntimeError("g++ not found; pla_amd.decode._C cannot be built")
-    out = binding_path()
+        raise RuntimeError("g++ not found; pla_amd.%s._C cannot be built" % package.replace(os.sep, "."))
+    src, defines = BINDINGS[package]
+    out = binding_path(package)
     tmp = out + ".tmp"
     incs = cpp_extension.include_paths() + [sysconfig.get_paths()["include"], "/opt/rocm/include"]
     libdirs = cpp_extension.library_paths() + [LIB_DIR]
+    up = "/".join([".."] * (package.count(os.sep) + 1))
     cmd = [cxx, "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-Wno-attributes",
            "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H", "-DUSE_ROCM", "-D__HIP_PLATFORM_AMD__=1",
-           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
-           *["-I" + p for p in incs], BINDING_SRC, "-o", tmp,
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI), *defines,
+           *["-I" + p for p in incs], src, "-o", tmp,
            *["-L" + p for p in libdirs], "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python",
-           "-lpla_gfx950", "-Wl,-rpath,$ORIGIN/../lib"]
+           "-lpla_gfx950", "-Wl,-rpath,$ORIGIN/%s/lib" % up]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
-        raise RuntimeError("building pla_amd.decode._C failed:\n%s\n%s" % (proc.stdout, proc.stderr[-4000:]))
+        raise RuntimeError("building pla_amd.%s._C failed:\n%s\n%s" % (package.replace(os.sep, "."), proc.stdout, proc.stderr[-4000:]))
     os.replace(tmp, out)
     if verbose:
         print("built", out)
     return out
 
 
+def build_bindings(verbose=True):
+    """All compiled host modules (three g++ runs side by side)."""
+    with ThreadPoolExecutor(max_workers=len(BINDINGS)) as pool:
+        return list(pool.map(lambda package: build_binding(verbose, package), BINDINGS))
+
+
 if __name__ == "__main__":
     build_library()
-    build_binding()
+    build_bindings()
     sys.exit(0)

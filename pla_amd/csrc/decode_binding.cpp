@@ -10,8 +10,12 @@
 #include <torch/extension.h>
 #include <c10/hip/HIPStream.h>
 
+#include <c10/core/DeviceGuard.h>
+
+#include <cmath>
 #include <cstdlib>
 #include <optional>
+#include <string>
 #include <variant>
 
 #include "../../include/pla_gfx950.h"
@@ -248,10 +252,171 @@ Tensor k_last_impl(const Tensor& A_log, const Tensor& a, const Tensor& dt_bias, 
   return o;
 }
 
+// Recurrent KDA decode from raw gate / beta projections (vLLM's fused_recurrent_kda plus a trailing is_sglang;
+// reference wrapper src/decode/k-last/fused_recurrent_kda.cpp:146-314): argument problems raise ValueError or
+// NotImplementedError as there, dt_bias is float32 and is narrowed to the activation dtype only for the pure-decode
+// path, a 2-D per-token slot table sets disable_state_update.  Returns (out, initial_state).
+std::pair<Tensor, Tensor> fused_recurrent_kda(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& raw_g,
+                                              const Tensor& raw_beta, const Tensor& A_log, const OptTensor& dt_bias,
+                                              std::optional<double> lower_bound, const Tensor& initial_state, const Tensor& cu_seqlens,
+                                              const Tensor& ssm_state_indices, const OptTensor& num_accepted_tokens,
+                                              const OptTensor& out, std::optional<bool> fuse_gate, bool is_sglang) {
+  namespace py = pybind11;
+  auto value_error = [](const std::string& m) { return py::value_error(m); };
+  auto not_implemented = [](const std::string& m) { PyErr_SetString(PyExc_NotImplementedError, m.c_str()); return py::error_already_set(); };
+  if (fuse_gate.has_value() && !*fuse_gate)
+    throw not_implemented("pla.decode.kda.fused_recurrent_kda only implements the fused-gate path (fuse_gate=True): pass the raw "
+                          "gate projection plus A_log/dt_bias and drop the separate _fused_kda_gate_beta call.");
+  if (!dt_bias.has_value()) throw value_error("dt_bias is required by the fused-gate kernel path.");
+  if (q.dim() != 4) throw value_error("q must be packed as [1, T, H, K], got " + std::to_string(q.dim()) + "D.");
+  const int64_t B = q.size(0), T = q.size(1), H = q.size(2), K = q.size(3), V = v.size(-1);
+  if (B != 1) throw value_error("q must be packed as [1, T, H, K], got batch " + std::to_string(B) + ".");
+  if (K != 128 || V != 128)
+    throw not_implemented("pla.decode.kda.fused_recurrent_kda requires head_dim K == V == 128, got K=" + std::to_string(K) +
+                          ", V=" + std::to_string(V) + ".");
+  auto torch_name = [](at::ScalarType t) { return std::string("torch.") + (t == at::kHalf ? "float16" : t == at::kBFloat16 ? "bfloat16" :
+                                           t == at::kFloat ? "float32" : t == at::kDouble ? "float64" : c10::toString(t)); };
+  if (initial_state.scalar_type() != at::kFloat) throw value_error("initial_state must be float32, got " + torch_name(initial_state.scalar_type()) + ".");
+  if (ssm_state_indices.dim() != 1 && ssm_state_indices.dim() != 2)
+    throw value_error("ssm_state_indices must be 1D or 2D, got " + std::to_string(ssm_state_indices.dim()) + "D");
+  const bool per_token_slots = ssm_state_indices.dim() == 2;
+  if (per_token_slots && is_sglang)
+    throw value_error("a 2D ssm_state_indices is the vLLM spec-decode layout; sglang uses a 1D table plus its own "
+                      "intermediate-state buffer.");
+  if (dt_bias->scalar_type() != at::kFloat) throw value_error("dt_bias must be float32, got " + torch_name(dt_bias->scalar_type()) + ".");
+
+  const at::ScalarType act = q.scalar_type();
+  const Tensor a = raw_g.reshape({B * T, H * K}).to(act).contiguous();
+  const Tensor b = raw_beta.reshape({B * T, H}).to(act).contiguous();
+  const Tensor k_c = k.contiguous();
+  const Tensor cu32 = cu_seqlens.to(at::kInt);
+  const Tensor idx = ssm_state_indices.to(at::kInt).contiguous();
+  Tensor dt = dt_bias->reshape({H, K});
+  // whether the k-last call takes the MTP-verify path, which reads dt_bias as float32
+  // (src/decode/k-last/fused_sigmoid_gating_cuda_k_last.cpp:225-236)
+  const int64_t t_max = packed_t_max(k_c, cu32.size(0) - 1, per_token_slots, 0, per_token_slots ? idx.size(1) : 0);
+  if (!(t_max > 1 || per_token_slots)) dt = dt.to(act);
+  dt = dt.contiguous();
+  StepsOrAccepted accepted;
+  if (num_accepted_tokens.has_value()) accepted = std::variant<Tensor, int64_t>(num_accepted_tokens->to(at::kInt).contiguous());
+  Tensor o = k_last_impl(A_log.reshape({-1}).contiguous(), a, dt, 1.0, 20.0, q.contiguous(), k_c, v.contiguous(), b, initial_state, idx,
+                         1.0 / std::sqrt((double)K), true, cu32, true, per_token_slots, std::nullopt, std::nullopt, accepted,
+                         std::nullopt, lower_bound, is_sglang, std::nullopt, std::nullopt);
+  if (out.has_value()) {
+    out->copy_(o);
+    o = *out;
+  }
+  return {o, initial_state};
+}
+
+// Causal conv1d update + SiLU, gate, delta-rule recurrence and optional gated RMSNorm in one launch: the checks of
+// the reference entry (src/decode/k-last/fused_kda_decode_mega_host.cpp:77-300), RuntimeError before anything is
+// written; conv_state, state and out are updated in place.
+void fused_kda_decode_mega_forward(const Tensor& x, const Tensor& weight, const OptTensor& bias, const Tensor& conv_state,
+                                   const Tensor& raw_g, const Tensor& raw_beta, const Tensor& a_log, const Tensor& dt_bias,
+                                   const Tensor& state_indices, const Tensor& state, const Tensor& out,
+                                   std::optional<double> lower_bound, const OptTensor& output_gate, const OptTensor& norm_weight,
+                                   double norm_eps) {
+  if (bypass()) return;
+  constexpr int64_t D = 128, W = 4;
+  TORCH_CHECK(x.is_cuda(), "x must be a CUDA tensor");
+  const at::ScalarType act = x.scalar_type();
+  TORCH_CHECK(act == at::kBFloat16 || act == at::kHalf, "x must be a bfloat16 or float16 tensor");
+  TORCH_CHECK(weight.is_cuda() && weight.scalar_type() == at::kFloat, "weight must be a CUDA float32 tensor");
+  TORCH_CHECK(conv_state.is_cuda() && conv_state.scalar_type() == act, "conv_state must be a CUDA tensor with the same dtype as x");
+  TORCH_CHECK(raw_g.is_cuda() && raw_g.scalar_type() == act, "raw_g must be a CUDA tensor with the same dtype as x");
+  TORCH_CHECK(raw_beta.is_cuda() && raw_beta.scalar_type() == act, "raw_beta must be a CUDA tensor with the same dtype as x");
+  TORCH_CHECK(a_log.is_cuda() && a_log.scalar_type() == at::kFloat, "A_log must be a CUDA float32 tensor");
+  TORCH_CHECK(dt_bias.is_cuda() && dt_bias.scalar_type() == at::kFloat, "dt_bias must be a CUDA float32 tensor");
+  TORCH_CHECK(state.is_cuda() && state.scalar_type() == at::kFloat, "state must be a CUDA float32 tensor");
+  TORCH_CHECK(out.is_cuda() && out.scalar_type() == act, "out must be a CUDA tensor with the same dtype as x");
+  TORCH_CHECK(state_indices.is_cuda() && state_indices.scalar_type() == at::kInt, "state_indices must be a CUDA int32 tensor");
+  TORCH_CHECK(x.dim() == 2 && x.size(1) % (3 * D) == 0, "x must have shape [B, 3 * H * 128]");
+  const int64_t B = x.size(0), H = x.size(1) / (3 * D);
+  bool known = false;
+  for (int64_t h : {4, 6, 8, 12, 16, 24, 48, 64, 96}) known = known || h == H;
+  TORCH_CHECK(known, "H must be 4, 6, 8, 12, 16, 24, 48, 64, or 96, got ", H);
+  TORCH_CHECK(B > 0, "KDA decode fusion requires at least one row");
+  const int64_t dim = H * D;
+  TORCH_CHECK(weight.dim() == 3 && weight.is_contiguous() && weight.size(0) == 3 && weight.size(1) == W && weight.size(2) == dim,
+              "weight must have shape [3, 4, H * 128]");
+  TORCH_CHECK(conv_state.dim() == 3 && conv_state.size(1) == 3 * dim && conv_state.size(2) == W - 1,
+              "conv_state must have shape [slots, 3 * H * 128, 3]");
+  TORCH_CHECK(raw_g.dim() == 4 && raw_g.size(0) == 1 && raw_g.size(1) == B && raw_g.size(2) == H && raw_g.size(3) == D,
+              "raw_g must have shape [1, B, H, 128]");
+  TORCH_CHECK(raw_beta.dim() == 3 && raw_beta.size(0) == 1 && raw_beta.size(1) == B && raw_beta.size(2) == H,
+              "raw_beta must have shape [1, B, H]");
+  TORCH_CHECK(a_log.is_contiguous() && a_log.numel() == H, "A_log must be contiguous with H elements");
+  TORCH_CHECK(dt_bias.is_contiguous() && dt_bias.numel() == dim, "dt_bias must be contiguous with H * 128 elements");
+  TORCH_CHECK(state_indices.is_contiguous() && state_indices.numel() == B, "state_indices must be contiguous with B elements");
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == D,
+              "state must have shape [slots, H, 128, 128]");
+  TORCH_CHECK(out.dim() == 4 && out.size(0) == 1 && out.size(1) == B && out.size(2) == H && out.size(3) == D,
+              "out must have shape [1, B, H, 128]");
+  TORCH_CHECK(x.stride(1) == 1, "x must be contiguous in its channel dimension");
+  TORCH_CHECK(conv_state.stride(0) >= 3 * dim * (W - 1) && conv_state.stride(1) == 1 && conv_state.stride(2) == 3 * dim,
+              "conv_state must use the SD cache layout");
+  TORCH_CHECK(state.stride(0) >= H * D * D && state.stride(1) == D * D && state.stride(2) == D && state.stride(3) == 1,
+              "state must have contiguous [H, 128, 128] slot contents");
+  TORCH_CHECK(raw_g.is_contiguous(), "raw_g must be contiguous");
+  TORCH_CHECK(raw_beta.stride(2) == 1, "raw_beta must be contiguous in its head dimension");
+  TORCH_CHECK(out.is_contiguous(), "out must be contiguous");
+  const bool apply_onorm = output_gate.has_value();
+  TORCH_CHECK(apply_onorm == norm_weight.has_value(), "output_gate and norm_weight must be provided together");
+  int64_t onorm_row = 0;
+  if (apply_onorm) {
+    TORCH_CHECK(output_gate->is_cuda() && output_gate->scalar_type() == act, "output_gate must be a CUDA tensor with the same dtype as x");
+    const bool gate_3d = output_gate->dim() == 3 && output_gate->size(0) == B && output_gate->size(1) == H && output_gate->size(2) == D;
+    const bool gate_4d = output_gate->dim() == 4 && output_gate->size(0) == 1 && output_gate->size(1) == B && output_gate->size(2) == H &&
+                         output_gate->size(3) == D;
+    TORCH_CHECK(gate_3d || gate_4d, "output_gate must have shape [B, H, 128] or [1, B, H, 128]");
+    const int row_dim = gate_3d ? 0 : 1;
+    TORCH_CHECK(output_gate->stride(-1) == 1, "output_gate must be contiguous in its last dimension");
+    TORCH_CHECK(output_gate->stride(row_dim + 1) == D, "output_gate must have contiguous head rows");
+    TORCH_CHECK(norm_weight->is_cuda() && norm_weight->scalar_type() == at::kFloat, "norm_weight must be a CUDA float32 tensor");
+    TORCH_CHECK(norm_weight->is_contiguous() && norm_weight->numel() == D, "norm_weight must be contiguous with 128 elements");
+    TORCH_CHECK(norm_eps >= 0.0, "norm_eps must be non-negative");
+    onorm_row = output_gate->stride(row_dim);
+  }
+  if (bias.has_value()) {
+    TORCH_CHECK(bias->is_cuda() && bias->scalar_type() == at::kFloat, "bias must be a CUDA float32 tensor");
+    TORCH_CHECK(bias->is_contiguous() && bias->numel() == 3 * dim, "bias must be contiguous with 3 * H * 128 elements");
+  }
+  const int64_t eb = x.element_size();
+  const char* xp = static_cast<const char*>(x.data_ptr());
+  const char* wp = static_cast<const char*>(weight.data_ptr());
+  char* cp = static_cast<char*>(conv_state.data_ptr());
+  const int64_t seg_b = dim * eb, wseg_b = dim * W * 4, cseg_b = dim * conv_state.stride(1) * eb;
+  const char* bp = bias.has_value() ? static_cast<const char*>(bias->data_ptr()) : nullptr;
+  const c10::DeviceGuard guard(x.device());
+  launched(pla_kda_decode_mega_launch(
+      dtype_code(act), apply_onorm ? 1 : 0, lower_bound.has_value() ? 1 : 0, a_log.data_ptr<float>(), raw_g.data_ptr(),
+      dt_bias.data_ptr<float>(), xp, xp + seg_b, xp + 2 * seg_b, raw_beta.data_ptr(),
+      reinterpret_cast<const float*>(wp), reinterpret_cast<const float*>(wp + wseg_b), reinterpret_cast<const float*>(wp + 2 * wseg_b),
+      reinterpret_cast<const float*>(bp), bp ? reinterpret_cast<const float*>(bp + dim * 4) : nullptr,
+      bp ? reinterpret_cast<const float*>(bp + 2 * dim * 4) : nullptr, cp, cp + cseg_b, cp + 2 * cseg_b, ptr(output_gate),
+      static_cast<const float*>(ptr(norm_weight)), (float)norm_eps, state.data_ptr<float>(), state_indices.data_ptr<int32_t>(),
+      out.data_ptr(), 1.0f / std::sqrt((float)D), lower_bound.has_value() ? (float)*lower_bound : 0.f, (int)B, (int)H, (int)H,
+      x.stride(0), raw_beta.stride(1), onorm_row, conv_state.stride(0), state.stride(0), stream_of(x)));
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   namespace py = pybind11;
+  m.def("fused_kda_decode_mega_forward", &fused_kda_decode_mega_forward,
+        "KDA decode step fused on gfx950: conv1d update + SiLU, gate, recurrence, optional gated RMSNorm (vLLM contract)",
+        py::arg("x"), py::arg("weight"), py::arg("bias") = py::none(), py::arg("conv_state"), py::arg("raw_g"), py::arg("raw_beta"),
+        py::arg("a_log"), py::arg("dt_bias"), py::arg("state_indices"), py::arg("state"), py::arg("out"),
+        py::arg("lower_bound") = py::none(), py::arg("output_gate") = py::none(), py::arg("norm_weight") = py::none(),
+        py::arg("norm_eps") = 1e-5);
+  m.def("fused_recurrent_kda", &fused_recurrent_kda,
+        "Recurrent KDA decode from raw gate / beta (vLLM fused_recurrent_kda contract; is_sglang selects the sglang pad-slot "
+        "convention).  Returns (out, initial_state); the state pool is updated in place.",
+        py::arg("q"), py::arg("k"), py::arg("v"), py::arg("raw_g"), py::arg("raw_beta"), py::arg("A_log"), py::arg("dt_bias"),
+        py::arg("lower_bound"), py::arg("initial_state"), py::arg("cu_seqlens"), py::arg("ssm_state_indices"),
+        py::arg("num_accepted_tokens") = py::none(), py::arg("out") = py::none(), py::arg("fuse_gate") = py::none(),
+        py::arg("is_sglang") = false);
   m.doc() = "pla.decode._C for MI355X: k-last gated delta-rule decode and MTP verify over libpla_gfx950.so";
   m.def(
       "fused_sigmoid_gating_delta_rule_forward_k_last",

@@ -34,10 +34,27 @@ def _takes_mtp_path(k, cu_seqlens, state_indices, disable_state_update):
     return t_max > 1 or disable_state_update or target_verify
 
 
+def _native():
+    """pla.decode._C when it is built and the PLA_SANITY_CHECK diagnostics are off (they live in the Python path)."""
+    from .. import _compiled, _sanity_enabled
+    module = _compiled()
+    return module if module and not _sanity_enabled() else None
+
+
 def fused_recurrent_kda(q, k, v, raw_g, raw_beta, A_log, dt_bias, lower_bound, initial_state,
                         cu_seqlens, ssm_state_indices, num_accepted_tokens=None, out=None,
                         fuse_gate=None, is_sglang=False):
     """Returns ``(out, initial_state)``; the state pool is updated in place."""
+    native = _native()
+    if native:
+        return native.fused_recurrent_kda(q, k, v, raw_g, raw_beta, A_log, dt_bias, lower_bound, initial_state, cu_seqlens,
+                                          ssm_state_indices, num_accepted_tokens, out, fuse_gate, is_sglang)
+    return _fused_recurrent_kda_impl(q, k, v, raw_g, raw_beta, A_log, dt_bias, lower_bound, initial_state, cu_seqlens,
+                                     ssm_state_indices, num_accepted_tokens, out, fuse_gate, is_sglang)
+
+
+def _fused_recurrent_kda_impl(q, k, v, raw_g, raw_beta, A_log, dt_bias, lower_bound, initial_state,
+                              cu_seqlens, ssm_state_indices, num_accepted_tokens, out, fuse_gate, is_sglang):
     if fuse_gate is not None and not fuse_gate:
         raise NotImplementedError(
             "pla.decode.kda.fused_recurrent_kda only implements the fused-gate path (fuse_gate=True): "
@@ -103,6 +120,17 @@ def fused_kda_decode_mega_forward(x, weight, bias=None, conv_state=None, raw_g=N
     anything is written.  A request whose ``state_indices`` entry is negative gets a zero output row
     and touches neither pool; slot 0 is an ordinary slot.
     """
+    native = _native()
+    if native:
+        return native.fused_kda_decode_mega_forward(x, weight, bias, conv_state, raw_g, raw_beta, a_log, dt_bias,
+                                                    state_indices, state, out, lower_bound, output_gate, norm_weight,
+                                                    norm_eps)
+    return _mega_impl(x, weight, bias, conv_state, raw_g, raw_beta, a_log, dt_bias, state_indices, state, out,
+                      lower_bound, output_gate, norm_weight, norm_eps)
+
+
+def _mega_impl(x, weight, bias, conv_state, raw_g, raw_beta, a_log, dt_bias, state_indices, state, out, lower_bound,
+               output_gate, norm_weight, norm_eps):
     if _BYPASS:
         return None
     D, W = 128, 4

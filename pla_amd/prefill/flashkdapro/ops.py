@@ -33,6 +33,23 @@ def _token_rows(name, t, H, width):
     return t, t.stride(0)
 
 
+# The compiled host layer (pla_amd/csrc/prefill_binding.cpp): see pla_amd/prefill/flashqla/ops.py.
+_native = None
+
+
+def _compiled():
+    global _native
+    if _native is None:
+        try:
+            import importlib
+            _native = importlib.import_module("._C", __package__)
+        except ModuleNotFoundError as exc:
+            if exc.name is None or not exc.name.endswith("_C"):
+                raise
+            _native = False
+    return _native
+
+
 def _workspace(T, N, H, device):
     nbytes = _lib.load().pla_kda_prefill_workspace_bytes(T, N, H)
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
@@ -57,6 +74,15 @@ def flashkda_fwd(
     raw_cu_seqlens: Optional[Tuple[int, ...]] = None,
 ) -> None:
     """FlashKDA prefill forward. Writes ``out`` (and ``final_state`` / ``state_pool``)."""
+    native = _compiled()
+    if native and (state_pool is None or (initial_state is None and final_state is None and state_indices is not None)):
+        first, last = (state_pool, state_pool) if state_pool is not None else (initial_state, final_state)
+        try:
+            if native.try_flashkda_fwd(q, k, v, g, beta, A_log, dt_bias, out, 128 ** -0.5 if scale is None else float(scale),
+                                       float(lower_bound), first, last, cu_seqlens, state_indices, raw_cu_seqlens):
+                return None
+        except TypeError:
+            pass                      # an argument of another type than the compiled signature: the checks below name it
     if not q.is_cuda:
         raise ValueError("q must be a CUDA tensor")
     for name, t in (("k", k), ("v", v), ("g", g), ("beta", beta), ("A_log", A_log), ("dt_bias", dt_bias), ("out", out)):

@@ -29,6 +29,26 @@ DK = 128
 DV = 128
 
 
+# The compiled host layer (pla_amd/csrc/prefill_binding.cpp, `python -m pla_amd.build`): every call is offered to it
+# first.  It takes calls in the plain serving form (dense rows on one GPU, FP32 k-last states, int32 offsets),
+# allocates and launches without Python in between, and returns None for any other form, which then runs below
+# with its conversions, diagnostics and error messages.  A tree without the module runs everything below.
+_native = None
+
+
+def _compiled():
+    global _native
+    if _native is None:
+        try:
+            import importlib
+            _native = importlib.import_module("._C", __package__)
+        except ModuleNotFoundError as exc:
+            if exc.name is None or not exc.name.endswith("_C"):
+                raise
+            _native = False
+    return _native
+
+
 def _workspace(T, N, Hg, H, device):
     nbytes = _lib.load().pla_gdn_prefill_workspace_bytes(T, N, Hg, H)
     return torch.empty(nbytes, dtype=torch.uint8, device=device), nbytes
@@ -64,6 +84,17 @@ def chunk_gated_delta_rule_fwd(
     ``final_state`` of the same shape is returned.  ``cu_seqlens`` may end before the physical
     token count; the padded suffix of ``O`` is zero and never touches a state.
     """
+    native = _compiled()
+    if native:
+        try:
+            taken = native.try_chunk_gated_delta_rule_fwd(
+                q, k, v, g, beta, scale, initial_state, initial_state_indices, cu_seqlens, bool(output_final_state),
+                overlap_warmup_threshold, bool(normalize_qk), raw_cu_seqlens, raw_gate_a, raw_beta_b, A_log, dt_bias,
+                final_state_dtype)
+        except TypeError:
+            taken = None              # an argument of another type than the compiled signature: the checks below name it
+        if taken is not None:
+            return taken
     if not q.is_cuda:
         raise ValueError("q must be a CUDA tensor")
     raw_gate_args = (raw_gate_a, raw_beta_b, A_log, dt_bias)
@@ -259,6 +290,17 @@ def gdn_prefill_packed_qkv_fwd(
 ):
     """GDN prefill directly on a post-convolution ``Q|K|V`` buffer (token stride may exceed the
     row width; features inside a token contiguous).  Q/K/V are aliases of ``packed_qkv``."""
+    native = _compiled()
+    if native:
+        try:
+            taken = native.try_gdn_prefill_packed_qkv_fwd(
+                packed_qkv, raw_gate_a, raw_beta_b, A_log, dt_bias, cu_seqlens, num_qk_heads, num_v_heads, scale,
+                initial_state, initial_state_indices, bool(output_final_state), overlap_warmup_threshold, raw_cu_seqlens,
+                final_state_dtype)
+        except TypeError:
+            taken = None
+        if taken is not None:
+            return taken
     if not packed_qkv.is_cuda:
         raise ValueError("packed_qkv must be a CUDA tensor")
     if packed_qkv.ndim != 2:

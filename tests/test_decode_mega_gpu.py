@@ -199,3 +199,71 @@ def test_mega_sanity_mode_rejects_aliased_slots_and_bad_values(monkeypatch):
     bad["state_indices"] = torch.tensor([4, -1, 2, 1], dtype=torch.int32, device="cuda")   # the poisoned row is a pad
     _run(bad, -5.0, True)
     assert not torch.equal(w["_cache"], snapshot)
+
+
+def test_compiled_and_python_layers_of_the_kda_entry_points_agree():
+    """fused_kda_decode_mega_forward and fused_recurrent_kda exist compiled (pla.decode._C, the path a call takes) and in
+    Python (the PLA_SANITY_CHECK path): the same refused calls raise the same exception type and message in both, and
+    an accepted call gives the same bits."""
+    import pla_amd.decode as dec
+    import pla_amd.decode.kda as kda
+    native = dec._compiled()
+    assert native and kda._native() is native
+    w = kda_decode_mega(2, 4, seed=3)
+    out = torch.empty(1, 2, 4, D, dtype=torch.bfloat16, device="cuda")
+    base = dict(x=w["x"], weight=w["weight"], bias=None, conv_state=w["conv_state"], raw_g=w["raw_g"], raw_beta=w["raw_beta"],
+                a_log=w["a_log"], dt_bias=w["dt_bias"], state_indices=w["state_indices"], state=w["state"], out=out,
+                lower_bound=-5.0, output_gate=w["output_gate"], norm_weight=w["norm_weight"], norm_eps=1e-5)
+    order = list(base)
+    edits = {
+        "cpu_x": dict(x=w["x"].cpu()), "x_dtype": dict(x=w["x"].float()), "weight_dtype": dict(weight=w["weight"].bfloat16()),
+        "heads": dict(x=torch.zeros(2, 3 * 5 * D, dtype=torch.bfloat16, device="cuda")),
+        "state_dtype": dict(state=w["state"].bfloat16()), "conv_layout": dict(conv_state=w["conv_state"].contiguous()),
+        "norm_pair": dict(norm_weight=None), "raw_g_shape": dict(raw_g=w["raw_g"][0]), "idx_dtype": dict(state_indices=w["state_indices"].long()),
+        "out_shape": dict(out=out[0]), "eps": dict(norm_eps=-1.0), "bias": dict(bias=torch.zeros(5, device="cuda")),
+        "gate_shape": dict(output_gate=w["output_gate"][..., :64]),
+    }
+    snapshot = w["_cache"].clone()
+    for name, edit in edits.items():
+        caught = []
+        for call in (native.fused_kda_decode_mega_forward, kda._mega_impl):
+            with pytest.raises(Exception) as info:
+                call(*[dict(base, **edit)[n] for n in order])
+            caught.append((type(info.value), str(info.value).splitlines()[0]))
+        assert caught[0] == caught[1] and caught[0][0] is RuntimeError, (name, caught)
+    torch.cuda.synchronize()
+    assert torch.equal(w["_cache"], snapshot)
+    # fused_recurrent_kda: refused calls
+    from pla_amd.workloads import kda_mtp_verify
+    H = 4
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(1, 3, H, 128, generator=g).bfloat16().cuda()
+    args = dict(q=q, k=q.clone(), v=q.clone(), raw_g=torch.randn(1, 3, H, 128, generator=g).bfloat16().cuda(),
+                raw_beta=torch.randn(1, 3, H, generator=g).bfloat16().cuda(), A_log=torch.zeros(H, device="cuda"),
+                dt_bias=torch.zeros(H, 128, device="cuda"), lower_bound=-5.0, initial_state=torch.zeros(5, H, 128, 128, device="cuda"),
+                cu_seqlens=torch.tensor([0, 1, 2, 3], dtype=torch.int32, device="cuda"),
+                ssm_state_indices=torch.tensor([1, 2, 4], dtype=torch.int32, device="cuda"), num_accepted_tokens=None, out=None,
+                fuse_gate=None, is_sglang=False)
+    korder = list(args)
+    kedits = {
+        "fuse_gate": dict(fuse_gate=False), "no_dt_bias": dict(dt_bias=None), "q_rank": dict(q=q[0]), "batch": dict(q=q.repeat(2, 1, 1, 1)),
+        "head_dim": dict(q=q[..., :64].contiguous()), "state_dtype": dict(initial_state=args["initial_state"].bfloat16()),
+        "idx_rank": dict(ssm_state_indices=args["ssm_state_indices"][None, None]),
+        "table_sglang": dict(ssm_state_indices=args["ssm_state_indices"][:, None].contiguous(), is_sglang=True),
+        "dt_dtype": dict(dt_bias=args["dt_bias"].bfloat16()),
+    }
+    for name, edit in kedits.items():
+        caught = []
+        for call in (native.fused_recurrent_kda, kda._fused_recurrent_kda_impl):
+            with pytest.raises(Exception) as info:
+                call(*[dict(args, **edit)[n] for n in korder])
+            caught.append((type(info.value), str(info.value).splitlines()[0]))
+        assert caught[0] == caught[1] and caught[0][0] in (ValueError, NotImplementedError), (name, caught)
+    # an accepted call: same output and state bits from both layers
+    outs = []
+    for call in (native.fused_recurrent_kda, kda._fused_recurrent_kda_impl):
+        state = torch.full((5, H, 128, 128), 0.01, device="cuda")
+        o, st = call(*[dict(args, initial_state=state)[n] for n in korder])
+        outs.append((o.clone(), st.clone()))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
