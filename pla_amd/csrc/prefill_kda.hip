@@ -51,8 +51,8 @@ struct KdaPrefillParams {
   // operand tiles of the sweeps, fp16 (every factor lies in (0, 1]; values below 6e-8 vanish)
   uint16_t* Kg; uint16_t* Qg;                      // [chunk, H, 64, 128]: k e^{G}, scale q e^{G}
   uint16_t* Kt;                                    // [chunk, H, 2, 64, 128]: k e^{G_last - G} as an fp16 hi + lo pair
-  uint16_t* W;                                     // [chunk, H, 2, 64, 64]: W = hi + lo
-  uint16_t* P;                                     // [chunk, H, 64, 64]
+  uint16_t* W;                                     // [chunk, H, 2, 6 blocks]: W = hi + lo in the six-block operand layout (prefill_common.h)
+  uint16_t* P;                                     // [chunk, H, 6 blocks]: P in the same layout
   float* eGlast;                                   // [chunk, H, 128]: e^{G_last}
   SegmentTable seg;                                // split long sequences (seg.seg_chunks > 0)
   StageTable stg;                                  // pipelined preparation and sweep (stg.stages > 0)
@@ -231,8 +231,15 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
     bf16x8_t Ql[4];
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
-      f32x4_t a, b;
-      decayed8(&sh.Kn[i_row][0], &sh.G[i_row][0], R, 1.0f, s, kb, a, b);
+      // the decay factors e^{G_i - R} of the lane's eight channels serve both the k and the q rows
+      const int c0 = 32 * s + 4 * kb, c1 = c0 + 16;
+      const float4 g0 = *reinterpret_cast<const float4*>(&sh.G[i_row][c0]), g1 = *reinterpret_cast<const float4*>(&sh.G[i_row][c1]);
+      const float4 r0 = *reinterpret_cast<const float4*>(R + c0), r1 = *reinterpret_cast<const float4*>(R + c1);
+      const f32x4_t e0 = {__expf(g0.x - r0.x), __expf(g0.y - r0.y), __expf(g0.z - r0.z), __expf(g0.w - r0.w)};
+      const f32x4_t e1 = {__expf(g1.x - r1.x), __expf(g1.y - r1.y), __expf(g1.z - r1.z), __expf(g1.w - r1.w)};
+      const uint2 k0 = *reinterpret_cast<const uint2*>(&sh.Kn[i_row][c0]), k1 = *reinterpret_cast<const uint2*>(&sh.Kn[i_row][c1]);
+      f32x4_t a = {lo16<bf16_t>(k0.x) * e0[0], hi16<bf16_t>(k0.x) * e0[1], lo16<bf16_t>(k0.y) * e0[2], hi16<bf16_t>(k0.y) * e0[3]};
+      f32x4_t b = {lo16<bf16_t>(k1.x) * e1[0], hi16<bf16_t>(k1.x) * e1[1], lo16<bf16_t>(k1.y) * e1[2], hi16<bf16_t>(k1.y) * e1[3]};
       Al[s] = split8(a, b);
       // the same normalised bf16 values as phase 1 formed: raw q times the row's inverse norm, rounded to bf16
       const float qi = sh.QI[i_row];
@@ -241,25 +248,20 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
       const uint32_t n1 = pack2<bf16_t>(lo16<bf16_t>(x0.y) * qi, hi16<bf16_t>(x0.y) * qi);
       const uint32_t n2 = pack2<bf16_t>(lo16<bf16_t>(x1.x) * qi, hi16<bf16_t>(x1.x) * qi);
       const uint32_t n3 = pack2<bf16_t>(lo16<bf16_t>(x1.y) * qi, hi16<bf16_t>(x1.y) * qi);
-      const int c0 = 32 * s + 4 * kb, c1 = c0 + 16;
-      const float4 g0 = *reinterpret_cast<const float4*>(&sh.G[i_row][c0]), g1 = *reinterpret_cast<const float4*>(&sh.G[i_row][c1]);
-      const float4 r0 = *reinterpret_cast<const float4*>(R + c0), r1 = *reinterpret_cast<const float4*>(R + c1);
-      a = f32x4_t{lo16<bf16_t>(n0) * __expf(g0.x - r0.x), hi16<bf16_t>(n0) * __expf(g0.y - r0.y),
-                  lo16<bf16_t>(n1) * __expf(g0.z - r0.z), hi16<bf16_t>(n1) * __expf(g0.w - r0.w)};
-      b = f32x4_t{lo16<bf16_t>(n2) * __expf(g1.x - r1.x), hi16<bf16_t>(n2) * __expf(g1.y - r1.y),
-                  lo16<bf16_t>(n3) * __expf(g1.z - r1.z), hi16<bf16_t>(n3) * __expf(g1.w - r1.w)};
+      a = f32x4_t{lo16<bf16_t>(n0) * e0[0], hi16<bf16_t>(n0) * e0[1], lo16<bf16_t>(n1) * e0[2], hi16<bf16_t>(n1) * e0[3]};
+      b = f32x4_t{lo16<bf16_t>(n2) * e1[0], hi16<bf16_t>(n2) * e1[1], lo16<bf16_t>(n3) * e1[2], hi16<bf16_t>(n3) * e1[3]};
       Ql[s] = round8(a, b);
     }
-    uint16_t* const Pt = p.P + tile * 4096;
+    // P leaves in the six-block operand layout (prefill_common.h): its product is formed transposed (A = k rows j,
+    // B = q rows i), so a lane holds four consecutive j of token i = 16 bi + r16, which is half of the 16 bytes it owns
+    // in block (row block bi, contraction half s = bj / 2); the halves of blocks above the diagonal are zero.
+    uint16_t* const Pt = p.P + tile * (TRI_BLOCKS * 512);
     f32x4_t mblock[4];
+    uint32_t ppk[4][2] = {{0u, 0u}, {0u, 0u}, {0u, 0u}, {0u, 0u}};
 #pragma unroll
     for (int bj = 0; bj < 4; ++bj) {
       const int j = 16 * bj + r16;
-      if (bj > bi) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) Pt[(16 * bi + 4 * kb + r) * 64 + j] = 0;
-        continue;
-      }
+      if (bj > bi) continue;
       f32x4_t m = {0.f, 0.f, 0.f, 0.f}, pq = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
@@ -269,15 +271,17 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
         m = mfma16(Al[s].hi, Br.hi, m);
         m = mfma16(Al[s].lo, Br.hi, m);
         m = mfma16(Al[s].hi, Br.lo, m);
-        pq = mfma16(Ql[s], Br.hi, pq);
+        pq = mfma16(Br.hi, Ql[s], pq);        // pq[r] = P[i = 16 bi + r16][j = 16 bj + 4 kb + r] / scale
       }
       mblock[bj] = m;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * bi + 4 * kb + r;
-        Pt[i * 64 + j] = from_float<f16_t>(i >= j ? p.scale * pq[r] : 0.f).bits;
+      {
+        const int i = 16 * bi + r16, j0 = 16 * bj + 4 * kb;
+        ppk[bj][0] = pack2<f16_t>(i >= j0 ? p.scale * pq[0] : 0.f, i >= j0 + 1 ? p.scale * pq[1] : 0.f);
+        ppk[bj][1] = pack2<f16_t>(i >= j0 + 2 ? p.scale * pq[2] : 0.f, i >= j0 + 3 ? p.scale * pq[3] : 0.f);
       }
     }
+    *reinterpret_cast<uint4*>(Pt + bi * 512 + lane * 8) = make_uint4(ppk[0][0], ppk[0][1], ppk[1][0], ppk[1][1]);
+    if (bi >= 2) *reinterpret_cast<uint4*>(Pt + (2 + bi) * 512 + lane * 8) = make_uint4(ppk[2][0], ppk[2][1], ppk[3][0], ppk[3][1]);
     __syncthreads();                     // Kn is dead from here on: L reuses its storage
 #pragma unroll
     for (int bj = 0; bj < 4; ++bj) {
@@ -294,7 +298,10 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 
   // ---- phase 4: W = L^-1 diag(beta) by blocks on one wavefront (which one rotates with the workgroup, so
   // that co-resident workgroups keep different SIMDs busy) -----------------------------------------
-  if (wave == (int)(blockIdx.x & 3)) block_inverse_store_w<true>(sh.L, sh.B, lane, p.W + tile * 8192);
+  if (wave == (int)(blockIdx.x & 3)) {
+    block_inverse_inplace(sh.L, lane);
+    store_w_operand_blocks(sh.L, sh.B, lane, p.W + tile * (2 * TRI_BLOCKS * 512));
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -314,7 +321,7 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
+  constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -329,10 +336,10 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
   __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
+  __shared__ __align__(16) uint16_t tW[2][W_HALVES];                // [parity][hi blocks, lo blocks]
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tP[CHUNK * PITCH64];
+  __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
   __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
   __shared__ __align__(16) float tE[128];
 
@@ -342,21 +349,20 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
     const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
     const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
     const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
-    const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
-    const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * 8192;
+    const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * (W_HALVES * 2);
+    const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * (TRI_BLOCKS * 1024);
     const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
     const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
-    const int64_t big_step = (int64_t)p.H * 16384, small_step = (int64_t)p.H * 8192, e_step = (int64_t)p.H * 512;
+    const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), p_step = (int64_t)p.H * (TRI_BLOCKS * 1024);
+    const int64_t e_step = (int64_t)p.H * 512;
     CopyWide plan_k, plan_v;
-    CopyNarrow plan_w;
     plan_k.plan(256, CHUNK - 1, 0, lane);
     plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, 0, lane);
-    plan_w.plan(128, CHUNK - 1, 0, lane);
     auto issue_kw = [&](int c) {                     // K e^G and W (hi, lo) into the buffers of c's parity
       const int par = c & 1;
       plan_k.issue(tK[par], kg_b + c * big_step, 0);
-      plan_w.issue(tW[par][0], w_b + c * big_step, 0);
-      plan_w.issue(tW[par][1], w_b + c * big_step + 8192, 0);
+#pragma unroll
+      for (int j = 0; j < 2 * TRI_BLOCKS; ++j) dma16(w_b + c * w_step, 1024u * j + 16u * lane, lds_address(tW[par]) + 1024u * j);
     };
     auto issue_v = [&](int c) {
       const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
@@ -371,12 +377,13 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
     };
     auto issue_second = [&](int c) {                 // scale Q e^G, P, K e^{G_last-G} (hi, lo), e^{G_last}
       plan_k.issue(tQ, qg_b + c * big_step, 0);
-      plan_w.issue(tP, pp_b + c * small_step, 0);
+#pragma unroll
+      for (int j = 0; j < TRI_BLOCKS; ++j) dma16(pp_b + c * p_step, 1024u * j + 16u * lane, lds_address(tP) + 1024u * j);
       plan_k.issue(tKt[0], kt_b + c * 2 * big_step, 0);
       plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, 0);
       if (lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
     };
-    constexpr int KW_COPIES = CopyWide::FIRST + 2 * CopyNarrow::FIRST;       // copies of one issue_kw
+    constexpr int KW_COPIES = CopyWide::FIRST + 2 * TRI_BLOCKS;              // copies of one issue_kw
     if (n_chunks > 0) {
       issue_kw(0);
       issue_v(0);
@@ -437,7 +444,12 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
     const uint16_t* const K = tK[par];
     // ---- KS = (K e^G) S^T ----
     f32x4_t KS[NB][4];
-    bf16x8_t wa[2][4], wl[2][4];
+    // W operands: block b of the six (row block tri_block_m(b), contraction half tri_block_s(b)), hi at block b, lo at
+    // block TRI_BLOCKS + b; one 16-byte read per lane
+    bf16x8_t wa[TRI_BLOCKS], wl[TRI_BLOCKS];
+    auto ldW = [&](int b, bool lo) {
+      return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][((lo ? TRI_BLOCKS : 0) + b) * 512 + lane * 8]));
+    };
     uint16_t vraw[NB][16];
     {
       bf16x8_t ka[2][4], sb[2][NB];
@@ -466,10 +478,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
               for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
             }
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
-            wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
-          }
+          for (int b = 0; b < 4; ++b) { wa[b] = ldW(b, false); wl[b] = ldW(b, true); }
         }
         __builtin_amdgcn_sched_barrier(0x000F);
         if (s < 3) {
@@ -486,10 +495,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
     f32x4_t U[NB][4];
     {
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
-        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
-      }
+      for (int b = 4; b < TRI_BLOCKS; ++b) { wa[b] = ldW(b, false); wl[b] = ldW(b, true); }
       __builtin_amdgcn_sched_barrier(0x000F);
       f32x4_t X[NB][4];
 #pragma unroll
@@ -507,14 +513,15 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
         bf16x8_t xb[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+        // lower triangular W: contraction half 1 only reaches row blocks 2 and 3
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+          for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wl[b], xb[nb], U[nb][tri_block_m(b)]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+          for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wa[b], xb[nb], U[nb][tri_block_m(b)]);
       }
     }
     // barrier B: Q, P, the K e^{G_last-G} pair and e^{G_last} of this chunk have landed
@@ -528,7 +535,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      bf16x8_t qa[2][4], sb[2][NB], pa[2][4];
+      bf16x8_t qa[2][4], sb[2][NB], pa[TRI_BLOCKS];
 #pragma unroll
       for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], 0, kb);
       __builtin_amdgcn_sched_barrier(0x000F);
@@ -541,9 +548,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
           for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], s + 1, kb);
         } else {
 #pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-            for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[(16 * ni + r16) * PITCH64], s2, kb);
+          for (int b = 0; b < TRI_BLOCKS; ++b) pa[b] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tP[b * 512 + lane * 8]));
         }
         __builtin_amdgcn_sched_barrier(0x000F);
         if (s < 3) {
@@ -572,7 +577,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(ur[nb], pa[s][ni], OT[nb][ni]);
+          for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) OT[nb][tri_block_m(b)] = mfma16h(ur[nb], pa[b], OT[nb][tri_block_m(b)]);
       }
       if (write_o) {
         const int len = chunk_len(ci);
@@ -661,7 +666,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
 __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
+  constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -686,7 +691,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
 
   __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
+  __shared__ __align__(16) uint16_t tW[2][W_HALVES];                // [parity][hi blocks, lo blocks]
   __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
   __shared__ __align__(16) float tE[128];
 
@@ -720,16 +725,14 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
   const int64_t tile0 = (int64_t)c_begin * p.H + h;
   const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
   const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * 16384;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * (W_HALVES * 2);
   const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
-  const int64_t big_step = (int64_t)p.H * 16384, e_step = (int64_t)p.H * 512;
+  const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), e_step = (int64_t)p.H * 512;
   CopyWide plan_k, plan_v;
-  CopyNarrow plan_w;
   if (m_side) {
     plan_k.plan(256, CHUNK - 1, cw, lane);
     plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
-    plan_w.plan(128, CHUNK - 1, cw, lane);
   }
   auto issue_first = [&](int c) {                    // K e^G, V, W (hi, lo) into the buffers of c's parity
     const int par = c & 1;
@@ -743,8 +746,9 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
       tail_v.issue(tV[par], vs, cw);
     }
-    plan_w.issue(tW[par][0], w_b + c * big_step, cw);
-    plan_w.issue(tW[par][1], w_b + c * big_step + 8192, cw);
+#pragma unroll
+    for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)      // twelve 1 KiB blocks, three per copying wavefront
+      dma16(w_b + c * w_step, 1024u * (4 * j + cw) + 16u * lane, lds_address(tW[par]) + 1024u * (4 * j + cw));
   };
   auto issue_second = [&](int c) {                   // K e^{G_last-G} (hi, lo), e^{G_last}
     plan_k.issue(tKt[0], kt_b + c * 2 * big_step, cw);
@@ -752,8 +756,8 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
     if (cw == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
   };
   // copies one wavefront issues in issue_first (constant: a tail plan has the same piece counts)
-  constexpr int FIRST_REST = 2 * (CopyWide::FIRST) + 2 * (CopyNarrow::FIRST);      // wavefront 4
-  constexpr int EACH_REST = 2 * (CopyWide::EACH) + 2 * (CopyNarrow::EACH);         // wavefronts 5-7
+  constexpr int FIRST_REST = 2 * (CopyWide::FIRST) + 2 * TRI_BLOCKS / 4;           // wavefront 4
+  constexpr int EACH_REST = 2 * (CopyWide::EACH) + 2 * TRI_BLOCKS / 4;             // wavefronts 5-7
 
   if (m_side && n_chunks > 0) issue_first(0);
 
@@ -773,7 +777,10 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       const uint16_t* const V = tV[par];
       // ---- KS = (K e^G) S^T ----
       f32x4_t KS[NB][4];
-      bf16x8_t wa[2][4], wl[2][4];
+      bf16x8_t wa[TRI_BLOCKS], wl[TRI_BLOCKS];          // W operand blocks (hi, lo), one 16-byte read per lane each
+      auto ldW = [&](int b, bool lo) {
+        return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][((lo ? TRI_BLOCKS : 0) + b) * 512 + lane * 8]));
+      };
       uint16_t vraw[NB][16];
       {
         bf16x8_t ka[2][4], sb[2][NB];
@@ -804,10 +811,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
                 }
             }
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) {
-              wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
-              wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
-            }
+            for (int b = 0; b < 4; ++b) { wa[b] = ldW(b, false); wl[b] = ldW(b, true); }
           }
           __builtin_amdgcn_sched_barrier(0x000F);
           if (s < 3) {
@@ -822,10 +826,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       }
       // ---- X = V - KS,  U = W X ----
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
-        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
-      }
+      for (int b = 4; b < TRI_BLOCKS; ++b) { wa[b] = ldW(b, false); wl[b] = ldW(b, true); }
       __builtin_amdgcn_sched_barrier(0x000F);
       f32x4_t X[NB][4];
 #pragma unroll
@@ -844,14 +845,15 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
         bf16x8_t xb[NB];
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
+        // lower triangular W: contraction half 1 only reaches row blocks 2 and 3
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+          for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wl[b], xb[nb], U[nb][tri_block_m(b)]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+          for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wa[b], xb[nb], U[nb][tri_block_m(b)]);
       }
     }
     // barrier B: the pair of this chunk has landed (copies issued after it may still be in flight)
@@ -937,9 +939,9 @@ static KdaWorkspaceLayout kda_layout(int T, int N, int H) {
   L.chunk_seq = take((size_t)L.NC_max * 4);
   L.chunk_tok = take((size_t)L.NC_max * 4);
   L.chunk_len = take((size_t)L.NC_max * 4);
-  const size_t big = (size_t)L.NC_max * H * 8192 * 2, small = (size_t)L.NC_max * H * 4096 * 2;
+  const size_t big = (size_t)L.NC_max * H * 8192 * 2, tri = (size_t)L.NC_max * H * TRI_BLOCKS * 1024;
   L.Kg = take(big); L.Qg = take(big); L.Kt = take(2 * big);
-  L.W = take(2 * small); L.P = take(small);
+  L.W = take(2 * tri); L.P = take(tri);
   L.eGlast = take((size_t)L.NC_max * H * 128 * 4);
   L.seg_chunks = pick_segment_chunks(T, N, H);
   L.max_segments = max_segments(T, N, L.seg_chunks);
