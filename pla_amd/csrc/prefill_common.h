@@ -479,7 +479,10 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
                                                   const SegmentTable& seg, const StageTable& stg, int stage,
                                                   const float* h0, const int32_t* h0_indices,
                                                   int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
-                                                  int64_t ht_slot_stride, bool resweep_first = false, int block = -1) {
+                                                  int64_t ht_slot_stride, bool resweep_first = false, int block = -1,
+                                                  const int3 inline_chunks = int3{-1, 0, 0}) {
+  // inline_chunks (pass 0 only, x >= 0): (first chunk, end chunk, stages in effect) of the workgroup's sequence worked
+  // out by the caller (inline_sequences) instead of read from the tables
   // block: the logical workgroup index when the caller remaps blockIdx (see xcd_grouped_index), else blockIdx.x
   // resweep_first: the first sweep publishes no output at all (first segments keep a copy of their start
   // state and only deliver the state they end in), the second sweep runs every segment with output.
@@ -498,8 +501,8 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     const int logical = block >= 0 ? block : (int)blockIdx.x;
     r.n = logical / heads;
     r.head = logical - r.n * heads;
-    r.c_begin = seq_chunk_off[r.n];
-    r.c_end = seq_chunk_off[r.n + 1];
+    r.c_begin = inline_chunks.x >= 0 ? inline_chunks.x : seq_chunk_off[r.n];
+    r.c_end = inline_chunks.x >= 0 ? inline_chunks.y : seq_chunk_off[r.n + 1];
     if (r.c_begin >= r.c_end) return r;              // empty sequence: state untouched, no output
     r.init = state_in(r.n, r.head);
     r.fin = state_out(r.n, r.head);
@@ -535,7 +538,7 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     }
   }
   if (carry != nullptr && stg.stages > 0) {
-    const int E = stg.stage_begin[MAX_STAGES + 1];                 // stages in effect (the table kernel's choice)
+    const int E = inline_chunks.x >= 0 ? inline_chunks.z : stg.stage_begin[MAX_STAGES + 1];   // stages in effect (the table kernel's choice)
     if (stage >= E) return r;                                      // an empty stage: the one before it delivered the state
     const int nc = r.c_end - r.c_begin, c0 = r.c_begin;
     r.c_begin = c0 + stage_cut(nc, stage, E);
@@ -545,6 +548,63 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
   }
   r.active = true;
   return r;
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same tables worked out by ONE wavefront in registers, for calls of whole sequences with at most 64
+// sequences: lane n holds sequence n, prefix sums run over the lanes.  A kernel that does this at its start needs no
+// table kernel before it (one launch and its gap less on the critical path of a call) and no dependent trips to
+// memory for its tile: one load of cu_seqlens per lane.  The results equal chunk_map / stage_map / staged_chunk /
+// select_sweep(pass 0) for the same offsets, including the rule that keeps a single stage for chains of nearly equal
+// length.  All 64 lanes of the wavefront must call these functions together.
+constexpr int INLINE_TABLE_SEQUENCES = 64;
+__device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int up = __shfl_up(x, d, 64);
+    if (lane >= d) x += up;
+  }
+  return x;
+}
+struct InlineSequences {
+  int start, len, nc, off;      // this lane's sequence: first token, tokens, chunks, first chunk (global index)
+  int total, E;                 // chunks of the call; stages in effect
+};
+__device__ __forceinline__ InlineSequences inline_sequences(const int32_t* cu_seqlens, int N, int stages, int lane) {
+  InlineSequences q;
+  const int a = lane < N ? cu_seqlens[lane] : 0, b = lane < N ? cu_seqlens[lane + 1] : 0;
+  q.start = a;
+  q.len = max(b - a, 0);
+  q.nc = (q.len + CHUNK - 1) / CHUNK;
+  const int incl = wave_inclusive_scan(q.nc, lane);
+  q.off = incl - q.nc;
+  q.total = __builtin_amdgcn_readlane(incl, 63);
+  int longest = q.nc;
+#pragma unroll
+  for (int d = 32; d > 0; d >>= 1) longest = max(longest, __shfl_xor(longest, d, 64));
+  longest = __builtin_amdgcn_readfirstlane(longest);
+  q.E = (stages > 0 && 5 * (int64_t)q.total < 4 * (int64_t)N * longest) ? stages : 1;
+  return q;
+}
+// Chunk `index` of stage `stage` (all chunks in order when the call is not staged): its global chunk id, first token
+// and length, or id -1 when the stage holds fewer chunks.
+struct InlineTile { int cb, t0, len; };
+__device__ __forceinline__ InlineTile inline_tile(const InlineSequences& q, int stage, int index, int NC_max, int lane) {
+  InlineTile t{-1, 0, 0};
+  if (stage >= q.E) return t;
+  const int lo = stage_cut(q.nc, stage, q.E), hi = stage_cut(q.nc, stage + 1, q.E);
+  const int cnt = hi - lo;
+  const int before = wave_inclusive_scan(cnt, lane) - cnt;
+  const unsigned long long owner = __ballot(index >= before && index < before + cnt);
+  if (owner == 0) return t;
+  const int n = __builtin_amdgcn_readfirstlane(__ffsll((long long)owner) - 1);
+  const int cc = __builtin_amdgcn_readlane(lo, n) + index - __builtin_amdgcn_readlane(before, n);
+  const int cb = __builtin_amdgcn_readlane(q.off, n) + cc;
+  if (cb >= NC_max) return t;                   // offsets that do not fit the workspace: the tile is skipped
+  t.cb = cb;
+  t.t0 = __builtin_amdgcn_readlane(q.start, n) + cc * CHUNK;
+  t.len = min(CHUNK, __builtin_amdgcn_readlane(q.len, n) - cc * CHUNK);
+  return t;
 }
 
 // Segments per sequence and the 128 x 128 identity.  Single workgroup, after chunk_map.

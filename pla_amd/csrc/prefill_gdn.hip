@@ -77,6 +77,8 @@ struct GdnPrefillParams {
   int stage;             // stage handled by this launch (per-chunk kernels and pass 3)
   int H, HV, NC_max;
   int qk_rows_16;        // q and k rows start on 16-byte boundaries (else on 4-byte ones)
+  int inline_tables;     // at most 64 whole sequences: kernels work the chunk tables out themselves (no table kernel)
+  int tail_blocks;       // workgroups appended to the preparation grid that zero the output rows beyond the last sequence
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -323,14 +325,27 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
 template <typename act_t, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefillParams p) {
   const int groups = p.HV / WAVES;
-  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
-  if (cb < 0) return;
+  const int lane = threadIdx.x & 63;
+  const int main_blocks = gridDim.x - p.tail_blocks;
+  if ((int)blockIdx.x >= main_blocks) {            // appended workgroups: zero the padded rows of o
+    zero_tail(reinterpret_cast<uint16_t*>(p.o), p.cu_seqlens, p.N, p.T, p.HV, blockIdx.x - main_blocks, p.tail_blocks);
+    return;
+  }
+  int cb, t0, len;
+  if (p.inline_tables) {
+    const InlineSequences seqs = inline_sequences(p.cu_seqlens, p.N, p.stg.stages, lane);
+    const InlineTile tile = inline_tile(seqs, p.stage, blockIdx.x / groups, p.NC_max, lane);
+    cb = tile.cb; t0 = tile.t0; len = tile.len;
+    if (cb < 0) return;
+  } else {
+    cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
+    if (cb < 0) return;
+    t0 = p.chunk_tok[cb];
+    len = p.chunk_len[cb];
+  }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int hv = (blockIdx.x % groups) * WAVES + wave;
   const int h = hv / (p.HV / p.H);
-  const int t0 = p.chunk_tok[cb];
-  const int len = p.chunk_len[cb];
-  const int lane = threadIdx.x & 63;
   const int r16 = lane & 15, kb = lane >> 4;
 
   __shared__ __align__(16) float Lm_all[WAVES][CHUNK][68];
@@ -1093,17 +1108,33 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   using CopyV = SwizzledTileCopy<AUX>;
   const int block = xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV);
   if (block < 0) return;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  // the chunks of this workgroup's sequence: from the tables, or worked out here (every wavefront for itself)
+  int3 inline_chunks{-1, 0, 0};
+  int seq_first_chunk = 0, seq_first_token = 0, seq_end_token = 0;
+  if (p.inline_tables) {
+    const InlineSequences seqs = inline_sequences(p.cu_seqlens, p.N, p.stg.stages, lane);
+    const int n0 = __builtin_amdgcn_readfirstlane(block / p.HV);
+    seq_first_chunk = __builtin_amdgcn_readlane(seqs.off, n0);
+    seq_first_token = __builtin_amdgcn_readlane(seqs.start, n0);
+    seq_end_token = seq_first_token + __builtin_amdgcn_readlane(seqs.len, n0);
+    inline_chunks = int3{seq_first_chunk, min(seq_first_chunk + __builtin_amdgcn_readlane(seqs.nc, n0), p.NC_max), seqs.E};
+  }
   const SweepRole role = select_sweep(0, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block, inline_chunks);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int h = hv / (p.HV / p.H);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
-  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
+  if (!p.inline_tables) {
+    seq_first_chunk = p.seq_chunk_off[n];
+    seq_first_token = p.cu_seqlens[n];
+    seq_end_token = p.cu_seqlens[n + 1];
+  }
+  const int seq_start = seq_first_token + (c_begin - seq_first_chunk) * CHUNK;
+  const int seq_len = min(seq_end_token - seq_start, (c_end - c_begin) * CHUNK);
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
@@ -1819,14 +1850,19 @@ static int gdn_prefill_run(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = stages;
   }
-  launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
-                segmented ? L.max_segments : N, o, HV);
+  // Whole sequences through the fused sweep, at most 64 of them: the kernels work the chunk tables out themselves and
+  // the first launch of the preparation also zeroes the padded rows of o, so no table kernel runs ahead of them.
+  p.inline_tables = fused && N <= INLINE_TABLE_SEQUENCES;
+  if (!p.inline_tables)
+    launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
+                  segmented ? L.max_segments : N, o, HV);
   const bool ok = launch_pipeline(
       s, stages, lease.get(), segmented, (unsigned)N * HV, (unsigned)L.max_segments * HV, &p.pass, &p.stage,
       [&](hipStream_t ps) {
         const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
         const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
-        const dim3 grid((unsigned)L.NC_max * (HV / waves)), block(64 * waves);
+        p.tail_blocks = (p.inline_tables && p.stage == 0) ? TABLE_WORKGROUPS - 1 : 0;
+        const dim3 grid((unsigned)L.NC_max * (HV / waves) + p.tail_blocks), block(64 * waves);
         if (fused) {
           if (half_act) {
             if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 4>), grid, block, 0, ps, p);

@@ -95,6 +95,34 @@ def test_gdn_prefill_small(lengths, tail_pad, H, HV):
     _check(w, fast=sum(lengths) > 3000)
 
 
+def test_gdn_prefill_64_sequences_and_65_give_the_same_bits():
+    """Calls of at most 64 whole sequences work their chunk tables out inside the kernels; with more sequences a
+    table kernel runs first.  64 ragged sequences (empty ones among them, a padded tail, both staged - chains of
+    unequal length - and unstaged) against the oracle, then the same tokens with one empty sequence appended (65
+    sequences: the table kernel) must give the same bits in o, g_cum and the 64 states."""
+    import random
+    from pla_amd.workloads import gdn_prefill_packed
+    rng = random.Random(5)
+    for longest, H, HV in ((300, 1, 2), (2200, 2, 4)):          # 128 chains of few chunks; 256 chains, staged
+        lengths = [rng.choice((0, 1, 63, 64, 65, 130, longest // 3)) for _ in range(64)]
+        lengths[7] = longest
+        lengths[63] = 77
+        results = []
+        _check(gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=70, seed=longest, tail_pad=9), fast=True)
+        for extra in ([], [0]):
+            w = gdn_prefill_packed(lengths + extra, H=H, HV=HV, pool_slots=70, seed=longest, tail_pad=9)
+            if not extra:
+                slots = w["initial_state_indices"]
+            else:                                               # the same slots for the 64, a free one for the empty sequence
+                free = (set(range(70)) - set(slots.cpu().tolist())).pop()
+                w["initial_state_indices"] = torch.cat([slots, torch.tensor([free], dtype=slots.dtype, device=slots.device)])
+            g_cum, _, o, _, final = _run_workload(w)
+            torch.cuda.synchronize()
+            results.append((o, g_cum.reshape(-1, HV)[:sum(lengths)], final[:64]))
+        for x, y in zip(*results):
+            assert torch.equal(x, y)
+
+
 @pytest.mark.parametrize("lengths,tail_pad", [([17], 3), ([200, 0, 33, 2049], 5), ([5555], 0)])
 def test_gdn_prefill_fp16_activations(lengths, tail_pad):
     """fp16 q / k / v / gates (the reference's FlashQLA takes both,
