@@ -24,20 +24,25 @@
 //                           gate, cumulative decay, decayed operand tiles (fp16), M / P on MFMA, the
 //                           inverse of I + L by 16 x 16 blocks, W and P (fp16)
 //   kda_sweep_kernel        one workgroup per (sequence, head) or second segment sweep: four computing
-//                           wavefronts x 32 V columns with a register-chained MFMA pipeline, one wavefront
-//                           that issues the asynchronous global -> LDS tile copies; writes o
+//                           wavefronts x 32 V columns with a register-chained MFMA pipeline, two wavefronts
+//                           that issue the asynchronous global -> LDS tile copies; writes o
 //   kda_lean_sweep_kernel   first sweep over segments: the zero-state sweep and the transition-matrix
 //                           sweep of two segments in one workgroup of eight wavefronts, no output
 // The operands of every sweep product are fp16 (v_mfma_f32_16x16x32_f16): the decayed tiles hold factors in
 // (0, 1].  W, K e^{G_last-G} and the U of the state update are hi + lo pairs; a float64 simulation of these
 // rounding points gives a final-state rel-L2 below 5e-4 from strong to weak decay (bound 1e-3); the pairs are
-// what keeps keys that repeat within a chunk inside the same bound.  The K e^{G_last-G} tile is stored row major like the others; its transposed
+// what keeps keys that repeat within a chunk inside the same bound (measured on such keys: 3.3e-4 .. 3.7e-4 with the
+// pairs, 1.7e-3 with K e^{G_last-G} rounded once).  The K e^{G_last-G} tile is stored row major like the others; its transposed
 // operands come from ds_read_b64_tr_b16.
 
 #include "prefill_common.h"
 
 namespace pla {
 
+// Wavefronts of kda_sweep_kernel that issue its global -> LDS copies.  One wavefront holds at most 63 memory
+// operations in flight (1 KiB each here); two share the issue work and that limit (config 4: 2.46 -> 2.44 ms, 2.43 ms
+// with three).
+constexpr int KDA_SWEEP_COPIERS = 2;
 struct KdaPrefillParams {
   const void* q; const void* k; const void* v; const void* g; const void* beta;   // bf16
   int64_t stride_q, stride_k, stride_v, stride_g, stride_beta;                    // token pitches (elements)
@@ -306,21 +311,23 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 
 // ---------------------------------------------------------------------------------------------
 // Sequential kernel with output (whole sequences, and the second sweep over segments): one workgroup per
-// (sequence or segment, head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
-// memory only to store their output rows; wavefront 4 issues every global -> LDS copy of the workgroup (an LDS
-// copy occupies its issuer for tens of cycles, about 2.5 k cycles per chunk in all).  S^T stays in MFMA
+// (sequence or segment, head) of SIX wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
+// memory only to store their output rows; wavefronts 4 and 5 issue the global -> LDS copies of the workgroup, every
+// tile dealt between them in 1 KiB pieces (an LDS copy occupies its issuer for tens of cycles, about 2.5 k cycles
+// per chunk in all, and a wavefront holds at most 63 of them in flight).  S^T stays in MFMA
 // accumulator layout (an accumulator tile pair is already a valid operand of the next product); the output product
 // is formed transposed, so that a lane holds four adjacent V columns of one token and stores them as 8 bytes.
-// 151 KB of LDS: K e^G and W (hi, lo) are double buffered by chunk parity, everything else is single, with two
+// 133 KiB of LDS: K e^G and W (hi, lo) are double buffered by chunk parity, everything else is single, with two
 // barriers per chunk:
 //   barrier A   K e^G, W, V of chunk c landed; chunk c - 1 finished     copy scale Q e^G, P, K e^{G_last-G} (hi, lo),
 //               KS = (K e^G) S^T,  X = V - KS,  U = W X                 e^{G_last} of c, then K e^G and W of c + 1
 //   barrier B   the tiles requested at A landed; V is free              copy V of c + 1
 //               O^T = S (scale Q e^G)^T + U^T P^T -> rows of o
 //               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U         (pairs: hi.lo + lo.hi + hi.hi)
-__global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParams p) {
+__global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2;
-  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
+  constexpr int NCOPY = KDA_SWEEP_COPIERS;
+  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, NCOPY>;  // 64 x 128 tile, its pieces dealt to the copying wavefronts
   constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -343,7 +350,8 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
   __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
   __shared__ __align__(16) float tE[128];
 
-  if (wave == 4) {
+  if (wave >= 4) {
+    const int cw = wave - 4;                         // which of the copying wavefronts
     // ---- the copying wavefront -------------------------------------------------------------
     const int64_t tile0 = (int64_t)c_begin * p.H + h;
     const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
@@ -356,34 +364,42 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
     const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), p_step = (int64_t)p.H * (TRI_BLOCKS * 1024);
     const int64_t e_step = (int64_t)p.H * 512;
     CopyWide plan_k, plan_v;
-    plan_k.plan(256, CHUNK - 1, 0, lane);
-    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, 0, lane);
+    plan_k.plan(256, CHUNK - 1, cw, lane);
+    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
     auto issue_kw = [&](int c) {                     // K e^G and W (hi, lo) into the buffers of c's parity
       const int par = c & 1;
-      plan_k.issue(tK[par], kg_b + c * big_step, 0);
+      plan_k.issue(tK[par], kg_b + c * big_step, cw);
 #pragma unroll
-      for (int j = 0; j < 2 * TRI_BLOCKS; ++j) dma16(w_b + c * w_step, 1024u * j + 16u * lane, lds_address(tW[par]) + 1024u * j);
+      for (int j0 = 0; j0 < 2 * TRI_BLOCKS / NCOPY; ++j0) {
+        const int j = NCOPY * j0 + cw;
+        dma16(w_b + c * w_step, 1024u * j + 16u * lane, lds_address(tW[par]) + 1024u * j);
+      }
     };
     auto issue_v = [&](int c) {
       const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
       const int len = chunk_len(c);
       if (len == CHUNK) {
-        plan_v.issue(tV, vs, 0);
+        plan_v.issue(tV, vs, cw);
       } else {                                       // rows past the sequence re-read its last row
         CopyWide tail_v;
-        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, 0, lane);
-        tail_v.issue(tV, vs, 0);
+        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
+        tail_v.issue(tV, vs, cw);
       }
     };
     auto issue_second = [&](int c) {                 // scale Q e^G, P, K e^{G_last-G} (hi, lo), e^{G_last}
-      plan_k.issue(tQ, qg_b + c * big_step, 0);
+      plan_k.issue(tQ, qg_b + c * big_step, cw);
 #pragma unroll
-      for (int j = 0; j < TRI_BLOCKS; ++j) dma16(pp_b + c * p_step, 1024u * j + 16u * lane, lds_address(tP) + 1024u * j);
-      plan_k.issue(tKt[0], kt_b + c * 2 * big_step, 0);
-      plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, 0);
-      if (lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
+      for (int j0 = 0; j0 < TRI_BLOCKS / NCOPY; ++j0) {
+        const int j = NCOPY * j0 + cw;
+        dma16(pp_b + c * p_step, 1024u * j + 16u * lane, lds_address(tP) + 1024u * j);
+      }
+      plan_k.issue(tKt[0], kt_b + c * 2 * big_step, cw);
+      plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, cw);
+      if (cw == NCOPY - 1 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
     };
-    constexpr int KW_COPIES = CopyWide::FIRST + 2 * TRI_BLOCKS;              // copies of one issue_kw
+    static_assert(2 * TRI_BLOCKS % NCOPY == 0 && TRI_BLOCKS % NCOPY == 0, "W and P pieces are dealt evenly");
+    // copies of one issue_kw by this wavefront (the first copying wavefront also takes the pieces left over)
+    constexpr int KW_FIRST = CopyWide::FIRST + 2 * TRI_BLOCKS / NCOPY, KW_OTHER = CopyWide::EACH + 2 * TRI_BLOCKS / NCOPY;
     if (n_chunks > 0) {
       issue_kw(0);
       issue_v(0);
@@ -395,7 +411,8 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
       issue_second(ci);
       if (more) {
         issue_kw(ci + 1);
-        wait_vmcnt<KW_COPIES>();                     // the second-half tiles of ci have landed (what follows may be in flight)
+        // the second-half tiles of ci have landed (what follows may be in flight)
+        if (cw == 0) wait_vmcnt<KW_FIRST>(); else wait_vmcnt<KW_OTHER>();
       } else {
         wait_vmcnt<0>();
       }
@@ -658,7 +675,7 @@ __global__ __launch_bounds__(320, 1) void kda_sweep_kernel(const KdaPrefillParam
 // from its real start state (of which they keep a copy for the second sweep).
 //
 // The tiles of a chunk's first half (K e^G, V, W hi / lo) are double buffered by chunk parity, the hi / lo pair of
-// K e^{G_last - G} and e^{G_last} single (142 KB of LDS), with two barriers per chunk:
+// K e^{G_last - G} and e^{G_last} single (127 KiB of LDS), with two barriers per chunk:
 //   barrier A   first-half tiles of chunk c landed, chunk c - 1 finished    copy K e^{G_last-G} (hi, lo), e^{G_last} of c,
 //               KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X             then the first-half tiles of chunk c + 1
 //   barrier B   the pair of c landed
@@ -1054,14 +1071,14 @@ extern "C" int pla_kda_prefill_launch(
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
         // the first sweep over segments publishes no output: both of its roles in one workgroup per (segment, head)
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(kda_sweep_kernel, dim3(grid), dim3(320), 0, s, p);
+        else hipLaunchKernelGGL(kda_sweep_kernel, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_sweep_kernel, dim3((unsigned)L.max_segments * H), dim3(320), 0, s, p);
+    hipLaunchKernelGGL(kda_sweep_kernel, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
