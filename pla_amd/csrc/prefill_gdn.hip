@@ -322,6 +322,10 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
 // with the raw cumulative log-decay appended for the sweep's P), normalised K in registers, K K^T on MFMA, the
 // inverse of I + L by 16 x 16 blocks, and W = (I + L)^-1 diag(beta) as an fp16 hi + lo pair in the six-block
 // operand layout (12 KiB per (chunk, value head) instead of 16 KiB row-major + 8 KiB of P + the normalised rows).
+// The blocks of L below the diagonal never leave the registers: the accumulators of K K^T are the operands of the
+// transposed block recursion as they stand, and its results are the lane's pieces of the W blocks.  Registers, not
+// LDS, then bound the occupancy (two wavefronts per SIMD; forcing three or four spills and is slower: config 3
+// 0.446 / 0.455 / 0.489 ms).
 template <typename act_t, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefillParams p) {
   const int groups = p.HV / WAVES;
@@ -348,10 +352,14 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   const int h = hv / (p.HV / p.H);
   const int r16 = lane & 15, kb = lane >> 4;
 
-  __shared__ __align__(16) float Lm_all[WAVES][CHUNK][68];
+  // Per wavefront only the four diagonal 16 x 16 blocks of L pass through LDS (rows of 20 floats, blocks 336 floats
+  // apart: the four groups of 16 lanes that walk one block each in the forward substitution stay on different banks);
+  // the six blocks below the diagonal stay in the accumulators of K K^T.  5.9 KB instead of a 64 x 68 FP32 tile.
+  constexpr int DIAG_PITCH = 20, DIAG_BLOCK = 336;
+  __shared__ __align__(16) float Ld_all[WAVES][4 * DIAG_BLOCK];
   __shared__ __align__(16) float Gs_all[WAVES][CHUNK];
   __shared__ __align__(16) float Bs_all[WAVES][CHUNK];
-  float (*const Lm)[68] = Lm_all[wave];
+  float* const Ld = Ld_all[wave];
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
@@ -458,25 +466,111 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   }
   __syncthreads();
 
-  // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
+  // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j}) by 16 x 16 blocks.  The accumulators of block (mi, ni) hold rows
+  // i = 4 kb + r of column j = r16: for a block below the diagonal that is the A operand of L_ab^T as it stands
+  // (Lr[mi][ni]); the diagonal blocks go to LDS, row major, for the forward substitution.
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t Lr[4][4];
 #pragma unroll
   for (int mi = 0; mi < 4; ++mi) {
+    const float4 Gi = *reinterpret_cast<const float4*>(&Gs[16 * mi + 4 * kb]);
+    const float4 Bi = *reinterpret_cast<const float4*>(&Bs[16 * mi + 4 * kb]);
+    const float gi[4] = {Gi.x, Gi.y, Gi.z, Gi.w}, bi[4] = {Bi.x, Bi.y, Bi.z, Bi.w};
 #pragma unroll
     for (int ni = 0; ni <= mi; ++ni) {
-      f32x4_t kk = {0.f, 0.f, 0.f, 0.f};
+      f32x4_t kk = zero;
 #pragma unroll
       for (int s = 0; s < 4; ++s) kk = mfma16h(Kop[mi][s], Kop[ni][s], kk);
-      const int j = 16 * ni + r16;
-      const float Gj = Gs[j];
+      const float Gj = Gs[16 * ni + r16];
+      if (ni < mi) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * mi + 4 * kb + r;
-        Lm[i][j] = i > j ? Bs[i] * kk[r] * __expf(Gs[i] - Gj) : 0.f;
+        for (int r = 0; r < 4; ++r) Lr[mi][ni][r] = bi[r] * kk[r] * __expf(gi[r] - Gj);
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          Ld[mi * DIAG_BLOCK + (4 * kb + r) * DIAG_PITCH + r16] = 4 * kb + r > r16 ? bi[r] * kk[r] * __expf(gi[r] - Gj) : 0.f;
       }
     }
   }
-  block_inverse_inplace(Lm, lane);
-  store_w_operand_blocks(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * (2 * TRI_BLOCKS * 512));
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // Diagonal blocks D_a = (I + L_aa)^-1: lane (a = kb, j = r16) solves column j by forward substitution over the 16
+  // rows, x_i = [i == j] - sum_{l < i} L_aa[i][l] x_l, and writes it over row j of the block (the block then holds
+  // D_a^T; every read of L_aa precedes the writes: one wavefront, LDS operations complete in order).
+  {
+    float* const La = Ld + kb * DIAG_BLOCK;
+    float x[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int l4 = 0; l4 < i; l4 += 4) {
+        const float4 row = *reinterpret_cast<const float4*>(&La[i * DIAG_PITCH + l4]);
+        acc0 = fmaf(row.x, x[l4], acc0);
+        if (l4 + 1 < i) acc1 = fmaf(row.y, x[l4 + 1], acc1);
+        if (l4 + 2 < i) acc0 = fmaf(row.z, x[l4 + 2], acc0);
+        if (l4 + 3 < i) acc1 = fmaf(row.w, x[l4 + 3], acc1);
+      }
+      x[i] = (i == r16 ? 1.f : 0.f) - (acc0 + acc1);
+    }
+#pragma unroll
+    for (int i4 = 0; i4 < 16; i4 += 4)
+      *reinterpret_cast<float4*>(&La[r16 * DIAG_PITCH + i4]) = make_float4(x[i4], x[i4 + 1], x[i4 + 2], x[i4 + 3]);
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // Dq[a]: D_a[r16][4 kb + r], the lane's piece of D_a as the operand of a product that contracts over its columns
+  // and, as it stands, of the W blocks; DTq[b]: D_b[4 kb + r][r16], the same for D_b^T.
+  f32x4_t Dq[4], DTq[3];
+#pragma unroll
+  for (int a = 0; a < 4; ++a)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) Dq[a][r] = Ld[a * DIAG_BLOCK + (4 * kb + r) * DIAG_PITCH + r16];
+#pragma unroll
+  for (int b = 0; b < 3; ++b) {
+    const float4 t = *reinterpret_cast<const float4*>(&Ld[b * DIAG_BLOCK + r16 * DIAG_PITCH + 4 * kb]);
+    DTq[b] = f32x4_t{t.x, t.y, t.z, t.w};
+  }
+  // The blocks of N = (I + L)^-1 below the diagonal, transposed: N_ab^T = -D_b^T sum_{b < c <= a} L_cb^T N_ac^T with
+  // N_aa = D_a, in order of a - b = 1, 2, 3.  Every product has the earlier result on its right, where an accumulator
+  // tile is an operand as it stands, and leaves N_ab^T in accumulator layout: rows j = 4 kb + r of column i = r16,
+  // which is the lane's piece N_ab[r16][4 kb + r] of a W block.  FP32 values cross the MFMA as bf16 hi / lo pairs.
+  auto negate = [](f32x4_t t) { return f32x4_t{-t.x, -t.y, -t.z, -t.w}; };
+  auto solve = [&](int b, f32x4_t y) { return negate(mfma_hilo(split8(DTq[b], zero), split8(y, zero), zero)); };
+  f32x4_t Nq[4][4];
+  Nq[1][0] = solve(0, mfma_hilo(split8(Lr[1][0], zero), split8(Dq[1], zero), zero));
+  Nq[2][1] = solve(1, mfma_hilo(split8(Lr[2][1], zero), split8(Dq[2], zero), zero));
+  Nq[3][2] = solve(2, mfma_hilo(split8(Lr[3][2], zero), split8(Dq[3], zero), zero));
+  Nq[2][0] = solve(0, mfma_hilo(split8(Lr[1][0], Lr[2][0]), split8(Nq[2][1], Dq[2]), zero));
+  Nq[3][1] = solve(1, mfma_hilo(split8(Lr[2][1], Lr[3][1]), split8(Nq[3][2], Dq[3]), zero));
+  {
+    f32x4_t y = mfma_hilo(split8(Lr[1][0], Lr[2][0]), split8(Nq[3][1], Nq[3][2]), zero);
+    y = mfma_hilo(split8(Lr[3][0], zero), split8(Dq[3], zero), y);
+    Nq[3][0] = solve(0, y);
+  }
+  // W = N diag(beta) as an fp16 hi + lo pair in the six-block operand layout: block (row block m, column half s) holds
+  // the lane's pieces of blocks (m, 2 s) and (m, 2 s + 1)
+  uint16_t* const Wt = p.W + ((int64_t)cb * p.HV + hv) * (2 * TRI_BLOCKS * 512);
+#pragma unroll
+  for (int b = 0; b < TRI_BLOCKS; ++b) {
+    const int m = tri_block_m(b), sh = tri_block_s(b);
+    uint32_t hi[4], lo[4];
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int cbk = 2 * sh + half;                       // column block
+      f32x4_t n4 = zero;
+      if (cbk < m) n4 = Nq[m][cbk];
+      else if (cbk == m) n4 = Dq[m];
+      const float4 b4 = *reinterpret_cast<const float4*>(&Bs[16 * cbk + 4 * kb]);
+      const bool diag = cbk == m;                          // a diagonal block keeps columns j <= i
+      const float w0 = !diag || 4 * kb <= r16 ? n4[0] * b4.x : 0.f, w1 = !diag || 4 * kb + 1 <= r16 ? n4[1] * b4.y : 0.f;
+      const float w2 = !diag || 4 * kb + 2 <= r16 ? n4[2] * b4.z : 0.f, w3 = !diag || 4 * kb + 3 <= r16 ? n4[3] * b4.w : 0.f;
+      pack2_pair(w0, w1, hi[2 * half], lo[2 * half]);
+      pack2_pair(w2, w3, hi[2 * half + 1], lo[2 * half + 1]);
+    }
+    *reinterpret_cast<uint4*>(Wt + b * 512 + lane * 8) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+    *reinterpret_cast<uint4*>(Wt + (TRI_BLOCKS + b) * 512 + lane * 8) = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
