@@ -21,7 +21,9 @@ Shapes outside head_dim 128 and other operator families (``mamba2_ssm``) are rep
 Decode shapes are timed as graph replays over rotating slot sets (the host-side argument checks cost
 more than the small kernels, and a fixed slot set would be served from the last-level cache).
 
-Command line: ``python -m pla_amd.caselist FILE [--limit N] [--csv OUT]``.
+Command line: ``python -m pla_amd.caselist FILE [--limit N] [--csv OUT]`` times every case;
+``python -m pla_amd.caselist FILE --check N`` checks N seeded small prefill shapes of the list instead (each against
+itself fed in two chained calls per sequence; ``check_case`` also takes a reference, which the tests use).
 """
 
 import argparse
@@ -222,6 +224,113 @@ def build_case(case, device="cuda", seed=0, sets=None):
     return [fn], dict(kind="kda_prefill", tokens=tokens, workload=w)
 
 
+def select_check_cases(cases, n, seed=0, max_tokens=2048):
+    """``n`` prefill cases of a list for a correctness check: drawn with a seeded generator from the served prefill
+    cases of at most ``max_tokens`` tokens (small enough for a CPU reference), in the order of the list."""
+    import random
+    small = [c for c in cases if c["phase"] == "P" and unsupported_reason(c) is None and c["cu_seqlens_q"][-1] <= max_tokens]
+    if len(small) <= n:
+        return small
+    keep = set(random.Random(seed).sample(range(len(small)), n))
+    return [c for i, c in enumerate(small) if i in keep]
+
+
+def run_prefill_case(case, device="cuda", seed=0, split=False):
+    """One prefill case on seeded synthetic inputs: returns ``(o, final_states, inputs)`` with ``o`` [T, HV, 128],
+    the final states [N, HV, 128, 128] and the input tensors (what a CPU reference needs).  With ``split`` every
+    sequence is fed in two calls - its first ``len // 2`` tokens, then the rest from the state the first call left -
+    and the outputs are put back into the order of the single call: both ways must agree to rounding."""
+    from . import workloads
+    from .prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from .prefill.flashkdapro import flashkda_fwd
+    dtype = torch.bfloat16 if case["dtype"] == "bf16" else torch.float16
+    H, HV = case["num_heads_qk"], case["num_heads_v"]
+    offs = list(case["cu_seqlens_q"])
+    N, T = len(offs) - 1, offs[-1]
+    lb = case.get("gate_lower_bound")
+    mids = [lo + (hi - lo) // 2 for lo, hi in zip(offs, offs[1:])]
+    # token rows of the two calls of a split run, and the offsets of each call
+    parts = [[(lo, mid) for lo, mid in zip(offs, mids)], [(mid, hi) for mid, hi in zip(mids, offs[1:])]] if split else \
+            [[(lo, hi) for lo, hi in zip(offs, offs[1:])]]
+
+    def rows_and_offsets(part):
+        rows = torch.cat([torch.arange(lo, hi) for lo, hi in part] + [torch.arange(0)]).to(device)
+        cu = [0]
+        for lo, hi in part:
+            cu.append(cu[-1] + hi - lo)
+        return rows, cu
+
+    if case["op"] == "gdn_attn":
+        w = workloads.gdn_prefill_packed([hi - lo for lo, hi in zip(offs, offs[1:])], H=H, HV=HV,
+                                         pool_slots=max(8, N + 3), seed=seed, device=device, dtype=dtype)
+        pool = w["initial_state"].clone()
+        idx = w["initial_state_indices"]
+        o = torch.zeros(T, HV, 128, dtype=dtype, device=device)
+        for part in parts:
+            rows, cu = rows_and_offsets(part)
+            if rows.numel() == 0:
+                continue
+            out = gdn_prefill_packed_qkv_fwd(
+                w["packed_qkv"][rows].contiguous(), w["raw_gate_a"][rows].contiguous(), w["raw_beta_b"][rows].contiguous(),
+                w["A_log"], w["dt_bias"], torch.tensor(cu, dtype=torch.int32, device=device), num_qk_heads=H,
+                num_v_heads=HV, scale=w["scale"], initial_state=pool, initial_state_indices=idx,
+                raw_cu_seqlens=tuple(cu), output_final_state=False)
+            o[rows] = out[2][0]
+        torch.cuda.synchronize()
+        return o, pool[idx.long()], w
+    g = torch.Generator().manual_seed(seed)
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    w = dict(q=rnd(T, H, 128).to(dtype).to(device), k=rnd(T, H, 128).to(dtype).to(device),
+             v=rnd(T, H, 128).to(dtype).to(device), g=rnd(T, H, 128).to(dtype).to(device),
+             beta=rnd(T, H).to(dtype).to(device), A_log=(rnd(H) * 0.5).to(device), dt_bias=(rnd(H, 128) * 0.1).to(device),
+             scale=128 ** -0.5, lower_bound=-5.0 if lb is None else lb, initial_state=(rnd(N, H, 128, 128) * 0.1).to(device),
+             offsets=offs)
+    o = torch.zeros(T, H, 128, dtype=dtype, device=device)
+    state = w["initial_state"]
+    for part in parts:
+        rows, cu = rows_and_offsets(part)
+        final = torch.empty(N, H, 128, 128, dtype=torch.float32, device=device)
+        if rows.numel() == 0:
+            continue
+        out = torch.empty(rows.numel(), H, 128, dtype=dtype, device=device)
+        flashkda_fwd(w["q"][rows].contiguous(), w["k"][rows].contiguous(), w["v"][rows].contiguous(),
+                     w["g"][rows].contiguous(), w["beta"][rows].contiguous(), w["A_log"], w["dt_bias"], out,
+                     scale=w["scale"], lower_bound=w["lower_bound"], initial_state=state, final_state=final,
+                     cu_seqlens=torch.tensor(cu, dtype=torch.int32, device=device))
+        o[rows] = out
+        state = final
+    torch.cuda.synchronize()
+    return o, state, w
+
+
+def check_case(case, reference=None, device="cuda", seed=0):
+    """Correctness of one prefill case.  ``reference(case, inputs) -> (o, final_states)`` supplies the expected
+    result (the tests pass the CPU oracle); without one the case is compared with itself fed in two chained calls
+    per sequence.  Returns a row with the largest output error in units of the tolerance ``2e-2 + 2e-2 |o|``
+    (``o_err`` <= 1 passes), the worst relative L2 error of a final state (bound 1e-3 against a reference, 2e-3
+    between the two ways of calling, which round differently) and ``ok``."""
+    o, final, w = run_prefill_case(case, device=device, seed=seed)
+    if reference is not None:
+        want_o, want_final = reference(case, w)
+        bound = 1e-3
+    else:
+        want_o, want_final, _ = run_prefill_case(case, device=device, seed=seed, split=True)
+        bound = 2e-3
+    want_o = want_o.to(o.device).float()
+    want_final = want_final.to(final.device).float()
+    o_err = float(((o.float() - want_o).abs() / (2e-2 + 2e-2 * want_o.abs())).max()) if o.numel() else 0.0
+    worst = 0.0
+    for n in range(final.shape[0]):
+        for h in range(final.shape[1]):
+            den = float(want_final[n, h].norm())
+            num = float((final[n, h] - want_final[n, h]).norm())
+            worst = max(worst, num / den if den > 0 else num)
+    finite = bool(torch.isfinite(o.float()).all() and torch.isfinite(final).all())
+    return dict(family=case["family"], heads=f"{case['num_heads_qk']}/{case['num_heads_v']}", batch=case["batch_size"],
+                tokens=case["cu_seqlens_q"][-1], against="reference" if reference is not None else "split calls",
+                o_err=round(o_err, 4), state_rel_l2=float("%.3e" % worst), ok=finite and o_err <= 1.0 and worst <= bound)
+
+
 def replay_case(case, device="cuda", reps=20, seed=0):
     """Runs and times one case.  Returns a result row (dict)."""
     row = dict(family=case["family"], phase=case["phase"], batch=case.get("batch_size"),
@@ -246,12 +355,26 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
     ap.add_argument("caselist")
     ap.add_argument("--limit", type=int, default=None)
+    ap.add_argument("--start", type=int, default=0, help="skip this many cases of the list (a long list replayed in parts)")
     ap.add_argument("--csv", default=None)
     ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--check", type=int, default=0, metavar="N",
+                    help="instead of timing, check N seeded small prefill shapes of the list: each case against itself "
+                         "fed in two chained calls per sequence; exit status 1 if a case fails")
+    ap.add_argument("--check-max-tokens", type=int, default=2048)
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         print("a GPU is required to replay a caselist", file=sys.stderr)
         return 2
+    if args.check > 0:
+        chosen = select_check_cases(read_caselist(args.caselist, args.limit), args.check, max_tokens=args.check_max_tokens)
+        failed = 0
+        for case in chosen:
+            row = check_case(case)
+            failed += not row["ok"]
+            print(row, flush=True)
+        print(f"checked {len(chosen)} cases, {failed} failed", flush=True)
+        return 1 if failed else 0
     # rows are written as they are measured, so that an interrupted replay keeps what it has
     keys = ["family", "phase", "kind", "batch", "heads", "seqlen_q", "tokens", "us", "tokens_per_s", "state_GBps",
             "status", "reason"]
@@ -260,7 +383,7 @@ def main(argv=None):
     if writer:
         writer.writeheader()
     try:
-        for case in read_caselist(args.caselist, args.limit):
+        for case in read_caselist(args.caselist, args.limit)[args.start:]:
             row = replay_case(case, reps=args.reps)
             print(row, flush=True)
             if writer:

@@ -1,4 +1,5 @@
-"""Caselist parsing (CPU) and replay of a sample of the reference's caselists with a parity check (GPU).
+"""Caselist parsing (CPU), replay of a sample of the reference's caselists with a parity check and the check of
+sampled prefill shapes against the oracle (GPU).
 
 ``tests/golden/caselist_sample.list`` holds seventeen lines of the reference's caselists (shapes only)."""
 import os
@@ -86,3 +87,63 @@ def test_replay_sample_and_check_against_oracle():
     torch.testing.assert_close(info["out"].cpu().float(), want_o.float(), atol=2e-2, rtol=2e-2)
     for slot in w["state_indices"].tolist():
         assert rel_l2(info["workload"]["state"][slot], want_s[slot]) <= 1e-3
+
+
+def _oracle_reference(case, w):
+    """Expected result of a prefill case from the CPU oracle (float64 chunked evaluation of the definition)."""
+    from oracle import chunked_delta_rule_fp64, softplus_gate, sigmoid_beta, l2norm, lower_bound_gate
+    offs = case["cu_seqlens_q"]
+    T = offs[-1]
+    if case["op"] == "gdn_attn":
+        H, HV = case["num_heads_qk"], case["num_heads_v"]
+        packed = w["packed_qkv"].cpu()
+        q = packed[:, : H * 128].reshape(T, H, 128)
+        k = packed[:, H * 128: 2 * H * 128].reshape(T, H, 128)
+        v = packed[:, 2 * H * 128:].reshape(T, HV, 128)
+        S0 = w["initial_state"][w["initial_state_indices"].long()].cpu()
+        gate = softplus_gate(w["raw_gate_a"].cpu(), w["dt_bias"].cpu(), w["A_log"].cpu())
+        beta = sigmoid_beta(w["raw_beta_b"].cpu())
+        scale = w["scale"]
+    else:
+        HV = case["num_heads_v"]
+        q, k, v = w["q"].cpu(), w["k"].cpu(), w["v"].cpu()
+        S0 = w["initial_state"].cpu()
+        gate = lower_bound_gate(w["g"].cpu(), w["dt_bias"].cpu(), w["A_log"].cpu(), w["lower_bound"])
+        beta = sigmoid_beta(w["beta"].cpu())
+        scale = w["scale"]
+    qn, kn = l2norm(q).to(q.dtype), l2norm(k).to(k.dtype)
+    o = torch.zeros(T, HV, 128, dtype=torch.float64)
+    final = S0.double().clone()
+    for n, (lo, hi) in enumerate(zip(offs, offs[1:])):
+        if hi > lo:
+            o[lo:hi], final[n] = chunked_delta_rule_fp64(qn[lo:hi], kn[lo:hi], v[lo:hi], gate[lo:hi], beta[lo:hi], S0[n], scale=scale)
+    return o, final
+
+
+def test_select_check_cases_is_seeded_and_small():
+    cases = caselist.read_caselist(PREFILL_EVERY50)
+    chosen = caselist.select_check_cases(cases, 24, seed=0, max_tokens=1800)
+    assert len(chosen) == 24 and chosen == caselist.select_check_cases(cases, 24, seed=0, max_tokens=1800)
+    assert all(c["phase"] == "P" and c["cu_seqlens_q"][-1] <= 1800 for c in chosen)
+    assert chosen != caselist.select_check_cases(cases, 24, seed=1, max_tokens=1800)
+    order = [cases.index(c) for c in chosen]
+    assert order == sorted(order)
+    assert len(caselist.select_check_cases(cases, 10 ** 6, max_tokens=500)) == sum(c["cu_seqlens_q"][-1] <= 500 for c in cases)
+
+
+@pytest.mark.gpu
+def test_check_24_sampled_prefill_shapes_against_the_oracle_and_split_calls():
+    """24 seeded shapes of the every-50th prefill list (up to 1800 tokens): each against the CPU oracle at the stated
+    tolerances, and the first eight also against themselves fed in two chained calls per sequence (what
+    ``python -m pla_amd.caselist FILE --check N`` runs)."""
+    cases = caselist.select_check_cases(caselist.read_caselist(PREFILL_EVERY50), 24, seed=0, max_tokens=1800)
+    assert len(cases) == 24
+    for i, case in enumerate(cases):
+        row = caselist.check_case(case, reference=_oracle_reference, seed=i)
+        print(row, flush=True)
+        assert row["ok"], row
+        if i < 8:
+            row = caselist.check_case(case, seed=i)
+            print(row, flush=True)
+            assert row["ok"], row
+    assert caselist.main([PREFILL_EVERY50, "--check", "3", "--check-max-tokens", "600"]) == 0
