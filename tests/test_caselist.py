@@ -138,12 +138,17 @@ def test_check_24_sampled_prefill_shapes_against_the_oracle_and_split_calls():
     ``python -m pla_amd.caselist FILE --check N`` runs)."""
     cases = caselist.select_check_cases(caselist.read_caselist(PREFILL_EVERY50), 24, seed=0, max_tokens=1800)
     assert len(cases) == 24
+    ties = 0
     for i, case in enumerate(cases):
         row = caselist.check_case(case, reference=_oracle_reference, seed=i)
         print(row, flush=True)
         assert row["ok"], row
+        ties += row["states_over_bound"]
         if i < 8:
             row = caselist.check_case(case, seed=i)
             print(row, flush=True)
             assert row["ok"], row
+    # states beyond 1e-3 are rounding ties of a normalised key under strong decay (see check_case): the first case has
+    # one (head 23: the whole last key row lies 1e-8 from the midpoints between bf16 values), none is expected elsewhere
+    assert ties <= 2, ties
     assert caselist.main([PREFILL_EVERY50, "--check", "3", "--check-max-tokens", "600"]) == 0
