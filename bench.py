@@ -132,7 +132,7 @@ KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00), summed over the kernels of
 # one call (profiles/gdn_prefill_kernels_32k.txt, profiles/kda_prefill_kernels_64k.txt)
 GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 1592000000
-KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11874000000
+KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11422000000
 
 
 def cpu_baseline_prefill(w):
@@ -209,7 +209,7 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
                               flop_per_token=GDN_FLOP_PER_TOKEN,
                               note="algorithmic flops (dense) over the whole call; fp16 operands, FP32 accumulation "
                                    "(v_mfma_f32_16x16x32_f16, the rate of the bf16 instruction): "
-                                   "table kernel + key-side preparation + fused sweeps, two pipelined stages, steady state after "
+                                   "key-side preparation + fused sweeps (chunk tables worked out inside them), two pipelined stages, steady state after "
                                    "%d warm-up calls; " % warmup +
                                    "traffic is a constant from rocprofv3 --pmc runs (profiles/gdn_prefill_kernels_32k.txt)"))
 
