@@ -218,12 +218,26 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
         qg[e] = pack2<f16_t>(p.scale * lo16<bf16_t>(qwv[e]) * e0, p.scale * hi16<bf16_t>(qwv[e]) * e1);
         pack2_pair(k0 * __expf(glast[c0 + 2 * e] - g0), k1 * __expf(glast[c0 + 2 * e + 1] - g1), kt[e], ktl[e]);
       }
-      const int64_t off = tile * 8192 + (int64_t)j * 128 + c0;
-      *reinterpret_cast<uint4*>(p.Kg + off) = make_uint4(kg[0], kg[1], kg[2], kg[3]);
-      *reinterpret_cast<uint4*>(p.Qg + off) = make_uint4(qg[0], qg[1], qg[2], qg[3]);
-      const int64_t off2 = tile * 16384 + (int64_t)j * 128 + c0;
-      *reinterpret_cast<uint4*>(p.Kt + off2) = make_uint4(kt[0], kt[1], kt[2], kt[3]);
-      *reinterpret_cast<uint4*>(p.Kt + off2 + 8192) = make_uint4(ktl[0], ktl[1], ktl[2], ktl[3]);
+      // The tiles leave in the layout the sweeps read from LDS (they copy them as linear memory): unpadded rows of
+      // 256 bytes with the swizzle of prefill_common.h, columns permuted inside groups of 32 so that an operand granule
+      // holds channels 32 s + 4 kb .. + 3 and 32 s + 16 + 4 kb .. + 3.  The thread's channels c0 .. c0 + 3 and
+      // c0 + 4 .. c0 + 7 are the same half of two neighbouring granules, and the thread two lanes away holds the other
+      // halves: the two exchange one piece each (a quad permutation) and then each stores one whole granule, so a
+      // wavefront still writes whole rows with one 16-byte store per lane.
+      const int lc = tid & 15;
+      const bool upper = lc & 2;                       // this thread holds the second halves of its granules
+      const int granule = 4 * (lc >> 2) + 2 * (lc & 1) + (upper ? 1 : 0);
+      auto whole_granule = [&](const uint32_t (&x)[4]) {
+        const uint32_t s0 = upper ? x[0] : x[2], s1 = upper ? x[1] : x[3];
+        const uint32_t r0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)s0, 0x4E, 0xF, 0xF, true);      // lane ^ 2
+        const uint32_t r1 = (uint32_t)__builtin_amdgcn_mov_dpp((int)s1, 0x4E, 0xF, 0xF, true);
+        return upper ? make_uint4(r0, r1, x[2], x[3]) : make_uint4(x[0], x[1], r0, r1);
+      };
+      const int64_t at = tile * 8192 + tile_offset(j, granule), at2 = tile * 16384 + tile_offset(j, granule);
+      *reinterpret_cast<uint4*>(p.Kg + at) = whole_granule(kg);
+      *reinterpret_cast<uint4*>(p.Qg + at) = whole_granule(qg);
+      *reinterpret_cast<uint4*>(p.Kt + at2) = whole_granule(kt);
+      *reinterpret_cast<uint4*>(p.Kt + at2 + 8192) = whole_granule(ktl);
     }
   }
 
@@ -342,12 +356,12 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(1024) uint16_t tK[2][TILE128_HALVES];       // swizzled operand tiles, as the preparation stored them
   __shared__ __align__(16) uint16_t tW[2][W_HALVES];                // [parity][hi blocks, lo blocks]
   __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tQ[CHUNK * PITCH128];
+  __shared__ __align__(1024) uint16_t tQ[TILE128_HALVES];
   __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
-  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
+  __shared__ __align__(1024) uint16_t tKt[2][TILE128_HALVES];      // hi, lo: the same layout, read transposed
   __shared__ __align__(16) float tE[128];
 
   if (wave >= 4) {
@@ -363,12 +377,19 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
     const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
     const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), p_step = (int64_t)p.H * (TRI_BLOCKS * 1024);
     const int64_t e_step = (int64_t)p.H * 512;
-    CopyWide plan_k, plan_v;
-    plan_k.plan(256, CHUNK - 1, cw, lane);
+    CopyWide plan_v;
     plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
+    // a 16 KiB operand tile is copied as it lies in memory, its sixteen 1 KiB pieces dealt to the copying wavefronts
+    auto copy_tile = [&](const uint16_t* dst, const char* src) {
+#pragma unroll
+      for (int j0 = 0; j0 < 16 / NCOPY; ++j0) {
+        const int j = NCOPY * j0 + cw;
+        dma16(src, 1024u * j + 16u * lane, lds_address(dst) + 1024u * j);
+      }
+    };
     auto issue_kw = [&](int c) {                     // K e^G and W (hi, lo) into the buffers of c's parity
       const int par = c & 1;
-      plan_k.issue(tK[par], kg_b + c * big_step, cw);
+      copy_tile(tK[par], kg_b + c * big_step);
 #pragma unroll
       for (int j0 = 0; j0 < 2 * TRI_BLOCKS / NCOPY; ++j0) {
         const int j = NCOPY * j0 + cw;
@@ -387,19 +408,18 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
       }
     };
     auto issue_second = [&](int c) {                 // scale Q e^G, P, K e^{G_last-G} (hi, lo), e^{G_last}
-      plan_k.issue(tQ, qg_b + c * big_step, cw);
+      copy_tile(tQ, qg_b + c * big_step);
 #pragma unroll
       for (int j0 = 0; j0 < TRI_BLOCKS / NCOPY; ++j0) {
         const int j = NCOPY * j0 + cw;
         dma16(pp_b + c * p_step, 1024u * j + 16u * lane, lds_address(tP) + 1024u * j);
       }
-      plan_k.issue(tKt[0], kt_b + c * 2 * big_step, cw);
-      plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, cw);
+      copy_tile(tKt[0], kt_b + c * 2 * big_step);
+      copy_tile(tKt[1], kt_b + c * 2 * big_step + 16384);
       if (cw == NCOPY - 1 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
     };
-    static_assert(2 * TRI_BLOCKS % NCOPY == 0 && TRI_BLOCKS % NCOPY == 0, "W and P pieces are dealt evenly");
-    // copies of one issue_kw by this wavefront (the first copying wavefront also takes the pieces left over)
-    constexpr int KW_FIRST = CopyWide::FIRST + 2 * TRI_BLOCKS / NCOPY, KW_OTHER = CopyWide::EACH + 2 * TRI_BLOCKS / NCOPY;
+    static_assert(2 * TRI_BLOCKS % NCOPY == 0 && TRI_BLOCKS % NCOPY == 0 && 16 % NCOPY == 0, "pieces are dealt evenly");
+    constexpr int KW_COPIES = (16 + 2 * TRI_BLOCKS) / NCOPY;                 // copies of one issue_kw by one wavefront
     if (n_chunks > 0) {
       issue_kw(0);
       issue_v(0);
@@ -412,7 +432,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
       if (more) {
         issue_kw(ci + 1);
         // the second-half tiles of ci have landed (what follows may be in flight)
-        if (cw == 0) wait_vmcnt<KW_FIRST>(); else wait_vmcnt<KW_OTHER>();
+        wait_vmcnt<KW_COPIES>();
       } else {
         wait_vmcnt<0>();
       }
@@ -471,7 +491,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_granule(K, 16 * mi + r16, 0, kb);
       __builtin_amdgcn_sched_barrier(0x000F);        // LDS requests stay above this line; ALU and MFMA work may cross it
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -483,7 +503,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
       for (int s = 0; s < 4; ++s) {
         if (s < 3) {
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_granule(K, 16 * mi + r16, s + 1, kb);
         } else {
           // under the last step: V and the first half of W
 #pragma unroll
@@ -554,7 +574,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
         for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       bf16x8_t qa[2][4], sb[2][NB], pa[TRI_BLOCKS];
 #pragma unroll
-      for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], 0, kb);
+      for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_granule(tQ, 16 * ni + r16, 0, kb);
       __builtin_amdgcn_sched_barrier(0x000F);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
@@ -562,7 +582,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
       for (int s = 0; s < 4; ++s) {
         if (s < 3) {
 #pragma unroll
-          for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&tQ[(16 * ni + r16) * PITCH128], s + 1, kb);
+          for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_granule(tQ, 16 * ni + r16, s + 1, kb);
         } else {
 #pragma unroll
           for (int b = 0; b < TRI_BLOCKS; ++b) pa[b] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tP[b * 512 + lane * 8]));
@@ -586,8 +606,8 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
           // under the last step: the first transposed key operands of the state update
 #pragma unroll
           for (int mc = 0; mc < 8; ++mc) {
-            kt[mc] = operand_transposed(tKt[0], 0, mc, kb, r16);
-            ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
+            kt[mc] = operand_granule_transposed(tKt[0], 0, mc, kb, r16);
+            ktl[mc] = operand_granule_transposed(tKt[1], 0, mc, kb, r16);
           }
           __builtin_amdgcn_sched_barrier(0x000F);
         }
@@ -634,7 +654,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
           for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
         if (s == 0) {
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_granule_transposed(tKt[1], 1, mc, kb, r16);
           __builtin_amdgcn_sched_barrier(0x000F);
         }
 #pragma unroll
@@ -647,7 +667,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
           for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
         if (s == 0) {
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(tKt[0], 1, mc, kb, r16);
+          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_granule_transposed(tKt[0], 1, mc, kb, r16);
           __builtin_amdgcn_sched_barrier(0x000F);
         }
       }
@@ -674,12 +694,14 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
 // wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
 // from its real start state (of which they keep a copy for the second sweep).
 //
-// The tiles of a chunk's first half (K e^G, V, W hi / lo) are double buffered by chunk parity, the hi / lo pair of
-// K e^{G_last - G} and e^{G_last} single (127 KiB of LDS), with two barriers per chunk:
-//   barrier A   first-half tiles of chunk c landed, chunk c - 1 finished    copy K e^{G_last-G} (hi, lo), e^{G_last} of c,
-//               KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X             then the first-half tiles of chunk c + 1
-//   barrier B   the pair of c landed
-//               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U              (pairs: hi.lo + lo.hi + hi.hi)
+// Every tile of a chunk (K e^G, V, W hi / lo, the hi / lo pair of K e^{G_last - G}, e^{G_last}) is double buffered by
+// chunk parity (155 KiB of LDS: the operand tiles are unpadded), so there is ONE barrier per chunk: at the barrier
+// that opens chunk c its tiles have landed and the buffers of chunk c - 1 are free; the copying wavefronts fill them
+// with chunk c + 1 at once, a whole chunk ahead, and then compute chunk c with the others:
+//     KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X
+//     S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U              (pairs: hi.lo + lo.hi + hi.hi)
+// (With the pair single buffered and requested half a chunk ahead, behind a second barrier, copies and computation
+// overlapped badly: 0.73 ms for config 4's first sweep where the copies alone take 0.47 and the computation 0.36.)
 __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefillParams p) {
   constexpr int NB = 2;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
@@ -706,11 +728,11 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
+  __shared__ __align__(1024) uint16_t tK[2][TILE128_HALVES];       // swizzled operand tiles, as the preparation stored them
   __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tW[2][W_HALVES];                // [parity][hi blocks, lo blocks]
-  __shared__ __align__(16) uint16_t tKt[2][CHUNK * PITCH128];       // hi, lo
-  __shared__ __align__(16) float tE[128];
+  __shared__ __align__(1024) uint16_t tKt[2][2][TILE128_HALVES];   // [parity][hi, lo]: the same layout, read transposed
+  __shared__ __align__(16) float tE[2][128];
 
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
   f32x4_t St[NB][8];
@@ -746,47 +768,58 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
   const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
   const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), e_step = (int64_t)p.H * 512;
-  CopyWide plan_k, plan_v;
-  if (m_side) {
-    plan_k.plan(256, CHUNK - 1, cw, lane);
-    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
-  }
-  auto issue_first = [&](int c) {                    // K e^G, V, W (hi, lo) into the buffers of c's parity
-    const int par = c & 1;
-    plan_k.issue(tK[par], kg_b + c * big_step, cw);
-    const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
-    const int len = chunk_len(c);
-    if (len == CHUNK) {
-      plan_v.issue(tV[par], vs, cw);
-    } else {                                         // rows past the sequence re-read its last row
-      CopyWide tail_v;
-      tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
-      tail_v.issue(tV[par], vs, cw);
-    }
+  CopyWide plan_v;
+  if (m_side) plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
+  // a 16 KiB operand tile is copied as it lies in memory, four of its sixteen 1 KiB pieces per copying wavefront
+  auto copy_tile = [&](const uint16_t* dst, const char* src) {
 #pragma unroll
-    for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)      // twelve 1 KiB blocks, three per copying wavefront
-      dma16(w_b + c * w_step, 1024u * (4 * j + cw) + 16u * lane, lds_address(tW[par]) + 1024u * (4 * j + cw));
+    for (int j0 = 0; j0 < 4; ++j0) {
+      const int j = 4 * j0 + cw;
+      dma16(src, 1024u * j + 16u * lane, lds_address(dst) + 1024u * j);
+    }
   };
-  auto issue_second = [&](int c) {                   // K e^{G_last-G} (hi, lo), e^{G_last}
-    plan_k.issue(tKt[0], kt_b + c * 2 * big_step, cw);
-    plan_k.issue(tKt[1], kt_b + c * 2 * big_step + 16384, cw);
-    if (cw == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE));
+  // Every tile of chunk c into the buffers of its parity, in four parts, issued together right after the barrier that
+  // frees the buffers.  Measured alternatives (config 4, this sweep 0.63-0.64 ms): half of the parts issued between the
+  // two phases of a chunk 0.68 ms; the pair requested by wavefronts 0-3 at a second barrier 0.66 ms; the parts spread
+  // over four points of the chunk spill registers (1.3 ms).  With wavefronts 4-7 only copying (a timing probe) the sweep
+  // takes the 0.48 ms of its copies alone, and its computation alone 0.36 ms: the two overlap only in part.
+  auto issue_part = [&](int c, int part) {
+    const int par = c & 1;
+    if (part == 0) {                                 // K e^G
+      copy_tile(tK[par], kg_b + c * big_step);
+    } else if (part == 1) {                          // V, W (hi, lo)
+      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
+      const int len = chunk_len(c);
+      if (len == CHUNK) {
+        plan_v.issue(tV[par], vs, cw);
+      } else {                                       // rows past the sequence re-read its last row
+        CopyWide tail_v;
+        tail_v.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
+        tail_v.issue(tV[par], vs, cw);
+      }
+#pragma unroll
+      for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)    // twelve 1 KiB blocks, three per copying wavefront
+        dma16(w_b + c * w_step, 1024u * (4 * j + cw) + 16u * lane, lds_address(tW[par]) + 1024u * (4 * j + cw));
+    } else if (part == 2) {                          // K e^{G_last-G}, hi
+      copy_tile(tKt[par][0], kt_b + c * 2 * big_step);
+    } else {                                         // K e^{G_last-G}, lo; e^{G_last}
+      copy_tile(tKt[par][1], kt_b + c * 2 * big_step + 16384);
+      if (cw == 0 && lane < 32) dma16(eg_b + c * e_step, 16u * lane, lds_address(tE[par]));
+    }
   };
-  // copies one wavefront issues in issue_first (constant: a tail plan has the same piece counts)
-  constexpr int FIRST_REST = 2 * (CopyWide::FIRST) + 2 * TRI_BLOCKS / 4;           // wavefront 4
-  constexpr int EACH_REST = 2 * (CopyWide::EACH) + 2 * TRI_BLOCKS / 4;             // wavefronts 5-7
 
-  if (m_side && n_chunks > 0) issue_first(0);
+  if (m_side && n_chunks > 0) {
+    for (int part = 0; part < 4; ++part) issue_part(0, part);
+  }
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
     const bool more = ci + 1 < n_chunks;
-    // barrier A
+    // the one barrier of a chunk: its tiles have landed, chunk ci - 1 is finished and its buffers are free
     if (m_side) wait_vmcnt<0>();
     __syncthreads();
-    if (m_side) {
-      issue_second(ci);
-      if (more) issue_first(ci + 1);
+    if (m_side && more) {
+      for (int part = 0; part < 4; ++part) issue_part(ci + 1, part);
     }
     f32x4_t U[NB][4];
     if (computing) {
@@ -802,7 +835,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       {
         bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+        for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_granule(K, 16 * mi + r16, 0, kb);
         __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
@@ -814,7 +847,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
         for (int s = 0; s < 4; ++s) {
           if (s < 3) {
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+            for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_granule(K, 16 * mi + r16, s + 1, kb);
           } else {
             // under the last step: V and the first half of W
             if (use_v) {
@@ -873,24 +906,17 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
           for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wa[b], xb[nb], U[nb][tri_block_m(b)]);
       }
     }
-    // barrier B: the pair of this chunk has landed (copies issued after it may still be in flight)
-    if (m_side) {
-      if (!more) wait_vmcnt<0>();
-      else if (cw == 0) wait_vmcnt<FIRST_REST>();
-      else wait_vmcnt<EACH_REST>();
-    }
-    __syncthreads();
     if (computing) {
       // ---- S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U ----
       bf16x8_t kt[8], ktl[8];
 #pragma unroll
       for (int mc = 0; mc < 8; ++mc) {
-        kt[mc] = operand_transposed(tKt[0], 0, mc, kb, r16);
-        ktl[mc] = operand_transposed(tKt[1], 0, mc, kb, r16);
+        kt[mc] = operand_granule_transposed(tKt[par][0], 0, mc, kb, r16);
+        ktl[mc] = operand_granule_transposed(tKt[par][1], 0, mc, kb, r16);
       }
       float4 eg[8];
 #pragma unroll
-      for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[16 * mc + 4 * kb]);
+      for (int mc = 0; mc < 8; ++mc) eg[mc] = *reinterpret_cast<const float4*>(&tE[par][16 * mc + 4 * kb]);
       __builtin_amdgcn_sched_barrier(0x000F);
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -910,7 +936,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
           for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(ktl[mc], ub[nb].hi, St[nb][mc]);
         if (s == 0) {
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_transposed(tKt[1], 1, mc, kb, r16);
+          for (int mc = 0; mc < 8; ++mc) ktl[mc] = operand_granule_transposed(tKt[par][1], 1, mc, kb, r16);
           __builtin_amdgcn_sched_barrier(0x000F);
         }
 #pragma unroll
@@ -923,7 +949,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
           for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[mc], ub[nb].hi, St[nb][mc]);
         if (s == 0) {
 #pragma unroll
-          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_transposed(tKt[0], 1, mc, kb, r16);
+          for (int mc = 0; mc < 8; ++mc) kt[mc] = operand_granule_transposed(tKt[par][0], 1, mc, kb, r16);
           __builtin_amdgcn_sched_barrier(0x000F);
         }
       }
