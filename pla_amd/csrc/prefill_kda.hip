@@ -689,15 +689,15 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
 // First sweep over segments, both roles in one workgroup.  A later segment is swept twice without output - from a
 // zero state (its B summary) and from the identity with v = 0 (its transition matrix M) - and both sweeps multiply
 // the same operand tiles.  One workgroup of eight wavefronts per (segment, head) therefore runs them side by side:
-// wavefronts 0-3 carry the B columns (32 each), wavefronts 4-7 the M columns and, having no values to subtract,
-// also issue every global -> LDS copy, so each tile crosses memory and LDS once for the two sweeps and two
-// wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
+// wavefronts 0-3 carry the B columns (32 each), wavefronts 4-7 the M columns; all eight issue the global -> LDS
+// copies, so each tile crosses memory and LDS once for the two sweeps and two wavefronts share a SIMD.  A first
+// segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
 // from its real start state (of which they keep a copy for the second sweep).
 //
 // Every tile of a chunk (K e^G, V, W hi / lo, the hi / lo pair of K e^{G_last - G}, e^{G_last}) is double buffered by
 // chunk parity (155 KiB of LDS: the operand tiles are unpadded), so there is ONE barrier per chunk: at the barrier
-// that opens chunk c its tiles have landed and the buffers of chunk c - 1 are free; the copying wavefronts fill them
-// with chunk c + 1 at once, a whole chunk ahead, and then compute chunk c with the others:
+// that opens chunk c its tiles have landed and the buffers of chunk c - 1 are free; the wavefronts fill them
+// with chunk c + 1 at once, a whole chunk ahead, and then compute chunk c:
 //     KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X
 //     S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U              (pairs: hi.lo + lo.hi + hi.hi)
 // (With the pair single buffered and requested half a chunk ahead, behind a second barrier, copies and computation
@@ -760,7 +760,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
   }
   const bool use_v = computing && !role.zero_v;                // the identity sweep runs with v = 0
 
-  // ---- copies (wavefronts 4-7) ----
+  // ---- copies ----
   const int64_t tile0 = (int64_t)c_begin * p.H + h;
   const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
   const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
@@ -778,10 +778,11 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       dma16(src, 1024u * j + 16u * lane, lds_address(dst) + 1024u * j);
     }
   };
-  // Every tile of chunk c into the buffers of its parity, in four parts, issued together right after the barrier that
-  // frees the buffers.  Measured alternatives (config 4, this sweep 0.63-0.64 ms): half of the parts issued between the
-  // two phases of a chunk 0.68 ms; the pair requested by wavefronts 0-3 at a second barrier 0.66 ms; the parts spread
-  // over four points of the chunk spill registers (1.3 ms).  With wavefronts 4-7 only copying (a timing probe) the sweep
+  // Every tile of chunk c into the buffers of its parity, in four parts, all issued right after the barrier that frees
+  // the buffers: wavefronts 4-7 take K e^G, V and W, wavefronts 0-3 the pair and e^{G_last} (0.60 ms for config 4's
+  // first sweep against 0.63 with wavefronts 4-7 issuing everything).  Measured alternatives: half of the parts issued
+  // between the two phases of a chunk 0.68 ms; the pair requested at a second barrier 0.66 ms; the parts spread over
+  // four points of the chunk spill registers (1.3 ms).  With wavefronts 4-7 only copying (a timing probe) the sweep
   // takes the 0.48 ms of its copies alone, and its computation alone 0.36 ms: the two overlap only in part.
   auto issue_part = [&](int c, int part) {
     const int par = c & 1;
@@ -808,18 +809,18 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
     }
   };
 
-  if (m_side && n_chunks > 0) {
-    for (int part = 0; part < 4; ++part) issue_part(0, part);
+  if (n_chunks > 0) {
+    if (m_side) { issue_part(0, 0); issue_part(0, 1); } else { issue_part(0, 2); issue_part(0, 3); }
   }
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
     const bool more = ci + 1 < n_chunks;
     // the one barrier of a chunk: its tiles have landed, chunk ci - 1 is finished and its buffers are free
-    if (m_side) wait_vmcnt<0>();
+    wait_vmcnt<0>();
     __syncthreads();
-    if (m_side && more) {
-      for (int part = 0; part < 4; ++part) issue_part(ci + 1, part);
+    if (more) {
+      if (m_side) { issue_part(ci + 1, 0); issue_part(ci + 1, 1); } else { issue_part(ci + 1, 2); issue_part(ci + 1, 3); }
     }
     f32x4_t U[NB][4];
     if (computing) {
