@@ -323,9 +323,11 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
 // inverse of I + L by 16 x 16 blocks, and W = (I + L)^-1 diag(beta) as an fp16 hi + lo pair in the six-block
 // operand layout (12 KiB per (chunk, value head) instead of 16 KiB row-major + 8 KiB of P + the normalised rows).
 // The blocks of L below the diagonal never leave the registers: the accumulators of K K^T are the operands of the
-// transposed block recursion as they stand, and its results are the lane's pieces of the W blocks.  Registers, not
-// LDS, then bound the occupancy (two wavefronts per SIMD; forcing three or four spills and is slower: config 3
-// 0.446 / 0.455 / 0.489 ms).
+// transposed block recursion as they stand, and its results are the lane's pieces of the W blocks.  The wavefronts
+// of a workgroup (the value heads of one q/k head) share the loading and normalising of the keys through LDS: a
+// quarter fewer vector instructions per tile and half the registers for raw rows, which brings three wavefronts
+// to a SIMD without spills (config 3 0.450 -> 0.440 ms, 8 x 2048 tokens 0.233 -> 0.224 ms; four per SIMD by a launch
+// bound measure the same: the kernel is bound by its vector instructions now, not by latency).
 template <typename act_t, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefillParams p) {
   const int groups = p.HV / WAVES;
@@ -356,10 +358,14 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   // apart: the four groups of 16 lanes that walk one block each in the forward substitution stay on different banks);
   // the six blocks below the diagonal stay in the accumulators of K K^T.  5.9 KB instead of a 64 x 68 FP32 tile.
   constexpr int DIAG_PITCH = 20, DIAG_BLOCK = 336;
-  __shared__ __align__(16) float Ld_all[WAVES][4 * DIAG_BLOCK];
+  // One buffer serves two purposes in turn: first the normalised keys the wavefronts hand each other ([row block][step]
+  // [lane], 16 KiB), then, behind a barrier, every wavefront's diagonal blocks.
+  constexpr int SHARE_BYTES = WAVES * 4 * DIAG_BLOCK * 4 > 16 * 64 * 16 ? WAVES * 4 * DIAG_BLOCK * 4 : 16 * 64 * 16;
+  __shared__ __align__(16) unsigned char share[SHARE_BYTES];
   __shared__ __align__(16) float Gs_all[WAVES][CHUNK];
   __shared__ __align__(16) float Bs_all[WAVES][CHUNK];
-  float* const Ld = Ld_all[wave];
+  uint4* const Kshare = reinterpret_cast<uint4*>(share);
+  float* const Ld = reinterpret_cast<float*>(share) + wave * 4 * DIAG_BLOCK;
   float* const Gs = Gs_all[wave];
   float* const Bs = Bs_all[wave];
 
@@ -378,15 +384,19 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
       a_log = p.A_log[hv];
     }
   }
-  // raw K operands, all 16 loads of a lane requested before the first use (rows are 16-byte aligned on this path)
-  uint4 kraw[4][4];
+  // Raw K operands.  The wavefronts of a workgroup work on the value heads of ONE q/k head and need the same
+  // normalised keys: each loads and normalises 4 / WAVES of the four row blocks and hands them to the others through
+  // LDS.  All loads of a lane are requested before the first use (rows are 16-byte aligned on this path).
+  constexpr int PER = 4 / WAVES;
+  static_assert(WAVES == 1 || WAVES == 2 || WAVES == 4, "row blocks are dealt evenly");
+  uint4 kraw[PER][4];
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const int row = 16 * mb + r16;
+  for (int i = 0; i < PER; ++i) {
+    const int row = 16 * (wave * PER + i) + r16;
     const int64_t t = t0 + (row < len ? row : 0);
     const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + 8 * kb;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) kraw[mb][s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
+    for (int s = 0; s < 4; ++s) kraw[i][s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
   }
 
   // ---- gate: lane = token ----
@@ -430,15 +440,17 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   bf16x8_t Kop[4][4];
   {
     const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    const bool first_group = (hv - wave) % (p.HV / p.H) == 0;           // this workgroup holds the head's first value heads
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
+    for (int i = 0; i < PER; ++i) {
+      const int mb = wave * PER + i;
       const bool ok = 16 * mb + r16 < len;
       float inv = 1.f;
       if (p.normalize_qk) {
         float ss = 0.f;
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          const uint32_t w[4] = {kraw[mb][s].x, kraw[mb][s].y, kraw[mb][s].z, kraw[mb][s].w};
+          const uint32_t w[4] = {kraw[i][s].x, kraw[i][s].y, kraw[i][s].z, kraw[i][s].w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const float a0 = lo16<act_t>(w[e]), a1 = hi16<act_t>(w[e]);
@@ -449,22 +461,31 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
         const LanePair r2 = swap_halves(r1.lo + r1.hi);
         inv = rsqrtf(r2.lo + r2.hi + 1e-6f);
         // the sweep scales the raw rows by the same factor, so both kernels hold the same rounded keys
-        if (ok && kb == 0 && hv % (p.HV / p.H) == 0) p.kinv[(int64_t)(t0 + 16 * mb + r16) * p.H + h] = inv;
+        if (ok && kb == 0 && first_group) p.kinv[(int64_t)(t0 + 16 * mb + r16) * p.H + h] = inv;
       }
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const uint32_t in[4] = {kraw[mb][s].x, kraw[mb][s].y, kraw[mb][s].z, kraw[mb][s].w};
+        const uint32_t in[4] = {kraw[i][s].x, kraw[i][s].y, kraw[i][s].z, kraw[i][s].w};
         uint32_t w[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const uint32_t a = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
           w[e] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
         }
-        Kop[mb][s] = ok ? __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3])) : __builtin_bit_cast(bf16x8_t, zero4);
+        const uint4 row_op = ok ? make_uint4(w[0], w[1], w[2], w[3]) : zero4;
+        if constexpr (WAVES == 1) Kop[i][s] = __builtin_bit_cast(bf16x8_t, row_op);
+        else Kshare[(mb * 4 + s) * 64 + lane] = row_op;
       }
     }
   }
   __syncthreads();
+  if constexpr (WAVES > 1) {
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int s = 0; s < 4; ++s) Kop[mb][s] = __builtin_bit_cast(bf16x8_t, Kshare[(mb * 4 + s) * 64 + lane]);
+    __syncthreads();                    // every wavefront holds the keys: the buffer is free for the diagonal blocks
+  }
 
   // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j}) by 16 x 16 blocks.  The accumulators of block (mi, ni) hold rows
   // i = 4 kb + r of column j = r16: for a block below the diagonal that is the A operand of L_ab^T as it stands
