@@ -555,20 +555,25 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
   // The blocks of N = (I + L)^-1 below the diagonal, transposed: N_ab^T = -D_b^T sum_{b < c <= a} L_cb^T N_ac^T with
   // N_aa = D_a, in order of a - b = 1, 2, 3.  Every product has the earlier result on its right, where an accumulator
   // tile is an operand as it stands, and leaves N_ab^T in accumulator layout: rows j = 4 kb + r of column i = r16,
-  // which is the lane's piece N_ab[r16][4 kb + r] of a W block.  FP32 values cross the MFMA as bf16 hi / lo pairs.
+  // which is the lane's piece N_ab[r16][4 kb + r] of a W block.  The products run on the FP32 MFMA
+  // (v_mfma_f32_16x16x4_f32, exact products): lane (r16, kb) supplies one element of row r16 per instruction, and with
+  // the contraction index taken as 4 kb + r for instruction r both operands are the lane's own quads, element r of
+  // each.  (As bf16 hi / lo pairs on the 16 x 16 x 32 instruction the same products cost a third of the matrix-pipe
+  // time but about 900 vector instructions per tile for the splits, in a kernel that its vector instructions bound.)
   auto negate = [](f32x4_t t) { return f32x4_t{-t.x, -t.y, -t.z, -t.w}; };
-  auto solve = [&](int b, f32x4_t y) { return negate(mfma_hilo(split8(DTq[b], zero), split8(y, zero), zero)); };
+  auto product = [](const f32x4_t& a, const f32x4_t& b, f32x4_t acc) {       // acc += A B over one 16-wide block
+#pragma unroll
+    for (int r = 0; r < 4; ++r) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[r], b[r], acc, 0, 0, 0);
+    return acc;
+  };
+  auto solve = [&](int b, const f32x4_t& y) { return negate(product(DTq[b], y, zero)); };
   f32x4_t Nq[4][4];
-  Nq[1][0] = solve(0, mfma_hilo(split8(Lr[1][0], zero), split8(Dq[1], zero), zero));
-  Nq[2][1] = solve(1, mfma_hilo(split8(Lr[2][1], zero), split8(Dq[2], zero), zero));
-  Nq[3][2] = solve(2, mfma_hilo(split8(Lr[3][2], zero), split8(Dq[3], zero), zero));
-  Nq[2][0] = solve(0, mfma_hilo(split8(Lr[1][0], Lr[2][0]), split8(Nq[2][1], Dq[2]), zero));
-  Nq[3][1] = solve(1, mfma_hilo(split8(Lr[2][1], Lr[3][1]), split8(Nq[3][2], Dq[3]), zero));
-  {
-    f32x4_t y = mfma_hilo(split8(Lr[1][0], Lr[2][0]), split8(Nq[3][1], Nq[3][2]), zero);
-    y = mfma_hilo(split8(Lr[3][0], zero), split8(Dq[3], zero), y);
-    Nq[3][0] = solve(0, y);
-  }
+  Nq[1][0] = solve(0, product(Lr[1][0], Dq[1], zero));
+  Nq[2][1] = solve(1, product(Lr[2][1], Dq[2], zero));
+  Nq[3][2] = solve(2, product(Lr[3][2], Dq[3], zero));
+  Nq[2][0] = solve(0, product(Lr[2][0], Dq[2], product(Lr[1][0], Nq[2][1], zero)));
+  Nq[3][1] = solve(1, product(Lr[3][1], Dq[3], product(Lr[2][1], Nq[3][2], zero)));
+  Nq[3][0] = solve(0, product(Lr[3][0], Dq[3], product(Lr[2][0], Nq[3][2], product(Lr[1][0], Nq[3][1], zero))));
   // W = N diag(beta) as an fp16 hi + lo pair in the six-block operand layout: block (row block m, column half s) holds
   // the lane's pieces of blocks (m, 2 s) and (m, 2 s + 1)
   uint16_t* const Wt = p.W + ((int64_t)cb * p.HV + hv) * (2 * TRI_BLOCKS * 512);
