@@ -391,7 +391,26 @@ struct StageTable {
 constexpr int MAX_STAGES = 2;
 // Chunks [stage_cut(nc, s, S), stage_cut(nc, s + 1, S)) of an item of `nc` chunks belong to stage s of the S stages in
 // effect (stages beyond S are empty).
-__device__ __forceinline__ int stage_cut(int nc, int s, int S) { return (int)((int64_t)nc * min(s, S) / S); }
+// The cut is described by a plan word: the number of stages in effect in its low byte and, above it, the sixteenths of
+// an item's chunks that the first of TWO stages takes.  Whoever sees the lengths on the device makes the plan
+// (stage_plan): one stage when the chains are of nearly equal length (their chunks fill 80 % or more of `items x
+// longest chain`: no CU falls idle before a sweep ends, so a later preparation would not run underneath it); else
+// the stages the host allowed, the first of two stages taking 3/8 of every chain when the chains fill less than
+// 5/8 of that rectangle and half otherwise: the preparation of the first stage is exposed, that of the second hides
+// under the first sweep only as far as chains that have ended leave CUs to it (measured, ms per call, first stage of
+// 8 / 7 / 6 / 5 / 4 sixteenths: 0.440 / 0.434 / 0.428 / 0.434 / 0.443 at a fill of 0.57; at fills of 0.66 half is the
+// better cut by 0.4-1.1 %, at 0.31 and 0.61 three eighths by 1.4-1.9 %).
+__device__ __forceinline__ int stage_plan(int64_t total, int n_items, int longest, int S) {
+  const int64_t rectangle = (int64_t)n_items * longest;
+  if (S <= 0 || 5 * total >= 4 * rectangle) return 1 | (8 << 8);
+  return S | ((S == 2 && 8 * total < 5 * rectangle ? 6 : 8) << 8);
+}
+__device__ __forceinline__ int plan_stages(int plan) { return plan & 0xff; }
+__device__ __forceinline__ int stage_cut(int nc, int s, int plan) {
+  const int S = plan & 0xff;
+  if (S == 2 && s == 1) return (int)((int64_t)nc * (plan >> 8) / 16);
+  return (int)((int64_t)nc * min(s, S) / S);
+}
 
 // Single workgroup of 256 threads with (stages + 1) * n_items_max + 1 words of LDS at `pair_begin`.  The items are sequences (`counts` null: item i holds chunks
 // starts[i] .. starts[i + 1]) or segments (chunks starts[i] .. starts[i] + counts[i]); `n_items` is read
@@ -416,7 +435,7 @@ __device__ __forceinline__ void stage_map(const int32_t* starts, const int32_t* 
     int64_t total = 0;
     int longest = 0;
     for (int i = 0; i < n_items; ++i) { total += count_of(i); longest = max(longest, count_of(i)); }
-    const int E = 5 * total < 4 * (int64_t)n_items * longest ? S : 1;      // idle share of the chains' rectangle above 20 %
+    const int E = stage_plan(total, n_items, longest, S);                  // the plan word: stages in effect and the cut
     stages_in_effect = E;
     t.stage_begin[MAX_STAGES + 1] = E;
     int k = 0;
@@ -538,13 +557,13 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     }
   }
   if (carry != nullptr && stg.stages > 0) {
-    const int E = inline_chunks.x >= 0 ? inline_chunks.z : stg.stage_begin[MAX_STAGES + 1];   // stages in effect (the table kernel's choice)
-    if (stage >= E) return r;                                      // an empty stage: the one before it delivered the state
+    const int E = inline_chunks.x >= 0 ? inline_chunks.z : stg.stage_begin[MAX_STAGES + 1];   // the plan word (stage_plan)
+    if (stage >= plan_stages(E)) return r;                                      // an empty stage: the one before it delivered the state
     const int nc = r.c_end - r.c_begin, c0 = r.c_begin;
     r.c_begin = c0 + stage_cut(nc, stage, E);
     r.c_end = c0 + stage_cut(nc, stage + 1, E);
     if (stage > 0) { r.init = carry; r.keep_init = nullptr; }      // the start state is kept by stage 0 only
-    if (stage < E - 1) r.fin = carry;
+    if (stage < plan_stages(E) - 1) r.fin = carry;
   }
   r.active = true;
   return r;
@@ -568,7 +587,7 @@ __device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
 }
 struct InlineSequences {
   int start, len, nc, off;      // this lane's sequence: first token, tokens, chunks, first chunk (global index)
-  int total, E;                 // chunks of the call; stages in effect
+  int total, E;                 // chunks of the call; the plan word (stage_plan)
 };
 __device__ __forceinline__ InlineSequences inline_sequences(const int32_t* cu_seqlens, int N, int stages, int lane) {
   InlineSequences q;
@@ -583,7 +602,7 @@ __device__ __forceinline__ InlineSequences inline_sequences(const int32_t* cu_se
 #pragma unroll
   for (int d = 32; d > 0; d >>= 1) longest = max(longest, __shfl_xor(longest, d, 64));
   longest = __builtin_amdgcn_readfirstlane(longest);
-  q.E = (stages > 0 && 5 * (int64_t)q.total < 4 * (int64_t)N * longest) ? stages : 1;
+  q.E = stage_plan(q.total, N, longest, stages);
   return q;
 }
 // Chunk `index` of stage `stage` (all chunks in order when the call is not staged): its global chunk id, first token
@@ -591,7 +610,7 @@ __device__ __forceinline__ InlineSequences inline_sequences(const int32_t* cu_se
 struct InlineTile { int cb, t0, len; };
 __device__ __forceinline__ InlineTile inline_tile(const InlineSequences& q, int stage, int index, int NC_max, int lane) {
   InlineTile t{-1, 0, 0};
-  if (stage >= q.E) return t;
+  if (stage >= plan_stages(q.E)) return t;
   const int lo = stage_cut(q.nc, stage, q.E), hi = stage_cut(q.nc, stage + 1, q.E);
   const int cnt = hi - lo;
   const int before = wave_inclusive_scan(cnt, lane) - cnt;
