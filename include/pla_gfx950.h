@@ -338,6 +338,27 @@ int pla_gdn_prefill_launch(
     int H, int HV, int K, int V, int act_dtype, void* stream);
 
 /*
+ * pla_gdn_prefill_launch with the sequence offsets on the host as well: raw_cu_seqlens points to N + 1 int32
+ * values in HOST memory that equal cu_seqlens (NULL: exactly pla_gdn_prefill_launch).  Replaces the
+ * `raw_cu_seqlens` argument of the reference's public ops (pla/prefill/flashqla/ops.py: "trusted host copy of
+ * cu_seqlens", which lets its planner decide without reading the device tensor back).  Here the host uses it for one
+ * decision only, by the rule the device applies anyway: a call whose sequences are of nearly equal length runs in
+ * one stage, and with the offsets at hand nothing is enqueued for a second one (two launches and four event
+ * operations less per call).  Results are bit-identical to pla_gdn_prefill_launch.  The values are read during the
+ * call and not kept.
+ */
+int pla_gdn_prefill_launch_raw(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens);
+
+/*
  * pla_gdn_prefill_launch for callers that cannot allocate (code under hipGraph capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments without the workspace pair, same results bit
  * for bit.  No counterpart in the reference.  The workspace is an array inside the library, one per GPU

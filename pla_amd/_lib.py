@@ -74,6 +74,14 @@ SIGNATURES = {
         _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
         _c_p, _c_p, _c_i64, _c_p, _c_p,
         _c_int, _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_gdn_prefill_launch_raw": [
+        _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64,
+        _c_p, _c_p, _c_i64, _c_i64,
+        _c_p, _c_p, _c_p, _c_p,
+        _c_p, _c_int, _c_int, _c_f, _c_int,
+        _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
+        _c_p, _c_p, _c_i64, _c_p, _c_p,
+        _c_int, _c_int, _c_int, _c_int, _c_int, _c_p, _c_p],
     "pla_gdn_prefill_launch_static": [
         _c_p, _c_p, _c_p, _c_i64, _c_i64, _c_i64,
         _c_p, _c_p, _c_i64, _c_i64,

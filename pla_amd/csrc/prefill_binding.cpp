@@ -47,17 +47,19 @@ bool plain_offsets(const OptTensor& cu, const Tensor& ref) {
          cu->is_contiguous();
 }
 // host offsets, when given, must describe the same packed batch (the facade's rule); None is fine
-bool plain_raw_offsets(const py::object& raw, int64_t batch, int64_t tokens) {
+bool plain_raw_offsets(const py::object& raw, int64_t batch, int64_t tokens, std::vector<int32_t>* values = nullptr) {
   if (raw.is_none()) return true;
   if (!py::isinstance<py::tuple>(raw) && !py::isinstance<py::list>(raw)) return false;
   const py::sequence seq = py::reinterpret_borrow<py::sequence>(raw);
   if ((int64_t)py::len(seq) != batch + 1) return false;
+  if (values) values->reserve(batch + 1);
   int64_t before = 0;
   for (int64_t i = 0; i <= batch; ++i) {
     if (!py::isinstance<py::int_>(seq[i])) return false;
     const int64_t x = seq[i].cast<int64_t>();
     if ((i == 0 && x != 0) || x < before || x > tokens) return false;
     before = x;
+    if (values) values->push_back((int32_t)x);
   }
   return true;
 }
@@ -86,7 +88,7 @@ struct GdnCall {
 py::object gdn_launch(const GdnCall& c, const OptTensor& g, const OptTensor& beta, const OptTensor& raw_gate_a,
                       const OptTensor& raw_beta_b, const OptTensor& A_log, const OptTensor& dt_bias, const Tensor& cu,
                       double scale, bool normalize_qk, const OptTensor& initial_state, const OptTensor& indices,
-                      bool output_final_state) {
+                      bool output_final_state, const std::vector<int32_t>& host_offsets) {
   const int64_t T = c.tokens, H = c.H, batch = cu.numel() - 1;
   const bool raw = raw_gate_a.has_value();
   if (raw) {
@@ -133,14 +135,15 @@ py::object gdn_launch(const GdnCall& c, const OptTensor& g, const OptTensor& bet
     ht = final_state.data_ptr<float>();
     ht_stride = final_state.stride(0);
   }
-  launched(pla_gdn_prefill_launch(
+  launched(pla_gdn_prefill_launch_raw(
       c.q, c.k, c.v, c.stride_q, c.stride_k, c.stride_v,
       raw ? raw_gate_a->data_ptr() : nullptr, raw ? raw_beta_b->data_ptr() : nullptr, raw ? raw_gate_a->stride(0) : 0,
       raw ? raw_beta_b->stride(0) : 0, raw ? A_log->data_ptr<float>() : nullptr, raw ? dt_bias->data_ptr<float>() : nullptr,
       raw ? nullptr : g->data_ptr<float>(), raw ? nullptr : beta->data_ptr<float>(),
       cu.data_ptr<int32_t>(), (int)batch, (int)T, (float)scale, normalize_qk ? 1 : 0,
       h0, idx, h0_stride, ht, idx, ht_stride, o.data_ptr(), ws.data_ptr(), ws_bytes, g_cum.data_ptr<float>(),
-      beta_act.data_ptr<float>(), (int)c.Hg, (int)H, 128, 128, c.act == at::kHalf ? PLA_F16 : PLA_BF16, stream_of(c.ref)));
+      beta_act.data_ptr<float>(), (int)c.Hg, (int)H, 128, 128, c.act == at::kHalf ? PLA_F16 : PLA_BF16, stream_of(c.ref),
+      host_offsets.empty() ? nullptr : host_offsets.data()));
   py::object final_obj = py::none();
   if (output_final_state) {
     if (indexed) final_obj = py::cast(initial_state->index_select(0, indices->to(at::kLong)));
@@ -172,14 +175,15 @@ py::object try_chunk_gated_delta_rule_fwd(
   }
   if (!plain_offsets(cu_seqlens, q)) return py::none();
   const int64_t batch = cu_seqlens->numel() - 1;
-  if (!plain_raw_offsets(raw_cu_seqlens, batch, T)) return py::none();
+  std::vector<int32_t> host_offsets;
+  if (!plain_raw_offsets(raw_cu_seqlens, batch, T, &host_offsets)) return py::none();
   if (!final_state_dtype.is_none()) {             // only the FP32 form is taken here
     const auto torch_mod = py::module_::import("torch");
     if (!final_state_dtype.is(torch_mod.attr("float32"))) return py::none();
   }
   GdnCall c{q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(1), k.stride(1), v.stride(1), T, Hg, H, act, q};
   return gdn_launch(c, g, beta, raw_gate_a, raw_beta_b, A_log, dt_bias, *cu_seqlens, scale.value_or(1.0 / std::sqrt(128.0)),
-                    normalize_qk, initial_state, initial_state_indices, output_final_state);
+                    normalize_qk, initial_state, initial_state_indices, output_final_state, host_offsets);
 }
 
 py::object try_gdn_prefill_packed_qkv_fwd(
@@ -201,7 +205,8 @@ py::object try_gdn_prefill_packed_qkv_fwd(
     if (!std::isfinite(overlap_warmup_threshold.cast<double>())) return py::none();
   }
   if (!plain_offsets(cu_seqlens, packed_qkv)) return py::none();
-  if (!plain_raw_offsets(raw_cu_seqlens, cu_seqlens->numel() - 1, T)) return py::none();
+  std::vector<int32_t> host_offsets;
+  if (!plain_raw_offsets(raw_cu_seqlens, cu_seqlens->numel() - 1, T, &host_offsets)) return py::none();
   if (!final_state_dtype.is_none()) {
     const auto torch_mod = py::module_::import("torch");
     if (!final_state_dtype.is(torch_mod.attr("float32"))) return py::none();
@@ -209,7 +214,8 @@ py::object try_gdn_prefill_packed_qkv_fwd(
   const char* base = static_cast<const char*>(packed_qkv.data_ptr());
   GdnCall c{base, base + Hg * 128 * 2, base + 2 * Hg * 128 * 2, pitch, pitch, pitch, T, Hg, H, act, packed_qkv};
   return gdn_launch(c, std::nullopt, std::nullopt, raw_gate_a, raw_beta_b, A_log, dt_bias, *cu_seqlens,
-                    scale.value_or(1.0 / std::sqrt(128.0)), true, initial_state, initial_state_indices, output_final_state);
+                    scale.value_or(1.0 / std::sqrt(128.0)), true, initial_state, initial_state_indices, output_final_state,
+                    host_offsets);
 }
 #endif  // PLA_BIND_FLASHQLA
 

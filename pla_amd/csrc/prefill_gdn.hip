@@ -1888,7 +1888,7 @@ static int gdn_prefill_run(
     float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
     void* o, void* workspace, int64_t workspace_bytes, bool static_scratch,
     float* gcum_out, float* beta_out,
-    int H, int HV, int K, int V, int act_dtype, void* stream) {
+    int H, int HV, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens = nullptr) {
   PLA_REQUIRE(K == 128 && V == 128, "GDN prefill requires head_dim K == V == 128, got K=%d, V=%d", K, V);
   PLA_REQUIRE(T > 0 && N > 0, "GDN prefill needs at least one token and one sequence");
   PLA_REQUIRE(H > 0 && HV >= H && HV % H == 0, "HV must be a positive multiple of H, got H=%d, HV=%d", H, HV);
@@ -1962,7 +1962,21 @@ static int gdn_prefill_run(
   }
   // the staged pipeline needs a side stream: without one (pool exhausted) the call runs unstaged, decided before
   // anything is launched
-  const SideStreamLease lease(s, L.stages > 0);
+  // With the offsets on the host as well the host applies the device's own rule (stage_plan) ahead of it: chains of
+  // nearly equal length run in one stage, and then nothing is enqueued for a second one (no side stream, no events,
+  // no launches that find nothing to do).
+  bool staged = L.stages > 0;
+  if (staged && raw_cu_seqlens != nullptr) {
+    int64_t total = 0;
+    int longest = 0;
+    for (int n = 0; n < N; ++n) {
+      const int nc = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+      total += nc;
+      longest = std::max(longest, nc);
+    }
+    staged = 5 * total < 4 * (int64_t)N * longest;
+  }
+  const SideStreamLease lease(s, staged);
   const int stages = lease.get() != nullptr ? L.stages : 0;
   if (stages > 0) {
     p.stg.order = reinterpret_cast<int32_t*>(ws + L.order);
@@ -2041,6 +2055,22 @@ extern "C" int pla_gdn_prefill_launch(
                          cu_seqlens, N, T, scale, normalize_qk, h0, h0_indices, h0_slot_stride, ht, ht_indices,
                          ht_slot_stride, o, workspace, workspace_bytes, false, gcum_out, beta_out, H, HV, K, V, act_dtype,
                          stream);
+}
+
+extern "C" int pla_gdn_prefill_launch_raw(
+    const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
+    const void* a, const void* b, int64_t stride_a, int64_t stride_b,
+    const float* A_log, const float* dt_bias, const float* g_in, const float* beta_in,
+    const int32_t* cu_seqlens, int N, int T, float scale, int normalize_qk,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    float* gcum_out, float* beta_out,
+    int H, int HV, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens) {
+  return gdn_prefill_run(q, k, v, stride_q, stride_k, stride_v, a, b, stride_a, stride_b, A_log, dt_bias, g_in, beta_in,
+                         cu_seqlens, N, T, scale, normalize_qk, h0, h0_indices, h0_slot_stride, ht, ht_indices,
+                         ht_slot_stride, o, workspace, workspace_bytes, false, gcum_out, beta_out, H, HV, K, V, act_dtype,
+                         stream, raw_cu_seqlens);
 }
 
 extern "C" int pla_gdn_prefill_launch_static(

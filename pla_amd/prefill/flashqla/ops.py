@@ -16,6 +16,7 @@ validated and otherwise unused).  States are FP32 and k-last ``[slots, H, DV, DK
 k-first ``[N, H, DK, DV]`` state form is not provided.
 """
 
+import ctypes
 import math
 from typing import Optional, Sequence, Tuple, Union
 
@@ -145,6 +146,7 @@ def chunk_gated_delta_rule_fwd(
     batch = cu32.numel() - 1
     if batch <= 0:
         raise ValueError("cu_seqlens must describe at least one sequence")
+    raw = None
     if raw_cu_seqlens is not None:
         if isinstance(raw_cu_seqlens, torch.Tensor):
             if (raw_cu_seqlens.device.type != "cpu" or raw_cu_seqlens.ndim != 1
@@ -251,15 +253,18 @@ def chunk_gated_delta_rule_fwd(
         sa = sb = 0
         g_ptr, bt_ptr = g32.data_ptr(), b32.data_ptr()
 
+    # host offsets, when the caller has them, go along (one decision is taken from them: see pla_gdn_prefill_launch_raw)
+    raw_host = (ctypes.c_int32 * (batch + 1))(*raw) if raw is not None else None
     _lib.call(
-        "pla_gdn_prefill_launch",
+        "pla_gdn_prefill_launch_raw",
         q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(1), k.stride(1), v.stride(1),
         a_ptr, b_ptr, sa, sb, al_ptr, dt_ptr, g_ptr, bt_ptr,
         cu32.data_ptr(), batch, num_tokens, float(scale), int(bool(normalize_qk)),
         _lib.ptr(h0), _lib.ptr(h0_idx), h0.stride(0) if h0 is not None else 0,
         _lib.ptr(ht), _lib.ptr(ht_idx), ht.stride(0) if ht is not None else 0,
         o.data_ptr(), ws.data_ptr(), ws_bytes, g_cum.data_ptr(), beta_act.data_ptr(),
-        Hg, H, DK, DV, _lib.dtype_code(q.dtype), _lib.current_stream(dev))
+        Hg, H, DK, DV, _lib.dtype_code(q.dtype), _lib.current_stream(dev),
+        ctypes.cast(raw_host, ctypes.c_void_p) if raw_host is not None else None)
 
     if output_final_state:
         final = initial_state[initial_state_indices.long()] if indexed else final

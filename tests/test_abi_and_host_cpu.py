@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     declared = _declared()
     assert {"pla_version", "pla_last_error", "pla_k_last_packed_launch", "pla_k_last_launch",
             "pla_kda_fold_launch", "pla_kda_fold_native_launch", "pla_kda_conv_native_launch", "pla_kda_commit_plan_launch", "pla_kda_decode_mega_launch", "pla_kda_verify_dspark_launch", "pla_kda_replay_verify_native_launch", "pla_conv_window_scatter_launch",
-            "pla_gdn_prefill_launch", "pla_gdn_prefill_workspace_bytes",
+            "pla_gdn_prefill_launch", "pla_gdn_prefill_launch_raw", "pla_gdn_prefill_workspace_bytes",
             "pla_kda_prefill_launch", "pla_kda_prefill_workspace_bytes"} <= set(declared)
     for name in declared:
         assert hasattr(lib, name), name

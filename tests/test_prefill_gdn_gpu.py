@@ -321,6 +321,30 @@ def test_gdn_prefill_equal_lengths_collapse_the_stages():
         _check(w, fast=True)
 
 
+def test_gdn_prefill_with_and_without_host_offsets_gives_the_same_bits():
+    """With ``raw_cu_seqlens`` the host applies the device's one-stage rule itself and enqueues nothing for a second
+    stage; without it the device collapses the stages.  Both must give the same bits, on either side of the rule, for
+    ragged lengths (staged either way) and through both host layers."""
+    from pla_amd.prefill.flashqla import ops
+    from pla_amd.workloads import gdn_prefill_packed
+    for lengths in ([1100] * 8, [1530, 1536, 1530, 1536, 955, 960, 890, 896], [1530, 1536, 1530, 1536, 955, 896, 890, 896],
+                    [2600, 300, 1900, 64, 0, 777, 1500, 2200]):
+        results = []
+        for native in (False, True):
+            for with_raw in (True, False):
+                ops._native = None if native else False
+                w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 3, seed=99)
+                if not with_raw:
+                    w["raw_cu_seqlens"] = None
+                g_cum, _, o, _, final = _run_workload(w)
+                torch.cuda.synchronize()
+                results.append((o, g_cum.reshape(-1, 16)[:sum(lengths)], final))
+        ops._native = False
+        for other in results[1:]:
+            for x, y in zip(results[0], other):
+                assert torch.equal(x, y), lengths
+
+
 def test_gdn_prefill_staged_pipeline_in_a_graph():
     """The staged call forks to a side stream and joins again, so it can be captured: three replays with
     eager work and synchronisation in between reproduce the eager result bit for bit."""
