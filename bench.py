@@ -65,13 +65,14 @@ def time_decode(prep, steps, warmup):
     """W untimed warm-up steps, then exactly K timed steps bracketed by synchronisations."""
     import torch
     step, bytes_state = prep["step"], prep["bytes_state"]
-    filler = torch.empty(32 << 20, dtype=torch.float32, device=prep["workload"]["mixed_qkv"].device)
+    filler = torch.empty(16 << 20, dtype=torch.float32, device=prep["workload"]["mixed_qkv"].device)
+    filler.zero_()                      # the fill kernel is loaded before anything is timed
     for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     # The op launches on torch's current stream, so torch events bracket exactly these launches.
     # One event pair around the K back-to-back launches: their mean is the kernel's average
-    # launch duration (rocprofv3 --kernel-trace reports the same average within 2 %).  A 128 MB fill runs
+    # launch duration (rocprofv3 --kernel-trace reports the same average within 2 %).  A 64 MB fill (about 13 us) runs
     # in front of the start event: while it runs the host enqueues the event and the first steps, so the event's
     # time stamp is followed at once by the first kernel and the K steps are back to back from the first one on
     # (with an idle stream the 10-20 us between enqueueing the event and the first launch would be counted, which
