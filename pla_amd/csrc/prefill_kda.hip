@@ -697,7 +697,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
 // Every tile of a chunk (K e^G, V, W hi / lo, the hi / lo pair of K e^{G_last - G}, e^{G_last}) is double buffered by
 // chunk parity (155 KiB of LDS: the operand tiles are unpadded), so there is ONE barrier per chunk: at the barrier
 // that opens chunk c its tiles have landed and the buffers of chunk c - 1 are free; the wavefronts fill them
-// with chunk c + 1 at once, a whole chunk ahead, and then compute chunk c:
+// with chunk c + 1 during chunk c, a whole chunk ahead of their use:
 //     KS = (K e^G) S^T,  X = V - KS (or -KS),  U = W X
 //     S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U              (pairs: hi.lo + lo.hi + hi.hi)
 // (With the pair single buffered and requested half a chunk ahead, behind a second barrier, copies and computation
@@ -778,12 +778,15 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       dma16(src, 1024u * j + 16u * lane, lds_address(dst) + 1024u * j);
     }
   };
-  // Every tile of chunk c into the buffers of its parity, in four parts, all issued right after the barrier that frees
-  // the buffers: wavefronts 4-7 take K e^G, V and W, wavefronts 0-3 the pair and e^{G_last} (0.60 ms for config 4's
-  // first sweep against 0.63 with wavefronts 4-7 issuing everything).  Measured alternatives: half of the parts issued
-  // between the two phases of a chunk 0.68 ms; the pair requested at a second barrier 0.66 ms; the parts spread over
-  // four points of the chunk spill registers (1.3 ms).  With wavefronts 4-7 only copying (a timing probe) the sweep
-  // takes the 0.48 ms of its copies alone, and its computation alone 0.36 ms: the two overlap only in part.
+  // Every tile of chunk c into the buffers of its parity, in four parts.  A wavefront that issues copies is held until
+  // the memory pipeline has taken them, so the two wavefronts of a SIMD issue at different times and one of them always
+  // computes: wavefronts 4-7 request K e^G, V and W right after the barrier that frees the buffers, wavefronts 0-3 the
+  // pair and e^{G_last} between the two phases of the chunk; everybody waits for its own copies before the next
+  // barrier.  Config 4's first sweep, ms: 0.59 this way; 0.62 with both groups issuing after the barrier; 0.63 with
+  // wavefronts 4-7 issuing everything there, 0.68 with them issuing half between the phases; 0.66 with the pair
+  // requested at a second barrier; the parts spread over four points of the chunk spill registers (1.3).  With
+  // wavefronts 4-7 only copying (a timing probe) the sweep takes the 0.48 ms of its copies alone, and its computation
+  // alone 0.36 ms.
   auto issue_part = [&](int c, int part) {
     const int par = c & 1;
     if (part == 0) {                                 // K e^G
@@ -819,9 +822,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
     // the one barrier of a chunk: its tiles have landed, chunk ci - 1 is finished and its buffers are free
     wait_vmcnt<0>();
     __syncthreads();
-    if (more) {
-      if (m_side) { issue_part(ci + 1, 0); issue_part(ci + 1, 1); } else { issue_part(ci + 1, 2); issue_part(ci + 1, 3); }
-    }
+    if (more && m_side) { issue_part(ci + 1, 0); issue_part(ci + 1, 1); }
     f32x4_t U[NB][4];
     if (computing) {
       const uint16_t* const K = tK[par];
@@ -907,6 +908,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
           for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) U[nb][tri_block_m(b)] = mfma16h(wa[b], xb[nb], U[nb][tri_block_m(b)]);
       }
     }
+    if (more && !m_side) { issue_part(ci + 1, 2); issue_part(ci + 1, 3); }
     if (computing) {
       // ---- S^T = e^{G_last} (.) S^T + (K e^{G_last - G})^T U ----
       bf16x8_t kt[8], ktl[8];
