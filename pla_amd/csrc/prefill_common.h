@@ -42,6 +42,12 @@ __device__ __forceinline__ uint2 read_tr4(const uint16_t* at) {
   return __builtin_bit_cast(uint2, v);
 }
 
+// Element r (0..3) of what read_tr4 returned, as FP32.
+template <typename T> __device__ __forceinline__ float quad_element(uint2 w, int r) {
+  const uint32_t pair = r < 2 ? w.x : w.y;
+  return (r & 1) ? hi16<T>(pair) : lo16<T>(pair);
+}
+
 // LDS tile pitches (bf16 elements): rows stay 16-byte aligned and consecutive rows start 4 (128-wide)
 // or 36 (64-wide) banks apart, which keeps the 8-byte operand reads of a wavefront conflict free.
 constexpr int PITCH128 = 136;

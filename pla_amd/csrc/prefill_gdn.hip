@@ -741,7 +741,7 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
     f32x4_t KS[NB][4];
     bf16x8_t wa[2][4], wl[2][4];
     float4 eg[4];
-    uint16_t vraw[NB][16];
+    uint2 vraw[NB][4];        // rows 16 mi + 4 kb .. + 3 of the lane's V column, one transposing read each
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
@@ -765,9 +765,7 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
             eg[mi] = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-              const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-              for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+              vraw[nb][mi] = read_tr4(&V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
             }
           }
 #pragma unroll
@@ -802,10 +800,10 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          X[nb][mi][0] = to_float(act_t{vraw[nb][4 * mi + 0]}) - eg[mi].x * KS[nb][mi][0];
-          X[nb][mi][1] = to_float(act_t{vraw[nb][4 * mi + 1]}) - eg[mi].y * KS[nb][mi][1];
-          X[nb][mi][2] = to_float(act_t{vraw[nb][4 * mi + 2]}) - eg[mi].z * KS[nb][mi][2];
-          X[nb][mi][3] = to_float(act_t{vraw[nb][4 * mi + 3]}) - eg[mi].w * KS[nb][mi][3];
+          X[nb][mi][0] = lo16<act_t>(vraw[nb][mi].x) - eg[mi].x * KS[nb][mi][0];
+          X[nb][mi][1] = hi16<act_t>(vraw[nb][mi].x) - eg[mi].y * KS[nb][mi][1];
+          X[nb][mi][2] = lo16<act_t>(vraw[nb][mi].y) - eg[mi].z * KS[nb][mi][2];
+          X[nb][mi][3] = hi16<act_t>(vraw[nb][mi].y) - eg[mi].w * KS[nb][mi][3];
         }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -1032,8 +1030,16 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   if (m_side) {
     plan_k.plan((uint32_t)tok_pitch_b, CHUNK - 1, cw, lane);
     plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
-    plan_w.plan(128, CHUNK - 1, cw, lane);
   }
+  // A wavefront that issues copies is held until the memory pipeline has taken them, so the two wavefronts of a SIMD
+  // issue at different times and one of them always computes: wavefronts 4-7 request the decay tile, K and V right
+  // after the barrier, wavefronts 0-3 the W pair between the two phases of the chunk.
+  auto issue_w = [&](int c) {
+    const int par = c & 1;
+    plan_w.plan(128, CHUNK - 1, cw, lane);           // worked out here: nothing is kept across the phases
+    plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, cw);
+    plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, cw);
+  };
   auto issue = [&](int c) {
     const int par = c & 1;
     const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
@@ -1050,14 +1056,14 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
       tail.plan((uint32_t)(p.stride_v * 2), len - 1, cw, lane);
       tail.issue(tV[par], vs, cw);
     }
-    plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, cw);
-    plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, cw);
   };
-  if (m_side && n_chunks > 0) issue(0);
+  if (n_chunks > 0) {
+    if (m_side) issue(0); else issue_w(0);
+  }
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
-    if (m_side) wait_vmcnt<0>();                     // chunk ci has landed
+    wait_vmcnt<0>();                                 // this wavefront's copies for chunk ci have landed
     __syncthreads();                                 // ... and chunk ci - 1 is finished: its buffers are free
     if (m_side && ci + 1 < n_chunks) issue(ci + 1);
     if (!computing) continue;
@@ -1068,7 +1074,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
     f32x4_t KS[NB][4];
     bf16x8_t wa[2][4], wl[2][4];
     float4 eg[4];
-    uint16_t vraw[NB][16];
+    uint2 vraw[NB][4];        // rows 16 mi + 4 kb .. + 3 of the lane's V column, one transposing read each
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
@@ -1093,9 +1099,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
             if (use_v) {
 #pragma unroll
               for (int nb = 0; nb < NB; ++nb) {
-                const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+                vraw[nb][mi] = read_tr4(&V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
               }
             }
           }
@@ -1131,10 +1135,10 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          X[nb][mi][0] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 0]}) : 0.f) - eg[mi].x * KS[nb][mi][0];
-          X[nb][mi][1] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 1]}) : 0.f) - eg[mi].y * KS[nb][mi][1];
-          X[nb][mi][2] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 2]}) : 0.f) - eg[mi].z * KS[nb][mi][2];
-          X[nb][mi][3] = (use_v ? to_float(act_t{vraw[nb][4 * mi + 3]}) : 0.f) - eg[mi].w * KS[nb][mi][3];
+          X[nb][mi][0] = (use_v ? lo16<act_t>(vraw[nb][mi].x) : 0.f) - eg[mi].x * KS[nb][mi][0];
+          X[nb][mi][1] = (use_v ? hi16<act_t>(vraw[nb][mi].x) : 0.f) - eg[mi].y * KS[nb][mi][1];
+          X[nb][mi][2] = (use_v ? lo16<act_t>(vraw[nb][mi].y) : 0.f) - eg[mi].z * KS[nb][mi][2];
+          X[nb][mi][3] = (use_v ? hi16<act_t>(vraw[nb][mi].y) : 0.f) - eg[mi].w * KS[nb][mi][3];
         }
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -1155,6 +1159,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
           for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
       }
     }
+    if (!m_side && ci + 1 < n_chunks) issue_w(ci + 1);
     // ---- S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U) ----
     {
 #pragma unroll

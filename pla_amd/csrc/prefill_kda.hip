@@ -487,7 +487,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
     auto ldW = [&](int b, bool lo) {
       return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][((lo ? TRI_BLOCKS : 0) + b) * 512 + lane * 8]));
     };
-    uint16_t vraw[NB][16];
+    uint2 vraw[NB][4];        // rows 16 mi + 4 kb .. + 3 of the lane's V column, one transposing read each
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
@@ -510,9 +510,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
           for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-              const uint16_t* vr = &tV[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-              for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+              vraw[nb][mi] = read_tr4(&tV[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
             }
 #pragma unroll
           for (int b = 0; b < 4; ++b) { wa[b] = ldW(b, false); wl[b] = ldW(b, true); }
@@ -540,7 +538,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) X[nb][mi][r] = to_float(bf16_t{vraw[nb][4 * mi + r]}) - KS[nb][mi][r];
+          for (int r = 0; r < 4; ++r) X[nb][mi][r] = quad_element<bf16_t>(vraw[nb][mi], r) - KS[nb][mi][r];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -833,7 +831,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
       auto ldW = [&](int b, bool lo) {
         return __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][((lo ? TRI_BLOCKS : 0) + b) * 512 + lane * 8]));
       };
-      uint16_t vraw[NB][16];
+      uint2 vraw[NB][4];        // rows 16 mi + 4 kb .. + 3 of the lane's V column, one transposing read each
       {
         bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
@@ -857,9 +855,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
               for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
-                  const uint16_t* vr = &V[(16 * mi + 4 * kb) * PITCH128 + vcol + 16 * nb];
-#pragma unroll
-                  for (int r = 0; r < 4; ++r) vraw[nb][4 * mi + r] = vr[r * PITCH128];
+                  vraw[nb][mi] = read_tr4(&V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
                 }
             }
 #pragma unroll
@@ -887,7 +883,7 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
         for (int mi = 0; mi < 4; ++mi)
 #pragma unroll
           for (int r = 0; r < 4; ++r)
-            X[nb][mi][r] = (use_v ? to_float(bf16_t{vraw[nb][4 * mi + r]}) : 0.f) - KS[nb][mi][r];
+            X[nb][mi][r] = (use_v ? quad_element<bf16_t>(vraw[nb][mi], r) : 0.f) - KS[nb][mi][r];
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
