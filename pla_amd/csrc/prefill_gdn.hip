@@ -24,21 +24,24 @@
 //
 // Kernels:
 //   prefill_tables_kernel    chunk / segment / stage tables from cu_seqlens (device side, graph-capturable)
-//   gdn_wsolve_kernel        preparation for the fused sweep, one wavefront per (chunk, value head): gate, beta and
-//                            their chunk-local cumsum, the decay-factor tile, normalised K, K K^T on MFMA, the
-//                            inverse of I + L by 16 x 16 blocks, W (hi, lo) in the six-block operand layout
-//   gdn_fused_sweep_kernel   whole sequences with 16-byte aligned q / k rows: one workgroup per (sequence, value
-//                            head) of four computing wavefronts (32 V columns of S^T each, in MFMA accumulator
-//                            layout, the chain K S^T -> X -> U -> S^T in registers) and four feeding wavefronts
-//                            that normalise the raw q / k rows into LDS tiles, form P and issue the global -> LDS
-//                            copies of V, W and the decay factors; two barriers per chunk
-//   gdn_prepare_kernel       preparation for the two kernels below: as gdn_wsolve_kernel, plus the normalised q / k
-//                            rows, Q K^T and P, W row-major (any 4-byte aligned q / k rows)
-//   gdn_sweep_kernel         sequential kernel with output for calls split into segments (second sweep) and for
-//                            q / k rows that are only 4-byte aligned: four computing wavefronts and one that issues
-//                            every global -> LDS copy; all tiles double buffered, one barrier per chunk
+//   gdn_wsolve_kernel        preparation for 16-byte aligned q / k rows, one wavefront per (chunk, value head): gate,
+//                            beta and their chunk-local cumsum, the decay-factor tile, normalised K, K K^T on MFMA,
+//                            the inverse of I + L by 16 x 16 blocks, W (hi, lo) in the six-block operand layout; for
+//                            calls split into segments also the normalised K rows
+//   gdn_fused_sweep_kernel   sequential kernel with output for 16-byte aligned q / k rows, over whole sequences or
+//                            (second sweep) over segments: one workgroup per (sequence or segment, value head) of four
+//                            computing wavefronts (32 V columns of S^T each, in MFMA accumulator layout, the chain
+//                            K S^T -> X -> U -> S^T in registers) and four feeding wavefronts that normalise the raw
+//                            q / k rows into LDS tiles, form P and issue the global -> LDS copies of V, W and the
+//                            decay factors; two barriers per chunk
 //   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
-//                            segment side by side in one workgroup of eight wavefronts that share every tile
+//                            segment side by side in one workgroup of eight wavefronts that share every tile; reads
+//                            what either preparation left (W in six blocks or row-major)
+//   gdn_prepare_kernel       preparation for q / k rows that are only 4-byte aligned: as gdn_wsolve_kernel, plus the
+//                            normalised q / k rows, Q K^T and P, W row-major
+//   gdn_sweep_kernel         sequential kernel with output after gdn_prepare_kernel (whole sequences and the second
+//                            sweep over segments): four computing wavefronts and one that issues every global -> LDS
+//                            copy; all tiles double buffered, one barrier per chunk
 
 #include <type_traits>
 
@@ -79,6 +82,7 @@ struct GdnPrefillParams {
   int qk_rows_16;        // q and k rows start on 16-byte boundaries (else on 4-byte ones)
   int inline_tables;     // at most 64 whole sequences: kernels work the chunk tables out themselves (no table kernel)
   int tail_blocks;       // workgroups appended to the preparation grid that zero the output rows beyond the last sequence
+  int store_kn;          // gdn_wsolve_kernel also stores the normalised K rows (kn): the first sweep over segments copies them
 };
 
 // ---------------------------------------------------------------------------------------------
@@ -327,14 +331,28 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
 // of a workgroup (the value heads of one q/k head) share the loading and normalising of the keys through LDS: a
 // quarter fewer vector instructions per tile and half the registers for raw rows, which brings three wavefronts
 // to a SIMD without spills (config 3 0.450 -> 0.440 ms, 8 x 2048 tokens 0.233 -> 0.224 ms; four per SIMD by a launch
-// bound measure the same: the kernel is bound by its vector instructions now, not by latency).
+// bound measure the same: the kernel is bound by its vector instructions now, not by latency).  For a call split
+// into segments (store_kn) the wavefront that normalised a row block also stores it: the first sweep over segments
+// copies its K tiles from those rows.
 template <typename act_t, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefillParams p) {
   const int groups = p.HV / WAVES;
   const int lane = threadIdx.x & 63;
   const int main_blocks = gridDim.x - p.tail_blocks;
-  if ((int)blockIdx.x >= main_blocks) {            // appended workgroups: zero the padded rows of o
-    zero_tail(reinterpret_cast<uint16_t*>(p.o), p.cu_seqlens, p.N, p.T, p.HV, blockIdx.x - main_blocks, p.tail_blocks);
+  if ((int)blockIdx.x >= main_blocks) {
+    // Appended workgroups: they zero the padded rows of o and, for a call split into segments, the first of them
+    // builds the chunk and segment tables the sweeps read (this kernel works its own tiles out by itself, so the
+    // tables only have to be complete when it ends).
+    const int extra = blockIdx.x - main_blocks;
+    const int builders = p.seg.seg_chunks > 0 ? 1 : 0;
+    if (extra < builders) {
+      chunk_map(p.cu_seqlens, p.N, p.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len);
+      __threadfence();
+      __syncthreads();
+      segment_map(p.seq_chunk_off, p.N, p.seg);
+    } else {
+      zero_tail(reinterpret_cast<uint16_t*>(p.o), p.cu_seqlens, p.N, p.T, p.HV, extra - builders, p.tail_blocks - builders);
+    }
     return;
   }
   int cb, t0, len;
@@ -475,6 +493,8 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
         const uint4 row_op = ok ? make_uint4(w[0], w[1], w[2], w[3]) : zero4;
         if constexpr (WAVES == 1) Kop[i][s] = __builtin_bit_cast(bf16x8_t, row_op);
         else Kshare[(mb * 4 + s) * 64 + lane] = row_op;
+        if (p.store_kn && ok && first_group)
+          *reinterpret_cast<uint4*>(p.kn + ((int64_t)(t0 + 16 * mb + r16) * p.H + h) * 128 + 32 * s + 8 * kb) = row_op;
       }
     }
   }
@@ -600,8 +620,8 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sequential kernel with output (whole sequences, and the second sweep over segments): one workgroup per
-// (sequence, value head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
+// Sequential kernel with output behind gdn_prepare_kernel (whole sequences, and the second sweep over segments): one
+// workgroup per (sequence or segment, value head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
 // memory only to store their output rows; wavefront 4 moves data: it issues every global -> LDS copy of the
 // workgroup (an LDS copy instruction occupies its issuer for tens of cycles, about 2 k cycles per chunk in all,
 // which the computing wavefronts no longer pay).  Every tile is double buffered by chunk parity, so there is
@@ -959,9 +979,11 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
 // wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
 // from its real start state (of which they keep a copy for the second sweep).  All tiles are double buffered by
 // chunk parity (109 KB of LDS) and there is one barrier per chunk, as in gdn_sweep_kernel.
-template <typename act_t>
+template <typename act_t, bool SIX>
 __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefillParams p) {
   constexpr int NB = 2;
+  // what gdn_wsolve_kernel (SIX) or gdn_prepare_kernel left per (chunk, value head): W and the tile of decay factors
+  constexpr int W_BYTES = SIX ? 2 * TRI_BLOCKS * 1024 : 16384, G_BYTES = SIX ? GTILE_FLOATS * 4 : 1024;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
   const int tid = threadIdx.x;
@@ -989,7 +1011,9 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 
   __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
   __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];      // [parity][hi, lo]
+  // W [parity]: the six-block operand layout (hi blocks, then lo blocks; SIX) or two padded row-major tiles (hi, lo)
+  constexpr int W_HI_LO = SIX ? TRI_BLOCKS * 512 : CHUNK * PITCH64;
+  __shared__ __align__(16) uint16_t tW[2][2 * W_HI_LO];
   // decay factors: [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
 
@@ -1023,8 +1047,8 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   const int64_t tok_pitch_b = (int64_t)p.H * 256;              // bytes between tokens of kn
   const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
   const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
-  const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
+  const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * W_BYTES;
+  const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * G_BYTES;
   CopyWide plan_k, plan_v;
   CopyNarrow plan_w;
   if (m_side) {
@@ -1036,16 +1060,23 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   // after the barrier, wavefronts 0-3 the W pair between the two phases of the chunk.
   auto issue_w = [&](int c) {
     const int par = c & 1;
-    plan_w.plan(128, CHUNK - 1, cw, lane);           // worked out here: nothing is kept across the phases
-    plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, cw);
-    plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, cw);
+    const char* const ws = w_b + (int64_t)c * p.HV * W_BYTES;
+    if constexpr (SIX) {                             // twelve 1 KiB blocks, three per wavefront, as they lie in memory
+#pragma unroll
+      for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)
+        dma16(ws, 1024u * (4 * j + cw) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (4 * j + cw));
+    } else {
+      plan_w.plan(128, CHUNK - 1, cw, lane);         // worked out here: nothing is kept across the phases
+      plan_w.issue(&tW[par][0], ws, cw);
+      plan_w.issue(&tW[par][W_HI_LO], ws + 8192, cw);
+    }
   };
   auto issue = [&](int c) {
     const int par = c & 1;
     const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
     const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
     const int len = chunk_len(c);
-    if (cw == 0) dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[par][0]));
+    if (cw == 0) dma16(gt_b + (int64_t)c * p.HV * G_BYTES, 16u * lane, lds_address(&tG[par][0]));
     if (len == CHUNK) {
       plan_k.issue(tK[par], ks, cw);
       plan_v.issue(tV[par], vs, cw);
@@ -1126,8 +1157,16 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          wa[s2][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], s2, kb);
-          wl[s2][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], s2, kb);
+          if constexpr (SIX) {
+            // block (row block mi, contraction half s2) of the lower triangle: 0-3 for s2 = 0, 4 and 5 (mi 2, 3) for s2 = 1
+            if (s2 == 1 && mi < 2) continue;
+            const int b = s2 == 0 ? mi : mi + 2;
+            wa[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][b * 512 + lane * 8]));
+            wl[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][(TRI_BLOCKS + b) * 512 + lane * 8]));
+          } else {
+            wa[s2][mi] = operand_from(&tW[par][(16 * mi + r16) * PITCH64], s2, kb);
+            wl[s2][mi] = operand_from(&tW[par][W_HI_LO + (16 * mi + r16) * PITCH64], s2, kb);
+          }
         }
       __builtin_amdgcn_sched_barrier(0x000F);
       f32x4_t X[NB][4];
@@ -1152,11 +1191,11 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+          for (int mi = (SIX && s == 1) ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+          for (int mi = (SIX && s == 1) ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
       }
     }
     if (!m_side && ci + 1 < n_chunks) issue_w(ci + 1);
@@ -1210,7 +1249,9 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused sweep for whole sequences: one workgroup of EIGHT wavefronts per (sequence, value head).  Wavefronts 0-3
+// Fused sweep, over whole sequences or as the second sweep over segments (pass 2: one 16 384-token sequence of 32
+// value heads 0.46 -> 0.36 ms against gdn_prepare_kernel / gdn_sweep_kernel there): one workgroup of EIGHT wavefronts
+// per (sequence or segment, value head).  Wavefronts 0-3
 // compute as in gdn_sweep_kernel (32 V columns of S^T each, the chain K S^T -> X -> U -> S^T in registers).
 // Wavefronts 4-7 feed them, so that neither the normalised rows nor P cross memory:
 //   rows   wavefronts 4, 5 take the raw K rows of the next chunk (32 rows each), 6, 7 the raw Q rows: loaded one
@@ -1231,14 +1272,16 @@ template <typename act_t>
 __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefillParams p) {
   constexpr int NB = 2, CW = 4, AUX = 4;
   using CopyV = SwizzledTileCopy<AUX>;
-  const int block = xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV);
+  // one workgroup per (sequence, value head), or per (segment, value head) in the second sweep over segments
+  const int block = xcd_grouped_index(blockIdx.x, p.HV / p.H, (p.pass == 2 ? p.seg.max_segments : p.N) * p.HV);
   if (block < 0) return;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   // the chunks of this workgroup's sequence: from the tables, or worked out here (every wavefront for itself)
   int3 inline_chunks{-1, 0, 0};
   int seq_first_chunk = 0, seq_first_token = 0, seq_end_token = 0;
-  if (p.inline_tables) {
+  const bool inline_tables = p.inline_tables && p.pass == 0;         // segments are looked up in the segment table
+  if (inline_tables) {
     const InlineSequences seqs = inline_sequences(p.cu_seqlens, p.N, p.stg.stages, lane);
     const int n0 = __builtin_amdgcn_readfirstlane(block / p.HV);
     seq_first_chunk = __builtin_amdgcn_readlane(seqs.off, n0);
@@ -1246,14 +1289,14 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     seq_end_token = seq_first_token + __builtin_amdgcn_readlane(seqs.len, n0);
     inline_chunks = int3{seq_first_chunk, min(seq_first_chunk + __builtin_amdgcn_readlane(seqs.nc, n0), p.NC_max), seqs.E};
   }
-  const SweepRole role = select_sweep(0, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
+  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride, true, block, inline_chunks);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int h = hv / (p.HV / p.H);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  if (!p.inline_tables) {
+  if (!inline_tables) {
     seq_first_chunk = p.seq_chunk_off[n];
     seq_first_token = p.cu_seqlens[n];
     seq_end_token = p.cu_seqlens[n + 1];
@@ -1950,8 +1993,11 @@ static int gdn_prefill_run(
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool segmented = L.seg_chunks > 0;
-  // whole sequences with 16-byte aligned q / k rows take the fused sweep (rows normalised and P formed inside it)
-  const bool fused = !segmented && p.qk_rows_16;
+  // 16-byte aligned q / k rows take the fused sweep (rows normalised and P formed inside it) after the lean preparation;
+  // for a call split into segments that is the second sweep, and the first one copies the normalised K rows the
+  // preparation then stores as well
+  const bool fused = p.qk_rows_16;
+  p.store_kn = segmented && fused;
   if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
@@ -1989,8 +2035,9 @@ static int gdn_prefill_run(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = stages;
   }
-  // Whole sequences through the fused sweep, at most 64 of them: the kernels work the chunk tables out themselves and
-  // the first launch of the preparation also zeroes the padded rows of o, so no table kernel runs ahead of them.
+  // 16-byte aligned rows and at most 64 sequences: no table kernel runs ahead of the preparation, whose first launch
+  // also zeroes the padded rows of o.  Whole sequences: every kernel works its chunks out by itself.  Segments: the
+  // preparation does, and one workgroup appended to it writes the chunk and segment tables for the sweeps.
   p.inline_tables = fused && N <= INLINE_TABLE_SEQUENCES;
   if (!p.inline_tables)
     launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
@@ -2000,7 +2047,7 @@ static int gdn_prefill_run(
       [&](hipStream_t ps) {
         const int ratio = HV / H;       // value heads per q/k head: as many wavefronts of a workgroup share K and Q
         const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
-        p.tail_blocks = (p.inline_tables && p.stage == 0) ? TABLE_WORKGROUPS - 1 : 0;
+        p.tail_blocks = (p.inline_tables && p.stage == 0) ? TABLE_WORKGROUPS - (segmented ? 0 : 1) : 0;
         const dim3 grid((unsigned)L.NC_max * (HV / waves) + p.tail_blocks), block(64 * waves);
         if (fused) {
           if (half_act) {
@@ -2024,8 +2071,11 @@ static int gdn_prefill_run(
       },
       [&](unsigned grid) {
         if (p.pass == 1) {        // first sweep over segments: no output, both roles in one workgroup per (segment, head)
-          if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(grid / 2), dim3(512), 0, s, p);
-          else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
+          if (fused) {
+            if (half_act) hipLaunchKernelGGL((gdn_lean_sweep_kernel<f16_t, true>), dim3(grid / 2), dim3(512), 0, s, p);
+            else hipLaunchKernelGGL((gdn_lean_sweep_kernel<bf16_t, true>), dim3(grid / 2), dim3(512), 0, s, p);
+          } else if (half_act) hipLaunchKernelGGL((gdn_lean_sweep_kernel<f16_t, false>), dim3(grid / 2), dim3(512), 0, s, p);
+          else hipLaunchKernelGGL((gdn_lean_sweep_kernel<bf16_t, false>), dim3(grid / 2), dim3(512), 0, s, p);
         } else {
           const unsigned g = xcd_grouped_grid(grid, (unsigned)(HV / H));
           if (fused) {
@@ -2040,7 +2090,11 @@ static int gdn_prefill_run(
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
                        ht_indices, ht_slot_stride);
     p.pass = 2;
-    if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+    if (fused) {
+      const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));
+      if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+      else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
+    } else if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
     else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
   }
   return check_launch("gdn prefill launch");
