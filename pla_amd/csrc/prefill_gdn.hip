@@ -319,6 +319,13 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefil
   }
 }
 
+// The value that lane ^ 32 holds.
+__device__ __forceinline__ uint32_t from_other_half(uint32_t x) {
+  uint32_t a = x, b = x;                // after the swap: a = the value of lanes 0-31 in both halves, b = that of lanes 32-63
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+  return (threadIdx.x & 32) ? a : b;
+}
+
 // ---------------------------------------------------------------------------------------------
 // Preparation for the fused sweep (gdn_fused_sweep_kernel), which normalises q and k and forms P itself: only what
 // needs the triangular solve leaves this kernel.  One wavefront per (chunk, value head) as above, the key side only:
@@ -493,8 +500,17 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
         const uint4 row_op = ok ? make_uint4(w[0], w[1], w[2], w[3]) : zero4;
         if constexpr (WAVES == 1) Kop[i][s] = __builtin_bit_cast(bf16x8_t, row_op);
         else Kshare[(mb * 4 + s) * 64 + lane] = row_op;
-        if (p.store_kn && ok && first_group)
-          *reinterpret_cast<uint4*>(p.kn + ((int64_t)(t0 + 16 * mb + r16) * p.H + h) * 128 + 32 * s + 8 * kb) = row_op;
+        if (p.store_kn && first_group) {
+          // The rows leave in the column order of an operand tile (prefill_common.h): granule 4 s + g of a row holds
+          // columns 32 s + 4 g .. + 3 and 32 s + 16 + 4 g .. + 3.  The lane's columns 32 s + 8 kb .. + 7 are one half of
+          // granules 2 (kb % 2) and 2 (kb % 2) + 1; lane kb ^ 2 (32 lanes away) holds the other halves, so the two
+          // exchange 8 bytes and each stores one whole granule.
+          const bool upper = kb >= 2;
+          const uint32_t r0 = from_other_half(upper ? row_op.x : row_op.z), r1 = from_other_half(upper ? row_op.y : row_op.w);
+          const uint4 granule = upper ? make_uint4(r0, r1, row_op.z, row_op.w) : make_uint4(row_op.x, row_op.y, r0, r1);
+          if (ok)
+            *reinterpret_cast<uint4*>(p.kn + ((int64_t)(t0 + 16 * mb + r16) * p.H + h) * 128 + 8 * (4 * s + 2 * (kb & 1) + (kb >> 1))) = granule;
+        }
       }
     }
   }
@@ -978,14 +994,18 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
 // also issue every global -> LDS copy, so each tile crosses memory and LDS once for the two sweeps and two
 // wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
 // from its real start state (of which they keep a copy for the second sweep).  All tiles are double buffered by
-// chunk parity (109 KB of LDS) and there is one barrier per chunk, as in gdn_sweep_kernel.
+// chunk parity (90 KB of LDS with the swizzled tiles, 109 KB with padded ones) and there is one barrier per chunk, as in
+// gdn_sweep_kernel.
 template <typename act_t, bool SIX>
 __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefillParams p) {
   constexpr int NB = 2;
   // what gdn_wsolve_kernel (SIX) or gdn_prepare_kernel left per (chunk, value head): W and the tile of decay factors
   constexpr int W_BYTES = SIX ? 2 * TRI_BLOCKS * 1024 : 16384, G_BYTES = SIX ? GTILE_FLOATS * 4 : 1024;
-  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 4>;      // 64 x 128 tile, issued by the four copying wavefronts
+  // K and V tiles, filled by the four copying wavefronts: swizzled and unpadded (SIX: the K rows come in the column
+  // order of an operand tile) or padded rows
+  using CopyWide = std::conditional_t<SIX, SwizzledTileCopy<4>, TileCopy<CHUNK, 2 * PITCH128, 256, 4>>;
   using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
+  constexpr int KV_HALVES = SIX ? TILE128_HALVES : CHUNK * PITCH128;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1009,8 +1029,8 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
+  __shared__ __align__(1024) uint16_t tK[2][KV_HALVES];
+  __shared__ __align__(1024) uint16_t tV[2][KV_HALVES];
   // W [parity]: the six-block operand layout (hi blocks, then lo blocks; SIX) or two padded row-major tiles (hi, lo)
   constexpr int W_HI_LO = SIX ? TRI_BLOCKS * 512 : CHUNK * PITCH64;
   __shared__ __align__(16) uint16_t tW[2][2 * W_HI_LO];
@@ -1042,6 +1062,19 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
     }
   }
   const bool use_v = computing && !role.zero_v;                // the identity sweep runs with v = 0
+  // LDS reads.  K operand of contraction step s for row block mi; the lane's V values of rows 16 mi + 4 kb .. + 3, column
+  // vcol + 16 nb, by one transposing read: lane t of a group of 16 addresses columns 32 cw + 16 nb + 4 (t % 4) .. + 3 of
+  // row 16 mi + 4 kb + t / 4, which in a swizzled tile is half (t % 2) of granule 4 cw + 2 nb + (t % 4) / 2; the
+  // swizzle 8 (kb & 1) + 2 (t / 4) of that row does not depend on mi, and nb = 1 differs in one bit of the granule index.
+  auto k_operand = [&](const uint16_t* K, int mi, int s) {
+    if constexpr (SIX) return operand_granule(K, 16 * mi + r16, s, kb);
+    else return operand_from(&K[(16 * mi + r16) * PITCH128], s, kb);
+  };
+  const int trV = (4 * kb + (r16 >> 2)) * 128 + 8 * ((4 * cw + ((r16 & 3) >> 1)) ^ (8 * (kb & 1) + 2 * (r16 >> 2))) + 4 * (r16 & 1);
+  auto v_at = [&](const uint16_t* V, int mi, int nb) {
+    if constexpr (SIX) return V + ((trV + 16 * 128 * mi) ^ (16 * nb));
+    else return &V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)];
+  };
 
   // ---- copies (wavefronts 4-7) ----
   const int64_t tok_pitch_b = (int64_t)p.H * 256;              // bytes between tokens of kn
@@ -1109,7 +1142,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
     {
       bf16x8_t ka[2][4], sb[2][NB];
 #pragma unroll
-      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
+      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = k_operand(K, mi, 0);
       __builtin_amdgcn_sched_barrier(0x000F);        // LDS requests stay above this line; ALU and MFMA work may cross it
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb)
@@ -1121,7 +1154,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
       for (int s = 0; s < 4; ++s) {
         if (s < 3) {
 #pragma unroll
-          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
+          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = k_operand(K, mi, s + 1);
         } else {
           // under the last step: V and e^G
 #pragma unroll
@@ -1130,7 +1163,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
             if (use_v) {
 #pragma unroll
               for (int nb = 0; nb < NB; ++nb) {
-                vraw[nb][mi] = read_tr4(&V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
+                vraw[nb][mi] = read_tr4(v_at(V, mi, nb));
               }
             }
           }
@@ -1204,7 +1237,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) kt[s2][mc] = operand_transposed(K, s2, mc, kb, r16);
+        for (int mc = 0; mc < 8; ++mc) kt[s2][mc] = SIX ? operand_granule_transposed(K, s2, mc, kb, r16) : operand_transposed(K, s2, mc, kb, r16);
         dg[s2][0] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 4 * kb]);
         dg[s2][1] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 16 + 4 * kb]);
       }
