@@ -345,12 +345,13 @@ def test_gdn_prefill_with_and_without_host_offsets_gives_the_same_bits():
                 assert torch.equal(x, y), lengths
 
 
-def test_gdn_prefill_staged_pipeline_in_a_graph():
+@pytest.mark.parametrize("lengths,H,HV", [([1500, 2100, 900, 1500, 1300, 1100, 700, 1200], 4, 16), ([2600, 70], 2, 4)])
+def test_gdn_prefill_staged_pipeline_in_a_graph(lengths, H, HV):
     """The staged call forks to a side stream and joins again, so it can be captured: three replays with
-    eager work and synchronisation in between reproduce the eager result bit for bit."""
+    eager work and synchronisation in between reproduce the eager result bit for bit.  The second case is a call
+    split into segments (two sweeps and the combine step, tables written by the preparation's appended workgroup)."""
     from pla_amd.workloads import gdn_prefill_packed
-    lengths = [1500, 2100, 900, 1500, 1300, 1100, 700, 1200]
-    w = gdn_prefill_packed(lengths, H=4, HV=16, pool_slots=len(lengths) + 2, seed=31)
+    w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 2, seed=31)
     pool0 = w["initial_state"].clone()
     _, _, o_eager, _, _ = _run_workload(w, output_final_state=False)
     torch.cuda.synchronize()
