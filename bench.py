@@ -133,7 +133,7 @@ KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00), summed over the kernels of
 # one call (profiles/gdn_prefill_kernels_32k.txt, profiles/kda_prefill_kernels_64k.txt)
 GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 1592000000
-KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11469000000
+KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11129000000
 
 
 def cpu_baseline_prefill(w):

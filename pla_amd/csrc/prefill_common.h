@@ -504,13 +504,15 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
                                                   const SegmentTable& seg, const StageTable& stg, int stage,
                                                   const float* h0, const int32_t* h0_indices,
                                                   int64_t h0_slot_stride, float* ht, const int32_t* ht_indices,
-                                                  int64_t ht_slot_stride, bool resweep_first = false, int block = -1,
+                                                  int64_t ht_slot_stride, int block = -1,
                                                   const int3 inline_chunks = int3{-1, 0, 0}) {
   // inline_chunks (pass 0 only, x >= 0): (first chunk, end chunk, stages in effect) of the workgroup's sequence worked
   // out by the caller (inline_sequences) instead of read from the tables
   // block: the logical workgroup index when the caller remaps blockIdx (see xcd_grouped_index), else blockIdx.x
-  // resweep_first: the first sweep publishes no output at all (first segments keep a copy of their start
-  // state and only deliver the state they end in), the second sweep runs every segment with output.
+  // Segments: the first sweep publishes no output at all (a first segment keeps a copy of its start state and only
+  // delivers the state it ends in), the second sweep runs every segment with output.  The LAST segment of a sequence
+  // has no part in the first sweep - nothing needs its summary -: the second sweep takes it from the state the combine
+  // step (or, for a sequence of one segment, the caller) provides and delivers the final state itself.
   SweepRole r{};
   r.write_o = true;
   auto state_in = [&](int n, int head) -> const float* {
@@ -545,21 +547,24 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     r.c_end = r.c_begin + seg.seg_nc[s];
     const int64_t tile = ((int64_t)s * heads + r.head) * 16384;
     if (pass == 1) {
+      if (last) return r;
+      r.write_o = false;
       if (first) {
         if (from_identity) return r;
         r.init = state_in(r.n, r.head);
-        r.fin = last ? state_out(r.n, r.head) : seg.B + tile;   // B of a first segment: the state entering the second
+        r.fin = seg.B + tile;                           // B of a first segment: the state entering the second
         carry = seg.B + tile;
-        if (resweep_first) { r.write_o = false; r.keep_init = seg.S + tile; }
+        r.keep_init = seg.S + tile;
       } else {
-        r.write_o = false;
         if (from_identity) { r.init = seg.identity; r.zero_v = true; r.fin = seg.M + tile; }
         else r.fin = seg.B + tile;
         carry = r.fin;
       }
     } else {
-      if (first && !resweep_first) return r;
-      r.init = seg.S + tile;                          // the state entering the segment (combine step, or kept copy)
+      // the state entering the segment: the caller's for a sequence of one segment, else the copy its first segment
+      // kept or what the combine step stored
+      r.init = (first && last) ? state_in(r.n, r.head) : seg.S + tile;
+      if (last) r.fin = state_out(r.n, r.head);
     }
   }
   if (carry != nullptr && stg.stages > 0) {
@@ -667,21 +672,20 @@ __device__ __forceinline__ void segment_map(const int32_t* seq_chunk_off, int N,
 }
 
 // Eight workgroups of 256 threads per (sequence, head), each owning 16 rows of the state (rows transform
-// independently): walks the sequence's segments, stores the state entering every later segment and the final
-// state.  A step S <- S M + B is a 16 x 128 x 128 product per workgroup on the FP32 MFMA
+// independently): walks the sequence's segments and stores the state entering every later segment (the last one
+// included: the second sweep carries it to the final state).  A step S <- S M + B is a 16 x 128 x 128 product per workgroup on the FP32 MFMA
 // (v_mfma_f32_16x16x4_f32, exact products, FP32 accumulation): wavefront w owns columns 32 w .. 32 w + 31 as two
 // accumulator tiles that start from B; the A operand is the workgroup's 16 rows of S from LDS (lane (r, kb) takes
 // S[r][16 s + 4 kb + e] for step (s, e)), the B operand the matching row of M straight from memory (lane (c, kb):
 // M[16 s + 4 kb + e][column c], 64 contiguous bytes per group of 16 lanes), all 64 loads of a step requested before
 // the first product.
 constexpr int COMBINE_SPLIT = 8;
-static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads, float* ht,
-                                                                     const int32_t* ht_indices, int64_t ht_slot_stride) {
+static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads) {
   const int part = blockIdx.x % COMBINE_SPLIT;
   const int chain = blockIdx.x / COMBINE_SPLIT;
   const int n = chain / heads, h = chain - n * heads;
   const int first = t.seq_seg_off[n], end = t.seq_seg_off[n + 1];
-  if (end - first < 2) return;                 // a single segment wrote its final state itself
+  if (end - first < 2) return;                 // a single segment starts from the caller's state
   __shared__ __align__(16) float S[16][132];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int c = lane & 15, kb = lane >> 4;
@@ -706,6 +710,7 @@ static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTabl
         t.S[tile + at(cb, v)] = acc[cb][v];
         S[4 * kb + v][col0 + 16 * cb] = acc[cb][v];
       }
+    if (seg + 1 == end) break;                 // the last segment: nothing follows it
     // M rows and the B tile of this segment, requested before the barrier
     const float* Mt = t.M + tile;
     float m[2][32];
@@ -733,16 +738,6 @@ static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTabl
           acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, m[cb][4 * s8 + e], acc[cb], 0, 0, 0);
       }
     __syncthreads();                           // every wavefront has read S before the next step overwrites it
-  }
-  if (ht != nullptr) {
-    const int slot = ht_indices ? ht_indices[n] : n;
-    if (slot >= 0) {
-      float* dst = ht + (int64_t)slot * ht_slot_stride + (int64_t)h * 16384;
-#pragma unroll
-      for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) dst[at(cb, v)] = acc[cb][v];
-    }
   }
 }
 

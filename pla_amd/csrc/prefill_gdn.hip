@@ -660,7 +660,7 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
   const int block = p.pass == 0 ? xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV) : (int)blockIdx.x;
   if (block < 0) return;
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, block);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int h = hv / (p.HV / p.H);
@@ -1016,10 +1016,10 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 
   // the two roles of this (segment, head): logical workgroups 2 i (zero state / real state) and 2 i + 1 (identity)
   const SweepRole lead = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x);
   if (!lead.active) return;
   const SweepRole mrole = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                       p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x + 1);
+                                       p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x + 1);
   const SweepRole& role = m_side ? mrole : lead;
   const bool computing = role.active;                          // wave-uniform; false: wavefronts 4-7 of a first segment
   const int n = lead.n, hv = lead.head, c_begin = lead.c_begin, c_end = lead.c_end;
@@ -1323,7 +1323,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
     inline_chunks = int3{seq_first_chunk, min(seq_first_chunk + __builtin_amdgcn_readlane(seqs.nc, n0), p.NC_max), seqs.E};
   }
   const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true, block, inline_chunks);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, block, inline_chunks);
   if (!role.active) return;
   const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int h = hv / (p.HV / p.H);
@@ -2120,8 +2120,7 @@ static int gdn_prefill_run(
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV, ht,
-                       ht_indices, ht_slot_stride);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV);
     p.pass = 2;
     if (fused) {
       const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));

@@ -348,7 +348,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true);
+                                      p.ht, p.ht_indices, p.ht_slot_stride);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
@@ -714,10 +714,10 @@ __global__ __launch_bounds__(512, 1) void kda_lean_sweep_kernel(const KdaPrefill
 
   // the two roles of this (segment, head): logical workgroups 2 i (zero state / real state) and 2 i + 1 (identity)
   const SweepRole lead = select_sweep(1, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, 0, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x);
   if (!lead.active) return;
   const SweepRole mrole = select_sweep(1, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, 0, p.h0, p.h0_indices, p.h0_slot_stride,
-                                       p.ht, p.ht_indices, p.ht_slot_stride, true, 2 * (int)blockIdx.x + 1);
+                                       p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x + 1);
   const SweepRole& role = m_side ? mrole : lead;
   const bool computing = role.active;                          // wave-uniform; false: wavefronts 4-7 of a first segment
   const int n = lead.n, h = lead.head, c_begin = lead.c_begin, c_end = lead.c_end;
@@ -1100,8 +1100,7 @@ extern "C" int pla_kda_prefill_launch(
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H, ht,
-                       ht_indices, ht_slot_stride);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H);
     p.pass = 2;
     hipLaunchKernelGGL(kda_sweep_kernel, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
