@@ -364,11 +364,12 @@ __device__ __forceinline__ void chunk_map(const int32_t* cu_seqlens, int N, int 
 // chip.  The per-token recurrence is affine in the state, S_out = S_in M + B, where for one segment
 // B is the state the segment produces from a zero state and M (K x K) is what it produces from the
 // identity with all values v = 0 (rows of the k-last state transform independently).  So:
-//   pass 1   every segment after the first of its sequence runs twice, from zero (-> B) and from the
-//            identity with v = 0 (-> M), without writing o; first segments run normally
-//   combine  per (sequence, head): S_in of every later segment, S <- S M + B in FP32, final state
-//   pass 2   the later segments run again from their true S_in and write o
-// which costs three sweeps over a later segment instead of one but runs them all concurrently.
+//   pass 1   no output.  A first segment runs from the caller's state, keeps a copy of it and delivers the state it
+//            ends in (its B); every segment between the first and the last of its sequence runs twice, from zero
+//            (-> B) and from the identity with v = 0 (-> M); the last segment does not run: nothing needs its summary
+//   combine  per (sequence, head): S_in of every later segment, S <- S M + B in FP32
+//   pass 2   every segment runs from its true S_in and writes o; the last one delivers the final state
+// which costs three sweeps over a middle segment instead of one but runs them all concurrently.
 struct SegmentTable {
   int32_t* seq_seg_off;   // [N + 1] first segment of each sequence
   int32_t* seg_seq;       // [segments] sequence of a segment
