@@ -29,6 +29,7 @@ itself fed in two chained calls per sequence; ``check_case`` also takes a refere
 import argparse
 import ast
 import csv
+import gzip
 import re
 import sys
 
@@ -68,8 +69,10 @@ def parse_case(line):
 
 
 def read_caselist(path, limit=None):
+    """The cases of a list file (plain text, or gzip when the name ends in .gz), in file order."""
     cases = []
-    with open(path) as fh:
+    opener = gzip.open if str(path).endswith(".gz") else open
+    with opener(path, "rt") as fh:
         for line in fh:
             case = parse_case(line)
             if case is not None:
@@ -134,6 +137,45 @@ def _eager_time_us(fn, reps):
     end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / reps * 1e3
+
+
+def _prefill_case_on_device(case, device, seed):
+    """A prefill case whose inputs are drawn on the GPU (same distributions as the CPU-seeded inputs of the checks,
+    other values): for replays of long lists, where drawing up to 32 768 tokens x 128 heads on the host would take
+    most of the time.  Returns ``(fn, kind)``."""
+    import math
+    from .prefill.flashqla import gdn_prefill_packed_qkv_fwd
+    from .prefill.flashkdapro import flashkda_fwd
+    dtype = torch.bfloat16 if case["dtype"] == "bf16" else torch.float16
+    H, HV = case["num_heads_qk"], case["num_heads_v"]
+    offs = list(case["cu_seqlens_q"])
+    N, T = len(offs) - 1, offs[-1]
+    lb = case.get("gate_lower_bound")
+    g = torch.Generator(device=device).manual_seed(seed)
+    rnd = lambda *s: torch.randn(*s, generator=g, device=device)
+    cu = torch.tensor(offs, dtype=torch.int32, device=device)
+    if case["op"] == "gdn_attn":
+        slots = max(8, N + 3)
+        packed = rnd(T, (2 * H + HV) * 128).to(dtype)
+        a, b = rnd(T, HV).to(dtype), rnd(T, HV).to(dtype)
+        A_log = torch.rand(HV, generator=g, device=device) * math.log(16.0)
+        dt_bias = torch.rand(HV, generator=g, device=device) * 2 - 1
+        pool = rnd(slots, HV, 128, 128) * 0.1
+        idx = torch.randperm(slots, generator=g, device=device)[:N].to(torch.int32)
+        fn = lambda: gdn_prefill_packed_qkv_fwd(packed, a, b, A_log, dt_bias, cu, num_qk_heads=H, num_v_heads=HV,
+                                                scale=128 ** -0.5, initial_state=pool, initial_state_indices=idx,
+                                                raw_cu_seqlens=tuple(offs), output_final_state=False)
+        return fn, "gdn_prefill"
+    q, k, v, gate = (rnd(T, H, 128).to(dtype) for _ in range(4))
+    beta = rnd(T, H).to(dtype)
+    A_log, dt_bias = rnd(H) * 0.5, rnd(H, 128) * 0.1
+    out = torch.empty(T, H, 128, dtype=dtype, device=device)
+    state = rnd(N, H, 128, 128) * 0.1
+    final = torch.empty(N, H, 128, 128, dtype=torch.float32, device=device)
+    fn = lambda: flashkda_fwd(q, k, v, gate, beta, A_log, dt_bias, out, scale=128 ** -0.5,
+                              lower_bound=-5.0 if lb is None else lb, initial_state=state, final_state=final,
+                              cu_seqlens=cu)
+    return fn, "kda_prefill"
 
 
 def build_case(case, device="cuda", seed=0, sets=None):
@@ -343,13 +385,19 @@ def check_case(case, reference=None, device="cuda", seed=0):
                 ok=finite and o_err <= 1.0 and states_ok)
 
 
-def replay_case(case, device="cuda", reps=20, seed=0):
-    """Runs and times one case.  Returns a result row (dict)."""
+def replay_case(case, device="cuda", reps=20, seed=0, device_inputs=False):
+    """Runs and times one case.  Returns a result row (dict).  device_inputs: prefill inputs are drawn on the GPU."""
     row = dict(family=case["family"], phase=case["phase"], batch=case.get("batch_size"),
                heads=f"{case.get('num_heads_qk')}/{case.get('num_heads_v')}", seqlen_q=case.get("seqlen_q"))
     reason = unsupported_reason(case)
     if reason is not None:
         row.update(status="skipped", reason=reason)
+        return row
+    if device_inputs and case["phase"] == "P":
+        fn, kind = _prefill_case_on_device(case, device, seed)
+        us = _eager_time_us(fn, max(3, reps // 4))
+        tokens = case["cu_seqlens_q"][-1]
+        row.update(status="ok", kind=kind, us=round(us, 1), tokens=tokens, tokens_per_s=round(tokens / us * 1e6))
         return row
     fns, info = build_case(case, device=device, seed=seed)
     if case["phase"] == "D":
@@ -374,6 +422,9 @@ def main(argv=None):
                     help="instead of timing, check N seeded small prefill shapes of the list: each case against itself "
                          "fed in two chained calls per sequence; exit status 1 if a case fails")
     ap.add_argument("--check-max-tokens", type=int, default=2048)
+    ap.add_argument("--device-inputs", action="store_true",
+                    help="draw prefill inputs on the GPU instead of the host (long lists; same distributions)")
+    ap.add_argument("--quiet", action="store_true", help="print every 500th row only (the CSV holds them all)")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         print("a GPU is required to replay a caselist", file=sys.stderr)
@@ -395,13 +446,15 @@ def main(argv=None):
     if writer:
         writer.writeheader()
     try:
-        for case in read_caselist(args.caselist, args.limit)[args.start:]:
-            row = replay_case(case, reps=args.reps)
-            print(row, flush=True)
+        for i, case in enumerate(read_caselist(args.caselist, args.limit)[args.start:]):
+            row = replay_case(case, reps=args.reps, device_inputs=args.device_inputs)
+            if not args.quiet or i % 500 == 0:
+                print(args.start + i, row, flush=True)
             if writer:
                 writer.writerow(row)
                 fh.flush()
-            torch.cuda.empty_cache()
+            if not args.device_inputs or i % 100 == 99:      # (the caching allocator reuses the blocks in between)
+                torch.cuda.empty_cache()
     finally:
         if fh:
             fh.close()

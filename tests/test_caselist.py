@@ -13,6 +13,7 @@ GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 SAMPLE = os.path.join(GOLDEN, "caselist_sample.list")
 DECODE_HEAD_SHAPES = os.path.join(GOLDEN, "caselist_decode_head_shapes.list")
 PREFILL_EVERY50 = os.path.join(GOLDEN, "caselist_prefill_every50.list")
+PREFILL_ALL = os.path.join(GOLDEN, "caselist_prefill_all.list.gz")
 
 
 def test_parse_sample_lines():
@@ -51,6 +52,11 @@ def test_full_caselist_fixtures_parse_and_are_served():
     assert all(caselist.unsupported_reason(c) is None for c in prefill)
     assert all(c["cu_seqlens_q"][0] == 0 and len(c["cu_seqlens_q"]) == c["batch_size"] + 1 for c in prefill)
     assert max(c["cu_seqlens_q"][-1] for c in prefill) == 32768
+    # every distinct line of the prefill caselists (gzip): all of them are served
+    everything = caselist.read_caselist(PREFILL_ALL)
+    assert len(everything) == 38971 and all(c["phase"] == "P" for c in everything)
+    assert all(caselist.unsupported_reason(c) is None for c in everything)
+    assert sum(c["cu_seqlens_q"][-1] for c in everything) == 677946457
 
 
 @pytest.mark.gpu
