@@ -310,8 +310,9 @@ int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV);
  * kkt_solve, fused_fwd) with one call that runs all stages on `stream`.
  *
  *   q,k [T,H,128], v [T,HV,128] in the activation dtype (act_dtype: PLA_BF16 or PLA_F16) with token
- *       pitches stride_q/k/v (views into a packed Q|K|V row are fine; q and k rows 4-byte aligned,
- *       v rows 16-byte aligned: v % 16 == 0, stride_v % 8 == 0); a,b [T,HV] raw gate / beta
+ *       pitches stride_q/k/v (views into a packed Q|K|V row are fine; q and k rows 4-byte aligned - rows that
+ *       are not 16-byte aligned are copied into the workspace first -, v rows 16-byte aligned: v % 16 == 0,
+ *       stride_v % 8 == 0); a,b [T,HV] raw gate / beta
  *       logits in the same dtype (pitches stride_a/b) with
  *       A_log, dt_bias [HV] float32:  g = -exp(A_log) softplus(a + dt_bias), beta = sigmoid(b);
  *       or g_in, beta_in [T,HV] float32 (log-decay per token, activated beta) instead.

@@ -167,7 +167,7 @@ py::object try_chunk_gated_delta_rule_fwd(
   const int64_t H = v.size(2);
   if (H <= 0 || H % Hg != 0 || !token_rows(q, T, Hg, 1) || !token_rows(k, T, Hg, 1) || !token_rows(v, T, H, 1)) return py::none();
   if (!same_gpu(k, q) || !same_gpu(v, q)) return py::none();
-  // q / k rows are read in 4-byte words, v rows are copied in 16-byte pieces (the facade materialises other views)
+  // q / k rows must start on 4-byte boundaries, v rows on 16-byte ones (the facade materialises other views)
   if (!aligned(q, 4) || q.stride(1) % 2 || !aligned(k, 4) || k.stride(1) % 2 || !aligned(v, 16) || v.stride(1) % 8) return py::none();
   if (!overlap_warmup_threshold.is_none()) {
     if (!py::isinstance<py::float_>(overlap_warmup_threshold) && !py::isinstance<py::int_>(overlap_warmup_threshold)) return py::none();

@@ -11,29 +11,7 @@ namespace pla {
 
 constexpr int CHUNK = 64;
 
-// A (or B) operand of one 16x16x32 MFMA step from a row-major bf16 tile: lane (r = lane%16,
-// kb = lane/16) takes columns [32s+4kb, +4) and [32s+16+4kb, +4) of row r, which is the
-// contraction order in which an accumulator tile pair (row blocks 2s, 2s+1) presents its rows.
-__device__ __forceinline__ bf16x8_t operand_from(const uint16_t* row_ptr, int s, int kb) {
-  const uint2 p0 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 4 * kb);
-  const uint2 p1 = *reinterpret_cast<const uint2*>(row_ptr + 32 * s + 16 + 4 * kb);
-  const uint4 u = make_uint4(p0.x, p0.y, p1.x, p1.y);
-  return __builtin_bit_cast(bf16x8_t, u);
-}
-
-// The same operand from the TRANSPOSE of a row-major 128-wide bf16 tile (row pitch PITCH128): lane
-// (r = lane%16, kb) takes rows [32s+4kb, +4) and [32s+16+4kb, +4) of column 16 m + r.  ds_read_b64_tr_b16
-// transposes inside each group of 16 lanes: lane t of the group addresses four consecutive columns
-// 16 m + 4 (t%4) .. +3 of row base + t/4, and lane i receives column 16 m + i of rows base .. base + 3.
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ bf16x8_t operand_transposed(const uint16_t* tile, int s, int m, int kb, int r) {
-  const uint16_t* at = tile + (32 * s + 4 * kb + (r >> 2)) * 136 + 16 * m + 4 * (r & 3);
-  const i16x4_t p0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)at);
-  const i16x4_t p1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) i16x4_t*)(at + 16 * 136));
-  typedef short i16x8_t __attribute__((ext_vector_type(8)));
-  const i16x8_t u = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-  return __builtin_bit_cast(bf16x8_t, u);
-}
 
 // One transposing read: lane i of a group of 16 receives column i of the four rows the group addresses (lane t
 // addresses columns 4 (t % 4) .. + 3 of row t / 4), packed as 16-bit (row 0, row 1), (row 2, row 3).
@@ -48,10 +26,9 @@ template <typename T> __device__ __forceinline__ float quad_element(uint2 w, int
   return (r & 1) ? hi16<T>(pair) : lo16<T>(pair);
 }
 
-// LDS tile pitches (bf16 elements): rows stay 16-byte aligned and consecutive rows start 4 (128-wide)
-// or 36 (64-wide) banks apart, which keeps the 8-byte operand reads of a wavefront conflict free.
+// Pitch of a padded 128-wide LDS tile (16-bit elements): rows stay 16-byte aligned and consecutive rows start 4 banks
+// apart, which keeps the 8-byte reads of a wavefront conflict free.
 constexpr int PITCH128 = 136;
-constexpr int PITCH64 = 72;
 
 // ---------------------------------------------------------------------------------------------
 // W = (I + L)^-1 diag(beta) for a strictly lower triangular 64 x 64 L (FP32, in LDS) on ONE wavefront, by
@@ -139,31 +116,6 @@ __device__ __forceinline__ void block_inverse_inplace(float (*L)[68], int lane) 
   put(1, 0, X10); put(2, 1, X21); put(3, 2, X32); put(2, 0, X20); put(3, 1, X31); put(3, 0, X30);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
-}
-
-// Row-major store.  PAIR: W leaves as two fp16 tiles, hi at W and lo at W + 4096 (W = hi + lo to about 22 bits),
-// else as one tile rounded to nearest.
-template <bool PAIR>
-__device__ __forceinline__ void block_inverse_store_w(float (*L)[68], const float* beta, int lane, uint16_t* W) {
-  block_inverse_inplace(L, lane);
-  // W[i][j] = N[i][j] beta_j for j <= i, zero above: lane -> row 8 pass + lane / 8, columns 8 (lane % 8) ..
-  const int c8 = 8 * (lane & 7);
-  const float4 b0 = *reinterpret_cast<const float4*>(&beta[c8]), b1 = *reinterpret_cast<const float4*>(&beta[c8 + 4]);
-#pragma unroll
-  for (int pass = 0; pass < 8; ++pass) {
-    const int i = 8 * pass + (lane >> 3);
-    const float4 lo = *reinterpret_cast<const float4*>(&L[i][c8]), hi = *reinterpret_cast<const float4*>(&L[i][c8 + 4]);
-    const float w[8] = {lo.x * b0.x, lo.y * b0.y, lo.z * b0.z, lo.w * b0.w, hi.x * b1.x, hi.y * b1.y, hi.z * b1.z, hi.w * b1.w};
-    uint32_t packed[4], rest[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float w0 = c8 + 2 * e <= i ? w[2 * e] : 0.f, w1 = c8 + 2 * e + 1 <= i ? w[2 * e + 1] : 0.f;
-      if constexpr (PAIR) pack2_pair(w0, w1, packed[e], rest[e]);
-      else packed[e] = pack2<f16_t>(w0, w1);
-    }
-    *reinterpret_cast<uint4*>(W + i * 64 + c8) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
-    if constexpr (PAIR) *reinterpret_cast<uint4*>(W + 4096 + i * 64 + c8) = make_uint4(rest[0], rest[1], rest[2], rest[3]);
-  }
 }
 
 // A lower triangular 64 x 64 tile as the A (or B) operands of the products that contract over its columns: only six

@@ -24,25 +24,21 @@
 //
 // Kernels:
 //   prefill_tables_kernel    chunk / segment / stage tables from cu_seqlens (device side, graph-capturable)
-//   gdn_wsolve_kernel        preparation for 16-byte aligned q / k rows, one wavefront per (chunk, value head): gate,
-//                            beta and their chunk-local cumsum, the decay-factor tile, normalised K, K K^T on MFMA,
-//                            the inverse of I + L by 16 x 16 blocks, W (hi, lo) in the six-block operand layout; for
-//                            calls split into segments also the normalised K rows
-//   gdn_fused_sweep_kernel   sequential kernel with output for 16-byte aligned q / k rows, over whole sequences or
-//                            (second sweep) over segments: one workgroup per (sequence or segment, value head) of four
-//                            computing wavefronts (32 V columns of S^T each, in MFMA accumulator layout, the chain
-//                            K S^T -> X -> U -> S^T in registers) and four feeding wavefronts that normalise the raw
-//                            q / k rows into LDS tiles, form P and issue the global -> LDS copies of V, W and the
-//                            decay factors; two barriers per chunk
+//   gdn_align_rows_kernel    q / k rows that start on 4-byte boundaries only are copied into dense buffers first
+//   gdn_wsolve_kernel        preparation, one wavefront per (chunk, value head): gate, beta and their chunk-local
+//                            cumsum, the decay-factor tile, normalised K, K K^T on MFMA, the inverse of I + L by
+//                            16 x 16 blocks, W (hi, lo) in the six-block operand layout; for calls split into
+//                            segments also the normalised K rows and (one appended workgroup) the tables
+//   gdn_fused_sweep_kernel   sequential kernel with output, over whole sequences or (second sweep) over segments: one
+//                            workgroup per (sequence or segment, value head) of four computing wavefronts (32 V
+//                            columns of S^T each, in MFMA accumulator layout, the chain K S^T -> X -> U -> S^T in
+//                            registers) and four feeding wavefronts that normalise the raw q / k rows into LDS
+//                            tiles, form P and issue the global -> LDS copies of V, W and the decay factors; two
+//                            barriers per chunk
 //   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
-//                            segment side by side in one workgroup of eight wavefronts that share every tile; reads
-//                            what either preparation left (W in six blocks or row-major)
-//   gdn_prepare_kernel       preparation for q / k rows that are only 4-byte aligned: as gdn_wsolve_kernel, plus the
-//                            normalised q / k rows, Q K^T and P, W row-major
-//   gdn_sweep_kernel         sequential kernel with output after gdn_prepare_kernel (whole sequences and the second
-//                            sweep over segments): four computing wavefronts and one that issues every global -> LDS
-//                            copy; all tiles double buffered, one barrier per chunk
+//                            segment side by side in one workgroup of eight wavefronts that share every tile
 
+#include <algorithm>
 #include <type_traits>
 
 #include "prefill_common.h"
@@ -68,254 +64,34 @@ struct GdnPrefillParams {
   void* o;                                            // [T, HV, 128] dense
   // workspace
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
-  uint16_t* qn; uint16_t* kn;
-  float* kinv;                                        // [T, H] 1 / |k| per row (fused sweep)
+  uint16_t* kn;                                       // [T, H, 128] normalised K rows in operand column order (calls split into segments)
+  float* kinv;                                        // [T, H] 1 / |k| per row
   float* gcum; float* beta;
-  uint16_t* W;                                        // fp16 [chunk, HV, 2, 64, 64]: W = hi + lo
-  uint16_t* P;                                        // fp16 [chunk, HV, 64, 64]
-  float* gtile;          // [chunk, HV, 256]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last}, ...
+  uint16_t* W;                                        // fp16 [chunk, HV, 12 blocks of 1 KiB]: W = hi + lo, six-block operand layout
+  float* gtile;          // [chunk, HV, 320]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last} | G
   SegmentTable seg;      // split long sequences (seg.seg_chunks > 0)
   StageTable stg;        // pipelined preparation and sweep (stg.stages > 0)
   int pass;              // 0: whole sequences; 1, 2: the two sweeps over segments
   int stage;             // stage handled by this launch (per-chunk kernels and pass 3)
   int H, HV, NC_max;
-  int qk_rows_16;        // q and k rows start on 16-byte boundaries (else on 4-byte ones)
   int inline_tables;     // at most 64 whole sequences: kernels work the chunk tables out themselves (no table kernel)
   int tail_blocks;       // workgroups appended to the preparation grid that zero the output rows beyond the last sequence
   int store_kn;          // gdn_wsolve_kernel also stores the normalised K rows (kn): the first sweep over segments copies them
 };
 
-// ---------------------------------------------------------------------------------------------
-// Preparation of a chunk, everything that does not depend on the state, in one kernel: one wavefront per
-// (chunk, value head); the WAVES wavefronts of a workgroup take consecutive value heads of one q/k head, so the
-// raw K and Q rows they all read meet in the CU's cache.  Per wavefront:
-//   gate      lane j = token j: g_j = -exp(A_log) softplus(a_j + dt_bias) and beta_j = sigmoid(b_j) (or the
-//             caller's g / beta), the chunk-local cumulative log-decay G by a scan over the lanes, the copies the
-//             call returns (g_cum, beta) and the chunk's tile of decay factors for the sequential kernel
-//   q, k      the raw rows are loaded directly in MFMA operand layout (lane (r, kb) holds 32 values of a row; the
-//             four lanes of a row meet through two lane swaps), L2-normalised, rounded to the activation dtype
-//             (the reference's operand) and held as fp16, which represents those values exactly; one wavefront of
-//             the q/k head stores the normalised K rows for the sequential kernel, another the Q rows
-//   products  K K^T and Q K^T on MFMA, L = strict_tril(beta_i (k_i.k_j) e^{G_i - G_j}), W = (I + L)^-1 diag(beta)
-//             by 16 x 16 blocks (an fp16 hi + lo pair), P = scale tril(q_i.k_j e^{G_i - G_j}) (fp16)
-template <typename act_t, int WAVES>
-__global__ __launch_bounds__(64 * WAVES) void gdn_prepare_kernel(const GdnPrefillParams p) {
-  const int groups = p.HV / WAVES;
-  const int cb = staged_chunk(p.stg, p.stage, blockIdx.x / groups, p.seq_chunk_off[p.N]);
-  if (cb < 0) return;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int hv0 = (blockIdx.x % groups) * WAVES;           // first value head of this workgroup
-  const int hv = hv0 + wave;
-  const int ratio = p.HV / p.H;
-  const int h = hv / ratio;
-  const int t0 = p.chunk_tok[cb];
-  const int len = p.chunk_len[cb];
-  const int lane = threadIdx.x & 63;
-  const int r16 = lane & 15, kb = lane >> 4;
-
-  __shared__ __align__(16) float Lm_all[WAVES][CHUNK][68];
-  __shared__ __align__(16) float Gs_all[WAVES][CHUNK];
-  __shared__ __align__(16) float Bs_all[WAVES][CHUNK];
-  float (*const Lm)[68] = Lm_all[wave];
-  float* const Gs = Gs_all[wave];
-  float* const Bs = Bs_all[wave];
-
-  // raw K and Q operands: 4 row blocks x 4 contraction steps of 16 bytes (lane (r, kb) takes elements 32 s + 8 kb .. + 7
-  // of its row; the contraction index may be assigned to operand slots in any order as long as both operands of a
-  // product agree); all 32 loads of a lane are requested before the first use (a SIMD holds two wavefronts, which
-  // hide no latency)
-  uint4 kraw[4][4], qraw[4][4];
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) {
-    const int row = 16 * mb + r16;
-    const int64_t t = t0 + (row < len ? row : 0);
-    const uint16_t* kr = reinterpret_cast<const uint16_t*>(p.k) + t * p.stride_k + h * 128 + 8 * kb;
-    const uint16_t* qr = reinterpret_cast<const uint16_t*>(p.q) + t * p.stride_q + h * 128 + 8 * kb;
-    if (p.qk_rows_16) {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) kraw[mb][s] = *reinterpret_cast<const uint4*>(kr + 32 * s);
-#pragma unroll
-      for (int s = 0; s < 4; ++s) qraw[mb][s] = *reinterpret_cast<const uint4*>(qr + 32 * s);
-    } else {                                             // rows aligned to 4 bytes only
-      auto four_words = [](const uint16_t* at) {
-        const uint32_t* w = reinterpret_cast<const uint32_t*>(at);
-        return make_uint4(w[0], w[1], w[2], w[3]);
-      };
-#pragma unroll
-      for (int s = 0; s < 4; ++s) kraw[mb][s] = four_words(kr + 32 * s);
-#pragma unroll
-      for (int s = 0; s < 4; ++s) qraw[mb][s] = four_words(qr + 32 * s);
-    }
-  }
-
-  // ---- gate: lane = token ----
-  {
-    float g = 0.f, bt = 0.f;
-    if (lane < len) {
-      const int64_t t = t0 + lane;
-      if (p.g_in) {
-        g = p.g_in[t * p.HV + hv];
-        bt = p.beta_in[t * p.HV + hv];
-      } else {
-        const float x = to_float(reinterpret_cast<const act_t*>(p.a)[t * p.stride_a + hv]) + p.dt_bias[hv];
-        const float sp = x <= 20.0f ? log1pf(expf(x)) : x;
-        g = -expf(p.A_log[hv]) * sp;
-        const float braw = to_float(reinterpret_cast<const act_t*>(p.b)[t * p.stride_b + hv]);
-        bt = 1.0f / (1.0f + expf(-braw));
-      }
-    }
-    // inclusive scan over the 64 lanes (rows beyond the chunk have g = 0 and so repeat G_last)
-    float cum = g;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const float up = __shfl_up(cum, d, 64);
-      if (lane >= d) cum += up;
-    }
-    const float glast = __shfl(cum, 63, 64);
-    if (lane < len) {
-      const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;
-      p.gcum[at] = cum;
-      p.beta[at] = bt;
-    }
-    Gs[lane] = cum;
-    Bs[lane] = bt;
-    // decay factors of the sequential kernel, one 1 KiB tile per (chunk, value head)
-    float* gt = p.gtile + ((int64_t)cb * p.HV + hv) * 256;
-    const float e = __expf(cum);
-    gt[lane] = p.scale * e;
-    gt[64 + lane] = e;
-    gt[128 + lane] = __expf(glast - cum);
-    gt[192 + lane] = __expf(glast);
-  }
-
-  // ---- q / k: normalise, round to the activation dtype, hold as fp16 (exact; saturating beyond its range) ----
-  bf16x8_t Kop[4][4], Qop[4][4];
-  {
-    auto row_scale = [&](const uint4 (&raw)[4]) {
-      float ss = 0.f;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const uint32_t w[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float a0 = lo16<act_t>(w[e]), a1 = hi16<act_t>(w[e]);
-          ss += a0 * a0 + a1 * a1;
-        }
-      }
-      const LanePair r1 = swap_rows16(ss);               // the four lanes of a row are 16 lanes apart
-      const LanePair r2 = swap_halves(r1.lo + r1.hi);
-      return rsqrtf(r2.lo + r2.hi + 1e-6f);
-    };
-    auto normalised = [&](const uint4& raw, float inv) {
-      const uint32_t in[4] = {raw.x, raw.y, raw.z, raw.w};
-      uint32_t w[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const uint32_t a = pack2<act_t>(lo16<act_t>(in[e]) * inv, hi16<act_t>(in[e]) * inv);
-        w[e] = pack2_rtz(lo16<act_t>(a), hi16<act_t>(a));
-      }
-      return __builtin_bit_cast(bf16x8_t, make_uint4(w[0], w[1], w[2], w[3]));
-    };
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
-    // the normalised rows go to the sequential kernel from one wavefront of the q/k head each (K from the first,
-    // Q from the second, or both from the only one)
-    const bool first_group = hv0 % ratio == 0;
-    const bool store_k = first_group && wave == 0, store_q = first_group && wave == (WAVES > 1 ? 1 : 0);
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      const int row = 16 * mb + r16;
-      const bool ok = row < len;
-      const float ki = p.normalize_qk ? row_scale(kraw[mb]) : 1.f;
-      const float qi = p.normalize_qk ? row_scale(qraw[mb]) : 1.f;
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const bf16x8_t kz = normalised(kraw[mb][s], ki), qz = normalised(qraw[mb][s], qi);
-        Kop[mb][s] = ok ? kz : __builtin_bit_cast(bf16x8_t, zero4);
-        Qop[mb][s] = ok ? qz : __builtin_bit_cast(bf16x8_t, zero4);
-      }
-      if (ok && (store_k || store_q)) {
-        uint16_t* dst = (store_k ? p.kn : p.qn) + ((int64_t)(t0 + row) * p.H + h) * 128 + 8 * kb;
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          *reinterpret_cast<uint4*>(dst + 32 * s) = __builtin_bit_cast(uint4, store_k ? Kop[mb][s] : Qop[mb][s]);
-        if (store_k && store_q) {                      // one wavefront per q/k head: it stores both
-          uint16_t* dq = p.qn + ((int64_t)(t0 + row) * p.H + h) * 128 + 8 * kb;
-#pragma unroll
-          for (int s = 0; s < 4; ++s) *reinterpret_cast<uint4*>(dq + 32 * s) = __builtin_bit_cast(uint4, Qop[mb][s]);
-        }
-      }
-    }
-  }
-  __syncthreads();
-
-  // L = strict_tril(beta_i (k_i . k_j) e^{G_i - G_j})
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-#pragma unroll
-    for (int ni = 0; ni <= mi; ++ni) {
-      f32x4_t kk = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 4; ++s) kk = mfma16h(Kop[mi][s], Kop[ni][s], kk);
-      const int j = 16 * ni + r16;
-      const float Gj = Gs[j];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * mi + 4 * kb + r;
-        Lm[i][j] = i > j ? Bs[i] * kk[r] * __expf(Gs[i] - Gj) : 0.f;
-      }
-    }
-  }
-
-  // P = scale * tril(q_i . k_j e^{G_i - G_j}), kept as packed fp16 until the solve has released the LDS tile
-  uint32_t Ppk[10][2];
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi) {
-#pragma unroll
-    for (int ni = 0; ni <= mi; ++ni) {
-      const int j = 16 * ni + r16;
-      f32x4_t qk = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 4; ++s) qk = mfma16h(Qop[mi][s], Kop[ni][s], qk);
-      const float Gj = Gs[j];
-      float pv[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int i = 16 * mi + 4 * kb + r;
-        pv[r] = i >= j ? p.scale * qk[r] * __expf(Gs[i] - Gj) : 0.f;
-      }
-      Ppk[mi * (mi + 1) / 2 + ni][0] = pack2_rtz(pv[0], pv[1]);
-      Ppk[mi * (mi + 1) / 2 + ni][1] = pack2_rtz(pv[2], pv[3]);
-    }
-  }
-
-  // W = (I + L)^-1 diag(beta): 16 x 16 blocks, the off-diagonal ones on MFMA
-  block_inverse_store_w<true>(Lm, Bs, lane, p.W + ((int64_t)cb * p.HV + hv) * 8192);
-  __syncthreads();
-
-  // P leaves through the released tile in 16-byte pieces; blocks above the diagonal are never written and read as zero
-  uint16_t* const Ps = reinterpret_cast<uint16_t*>(&Lm[0][0]);          // rows of 136 halves
-#pragma unroll
-  for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-    for (int ni = 0; ni <= mi; ++ni) {
-      uint16_t* dst = Ps + (16 * mi + 4 * kb) * 136 + 16 * ni + r16;
-      const uint32_t w0 = Ppk[mi * (mi + 1) / 2 + ni][0], w1 = Ppk[mi * (mi + 1) / 2 + ni][1];
-      dst[0] = (uint16_t)w0; dst[136] = (uint16_t)(w0 >> 16); dst[272] = (uint16_t)w1; dst[408] = (uint16_t)(w1 >> 16);
-    }
-  __syncthreads();
-  uint16_t* const Pt = p.P + ((int64_t)cb * p.HV + hv) * 4096;
-  const int c8 = 8 * (lane & 7);
-#pragma unroll
-  for (int pass = 0; pass < 8; ++pass) {
-    const int i = 8 * pass + (lane >> 3);
-    uint4 w = *reinterpret_cast<const uint4*>(Ps + i * 136 + c8);
-    uint32_t* we = reinterpret_cast<uint32_t*>(&w);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (c8 + 2 * e > i) we[e] = 0u;
-      else if (c8 + 2 * e + 1 > i) we[e] &= 0xffffu;
-    }
-    *reinterpret_cast<uint4*>(Pt + i * 64 + c8) = w;
+// q and k rows that start on 4-byte boundaries only (a packed view shifted inside its buffer) are copied into dense
+// [T, H, 128] buffers first, which the kernels below read in 16-byte pieces: one piece per thread and trip.
+static __global__ __launch_bounds__(256) void gdn_align_rows_kernel(const uint16_t* q, const uint16_t* k, int64_t stride_q,
+                                                                    int64_t stride_k, int T, int H, uint16_t* q_out,
+                                                                    uint16_t* k_out) {
+  const int64_t pieces = (int64_t)T * H * 16;                  // 16-byte pieces per tensor
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < 2 * pieces; i += (int64_t)gridDim.x * 256) {
+    const bool keys = i >= pieces;
+    const int64_t j = keys ? i - pieces : i;
+    const int64_t t = j / (H * 16);
+    const int c = (int)(j - t * (H * 16));                     // piece c of token t
+    const uint32_t* src = reinterpret_cast<const uint32_t*>((keys ? k : q) + t * (keys ? stride_k : stride_q) + 8 * c);
+    *reinterpret_cast<uint4*>((keys ? k_out : q_out) + 8 * j) = make_uint4(src[0], src[1], src[2], src[3]);
   }
 }
 
@@ -327,12 +103,16 @@ __device__ __forceinline__ uint32_t from_other_half(uint32_t x) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Preparation for the fused sweep (gdn_fused_sweep_kernel), which normalises q and k and forms P itself: only what
-// needs the triangular solve leaves this kernel.  One wavefront per (chunk, value head) as above, the key side only:
-// gate, beta and their cumulative sum (g_cum and beta as the call returns them, the chunk's tile of decay factors
-// with the raw cumulative log-decay appended for the sweep's P), normalised K in registers, K K^T on MFMA, the
+// Preparation of a chunk: what does not depend on the state and needs the triangular solve.  The sweep
+// (gdn_fused_sweep_kernel) normalises q and k and forms P itself, so only the key side is here.  One wavefront per
+// (chunk, value head); the WAVES wavefronts of a workgroup take consecutive value heads of one q/k head:
+// gate, beta and their cumulative sum (lane j = token j: g_j = -exp(A_log) softplus(a_j + dt_bias), beta_j =
+// sigmoid(b_j), or the caller's g / beta; a scan over the lanes; g_cum and beta as the call returns them, the chunk's
+// tile of decay factors with the raw cumulative log-decay appended for the sweep's P), normalised K in registers (rows
+// loaded directly in MFMA operand layout, L2-normalised, rounded to the activation dtype - the reference's operand -
+// and held as fp16, which represents those values exactly), K K^T on MFMA, the
 // inverse of I + L by 16 x 16 blocks, and W = (I + L)^-1 diag(beta) as an fp16 hi + lo pair in the six-block
-// operand layout (12 KiB per (chunk, value head) instead of 16 KiB row-major + 8 KiB of P + the normalised rows).
+// operand layout (12 KiB per (chunk, value head)).
 // The blocks of L below the diagonal never leave the registers: the accumulators of K K^T are the operands of the
 // transposed block recursion as they stand, and its results are the lane's pieces of the W blocks.  The wavefronts
 // of a workgroup (the value heads of one q/k head) share the loading and normalising of the keys through LDS: a
@@ -636,357 +416,6 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
 }
 
 // ---------------------------------------------------------------------------------------------
-// Sequential kernel with output behind gdn_prepare_kernel (whole sequences, and the second sweep over segments): one
-// workgroup per (sequence or segment, value head) of FIVE wavefronts.  Wavefronts 0-3 compute, each on its own 32 V columns, and touch
-// memory only to store their output rows; wavefront 4 moves data: it issues every global -> LDS copy of the
-// workgroup (an LDS copy instruction occupies its issuer for tens of cycles, about 2 k cycles per chunk in all,
-// which the computing wavefronts no longer pay).  Every tile is double buffered by chunk parity, so there is
-// ONE barrier per chunk: at the barrier that opens chunk c the tiles of c have landed (the copying wavefront
-// waited for them) and the buffers of chunk c - 1 are free, so it fills them with chunk c + 1 while the others
-// compute chunk c.  Per chunk and computing wavefront, nothing crossing wavefronts:
-//     KS = K S^T,  X = V - e^G (.) KS,  U = W X                  (W as an fp16 hi + lo pair)
-//     O^T = scale e^G (.) (S Q^T) + U^T P^T  -> rows of o         (the output product is formed transposed: a lane
-//                                                                  then holds four adjacent V columns of one token
-//                                                                  and stores them as 8 bytes, no LDS tile)
-//     S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)          (U as an fp16 hi + lo pair)
-// The query product is formed after U, so its accumulators and those of K S^T never live together and a
-// computing wavefront stays within 256 registers (five wavefronts put two on one SIMD).
-template <typename act_t, int NB>
-__global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const GdnPrefillParams p) {
-  constexpr int CW = 8 / NB;                                  // computing wavefronts, NB 16-column blocks of V each
-  using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, 1>;      // 64 x 128 tile, all pieces issued by one wavefront
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 1>;     // 64 x 64 tile
-  // whole sequences: the value heads of a q/k head run on one XCD, so that K and Q reach its L2 once
-  const int block = p.pass == 0 ? xcd_grouped_index(blockIdx.x, p.HV / p.H, p.N * p.HV) : (int)blockIdx.x;
-  if (block < 0) return;
-  const SweepRole role = select_sweep(p.pass, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, block);
-  if (!role.active) return;
-  const int n = role.n, hv = role.head, c_begin = role.c_begin, c_end = role.c_end;
-  const int h = hv / (p.HV / p.H);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int r16 = lane & 15, kb = lane >> 4;
-  const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
-  const int seq_len = min(p.cu_seqlens[n + 1] - seq_start, (c_end - c_begin) * CHUNK);
-  const int n_chunks = c_end - c_begin;
-  auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
-
-  __shared__ __align__(16) uint16_t tK[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tQ[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tV[2][CHUNK * PITCH128];
-  __shared__ __align__(16) uint16_t tW[2][2][CHUNK * PITCH64];     // [parity][hi, lo]
-  __shared__ __align__(16) uint16_t tP[2][CHUNK * PITCH64];
-  // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
-  __shared__ __align__(16) float tG[2][256];
-
-  if (wave == CW) {
-    // ---- the copying wavefront -------------------------------------------------------------
-    const int64_t tok_pitch_b = (int64_t)p.H * 256;            // bytes between tokens of kn / qn
-    const char* const kn_b = reinterpret_cast<const char*>(p.kn) + ((int64_t)seq_start * p.H + h) * 256;
-    const char* const qn_b = reinterpret_cast<const char*>(p.qn) + ((int64_t)seq_start * p.H + h) * 256;
-    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
-    const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * 16384;
-    const char* const pp_b = reinterpret_cast<const char*>(p.P) + ((int64_t)c_begin * p.HV + hv) * 8192;
-    const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * 1024;
-    CopyWide plan_kq, plan_v;
-    CopyNarrow plan_w;
-    plan_kq.plan((uint32_t)tok_pitch_b, CHUNK - 1, 0, lane);
-    plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, 0, lane);
-    plan_w.plan(128, CHUNK - 1, 0, lane);
-    auto issue = [&](int c) {
-      const int par = c & 1;
-      const char* ks = kn_b + (int64_t)c * CHUNK * tok_pitch_b;
-      const char* qs = qn_b + (int64_t)c * CHUNK * tok_pitch_b;
-      const char* vs = v_b + (int64_t)c * CHUNK * p.stride_v * 2;
-      const int len = chunk_len(c);
-      dma16(gt_b + (int64_t)c * p.HV * 1024, 16u * lane, lds_address(&tG[par][0]));
-      if (len == CHUNK) {
-        plan_kq.issue(tK[par], ks, 0);
-        plan_v.issue(tV[par], vs, 0);
-      } else {                                       // rows past the sequence end re-read its last row
-        CopyWide tail;
-        tail.plan((uint32_t)tok_pitch_b, len - 1, 0, lane);
-        tail.issue(tK[par], ks, 0);
-        tail.issue(tQ[par], qs, 0);
-        tail.plan((uint32_t)(p.stride_v * 2), len - 1, 0, lane);
-        tail.issue(tV[par], vs, 0);
-      }
-      plan_w.issue(tW[par][0], w_b + (int64_t)c * p.HV * 16384, 0);
-      plan_w.issue(tW[par][1], w_b + (int64_t)c * p.HV * 16384 + 8192, 0);
-      if (len == CHUNK) plan_kq.issue(tQ[par], qs, 0);
-      plan_w.issue(tP[par], pp_b + (int64_t)c * p.HV * 8192, 0);
-    };
-    if (n_chunks > 0) issue(0);
-    for (int ci = 0; ci < n_chunks; ++ci) {
-      wait_vmcnt<0>();                               // chunk ci has landed
-      __syncthreads();                               // ... and chunk ci - 1 is finished: its buffers are free
-      if (ci + 1 < n_chunks) issue(ci + 1);
-    }
-    return;
-  }
-
-  // ---- the computing wavefronts ------------------------------------------------------------
-  const int vbase = 16 * NB * wave;                  // this wavefront's V columns: vbase .. vbase + 16 NB - 1
-  const int vcol = vbase + r16;                      // state / KS / U layout: the lane's column (second block: + 16)
-  // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
-  f32x4_t St[NB][8];
-#pragma unroll
-  for (int nb = 0; nb < NB; ++nb)
-    if (role.init != nullptr) {
-      const float* src = role.init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) {
-        const float4 t4 = *reinterpret_cast<const float4*>(src + 16 * mc);
-        St[nb][mc] = f32x4_t{t4.x, t4.y, t4.z, t4.w};
-      }
-    } else {
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) St[nb][mc] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
-  if (role.keep_init != nullptr) {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float* dst = role.keep_init + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
-    }
-  }
-  // output rows: in the transposed product a lane holds V columns vbase + 16 nb + 4 kb .. + 3 of token 16 ni + r16
-  uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.HV + hv) * 128 + vbase + 4 * kb;
-  const bool write_o = role.write_o;
-
-  // Software pipeline of a chunk: the LDS operands of a product are requested one contraction step ahead, and the
-  // first operands of the next product under the last MFMAs of the current one.  The scheduling fences below pin
-  // memory operations only: arithmetic may move across them freely.
-  for (int ci = 0; ci < n_chunks; ++ci) {
-    const int par = ci & 1;
-    // A bare barrier: the tiles were written by the copying wavefront's LDS copies, which it waited for before it
-    // arrived, and this wavefront's own LDS reads of the previous chunk are complete (their MFMAs have issued).  A
-    // full workgroup fence would also wait for this wavefront's output stores, which nobody in the workgroup reads.
-    __builtin_amdgcn_s_waitcnt(0xc07f);              // lgkmcnt(0) only
-    __builtin_amdgcn_s_barrier();
-    const uint16_t* const K = tK[par];
-    const uint16_t* const Q = tQ[par];
-    const uint16_t* const V = tV[par];
-    const float* const G = tG[par];
-
-    // ---- KS = K S^T ----
-    f32x4_t KS[NB][4];
-    bf16x8_t wa[2][4], wl[2][4];
-    float4 eg[4];
-    uint2 vraw[NB][4];        // rows 16 mi + 4 kb .. + 3 of the lane's V column, one transposing read each
-    {
-      bf16x8_t ka[2][4], sb[2][NB];
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) ka[0][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], 0, kb);
-      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        if (s < 3) {
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) ka[(s + 1) & 1][mi] = operand_from(&K[(16 * mi + r16) * PITCH128], s + 1, kb);
-        } else {
-          // under the last step: V, e^G and the first half of W
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            eg[mi] = *reinterpret_cast<const float4*>(&G[64 + 16 * mi + 4 * kb]);
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              vraw[nb][mi] = read_tr4(&V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)]);
-            }
-          }
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) {
-            wa[0][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 0, kb);
-            wl[0][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 0, kb);
-          }
-        }
-        __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-        if (s < 3) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) KS[nb][mi] = mfma16h(ka[s & 1][mi], sb[s & 1][nb], KS[nb][mi]);
-      }
-    }
-    // ---- X = V - e^G (.) KS,  U = W X ----
-    f32x4_t U[NB][4];
-    bf16x8_t qa[2][4];
-    {
-#pragma unroll
-      for (int mi = 0; mi < 4; ++mi) {
-        wa[1][mi] = operand_from(&tW[par][0][(16 * mi + r16) * PITCH64], 1, kb);
-        wl[1][mi] = operand_from(&tW[par][1][(16 * mi + r16) * PITCH64], 1, kb);
-      }
-      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-      f32x4_t X[NB][4];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) {
-          X[nb][mi][0] = lo16<act_t>(vraw[nb][mi].x) - eg[mi].x * KS[nb][mi][0];
-          X[nb][mi][1] = hi16<act_t>(vraw[nb][mi].x) - eg[mi].y * KS[nb][mi][1];
-          X[nb][mi][2] = lo16<act_t>(vraw[nb][mi].y) - eg[mi].z * KS[nb][mi][2];
-          X[nb][mi][3] = hi16<act_t>(vraw[nb][mi].y) - eg[mi].w * KS[nb][mi][3];
-        }
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mi = 0; mi < 4; ++mi) U[nb][mi] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        bf16x8_t xb[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) xb[nb] = half8_sat(X[nb][2 * s], X[nb][2 * s + 1]);
-        if (s == 1) {
-          // under the last step: the first query operands
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) qa[0][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], 0, kb);
-          __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mi = 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
-      }
-    }
-    // ---- O^T = scale e^G (.) (S Q^T) + U^T P^T -> o ----
-    bf16x8_t kt[2][8];
-    float4 dg[2][2];
-    float egl;
-    {
-      f32x4_t OT[NB][4];                             // OT[nb][ni][r] = o[token 16 ni + r16][v = vbase + 16 nb + 4 kb + r]
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      bf16x8_t sb[2][NB], pa[2][4];
-      float sq[4];
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) sb[0][nb] = half8_rtz(St[nb][0], St[nb][1]);
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        if (s < 3) {
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) qa[(s + 1) & 1][ni] = operand_from(&Q[(16 * ni + r16) * PITCH128], s + 1, kb);
-        } else {
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2)
-#pragma unroll
-            for (int ni = 0; ni < 4; ++ni) pa[s2][ni] = operand_from(&tP[par][(16 * ni + r16) * PITCH64], s2, kb);
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) sq[ni] = G[16 * ni + r16];
-        }
-        __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-        if (s < 3) {
-#pragma unroll
-          for (int nb = 0; nb < NB; ++nb) sb[(s + 1) & 1][nb] = half8_rtz(St[nb][2 * s + 2], St[nb][2 * s + 3]);
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(sb[s & 1][nb], qa[s & 1][ni], OT[nb][ni]);
-      }
-#pragma unroll
-      for (int ni = 0; ni < 4; ++ni)
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) OT[nb][ni] *= sq[ni];
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        bf16x8_t ur[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) ur[nb] = half8_rtz(U[nb][2 * s], U[nb][2 * s + 1]);
-        if (s == 1) {
-          // under the last step: the transposed key operands and the decay factors of the state update
-#pragma unroll
-          for (int mc = 0; mc < 8; ++mc) kt[0][mc] = operand_transposed(K, 0, mc, kb, r16);
-#pragma unroll
-          for (int s2 = 0; s2 < 2; ++s2) {
-            dg[s2][0] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 4 * kb]);
-            dg[s2][1] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 16 + 4 * kb]);
-          }
-          egl = G[192];
-          __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int ni = 0; ni < 4; ++ni) OT[nb][ni] = mfma16h(ur[nb], pa[s][ni], OT[nb][ni]);
-      }
-      if (write_o) {
-        const int len = chunk_len(ci);
-        uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.HV * 128;
-#pragma unroll
-        for (int ni = 0; ni < 4; ++ni)
-          if (16 * ni + r16 < len) {
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-              const uint2 packed = make_uint2(pack2<act_t>(OT[nb][ni][0], OT[nb][ni][1]), pack2<act_t>(OT[nb][ni][2], OT[nb][ni][3]));
-              *reinterpret_cast<uint2*>(dst + (int64_t)16 * ni * p.HV * 128 + 16 * nb) = packed;
-            }
-          }
-      }
-    }
-    // ---- S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U) ----
-    {
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc) kt[1][mc] = operand_transposed(K, 1, mc, kb, r16);
-      __builtin_amdgcn_sched_barrier(0x000F);      // LDS requests stay above this line; ALU and MFMA work may cross it
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-        for (int mc = 0; mc < 8; ++mc) St[nb][mc] *= egl;
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        HalfPair ub[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          const f32x4_t u0 = {U[nb][2 * s][0] * dg[s][0].x, U[nb][2 * s][1] * dg[s][0].y, U[nb][2 * s][2] * dg[s][0].z,
-                              U[nb][2 * s][3] * dg[s][0].w};
-          const f32x4_t u1 = {U[nb][2 * s + 1][0] * dg[s][1].x, U[nb][2 * s + 1][1] * dg[s][1].y,
-                              U[nb][2 * s + 1][2] * dg[s][1].z, U[nb][2 * s + 1][3] * dg[s][1].w};
-          ub[nb] = half8_pair(u0, u1);
-        }
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].lo, St[nb][mc]);
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-          for (int mc = 0; mc < 8; ++mc) St[nb][mc] = mfma16h(kt[s][mc], ub[nb].hi, St[nb][mc]);
-      }
-    }
-  }
-
-  if (role.fin != nullptr) {
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-      float* dst = role.fin + (int64_t)(vcol + 16 * nb) * 128 + 4 * kb;
-#pragma unroll
-      for (int mc = 0; mc < 8; ++mc)
-        *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
-    }
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
 // First sweep over segments, both roles in one workgroup.  A later segment is swept twice without output - from a
 // zero state (its B summary) and from the identity with v = 0 (its transition matrix M) - and both sweeps multiply
 // the same K and W tiles.  One workgroup of eight wavefronts per (segment, value head) runs them side by side:
@@ -994,18 +423,18 @@ __global__ __launch_bounds__(64 * (8 / NB + 1), 1) void gdn_sweep_kernel(const G
 // also issue every global -> LDS copy, so each tile crosses memory and LDS once for the two sweeps and two
 // wavefronts share a SIMD.  A first segment has no M role: its wavefronts 4-7 only copy, wavefronts 0-3 sweep it
 // from its real start state (of which they keep a copy for the second sweep).  All tiles are double buffered by
-// chunk parity (90 KB of LDS with the swizzled tiles, 109 KB with padded ones) and there is one barrier per chunk, as in
-// gdn_sweep_kernel.
-template <typename act_t, bool SIX>
+// chunk parity (90 KB of LDS: K and V in swizzled unpadded tiles, 134 us -> 124 us per sweep of 32 chunks against rows
+// padded to 272 bytes) and there is one barrier per chunk: at the barrier that opens chunk c its tiles have landed (every
+// wavefront waited for its own copies) and the buffers of chunk c - 1 are free for the copies of chunk c + 1.
+template <typename act_t>
 __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefillParams p) {
   constexpr int NB = 2;
-  // what gdn_wsolve_kernel (SIX) or gdn_prepare_kernel left per (chunk, value head): W and the tile of decay factors
-  constexpr int W_BYTES = SIX ? 2 * TRI_BLOCKS * 1024 : 16384, G_BYTES = SIX ? GTILE_FLOATS * 4 : 1024;
-  // K and V tiles, filled by the four copying wavefronts: swizzled and unpadded (SIX: the K rows come in the column
-  // order of an operand tile) or padded rows
-  using CopyWide = std::conditional_t<SIX, SwizzledTileCopy<4>, TileCopy<CHUNK, 2 * PITCH128, 256, 4>>;
-  using CopyNarrow = TileCopy<CHUNK, 2 * PITCH64, 128, 4>;     // 64 x 64 tile
-  constexpr int KV_HALVES = SIX ? TILE128_HALVES : CHUNK * PITCH128;
+  // what gdn_wsolve_kernel left per (chunk, value head): W (six blocks hi, six lo) and the tile of decay factors
+  constexpr int W_BYTES = 2 * TRI_BLOCKS * 1024, G_BYTES = GTILE_FLOATS * 4;
+  // K and V tiles, filled by the four copying wavefronts: swizzled and unpadded (the K rows come in the column order
+  // of an operand tile, V with its columns in order)
+  using CopyWide = SwizzledTileCopy<4>;
+  constexpr int KV_HALVES = TILE128_HALVES;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1031,9 +460,8 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 
   __shared__ __align__(1024) uint16_t tK[2][KV_HALVES];
   __shared__ __align__(1024) uint16_t tV[2][KV_HALVES];
-  // W [parity]: the six-block operand layout (hi blocks, then lo blocks; SIX) or two padded row-major tiles (hi, lo)
-  constexpr int W_HI_LO = SIX ? TRI_BLOCKS * 512 : CHUNK * PITCH64;
-  __shared__ __align__(16) uint16_t tW[2][2 * W_HI_LO];
+  // W [parity]: the six-block operand layout (hi blocks, then lo blocks)
+  __shared__ __align__(16) uint16_t tW[2][2 * TRI_BLOCKS * 512];
   // decay factors: [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}
   __shared__ __align__(16) float tG[2][256];
 
@@ -1066,15 +494,9 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   // vcol + 16 nb, by one transposing read: lane t of a group of 16 addresses columns 32 cw + 16 nb + 4 (t % 4) .. + 3 of
   // row 16 mi + 4 kb + t / 4, which in a swizzled tile is half (t % 2) of granule 4 cw + 2 nb + (t % 4) / 2; the
   // swizzle 8 (kb & 1) + 2 (t / 4) of that row does not depend on mi, and nb = 1 differs in one bit of the granule index.
-  auto k_operand = [&](const uint16_t* K, int mi, int s) {
-    if constexpr (SIX) return operand_granule(K, 16 * mi + r16, s, kb);
-    else return operand_from(&K[(16 * mi + r16) * PITCH128], s, kb);
-  };
+  auto k_operand = [&](const uint16_t* K, int mi, int s) { return operand_granule(K, 16 * mi + r16, s, kb); };
   const int trV = (4 * kb + (r16 >> 2)) * 128 + 8 * ((4 * cw + ((r16 & 3) >> 1)) ^ (8 * (kb & 1) + 2 * (r16 >> 2))) + 4 * (r16 & 1);
-  auto v_at = [&](const uint16_t* V, int mi, int nb) {
-    if constexpr (SIX) return V + ((trV + 16 * 128 * mi) ^ (16 * nb));
-    else return &V[(16 * mi + 4 * kb + (r16 >> 2)) * PITCH128 + (vcol - r16) + 16 * nb + 4 * (r16 & 3)];
-  };
+  auto v_at = [&](const uint16_t* V, int mi, int nb) { return V + ((trV + 16 * 128 * mi) ^ (16 * nb)); };
 
   // ---- copies (wavefronts 4-7) ----
   const int64_t tok_pitch_b = (int64_t)p.H * 256;              // bytes between tokens of kn
@@ -1083,7 +505,6 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * W_BYTES;
   const char* const gt_b = reinterpret_cast<const char*>(p.gtile) + ((int64_t)c_begin * p.HV + hv) * G_BYTES;
   CopyWide plan_k, plan_v;
-  CopyNarrow plan_w;
   if (m_side) {
     plan_k.plan((uint32_t)tok_pitch_b, CHUNK - 1, cw, lane);
     plan_v.plan((uint32_t)(p.stride_v * 2), CHUNK - 1, cw, lane);
@@ -1094,15 +515,9 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   auto issue_w = [&](int c) {
     const int par = c & 1;
     const char* const ws = w_b + (int64_t)c * p.HV * W_BYTES;
-    if constexpr (SIX) {                             // twelve 1 KiB blocks, three per wavefront, as they lie in memory
 #pragma unroll
-      for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)
-        dma16(ws, 1024u * (4 * j + cw) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (4 * j + cw));
-    } else {
-      plan_w.plan(128, CHUNK - 1, cw, lane);         // worked out here: nothing is kept across the phases
-      plan_w.issue(&tW[par][0], ws, cw);
-      plan_w.issue(&tW[par][W_HI_LO], ws + 8192, cw);
-    }
+    for (int j = 0; j < 2 * TRI_BLOCKS / 4; ++j)     // twelve 1 KiB blocks, three per wavefront, as they lie in memory
+      dma16(ws, 1024u * (4 * j + cw) + 16u * lane, lds_address(&tW[par][0]) + 1024u * (4 * j + cw));
   };
   auto issue = [&](int c) {
     const int par = c & 1;
@@ -1190,16 +605,12 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
       for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
         for (int mi = 0; mi < 4; ++mi) {
-          if constexpr (SIX) {
-            // block (row block mi, contraction half s2) of the lower triangle: 0-3 for s2 = 0, 4 and 5 (mi 2, 3) for s2 = 1
-            if (s2 == 1 && mi < 2) continue;
-            const int b = s2 == 0 ? mi : mi + 2;
-            wa[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][b * 512 + lane * 8]));
-            wl[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][(TRI_BLOCKS + b) * 512 + lane * 8]));
-          } else {
-            wa[s2][mi] = operand_from(&tW[par][(16 * mi + r16) * PITCH64], s2, kb);
-            wl[s2][mi] = operand_from(&tW[par][W_HI_LO + (16 * mi + r16) * PITCH64], s2, kb);
-          }
+          // block (row block mi, contraction half s2) of the lower triangle: 0-3 for s2 = 0, 4 and 5 (mi 2, 3) for s2 = 1;
+          // the two blocks above the diagonal (s2 = 1, mi < 2) are zero and cost neither a read nor an MFMA
+          if (s2 == 1 && mi < 2) continue;
+          const int b = s2 == 0 ? mi : mi + 2;
+          wa[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][b * 512 + lane * 8]));
+          wl[s2][mi] = __builtin_bit_cast(bf16x8_t, *reinterpret_cast<const uint4*>(&tW[par][(TRI_BLOCKS + b) * 512 + lane * 8]));
         }
       __builtin_amdgcn_sched_barrier(0x000F);
       f32x4_t X[NB][4];
@@ -1224,11 +635,11 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = (SIX && s == 1) ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
+          for (int mi = s == 1 ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wl[s][mi], xb[nb], U[nb][mi]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int mi = (SIX && s == 1) ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
+          for (int mi = s == 1 ? 2 : 0; mi < 4; ++mi) U[nb][mi] = mfma16h(wa[s][mi], xb[nb], U[nb][mi]);
       }
     }
     if (!m_side && ci + 1 < n_chunks) issue_w(ci + 1);
@@ -1237,7 +648,7 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 #pragma unroll
       for (int s2 = 0; s2 < 2; ++s2) {
 #pragma unroll
-        for (int mc = 0; mc < 8; ++mc) kt[s2][mc] = SIX ? operand_granule_transposed(K, s2, mc, kb, r16) : operand_transposed(K, s2, mc, kb, r16);
+        for (int mc = 0; mc < 8; ++mc) kt[s2][mc] = operand_granule_transposed(K, s2, mc, kb, r16);
         dg[s2][0] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 4 * kb]);
         dg[s2][1] = *reinterpret_cast<const float4*>(&G[128 + 32 * s2 + 16 + 4 * kb]);
       }
@@ -1282,10 +693,16 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused sweep, over whole sequences or as the second sweep over segments (pass 2: one 16 384-token sequence of 32
-// value heads 0.46 -> 0.36 ms against gdn_prepare_kernel / gdn_sweep_kernel there): one workgroup of EIGHT wavefronts
-// per (sequence or segment, value head).  Wavefronts 0-3
-// compute as in gdn_sweep_kernel (32 V columns of S^T each, the chain K S^T -> X -> U -> S^T in registers).
+// Fused sweep, over whole sequences or as the second sweep over segments (pass 2): one workgroup of EIGHT wavefronts
+// per (sequence or segment, value head).  Per chunk:
+//     KS = K S^T,  X = V - e^G (.) KS,  U = W X                  (W as an fp16 hi + lo pair)
+//     O^T = scale e^G (.) (S Q^T) + U^T P^T  -> rows of o         (the output product is formed transposed: a lane
+//                                                                  then holds four adjacent V columns of one token
+//                                                                  and stores them as 8 bytes, no LDS tile)
+//     S^T = e^{G_last} S^T + K^T (e^{G_last - G} (.) U)          (U as an fp16 hi + lo pair)
+// Wavefronts 0-3 compute, each on its own 32 V columns of S^T, nothing crossing wavefronts (the chain K S^T -> X -> U
+// -> S^T stays in registers; the query product is formed after U, so its accumulators and those of K S^T never live
+// together).
 // Wavefronts 4-7 feed them, so that neither the normalised rows nor P cross memory:
 //   rows   wavefronts 4, 5 take the raw K rows of the next chunk (32 rows each), 6, 7 the raw Q rows: loaded one
 //          chunk ahead into registers (16 lanes per row, 16 bytes per lane).  K rows are scaled by the row's 1 / |k|
@@ -1877,11 +1294,8 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 }
 #undef SB
 
-// 16-column V blocks per computing wavefront of gdn_sweep_kernel: 2 = four computing wavefronts (one per SIMD); 1 =
-// eight (two per SIMD, twice the LDS operand traffic) measures the same on config 3 (0.767 against 0.765 ms)
-constexpr int SWEEP_NB = 2;
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, qn, kn, kinv, gcum, beta, gtile, W, P;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, q_rows, k_rows, kn, kinv, gcum, beta, gtile, W;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -1895,14 +1309,14 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_sta
   L.chunk_seq = take((size_t)L.NC_max * 4);
   L.chunk_tok = take((size_t)L.NC_max * 4);
   L.chunk_len = take((size_t)L.NC_max * 4);
-  L.qn = take((size_t)T * H * 128 * 2);
+  L.q_rows = take((size_t)T * H * 128 * 2);              // aligned copies of q and k rows that are not
+  L.k_rows = take((size_t)T * H * 128 * 2);
   L.kn = take((size_t)T * H * 128 * 2);
   L.kinv = take((size_t)T * H * 4);
   L.gcum = take((size_t)T * HV * 4);
   L.beta = take((size_t)T * HV * 4);
   L.gtile = take((size_t)L.NC_max * HV * GTILE_FLOATS * 4);
-  L.W = take((size_t)L.NC_max * HV * 8192 * 2);
-  L.P = take((size_t)L.NC_max * HV * 4096 * 2);
+  L.W = take((size_t)L.NC_max * HV * 2 * TRI_BLOCKS * 1024);
   L.seg_chunks = pick_segment_chunks(T, N, HV);
   L.max_segments = max_segments(T, N, L.seg_chunks);
   if (L.seg_chunks > 0) {
@@ -2013,24 +1427,29 @@ static int gdn_prefill_run(
   p.chunk_seq = reinterpret_cast<int32_t*>(ws + L.chunk_seq);
   p.chunk_tok = reinterpret_cast<int32_t*>(ws + L.chunk_tok);
   p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
-  p.qn = reinterpret_cast<uint16_t*>(ws + L.qn);
   p.kn = reinterpret_cast<uint16_t*>(ws + L.kn);
   p.kinv = reinterpret_cast<float*>(ws + L.kinv);
   p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
   p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
   p.gtile = reinterpret_cast<float*>(ws + L.gtile);
   p.W = reinterpret_cast<uint16_t*>(ws + L.W);
-  p.P = reinterpret_cast<uint16_t*>(ws + L.P);
   p.H = H; p.HV = HV; p.NC_max = L.NC_max;
-  p.qk_rows_16 = (uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && stride_q % 8 == 0 && stride_k % 8 == 0;
 
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   const bool segmented = L.seg_chunks > 0;
-  // 16-byte aligned q / k rows take the fused sweep (rows normalised and P formed inside it) after the lean preparation;
-  // for a call split into segments that is the second sweep, and the first one copies the normalised K rows the
-  // preparation then stores as well
-  const bool fused = p.qk_rows_16;
-  p.store_kn = segmented && fused;
+  // the kernels read q and k rows in 16-byte pieces: rows that start on 4-byte boundaries only are copied first
+  if (!((uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && stride_q % 8 == 0 && stride_k % 8 == 0)) {
+    uint16_t* const q_rows = reinterpret_cast<uint16_t*>(ws + L.q_rows);
+    uint16_t* const k_rows = reinterpret_cast<uint16_t*>(ws + L.k_rows);
+    const int64_t threads = (int64_t)T * H * 32;
+    hipLaunchKernelGGL(gdn_align_rows_kernel, dim3((unsigned)std::min<int64_t>((threads + 255) / 256, 8192)), dim3(256), 0, s,
+                       reinterpret_cast<const uint16_t*>(q), reinterpret_cast<const uint16_t*>(k), stride_q, stride_k, T, H,
+                       q_rows, k_rows);
+    p.q = q_rows; p.k = k_rows;
+    p.stride_q = p.stride_k = (int64_t)H * 128;
+  }
+  // a call split into segments: the preparation also stores the normalised K rows, which the first sweep copies
+  p.store_kn = segmented;
   if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
@@ -2068,10 +1487,10 @@ static int gdn_prefill_run(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = stages;
   }
-  // 16-byte aligned rows and at most 64 sequences: no table kernel runs ahead of the preparation, whose first launch
-  // also zeroes the padded rows of o.  Whole sequences: every kernel works its chunks out by itself.  Segments: the
+  // At most 64 sequences: no table kernel runs ahead of the preparation, whose first launch also zeroes the padded
+  // rows of o.  Whole sequences: every kernel works its chunks out by itself.  Segments: the
   // preparation does, and one workgroup appended to it writes the chunk and segment tables for the sweeps.
-  p.inline_tables = fused && N <= INLINE_TABLE_SEQUENCES;
+  p.inline_tables = N <= INLINE_TABLE_SEQUENCES;
   if (!p.inline_tables)
     launch_tables(s, cu_seqlens, N, T, L.NC_max, p.seq_chunk_off, p.chunk_seq, p.chunk_tok, p.chunk_len, p.seg, p.stg,
                   segmented ? L.max_segments : N, o, HV);
@@ -2082,52 +1501,33 @@ static int gdn_prefill_run(
         const int waves = ratio % 4 == 0 ? 4 : ratio % 2 == 0 ? 2 : 1;
         p.tail_blocks = (p.inline_tables && p.stage == 0) ? TABLE_WORKGROUPS - (segmented ? 0 : 1) : 0;
         const dim3 grid((unsigned)L.NC_max * (HV / waves) + p.tail_blocks), block(64 * waves);
-        if (fused) {
-          if (half_act) {
-            if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 4>), grid, block, 0, ps, p);
-            else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 2>), grid, block, 0, ps, p);
-            else hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 1>), grid, block, 0, ps, p);
-          } else {
-            if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 4>), grid, block, 0, ps, p);
-            else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 2>), grid, block, 0, ps, p);
-            else hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 1>), grid, block, 0, ps, p);
-          }
-        } else if (half_act) {
-          if (waves == 4) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 4>), grid, block, 0, ps, p);
-          else if (waves == 2) hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 2>), grid, block, 0, ps, p);
-          else hipLaunchKernelGGL((gdn_prepare_kernel<f16_t, 1>), grid, block, 0, ps, p);
+        if (half_act) {
+          if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 4>), grid, block, 0, ps, p);
+          else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 2>), grid, block, 0, ps, p);
+          else hipLaunchKernelGGL((gdn_wsolve_kernel<f16_t, 1>), grid, block, 0, ps, p);
         } else {
-          if (waves == 4) hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 4>), grid, block, 0, ps, p);
-          else if (waves == 2) hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 2>), grid, block, 0, ps, p);
-          else hipLaunchKernelGGL((gdn_prepare_kernel<bf16_t, 1>), grid, block, 0, ps, p);
+          if (waves == 4) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 4>), grid, block, 0, ps, p);
+          else if (waves == 2) hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 2>), grid, block, 0, ps, p);
+          else hipLaunchKernelGGL((gdn_wsolve_kernel<bf16_t, 1>), grid, block, 0, ps, p);
         }
       },
       [&](unsigned grid) {
         if (p.pass == 1) {        // first sweep over segments: no output, both roles in one workgroup per (segment, head)
-          if (fused) {
-            if (half_act) hipLaunchKernelGGL((gdn_lean_sweep_kernel<f16_t, true>), dim3(grid / 2), dim3(512), 0, s, p);
-            else hipLaunchKernelGGL((gdn_lean_sweep_kernel<bf16_t, true>), dim3(grid / 2), dim3(512), 0, s, p);
-          } else if (half_act) hipLaunchKernelGGL((gdn_lean_sweep_kernel<f16_t, false>), dim3(grid / 2), dim3(512), 0, s, p);
-          else hipLaunchKernelGGL((gdn_lean_sweep_kernel<bf16_t, false>), dim3(grid / 2), dim3(512), 0, s, p);
+          if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(grid / 2), dim3(512), 0, s, p);
+          else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
         } else {
           const unsigned g = xcd_grouped_grid(grid, (unsigned)(HV / H));
-          if (fused) {
-            if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
-            else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
-          } else if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
-          else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3(g), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+          if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+          else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
         }
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV);
     p.pass = 2;
-    if (fused) {
-      const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));
-      if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
-      else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
-    } else if (half_act) hipLaunchKernelGGL((gdn_sweep_kernel<f16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
-    else hipLaunchKernelGGL((gdn_sweep_kernel<bf16_t, SWEEP_NB>), dim3((unsigned)L.max_segments * HV), dim3(64 * (8 / SWEEP_NB + 1)), 0, s, p);
+    const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));
+    if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+    else hipLaunchKernelGGL(gdn_fused_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
   }
   return check_launch("gdn prefill launch");
 }

@@ -122,8 +122,8 @@ def chunk_gated_delta_rule_fwd(
     for name, t in (("q", q), ("k", k), ("v", v)):
         if t.stride(3) != 1 or t.stride(2) != 128:
             raise ValueError(f"{name} head/feature axes must be contiguous")
-    # q / k rows are read in 4-byte words, v rows are copied to LDS in 16-byte pieces:
-    # a view that breaks those alignments is materialised once
+    # q / k rows must start on 4-byte boundaries (the library copies rows that are not 16-byte aligned itself), v rows
+    # are copied to LDS in 16-byte pieces: a view that breaks those alignments is materialised once
     if q.data_ptr() % 4 or q.stride(1) % 2:
         q = q.contiguous()
     if k.data_ptr() % 4 or k.stride(1) % 2:
