@@ -366,7 +366,7 @@ int pla_gdn_prefill_launch_raw(
  * (PLA_GDN_PREFILL_STATIC_BYTES, held until the process ends); the call allocates nothing, creates no
  * stream or event, and runs every kernel on `stream`.  Accepted: every shape whose
  * pla_gdn_prefill_workspace_bytes(T, N, H, HV) is within PLA_GDN_PREFILL_STATIC_BYTES (about 2 000 to
- * 2 900 tokens at H = 16, HV = 32, depending on the number of sequences); larger calls are rejected before any launch.  All calls on one GPU share that
+ * 3 300 tokens at H = 16, HV = 32, depending on the number of sequences); larger calls are rejected before any launch.  All calls on one GPU share that
  * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race and must be
  * serialised by the caller.
  */
