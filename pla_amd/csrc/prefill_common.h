@@ -451,7 +451,7 @@ struct SweepRole {
   const float* init;      // [V, K] tile the state starts from (nullptr: zero)
   float* fin;             // [V, K] tile that receives the state at the end (nullptr: none)
   float* keep_init;       // [V, K] tile that receives a copy of the start state (nullptr: none)
-  bool zero_v, write_o, active;
+  bool zero_v, active;
 };
 __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, const int32_t* seq_chunk_off,
                                                   const SegmentTable& seg, const StageTable& stg, int stage,
@@ -467,7 +467,6 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
   // has no part in the first sweep - nothing needs its summary -: the second sweep takes it from the state the combine
   // step (or, for a sequence of one segment, the caller) provides and delivers the final state itself.
   SweepRole r{};
-  r.write_o = true;
   auto state_in = [&](int n, int head) -> const float* {
     const int slot = (h0 != nullptr) ? (h0_indices ? h0_indices[n] : n) : -1;
     return slot >= 0 ? h0 + (int64_t)slot * h0_slot_stride + (int64_t)head * 16384 : nullptr;
@@ -501,7 +500,6 @@ __device__ __forceinline__ SweepRole select_sweep(int pass, int heads, int N, co
     const int64_t tile = ((int64_t)s * heads + r.head) * 16384;
     if (pass == 1) {
       if (last) return r;
-      r.write_o = false;
       if (first) {
         if (from_identity) return r;
         r.init = state_in(r.n, r.head);

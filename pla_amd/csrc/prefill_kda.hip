@@ -471,7 +471,6 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   }
   // output rows: in the transposed product a lane holds V columns vbase + 16 nb + 4 kb .. + 3 of token 16 ni + r16
   uint16_t* const o_lane = reinterpret_cast<uint16_t*>(p.o) + ((int64_t)(seq_start + r16) * p.H + h) * 128 + vbase + 4 * kb;
-  const bool write_o = role.write_o;
 
   for (int ci = 0; ci < n_chunks; ++ci) {
     const int par = ci & 1;
@@ -614,7 +613,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
 #pragma unroll
           for (int b = (s == 0 ? 0 : 4); b < (s == 0 ? 4 : TRI_BLOCKS); ++b) OT[nb][tri_block_m(b)] = mfma16h(ur[nb], pa[b], OT[nb][tri_block_m(b)]);
       }
-      if (write_o) {
+      {
         const int len = chunk_len(ci);
         uint16_t* const dst = o_lane + (int64_t)ci * CHUNK * p.H * 128;
 #pragma unroll
