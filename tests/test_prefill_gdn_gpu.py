@@ -217,20 +217,21 @@ def test_gdn_prefill_split_inputs_and_compact_state():
     torch.testing.assert_close(g_cum[0].cpu(), want, rtol=1e-5, atol=1e-6)
 
 
-def test_gdn_prefill_without_normalisation_on_a_poisoned_workspace_fused_sweep():
-    """normalize_qk=False through the fused sweep (16-byte aligned rows, whole sequences, several chunks): the
-    preparation then writes no 1 / |k| factors, and the sweep must not read them (the workspace holds NaN)."""
+@pytest.mark.parametrize("offs", [[0, 130, 130, 700], [0, 2300, 2300, 2600]])
+def test_gdn_prefill_without_normalisation_on_a_poisoned_workspace_fused_sweep(offs):
+    """normalize_qk=False (several chunks; whole sequences, and - the second case - a call split into segments, whose
+    first sweep copies the K rows the preparation stored): the preparation then writes no 1 / |k| factors, and the
+    sweeps must not read them (the workspace holds NaN)."""
     from pla_amd.prefill.flashqla import chunk_gated_delta_rule_fwd
     from oracle.prefill import token_recurrence
     g = torch.Generator().manual_seed(11)
-    T, H, HV = 700, 2, 4
+    T, H, HV = offs[-1], 2, 4
     q = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
     k = l2norm(torch.randn(T, H, 128, generator=g)).bfloat16()
     v = torch.randn(T, HV, 128, generator=g).bfloat16()
     gate = -torch.rand(T, HV, generator=g) * 0.3
     beta = torch.rand(T, HV, generator=g)
     S0 = torch.randn(3, HV, 128, 128, generator=g) * 0.1
-    offs = [0, 130, 130, 700]
     exp_o, exp_final = token_recurrence(q, k, v, gate, beta, offs, S0, scale=128 ** -0.5)
     dev = "cuda"
     cu = torch.tensor(offs, dtype=torch.int32, device=dev)
