@@ -141,20 +141,28 @@ def test_select_check_cases_is_seeded_and_small():
 def test_check_24_sampled_prefill_shapes_against_the_oracle_and_split_calls():
     """24 seeded shapes of the every-50th prefill list (up to 1800 tokens): each against the CPU oracle at the stated
     tolerances, and the first eight also against themselves fed in two chained calls per sequence (what
-    ``python -m pla_amd.caselist FILE --check N`` runs)."""
-    cases = caselist.select_check_cases(caselist.read_caselist(PREFILL_EVERY50), 24, seed=0, max_tokens=1800)
-    assert len(cases) == 24
+    ``python -m pla_amd.caselist FILE --check N`` runs).  With PLA_CASELIST_ORACLE_CASES=N in the environment the same
+    check draws N shapes from the list of every distinct prefill shape instead (a longer run, for a record)."""
+    wanted = int(os.environ.get("PLA_CASELIST_ORACLE_CASES", "24"))
+    source = PREFILL_EVERY50 if wanted == 24 else PREFILL_ALL
+    cases = caselist.select_check_cases(caselist.read_caselist(source), wanted, seed=0, max_tokens=1800)
+    assert len(cases) == wanted
     ties = 0
+    worst_o = worst_state = 0.0
     for i, case in enumerate(cases):
         row = caselist.check_case(case, reference=_oracle_reference, seed=i)
         print(row, flush=True)
         assert row["ok"], row
         ties += row["states_over_bound"]
+        worst_o, worst_state = max(worst_o, row["o_err"]), max(worst_state, row["state_rel_l2"])
         if i < 8:
             row = caselist.check_case(case, seed=i)
             print(row, flush=True)
             assert row["ok"], row
-    # states beyond 1e-3 are rounding ties of a normalised key under strong decay (see check_case): the first case has
-    # one (head 23: the whole last key row lies 1e-8 from the midpoints between bf16 values), none is expected elsewhere
-    assert ties <= 2, ties
+    print(f"{wanted} cases against the oracle: largest output difference {worst_o}, largest state rel-L2 {worst_state}, "
+          f"{ties} states beyond 1e-3", flush=True)
+    # states beyond 1e-3 are rounding ties of a normalised key under strong decay (see check_case): the first case of
+    # the 24 has one (head 23: the whole last key row lies 1e-8 from the midpoints between bf16 values), none is
+    # expected elsewhere
+    assert ties <= max(2, wanted // 12), ties
     assert caselist.main([PREFILL_EVERY50, "--check", "3", "--check-max-tokens", "600"]) == 0
