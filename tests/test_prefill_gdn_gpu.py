@@ -255,11 +255,13 @@ def test_config3_gdn_prefill_32k_varlen(seed, tokens):
     _check(w, fast=True)
 
 
-@pytest.mark.parametrize("lengths,tail_pad,H,HV", [([2500, 0, 1111, 40], 5, 1, 2), ([4096], 0, 2, 2), ([1030, 2049], 0, 1, 4)])
+@pytest.mark.parametrize("lengths,tail_pad,H,HV", [([2500, 0, 1111, 40], 5, 1, 2), ([4096], 0, 2, 2), ([1030, 2049], 0, 1, 4),
+                                                    ([16384], 0, 16, 32)])
 def test_gdn_prefill_split_sequences_match_oracle(lengths, tail_pad, H, HV):
     """Calls with few (sequence, head) chains and long sequences are split into 16-chunk segments that
     are swept concurrently (zero-state and identity sweeps, a combine step, a second sweep): ragged
-    lengths, an empty sequence, a sequence shorter than one segment, indexed pool, against the oracle."""
+    lengths, an empty sequence, a sequence shorter than one segment, indexed pool, against the oracle.  The last case is
+    the reference report's single 16 384-token sequence of 32 value heads (8 segments of 32 chunks per head)."""
     from pla_amd import _lib
     from pla_amd.workloads import gdn_prefill_packed
     T, N = sum(lengths) + tail_pad, len(lengths)
