@@ -325,7 +325,7 @@ int64_t pla_gdn_prefill_workspace_bytes(int T, int N, int H, int HV);
  *       array is NULL; zero state when h0 is NULL) and written at ht_indices[n].  h0 == ht with
  *       the same indices updates an indexed pool in place.
  *   o [T,HV,128] activation dtype, dense.   gcum_out / beta_out: optional [T,HV] float32 copies of the
- *       chunk-local cumulative log-decay and of beta (NULL keeps them in the workspace).
+ *       chunk-local cumulative log-decay and of beta (NULL: not written; no kernel reads them back).
  */
 int pla_gdn_prefill_launch(
     const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,

@@ -115,7 +115,6 @@ py::object gdn_launch(const GdnCall& c, const OptTensor& g, const OptTensor& bet
   const auto dev = c.ref.options();
   Tensor o = at::empty({1, T, H, 128}, dev.dtype(c.act));
   Tensor g_cum = at::empty({1, T, H}, dev.dtype(at::kFloat));
-  Tensor beta_act = at::empty({1, T, H}, dev.dtype(at::kFloat));
   const int64_t ws_bytes = pla_gdn_prefill_workspace_bytes((int)T, (int)batch, (int)c.Hg, (int)H);
   Tensor ws = at::empty({ws_bytes}, dev.dtype(at::kByte));
   const float* h0 = initial_state ? initial_state->data_ptr<float>() : nullptr;
@@ -142,7 +141,7 @@ py::object gdn_launch(const GdnCall& c, const OptTensor& g, const OptTensor& bet
       raw ? nullptr : g->data_ptr<float>(), raw ? nullptr : beta->data_ptr<float>(),
       cu.data_ptr<int32_t>(), (int)batch, (int)T, (float)scale, normalize_qk ? 1 : 0,
       h0, idx, h0_stride, ht, idx, ht_stride, o.data_ptr(), ws.data_ptr(), ws_bytes, g_cum.data_ptr<float>(),
-      beta_act.data_ptr<float>(), (int)c.Hg, (int)H, 128, 128, c.act == at::kHalf ? PLA_F16 : PLA_BF16, stream_of(c.ref),
+      nullptr, (int)c.Hg, (int)H, 128, 128, c.act == at::kHalf ? PLA_F16 : PLA_BF16, stream_of(c.ref),
       host_offsets.empty() ? nullptr : host_offsets.data()));
   py::object final_obj = py::none();
   if (output_final_state) {

@@ -227,8 +227,11 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
     const float glast = __shfl(cum, 63, 64);
     if (lane < len) {
       const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;
-      p.gcum[at] = cum;
-      p.beta[at] = bt;
+      // Copies for the caller, [T, HV]: each word is a 4-byte store into a line of its own (the other value heads of a
+      // token are written by other wavefronts at other times), which costs the call 1.5 % per copy - only on request.
+      // (Measured: workgroups of their own that write a chunk's 64 x HV words as one contiguous block cost as much.)
+      if (p.gcum != nullptr) p.gcum[at] = cum;
+      if (p.beta != nullptr) p.beta[at] = bt;
     }
     Gs[lane] = cum;
     Bs[lane] = bt;
@@ -1295,7 +1298,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 #undef SB
 
 struct GdnWorkspaceLayout {
-  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, q_rows, k_rows, kn, kinv, gcum, beta, gtile, W;
+  size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, q_rows, k_rows, kn, kinv, gtile, W;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
@@ -1313,8 +1316,6 @@ static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_sta
   L.k_rows = take((size_t)T * H * 128 * 2);
   L.kn = take((size_t)T * H * 128 * 2);
   L.kinv = take((size_t)T * H * 4);
-  L.gcum = take((size_t)T * HV * 4);
-  L.beta = take((size_t)T * HV * 4);
   L.gtile = take((size_t)L.NC_max * HV * GTILE_FLOATS * 4);
   L.W = take((size_t)L.NC_max * HV * 2 * TRI_BLOCKS * 1024);
   L.seg_chunks = pick_segment_chunks(T, N, HV);
@@ -1429,8 +1430,8 @@ static int gdn_prefill_run(
   p.chunk_len = reinterpret_cast<int32_t*>(ws + L.chunk_len);
   p.kn = reinterpret_cast<uint16_t*>(ws + L.kn);
   p.kinv = reinterpret_cast<float*>(ws + L.kinv);
-  p.gcum = gcum_out ? gcum_out : reinterpret_cast<float*>(ws + L.gcum);
-  p.beta = beta_out ? beta_out : reinterpret_cast<float*>(ws + L.beta);
+  p.gcum = gcum_out;
+  p.beta = beta_out;
   p.gtile = reinterpret_cast<float*>(ws + L.gtile);
   p.W = reinterpret_cast<uint16_t*>(ws + L.W);
   p.H = H; p.HV = HV; p.NC_max = L.NC_max;

@@ -218,7 +218,6 @@ def chunk_gated_delta_rule_fwd(
     dev = q.device
     o = torch.empty(1, num_tokens, H, DV, dtype=q.dtype, device=dev)
     g_cum = torch.empty(1, num_tokens, H, dtype=torch.float32, device=dev)
-    beta_act = torch.empty(1, num_tokens, H, dtype=torch.float32, device=dev)
     ws, ws_bytes = _workspace(num_tokens, batch, Hg, H, dev)
 
     if indexed:
@@ -262,7 +261,7 @@ def chunk_gated_delta_rule_fwd(
         cu32.data_ptr(), batch, num_tokens, float(scale), int(bool(normalize_qk)),
         _lib.ptr(h0), _lib.ptr(h0_idx), h0.stride(0) if h0 is not None else 0,
         _lib.ptr(ht), _lib.ptr(ht_idx), ht.stride(0) if ht is not None else 0,
-        o.data_ptr(), ws.data_ptr(), ws_bytes, g_cum.data_ptr(), beta_act.data_ptr(),
+        o.data_ptr(), ws.data_ptr(), ws_bytes, g_cum.data_ptr(), None,
         Hg, H, DK, DV, _lib.dtype_code(q.dtype), _lib.current_stream(dev),
         ctypes.cast(raw_host, ctypes.c_void_p) if raw_host is not None else None)
 
