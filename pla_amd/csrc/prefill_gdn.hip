@@ -65,7 +65,7 @@ struct GdnPrefillParams {
   // workspace
   int32_t* seq_chunk_off; int32_t* chunk_seq; int32_t* chunk_tok; int32_t* chunk_len;
   uint16_t* kn;                                       // [T, H, 128] normalised K rows in operand column order (calls split into segments)
-  float* kinv;                                        // [T, H] 1 / |k| per row
+  float* kinv;                                        // [H, T] 1 / |k| per row (a head's tokens are contiguous)
   float* gcum; float* beta;
   uint16_t* W;                                        // fp16 [chunk, HV, 12 blocks of 1 KiB]: W = hi + lo, six-block operand layout
   float* gtile;          // [chunk, HV, 320]: scale e^{G} | e^{G} | e^{G_last - G} | e^{G_last} | G
@@ -225,14 +225,6 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
       if (lane >= d) cum += up;
     }
     const float glast = __shfl(cum, 63, 64);
-    if (lane < len) {
-      const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;
-      // Copies for the caller, [T, HV]: each word is a 4-byte store into a line of its own (the other value heads of a
-      // token are written by other wavefronts at other times), which costs the call 1.5 % per copy - only on request.
-      // (Measured: workgroups of their own that write a chunk's 64 x HV words as one contiguous block cost as much.)
-      if (p.gcum != nullptr) p.gcum[at] = cum;
-      if (p.beta != nullptr) p.beta[at] = bt;
-    }
     Gs[lane] = cum;
     Bs[lane] = bt;
     float* gt = p.gtile + ((int64_t)cb * p.HV + hv) * GTILE_FLOATS;
@@ -269,7 +261,7 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
         const LanePair r2 = swap_halves(r1.lo + r1.hi);
         inv = rsqrtf(r2.lo + r2.hi + 1e-6f);
         // the sweep scales the raw rows by the same factor, so both kernels hold the same rounded keys
-        if (ok && kb == 0 && first_group) p.kinv[(int64_t)(t0 + 16 * mb + r16) * p.H + h] = inv;
+        if (ok && kb == 0 && first_group) p.kinv[(int64_t)h * p.T + t0 + 16 * mb + r16] = inv;
       }
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
@@ -298,6 +290,21 @@ __global__ __launch_bounds__(64 * WAVES) void gdn_wsolve_kernel(const GdnPrefill
     }
   }
   __syncthreads();
+  // Copies for the caller, [T, HV] FP32, only on request: the words of a token's other value heads are written by other
+  // workgroups at other times, so every store here is a piece of a line of its own (measured: 1.5 % of a call per copy
+  // with 4-byte stores).  The first wavefront writes the values of all WAVES heads of the workgroup as one piece per
+  // token.  (Measured as well: workgroups of their own that write a chunk's 64 x HV words as one contiguous block
+  // cost as much as they save.)
+  if (wave == 0 && lane < len) {
+    const int64_t at = (int64_t)(t0 + lane) * p.HV + hv;        // hv: the workgroup's first head, a multiple of WAVES
+    auto put = [&](float* out, const float (&all)[WAVES][CHUNK]) {
+      if constexpr (WAVES == 4) *reinterpret_cast<float4*>(out + at) = make_float4(all[0][lane], all[1][lane], all[2][lane], all[3][lane]);
+      else if constexpr (WAVES == 2) *reinterpret_cast<float2*>(out + at) = make_float2(all[0][lane], all[1][lane]);
+      else out[at] = all[0][lane];
+    };
+    if (p.gcum != nullptr) put(p.gcum, Gs_all);
+    if (p.beta != nullptr) put(p.beta, Bs_all);
+  }
   if constexpr (WAVES > 1) {
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
@@ -788,7 +795,7 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       const int64_t row_pitch = q_side ? p.stride_q : p.stride_k;
       // bases of the sequence part (wave-uniform, 64-bit) and offsets inside a chunk (per lane, 32-bit)
       const char* const rows_b = reinterpret_cast<const char*>(q_side ? p.q : p.k) + ((int64_t)seq_start * row_pitch + h * 128) * 2;
-      const char* const kinv_b = reinterpret_cast<const char*>(p.kinv + (int64_t)seq_start * p.H + h);
+      const char* const kinv_b = reinterpret_cast<const char*>(p.kinv + (int64_t)h * p.T + seq_start);
       const int64_t chunk_pitch_b = (int64_t)CHUNK * row_pitch * 2;
       const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + hv * 128) * 2;
       const char* const w_b = reinterpret_cast<const char*>(p.W) + ((int64_t)c_begin * p.HV + hv) * (2 * TRI_BLOCKS * 1024);
@@ -818,14 +825,14 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
       // raw rows of chunk c into registers (rows past the end of the sequence part re-read its last row)
       auto load_rows = [&](int c, uint4 (&raw)[8], float (&inv)[8]) {
         const char* const cb = rows_b + (int64_t)c * chunk_pitch_b;
-        const char* const ib = kinv_b + (int64_t)c * CHUNK * p.H * 4;
+        const char* const ib = kinv_b + (int64_t)c * CHUNK * 4;
         const int last = seq_len - 1 - c * CHUNK;          // last valid row of this chunk (>= 63 for a full one)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
           const uint32_t row = (uint32_t)min(row0 + 4 * j + lr, last);
           raw[j] = *reinterpret_cast<const uint4*>(cb + row * (uint32_t)(row_pitch * 2) + 16u * lc);
           // without normalisation the preparation never writes 1 / |k|: the workspace words are not read at all
-          inv[j] = (q_side || !p.normalize_qk) ? 1.f : *reinterpret_cast<const float*>(ib + row * (uint32_t)(p.H * 4));
+          inv[j] = (q_side || !p.normalize_qk) ? 1.f : *reinterpret_cast<const float*>(ib + row * 4u);
         }
       };
       // K rows: scaled by 1 / |k|, rounded to the activation dtype (the operand of the reference), written as fp16,
@@ -1397,6 +1404,7 @@ static int gdn_prefill_run(
               "q/k rows require 4-byte alignment");
   PLA_REQUIRE((uintptr_t)v % 16 == 0 && stride_v % 8 == 0, "v rows require 16-byte alignment (they are copied to LDS in 16-byte pieces)");
   PLA_REQUIRE((uintptr_t)o % 16 == 0, "o requires 16-byte alignment");
+  PLA_REQUIRE((uintptr_t)gcum_out % 16 == 0 && (uintptr_t)beta_out % 16 == 0, "gcum_out and beta_out require 16-byte alignment");
   const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV, !static_scratch);
   if (static_scratch) {
     PLA_REQUIRE((int64_t)L.total <= PLA_GDN_PREFILL_STATIC_BYTES,
