@@ -132,7 +132,7 @@ GDN_FLOP_PER_TOKEN = 4718592      # 2 * [HV (3 K V + 2 C V) + H (2 C K)], C = 64
 KDA_FLOP_PER_TOKEN = 5242880      # same with HV = H = 32 (one gram per head)
 # HBM bytes per call from rocprofv3 --pmc FETCH_SIZE (x2.00) and WRITE_SIZE (x1.00), summed over the kernels of
 # one call (profiles/gdn_prefill_kernels_32k.txt, profiles/kda_prefill_kernels_64k.txt)
-GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 1592000000
+GDN_PREFILL_TRAFFIC_BYTES_PER_CALL = 1532000000
 KDA_PREFILL_TRAFFIC_BYTES_PER_CALL = 11129000000
 
 
