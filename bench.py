@@ -261,10 +261,8 @@ def bench_prefill_kda(steps, device, cpu_leg=False):
                      lower_bound=c["lower_bound"], initial_state=c["initial_state"], final_state=c["final_state"],
                      cu_seqlens=c["cu_seqlens"])
 
-    ms = time_calls(run, steps, 3, device)
-    tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     extra = {}
-    if cpu_leg:
+    if cpu_leg:                                   # ahead of the GPU leg: what follows this function finds a busy GPU
         # the CPU oracle's token recurrence over a prefix of the same sequence (the whole of it would take minutes)
         import time as _time
         from oracle import kda_prefill_reference
@@ -281,6 +279,8 @@ def bench_prefill_kda(steps, device, cpu_leg=False):
                                      sample="the first %d tokens of the 65 536-token sequence, all 32 heads, one pass of "
                                             "the token recurrence (%.1f s)" % (prefix, t),
                                      threads_torch=torch.get_num_threads())
+    ms = time_calls(run, steps, 3, device)
+    tflops = KDA_FLOP_PER_TOKEN * T / (ms * 1e-3) / 1e12
     return dict(tokens=T, steps=steps, warmup=3, ms_per_call=round(ms, 4), tokens_per_s=round(T / ms * 1e3, 1), **extra,
                 roofline=dict(bound="mfma", achieved=round(tflops, 2), peak=BF16_PEAK_TFLOPS, unit="TFLOP/s",
                               frac=round(tflops / BF16_PEAK_TFLOPS, 4), traffic=KDA_PREFILL_TRAFFIC_BYTES_PER_CALL,
@@ -619,12 +619,13 @@ def main():
         extra["replay_verify"] = bench_replay_verify(device)
         extra["replay_paged"] = bench_replay_paged(device)
         torch.cuda.empty_cache()
+        # (the host-time leg keeps the GPU nearly idle, so it does not run last: what precedes the headline is GPU work)
+        extra["prefill_host_us"] = bench_prefill_host_time(device)
+        torch.cuda.empty_cache()
         extra["prefill"] = bench_prefill(max(args.steps, 50), 50, device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
         extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 2, 10), device)
         extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device, cpu_leg=not args.no_cpu_baseline)
-        torch.cuda.empty_cache()
-        extra["prefill_host_us"] = bench_prefill_host_time(device)
         torch.cuda.empty_cache()
     d = time_decode(prep, args.steps, args.warmup)
     result = {
