@@ -338,8 +338,9 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 //   barrier B   the tiles requested at A landed; V is free              copy V of c + 1
 //               O^T = S (scale Q e^G)^T + U^T P^T -> rows of o
 //               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U         (pairs: hi.lo + lo.hi + hi.hi)
+template <int NB>
 __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_kernel(const KdaPrefillParams p) {
-  constexpr int NB = 2;
+  constexpr int HALVES = 2 / NB;             // workgroups per chain: NB = 1 sweeps 64 of the 128 V columns
   constexpr int NCOPY = KDA_SWEEP_COPIERS;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, NCOPY>;  // 64 x 128 tile, its pieces dealt to the copying wavefronts
   constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
@@ -347,8 +348,9 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
+  const int v_half = (int)blockIdx.x % HALVES;
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, (int)blockIdx.x / HALVES);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
@@ -443,7 +445,7 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   }
 
   // ---- the computing wavefronts ------------------------------------------------------------
-  const int vbase = 32 * wave;
+  const int vbase = 64 * v_half + 16 * NB * wave;
   const int vcol = vbase + r16;                      // state / KS / U layout: the lane's column (second block: + 16)
   // S^T slices in accumulator layout: St[nb][mc][r] = S[v = vcol + 16 nb][c = 16 mc + 4 kb + r]
   f32x4_t St[NB][8];
@@ -1078,6 +1080,7 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
   }
+  const bool v_halves = !segmented && (int64_t)N * H > 64 && (int64_t)N * H <= 128;
   const SideStreamLease lease(s, L.stages > 0);
   const int stages = lease.get() != nullptr ? L.stages : 0;
   if (stages > 0) {
@@ -1095,13 +1098,16 @@ extern "C" int pla_kda_prefill_launch(
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
         // the first sweep over segments publishes no output: both of its roles in one workgroup per (segment, head)
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
-        else hipLaunchKernelGGL(kda_sweep_kernel, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+        // Whole sequences that give 65 to 128 chains (fewer are split into segments) leave half of the CUs idle: two
+        // workgroups then sweep a chain, 64 V columns each (the columns of V are independent: the same bits).
+        else if (v_halves) hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(2 * grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+        else hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_sweep_kernel, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+    hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
