@@ -1548,9 +1548,26 @@ static int gdn_prefill_run(
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV);
     p.pass = 2;
-    const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));
-    if (half_act) hipLaunchKernelGGL((gdn_fused_sweep_kernel<f16_t, 2>), dim3(g), dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((gdn_fused_sweep_kernel<bf16_t, 2>), dim3(g), dim3(512), 0, s, p);
+    // Segments are at least 16 chunks long, so short calls and calls of few heads give fewer (segment, head) pairs than
+    // half of the CUs: the second sweep then runs two workgroups per pair, 64 V columns each, as above.  The number of
+    // segments is known exactly where the caller passed the offsets on the host, else from the tokens alone.
+    int64_t segments = N == 1 ? ((T + CHUNK - 1) / CHUNK + L.seg_chunks - 1) / L.seg_chunks : (int64_t)(T / CHUNK + N) / L.seg_chunks + N;
+    if (raw_cu_seqlens != nullptr) {
+      segments = 0;
+      for (int n = 0; n < N; ++n) {
+        const int nc = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+        segments += (nc + L.seg_chunks - 1) / L.seg_chunks;
+      }
+    }
+    if (segments * HV <= 128) {
+      const unsigned g = xcd_grouped_grid(2 * (unsigned)L.max_segments * HV, 2 * (unsigned)(HV / H));
+      if (half_act) hipLaunchKernelGGL((gdn_fused_sweep_kernel<f16_t, 1>), dim3(g), dim3(512), 0, s, p);
+      else hipLaunchKernelGGL((gdn_fused_sweep_kernel<bf16_t, 1>), dim3(g), dim3(512), 0, s, p);
+    } else {
+      const unsigned g = xcd_grouped_grid((unsigned)L.max_segments * HV, (unsigned)(HV / H));
+      if (half_act) hipLaunchKernelGGL((gdn_fused_sweep_kernel<f16_t, 2>), dim3(g), dim3(512), 0, s, p);
+      else hipLaunchKernelGGL((gdn_fused_sweep_kernel<bf16_t, 2>), dim3(g), dim3(512), 0, s, p);
+    }
   }
   return check_launch("gdn prefill launch");
 }

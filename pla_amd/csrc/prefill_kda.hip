@@ -1107,7 +1107,12 @@ extern "C" int pla_kda_prefill_launch(
   if (segmented) {
     hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H);
     p.pass = 2;
-    hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+    // fewer (segment, head) pairs than half of the CUs (segments are at least 16 chunks long): two workgroups per pair
+    // (an upper bound of their number from the token count alone: exact for a single sequence)
+    if ((N == 1 ? ((T + CHUNK - 1) / CHUNK + L.seg_chunks - 1) / L.seg_chunks : (int64_t)(T / CHUNK + N) / L.seg_chunks + N) * H <= 128)
+      hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(2 * (unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+    else
+      hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
   return check_launch("kda prefill launch");
 }
