@@ -1462,7 +1462,7 @@ static int gdn_prefill_run(
   }
   // a call split into segments: the preparation also stores the normalised K rows, which the first sweep copies
   p.store_kn = segmented;
-  const bool v_halves = !segmented && (int64_t)N * HV > 64 && (int64_t)N * HV <= 128;
+  const bool v_halves = !segmented && (int64_t)N * HV <= 128;
   if (segmented) {
     // few, long sequences: sweep their segments concurrently (two sweeps and a combine step)
     p.seg.seq_seg_off = reinterpret_cast<int32_t*>(ws + L.seq_seg_off);
@@ -1529,7 +1529,7 @@ static int gdn_prefill_run(
           if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(grid / 2), dim3(512), 0, s, p);
           else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
         } else {
-          // Whole sequences that give 65 to 128 chains (fewer are split into segments) leave half of the CUs idle: two
+          // Whole sequences that give at most 128 chains (few long ones are split into segments instead) leave half of the CUs idle: two
           // workgroups then sweep a chain, 64 V columns each - the columns of V are independent, so the results are the
           // same bits.  A half costs 0.86 to 0.93 of a whole chain's chunk time (K, Q, W and P are fetched and formed once
           // per workgroup whatever its width): 4 x 4096 tokens of 32 value heads 0.248 -> 0.236 ms, 3 x 4096 0.227 -> 0.205.

@@ -1080,7 +1080,7 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.seg_chunks = L.seg_chunks;
     p.seg.max_segments = L.max_segments;
   }
-  const bool v_halves = !segmented && (int64_t)N * H > 64 && (int64_t)N * H <= 128;
+  const bool v_halves = !segmented && (int64_t)N * H <= 128;
   const SideStreamLease lease(s, L.stages > 0);
   const int stages = lease.get() != nullptr ? L.stages : 0;
   if (stages > 0) {
@@ -1098,7 +1098,7 @@ extern "C" int pla_kda_prefill_launch(
         // the first sweep over segments publishes no output: the lean variant, two workgroups per CU
         // the first sweep over segments publishes no output: both of its roles in one workgroup per (segment, head)
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
-        // Whole sequences that give 65 to 128 chains (fewer are split into segments) leave half of the CUs idle: two
+        // Whole sequences that give at most 128 chains (few long ones are split into segments instead) leave half of the CUs idle: two
         // workgroups then sweep a chain, 64 V columns each (the columns of V are independent: the same bits).
         else if (v_halves) hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(2 * grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
         else hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
