@@ -631,9 +631,12 @@ __device__ __forceinline__ void segment_map(const int32_t* seq_chunk_off, int N,
 // M[16 s + 4 kb + e][column c], 64 contiguous bytes per group of 16 lanes), all 64 loads of a step requested before
 // the first product.
 constexpr int COMBINE_SPLIT = 8;
-static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads) {
-  const int part = blockIdx.x % COMBINE_SPLIT;
-  const int chain = blockIdx.x / COMBINE_SPLIT;
+static __global__ __launch_bounds__(256) void segment_combine_kernel(SegmentTable t, int heads, int chains) {
+  // the eight workgroups of a chain read the same M tiles: on one XCD they come from memory once (xcd_grouped_index)
+  const int logical = xcd_grouped_index(blockIdx.x, COMBINE_SPLIT, chains * COMBINE_SPLIT);
+  if (logical < 0) return;
+  const int part = logical % COMBINE_SPLIT;
+  const int chain = logical / COMBINE_SPLIT;
   const int n = chain / heads, h = chain - n * heads;
   const int first = t.seq_seg_off[n], end = t.seq_seg_off[n + 1];
   if (end - first < 2) return;                 // a single segment starts from the caller's state

@@ -1546,7 +1546,8 @@ static int gdn_prefill_run(
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * HV * COMBINE_SPLIT), dim3(256), 0, s, p.seg, HV);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3(xcd_grouped_grid((unsigned)N * HV * COMBINE_SPLIT, COMBINE_SPLIT)), dim3(256), 0, s, p.seg, HV,
+                       N * HV);
     p.pass = 2;
     // Segments are at least 16 chunks long, so short calls and calls of few heads give fewer (segment, head) pairs than
     // half of the CUs: the second sweep then runs two workgroups per pair, 64 V columns each, as above.  The number of

@@ -1105,7 +1105,8 @@ extern "C" int pla_kda_prefill_launch(
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
   if (segmented) {
-    hipLaunchKernelGGL(segment_combine_kernel, dim3((unsigned)N * H * COMBINE_SPLIT), dim3(256), 0, s, p.seg, H);
+    hipLaunchKernelGGL(segment_combine_kernel, dim3(xcd_grouped_grid((unsigned)N * H * COMBINE_SPLIT, COMBINE_SPLIT)), dim3(256), 0, s, p.seg, H,
+                       N * H);
     p.pass = 2;
     // fewer (segment, head) pairs than half of the CUs (segments are at least 16 chunks long): two workgroups per pair
     // (an upper bound of their number from the token count alone: exact for a single sequence)
