@@ -454,11 +454,14 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
   const int vcol = 32 * cw + r16;
 
   // the two roles of this (segment, head): logical workgroups 2 i (zero state / real state) and 2 i + 1 (identity)
+  // the value heads of a q/k head copy the same K rows: on one XCD they come from memory once
+  const int pair = xcd_grouped_index(blockIdx.x, p.HV / p.H, p.seg.max_segments * p.HV);
+  if (pair < 0) return;
   const SweepRole lead = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, 2 * pair);
   if (!lead.active) return;
   const SweepRole mrole = select_sweep(1, p.HV, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                       p.ht, p.ht_indices, p.ht_slot_stride, 2 * (int)blockIdx.x + 1);
+                                       p.ht, p.ht_indices, p.ht_slot_stride, 2 * pair + 1);
   const SweepRole& role = m_side ? mrole : lead;
   const bool computing = role.active;                          // wave-uniform; false: wavefronts 4-7 of a first segment
   const int n = lead.n, hv = lead.head, c_begin = lead.c_begin, c_end = lead.c_end;
@@ -1526,8 +1529,9 @@ static int gdn_prefill_run(
       },
       [&](unsigned grid) {
         if (p.pass == 1) {        // first sweep over segments: no output, both roles in one workgroup per (segment, head)
-          if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(grid / 2), dim3(512), 0, s, p);
-          else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(grid / 2), dim3(512), 0, s, p);
+          const unsigned g = xcd_grouped_grid(grid / 2, (unsigned)(HV / H));
+          if (half_act) hipLaunchKernelGGL(gdn_lean_sweep_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+          else hipLaunchKernelGGL(gdn_lean_sweep_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
         } else {
           // Whole sequences that give at most 128 chains (few long ones are split into segments instead) leave half of the CUs idle: two
           // workgroups then sweep a chain, 64 V columns each - the columns of V are independent, so the results are the

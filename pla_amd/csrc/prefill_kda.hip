@@ -348,9 +348,13 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  const int v_half = (int)blockIdx.x % HALVES;
+  // the two halves of a chain copy the same tiles: on one XCD they come from memory once (xcd_grouped_index)
+  const int wide = HALVES == 1 ? (int)blockIdx.x
+                               : xcd_grouped_index(blockIdx.x, HALVES, HALVES * (p.pass == 2 ? p.seg.max_segments : p.N) * p.H);
+  if (wide < 0) return;
+  const int v_half = wide % HALVES;
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
-                                      p.ht, p.ht_indices, p.ht_slot_stride, (int)blockIdx.x / HALVES);
+                                      p.ht, p.ht_indices, p.ht_slot_stride, wide / HALVES);
   if (!role.active) return;
   const int n = role.n, h = role.head, c_begin = role.c_begin, c_end = role.c_end;
   const int seq_start = p.cu_seqlens[n] + (c_begin - p.seq_chunk_off[n]) * CHUNK;
@@ -1100,7 +1104,7 @@ extern "C" int pla_kda_prefill_launch(
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
         // Whole sequences that give at most 128 chains (few long ones are split into segments instead) leave half of the CUs idle: two
         // workgroups then sweep a chain, 64 V columns each (the columns of V are independent: the same bits).
-        else if (v_halves) hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(2 * grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+        else if (v_halves) hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(xcd_grouped_grid(2 * grid, 2)), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
         else hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
       });
   PLA_REQUIRE(ok, "an event call of the staged prefill failed: %s", hipGetErrorString(hipGetLastError()));
@@ -1111,7 +1115,7 @@ extern "C" int pla_kda_prefill_launch(
     // fewer (segment, head) pairs than half of the CUs (segments are at least 16 chunks long): two workgroups per pair
     // (an upper bound of their number from the token count alone: exact for a single sequence)
     if ((N == 1 ? ((T + CHUNK - 1) / CHUNK + L.seg_chunks - 1) / L.seg_chunks : (int64_t)(T / CHUNK + N) / L.seg_chunks + N) * H <= 128)
-      hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(2 * (unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
+      hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(xcd_grouped_grid(2 * (unsigned)L.max_segments * H, 2)), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
     else
       hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
