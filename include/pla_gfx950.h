@@ -342,11 +342,13 @@ int pla_gdn_prefill_launch(
  * pla_gdn_prefill_launch with the sequence offsets on the host as well: raw_cu_seqlens points to N + 1 int32
  * values in HOST memory that equal cu_seqlens (NULL: exactly pla_gdn_prefill_launch).  Replaces the
  * `raw_cu_seqlens` argument of the reference's public ops (pla/prefill/flashqla/ops.py: "trusted host copy of
- * cu_seqlens", which lets its planner decide without reading the device tensor back).  Here the host uses it for one
- * decision only, by the rule the device applies anyway: a call whose sequences are of nearly equal length runs in
- * one stage, and with the offsets at hand nothing is enqueued for a second one (two launches and four event
- * operations less per call).  Results are bit-identical to pla_gdn_prefill_launch.  The values are read during the
- * call and not kept.
+ * cu_seqlens", which lets its planner decide without reading the device tensor back).  Here the host takes two
+ * decisions from it, neither of which changes a bit of the results (they equal pla_gdn_prefill_launch's): by the rule
+ * the device applies anyway, a call whose sequences are of nearly equal length runs in one stage, and with the offsets
+ * at hand nothing is enqueued for a second one (two launches and four event operations less per call); and a call of
+ * at most 64 ragged whole sequences with more than 128 chains sweeps the chains of its longest sequences as two
+ * workgroups of 64 V columns each where idle CUs make that shorter (pla_gdn_prefill_halved_sequences).  The values
+ * are read during the call and not kept.
  */
 int pla_gdn_prefill_launch_raw(
     const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
@@ -358,6 +360,14 @@ int pla_gdn_prefill_launch_raw(
     void* o, void* workspace, int64_t workspace_bytes,
     float* gcum_out, float* beta_out,
     int H, int HV, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens);
+
+/*
+ * The number of sequences whose chains pla_gdn_prefill_launch_raw would sweep as two workgroups each in its last
+ * sweep, for these host offsets (0: none, or the call is not one of ragged whole sequences).  Host arithmetic only:
+ * no GPU call.  No counterpart in the reference (its planner, pla/prefill/flashqla/private, decides on context-parallel
+ * splits instead); for tests and for callers who log the plan.
+ */
+int pla_gdn_prefill_halved_sequences(const int32_t* raw_cu_seqlens, int N, int T, int H, int HV);
 
 /*
  * pla_gdn_prefill_launch for callers that cannot allocate (code under hipGraph capture, tight serving

@@ -359,16 +359,16 @@ constexpr int MAX_STAGES = 2;
 // under the first sweep only as far as chains that have ended leave CUs to it (measured, ms per call, first stage of
 // 8 / 7 / 6 / 5 / 4 sixteenths: 0.440 / 0.434 / 0.428 / 0.434 / 0.443 at a fill of 0.57; at fills of 0.66 half is the
 // better cut by 0.4-1.1 %, at 0.31 and 0.61 three eighths by 1.4-1.9 %).
-__device__ __forceinline__ int stage_plan(int64_t total, int n_items, int longest, int S) {
+__host__ __device__ __forceinline__ int stage_plan(int64_t total, int n_items, int longest, int S) {
   const int64_t rectangle = (int64_t)n_items * longest;
   if (S <= 0 || 5 * total >= 4 * rectangle) return 1 | (8 << 8);
   return S | ((S == 2 && 8 * total < 5 * rectangle ? 6 : 8) << 8);
 }
-__device__ __forceinline__ int plan_stages(int plan) { return plan & 0xff; }
-__device__ __forceinline__ int stage_cut(int nc, int s, int plan) {
+__host__ __device__ __forceinline__ int plan_stages(int plan) { return plan & 0xff; }
+__host__ __device__ __forceinline__ int stage_cut(int nc, int s, int plan) {
   const int S = plan & 0xff;
   if (S == 2 && s == 1) return (int)((int64_t)nc * (plan >> 8) / 16);
-  return (int)((int64_t)nc * min(s, S) / S);
+  return (int)((int64_t)nc * (s < S ? s : S) / S);
 }
 
 // Single workgroup of 256 threads with (stages + 1) * n_items_max + 1 words of LDS at `pair_begin`.  The items are sequences (`counts` null: item i holds chunks

@@ -77,6 +77,10 @@ struct GdnPrefillParams {
   int inline_tables;     // at most 64 whole sequences: kernels work the chunk tables out themselves (no table kernel)
   int tail_blocks;       // workgroups appended to the preparation grid that zero the output rows beyond the last sequence
   int store_kn;          // gdn_wsolve_kernel also stores the normalised K rows (kn): the first sweep over segments copies them
+  // gdn_fused_sweep_mixed_kernel: the first `split_grid` workgroups sweep the chains of sequences seq_order[0 .. n_long)
+  // as two halves, the others those of seq_order[n_long .. N) whole
+  unsigned split_grid; int n_long;
+  unsigned char seq_order[INLINE_TABLE_SEQUENCES];
 };
 
 // q and k rows that start on 4-byte boundaries only (a packed view shifted inside its buffer) are copied into dense
@@ -732,14 +736,20 @@ __global__ __launch_bounds__(512, 1) void gdn_lean_sweep_kernel(const GdnPrefill
 // operand is requested a fixed number of steps before the MFMA that uses it and the VALU work (conversions, X, the
 // hi / lo split of U, the decay of S) is placed under the MFMAs; scheduling barriers keep that order.
 #define SB() __builtin_amdgcn_sched_barrier(0)
+// LDS of one workgroup of the fused sweep (layout in fused_sweep below)
+constexpr int FUSED_W_HALVES = 2 * TRI_BLOCKS * 512;       // hi blocks, then lo blocks
+constexpr int FUSED_OFF_P = 0, FUSED_OFF_G = FUSED_OFF_P + TRI_BLOCKS * 1024, FUSED_OFF_RQ = FUSED_OFF_G + 2 * 2048;
+constexpr int FUSED_OFF_W = (FUSED_OFF_RQ + 2 * CHUNK * 4 + 1023) / 1024 * 1024, FUSED_OFF_Q = FUSED_OFF_W + 2 * FUSED_W_HALVES * 2;
+constexpr int FUSED_OFF_K = FUSED_OFF_Q + 2 * TILE128_HALVES * 2, FUSED_OFF_V = FUSED_OFF_K + 2 * TILE128_HALVES * 2;
+constexpr int FUSED_LDS_BYTES = FUSED_OFF_V + 2 * TILE128_HALVES * 2;
+
+// The sweep of one workgroup.  `wide`: 2 / NB x the chain's logical index (sequence x HV + value head, or segment x
+// HV + value head in the second sweep over segments) plus, for NB = 1, the half of the V columns it takes.
 template <typename act_t, int NB>
-__global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefillParams p) {
+__device__ __forceinline__ void fused_sweep(const GdnPrefillParams& p, unsigned char* const lds_all, const int wide) {
   constexpr int CW = 4, AUX = 4;
   constexpr int HALVES = 2 / NB;             // workgroups per chain: NB = 1 sweeps 64 of the 128 V columns
   using CopyV = SwizzledTileCopy<AUX>;
-  // one workgroup per (sequence, value head), or per (segment, value head) in the second sweep over segments
-  const int wide = xcd_grouped_index(blockIdx.x, HALVES * (p.HV / p.H), HALVES * (p.pass == 2 ? p.seg.max_segments : p.N) * p.HV);
-  if (wide < 0) return;
   const int block = wide / HALVES, v_half = wide % HALVES;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -776,12 +786,9 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
   // workgroup's LDS is ONE array with a fixed layout: what is read at many constant offsets from one per-lane address
   // (the blocks of P and W, the decay factors) lies in the first 64 KiB, where those offsets fit the 16-bit offset
   // field of an LDS instruction; above that every distinct offset would cost a register for its address.
-  constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;       // hi blocks, then lo blocks
-  constexpr int OFF_P = 0, OFF_G = OFF_P + TRI_BLOCKS * 1024, OFF_RQ = OFF_G + 2 * 2048;
-  constexpr int OFF_W = (OFF_RQ + 2 * CHUNK * 4 + 1023) / 1024 * 1024, OFF_Q = OFF_W + 2 * W_HALVES * 2;
-  constexpr int OFF_K = OFF_Q + 2 * TILE128_HALVES * 2, OFF_V = OFF_K + 2 * TILE128_HALVES * 2;
-  constexpr int LDS_BYTES = OFF_V + 2 * TILE128_HALVES * 2;
-  __shared__ __align__(1024) unsigned char lds_all[LDS_BYTES];
+  constexpr int W_HALVES = FUSED_W_HALVES;
+  constexpr int OFF_P = FUSED_OFF_P, OFF_G = FUSED_OFF_G, OFF_RQ = FUSED_OFF_RQ, OFF_W = FUSED_OFF_W, OFF_Q = FUSED_OFF_Q;
+  constexpr int OFF_K = FUSED_OFF_K, OFF_V = FUSED_OFF_V;
   uint16_t* const tP = reinterpret_cast<uint16_t*>(lds_all + OFF_P);
   // decay factors: [0,64) scale e^{G}, [64,128) e^{G}, [128,192) e^{G_last - G}, [192] e^{G_last}, [256,320) G
   float (*const tG)[512] = reinterpret_cast<float (*)[512]>(lds_all + OFF_G);                       // [2][512]
@@ -1310,12 +1317,99 @@ __global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefil
 }
 #undef SB
 
+// One workgroup per (sequence, value head), or per (segment, value head) in the second sweep over segments (NB = 2);
+// NB = 1: two per chain, 64 V columns each (the columns of V are independent: same bits).
+template <typename act_t, int NB>
+__global__ __launch_bounds__(512, 1) void gdn_fused_sweep_kernel(const GdnPrefillParams p) {
+  constexpr int HALVES = 2 / NB;
+  __shared__ __align__(1024) unsigned char lds_all[FUSED_LDS_BYTES];
+  const int wide = xcd_grouped_index(blockIdx.x, HALVES * (p.HV / p.H), HALVES * (p.pass == 2 ? p.seg.max_segments : p.N) * p.HV);
+  if (wide < 0) return;
+  fused_sweep<act_t, NB>(p, lds_all, wide);
+}
+
+// Whole sequences of unequal length, swept in one launch whose longest chains decide how long it lasts while the CUs
+// of chains that have ended stand idle: the chains of the longest sequences are swept as two halves (which start
+// first: workgroups are dispatched in index order), those of the others whole, longest first.
+template <typename act_t>
+__global__ __launch_bounds__(512, 1) void gdn_fused_sweep_mixed_kernel(const GdnPrefillParams p) {
+  __shared__ __align__(1024) unsigned char lds_all[FUSED_LDS_BYTES];
+  const int ratio = p.HV / p.H;
+  if (blockIdx.x < p.split_grid) {
+    const int wide = xcd_grouped_index(blockIdx.x, 2 * ratio, 2 * p.n_long * p.HV);
+    if (wide < 0) return;
+    const int chain = wide >> 1, k = chain / p.HV;
+    fused_sweep<act_t, 1>(p, lds_all, 2 * (p.seq_order[k] * p.HV + chain - k * p.HV) + (wide & 1));
+  } else {
+    const int chain = xcd_grouped_index(blockIdx.x - p.split_grid, ratio, (p.N - p.n_long) * p.HV);
+    if (chain < 0) return;
+    const int k = chain / p.HV;
+    fused_sweep<act_t, 2>(p, lds_all, p.seq_order[p.n_long + k] * p.HV + chain - k * p.HV);
+  }
+}
+
 struct GdnWorkspaceLayout {
   size_t seq_chunk_off, chunk_seq, chunk_tok, chunk_len, q_rows, k_rows, kn, kinv, gtile, W;
   size_t seq_seg_off, seg_seq, seg_c0, seg_nc, segM, segB, segS, identity;
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
 };
+// Plan of the mixed sweep (gdn_fused_sweep_mixed_kernel) for sequences that sweep `r[n]` chunks in one launch:
+// order[] receives the sequences longest first, the return value is the number of leading ones whose chains are swept
+// as two halves (0: sweep all chains whole).  The launch is priced in chunk times of a whole chain on an idle chip:
+// a half takes 0.9 of that, the launch lasts as long as its longest chain (or as the whole chains need on the CUs the
+// halves leave them, or as all the work needs on all CUs), and a chunk takes up to 17 % longer as the chip fills (3.0
+// us with a third of the CUs busy, 3.5 us with all of them: the sweeps share the memory system).  The split is taken
+// where the price falls by 5 % or more.
+constexpr int CUS = 256;
+static int mixed_sweep_plan(const int* r, int N, int HV, unsigned char* order) {
+  for (int n = 0; n < N; ++n) {
+    int at = n;
+    for (; at > 0 && r[order[at - 1]] < r[n]; --at) order[at] = order[at - 1];
+    order[at] = (unsigned char)n;
+  }
+  double rest = 0, halves = 0;
+  for (int n = 0; n < N; ++n) rest += r[n];
+  if (rest == 0) return 0;
+  double whole_price = 0, best = 0;
+  int best_k = 0;
+  for (int k = 0; k <= N && 2 * k * HV <= CUS; ++k) {
+    if (k > 0) { halves += r[order[k - 1]]; rest -= r[order[k - 1]]; }
+    const double work = (1.8 * halves + rest) * HV;
+    double span = std::max(k > 0 ? 0.9 * r[order[0]] : 0.0, work / CUS);
+    if (k < N) {
+      span = std::max(span, (double)r[order[k]]);
+      if ((int64_t)(N + k) * HV > CUS) {          // whole chains wait for CUs: longest first on those the halves leave
+        const int free_cus = CUS - 2 * k * HV;
+        if (free_cus <= 0) break;
+        span = std::max(span, rest * HV / free_cus + 0.5 * r[order[N - 1]]);
+      }
+    }
+    const double price = span * (1.0 + 0.17 * std::min(1.0, work / (CUS * span)));
+    if (k == 0) whole_price = best = price;
+    else if (price < best) { best = price; best_k = k; }
+  }
+  return best <= 0.95 * whole_price ? best_k : 0;
+}
+
+// The plan for a call of N <= INLINE_TABLE_SEQUENCES whole sequences run in `stages` stages (0: unstaged): *stage
+// receives the stage whose sweep is the last one.
+static int mixed_sweep_from_offsets(const int32_t* raw_cu_seqlens, int N, int HV, int stages, unsigned char* order, int* stage) {
+  int nc[INLINE_TABLE_SEQUENCES], r[INLINE_TABLE_SEQUENCES];
+  int64_t total = 0;
+  int longest = 0;
+  for (int n = 0; n < N; ++n) {
+    nc[n] = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+    total += nc[n];
+    longest = std::max(longest, nc[n]);
+  }
+  const int plan = stage_plan(total, N, longest, stages);
+  const int last = plan_stages(plan) - 1;
+  for (int n = 0; n < N; ++n) r[n] = stage_cut(nc[n], last + 1, plan) - stage_cut(nc[n], last, plan);
+  *stage = last;
+  return mixed_sweep_plan(r, N, HV, order);
+}
+
 static GdnWorkspaceLayout gdn_layout(int T, int N, int H, int HV, bool allow_stages = true) {
   GdnWorkspaceLayout L;
   L.NC_max = T / CHUNK + N;
@@ -1503,6 +1597,14 @@ static int gdn_prefill_run(
     p.stg.carry = segmented ? nullptr : reinterpret_cast<float*>(ws + L.carry);
     p.stg.stages = stages;
   }
+  // Ragged whole sequences whose offsets the host holds: the last (or only) sweep runs the chains of the longest
+  // sequences as two halves where that shortens it (mixed_sweep_plan)
+  int mixed_stage = -1;
+  if (!segmented && !v_halves && raw_cu_seqlens != nullptr && N <= INLINE_TABLE_SEQUENCES) {
+    p.n_long = mixed_sweep_from_offsets(raw_cu_seqlens, N, HV, stages, p.seq_order, &mixed_stage);
+    if (p.n_long > 0) p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * HV, 2 * (unsigned)(HV / H));
+    else mixed_stage = -1;
+  }
   // At most 64 sequences: no table kernel runs ahead of the preparation, whose first launch also zeroes the padded
   // rows of o.  Whole sequences: every kernel works its chunks out by itself.  Segments: the
   // preparation does, and one workgroup appended to it writes the chunk and segment tables for the sweeps.
@@ -1537,7 +1639,11 @@ static int gdn_prefill_run(
           // workgroups then sweep a chain, 64 V columns each - the columns of V are independent, so the results are the
           // same bits.  A half costs 0.86 to 0.93 of a whole chain's chunk time (K, Q, W and P are fetched and formed once
           // per workgroup whatever its width): 4 x 4096 tokens of 32 value heads 0.248 -> 0.236 ms, 3 x 4096 0.227 -> 0.205.
-          if (v_halves) {
+          if (p.stage == mixed_stage) {
+            const unsigned g = p.split_grid + xcd_grouped_grid((unsigned)(N - p.n_long) * HV, (unsigned)(HV / H));
+            if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_mixed_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
+            else hipLaunchKernelGGL(gdn_fused_sweep_mixed_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);
+          } else if (v_halves) {
             const unsigned g = xcd_grouped_grid(2 * grid, 2 * (unsigned)(HV / H));
             if (half_act) hipLaunchKernelGGL((gdn_fused_sweep_kernel<f16_t, 1>), dim3(g), dim3(512), 0, s, p);
             else hipLaunchKernelGGL((gdn_fused_sweep_kernel<bf16_t, 1>), dim3(g), dim3(512), 0, s, p);
@@ -1607,6 +1713,15 @@ extern "C" int pla_gdn_prefill_launch_raw(
                          cu_seqlens, N, T, scale, normalize_qk, h0, h0_indices, h0_slot_stride, ht, ht_indices,
                          ht_slot_stride, o, workspace, workspace_bytes, false, gcum_out, beta_out, H, HV, K, V, act_dtype,
                          stream, raw_cu_seqlens);
+}
+
+extern "C" int pla_gdn_prefill_halved_sequences(const int32_t* raw_cu_seqlens, int N, int T, int H, int HV) {
+  if (raw_cu_seqlens == nullptr || N <= 0 || N > INLINE_TABLE_SEQUENCES || T <= 0 || H <= 0 || HV < H || HV % H != 0) return 0;
+  const GdnWorkspaceLayout L = gdn_layout(T, N, H, HV);
+  if (L.seg_chunks > 0 || (int64_t)N * HV <= 128) return 0;
+  unsigned char order[INLINE_TABLE_SEQUENCES];
+  int stage = 0;
+  return mixed_sweep_from_offsets(raw_cu_seqlens, N, HV, L.stages, order, &stage);
 }
 
 extern "C" int pla_gdn_prefill_launch_static(

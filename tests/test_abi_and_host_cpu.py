@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     declared = _declared()
     assert {"pla_version", "pla_last_error", "pla_k_last_packed_launch", "pla_k_last_launch",
             "pla_kda_fold_launch", "pla_kda_fold_native_launch", "pla_kda_conv_native_launch", "pla_kda_commit_plan_launch", "pla_kda_decode_mega_launch", "pla_kda_verify_dspark_launch", "pla_kda_replay_verify_native_launch", "pla_conv_window_scatter_launch",
-            "pla_gdn_prefill_launch", "pla_gdn_prefill_launch_raw", "pla_gdn_prefill_workspace_bytes",
+            "pla_gdn_prefill_launch", "pla_gdn_prefill_launch_raw", "pla_gdn_prefill_workspace_bytes", "pla_gdn_prefill_halved_sequences",
             "pla_kda_prefill_launch", "pla_kda_prefill_workspace_bytes"} <= set(declared)
     for name in declared:
         assert hasattr(lib, name), name
@@ -53,6 +53,29 @@ def test_workspace_sizes_are_monotone_and_aligned():
     assert lib.pla_gdn_prefill_workspace_bytes(0, 1, 1, 1) == 0
     c = lib.pla_kda_prefill_workspace_bytes(4096, 1, 32)
     assert c > 0 and c % 256 == 0
+
+
+def test_plan_of_the_halved_sequences_is_host_arithmetic():
+    """Which sequences the last sweep of a ragged GDN prefill call runs as two workgroups per chain is decided from
+    the host offsets alone: more than 128 chains of whole sequences, a price that falls by 5 % or more."""
+    from pla_amd import _lib
+    lib = _lib.load()
+
+    def plan(lengths, H, HV):
+        offs = [0]
+        for n in lengths:
+            offs.append(offs[-1] + n)
+        return lib.pla_gdn_prefill_halved_sequences((ctypes.c_int32 * len(offs))(*offs), len(lengths), offs[-1], H, HV)
+    assert plan([8000, 7000, 1000, 2000, 3000], 16, 32) == 1           # 0.9 x 79 chunks is still above the runner-up's 69
+    assert plan([5000, 4800, 300, 2000, 1000, 100, 64], 16, 32) == 2   # two long sequences of nearly equal length
+    assert plan([4000] * 4 + [1000], 16, 32) == 0                      # four long ones as halves would fill every CU
+    assert plan([2646, 6988, 1342, 6924, 3410, 2250, 1978, 7272], 16, 32) == 0      # 256 chains: no idle CU to gain from
+    assert plan([4000, 3900, 3800, 3700, 500, 600, 700, 800, 900], 16, 32) == 0
+    assert plan([1500, 200, 300, 400, 700], 16, 32) == 1               # a single sweep (too short for stages)
+    assert plan([16384], 16, 32) == 0                                  # split into segments instead
+    assert plan([3000, 100], 16, 32) == 0                              # at most 128 chains: every chain runs as halves anyway
+    assert plan([100] * 65, 16, 32) == 0                               # more than 64 sequences: table kernel path
+    assert lib.pla_gdn_prefill_halved_sequences(None, 5, 1000, 16, 32) == 0
 
 
 def test_native_entry_points_reject_bad_arguments_without_a_gpu():

@@ -348,6 +348,41 @@ def test_gdn_prefill_with_and_without_host_offsets_gives_the_same_bits():
                 assert torch.equal(x, y), lengths
 
 
+@pytest.mark.parametrize("lengths,H,HV,halved,dtype", [
+    ([3000, 2600, 300, 64, 0, 777, 500, 200, 900, 400], 8, 16, 1, torch.bfloat16),       # one sweep (not staged)
+    ([4000, 3500, 500, 1000, 1500], 16, 32, 1, torch.bfloat16),                         # two stages: the second sweep
+    ([2000, 100, 200, 300, 2000, 64, 1, 0, 500], 16, 16, 2, torch.float16),             # as many value heads as q/k heads
+    ([1800, 1750, 100, 64, 0, 300, 200, 150, 400, 130, 77], 4, 12, 2, torch.bfloat16),  # three value heads per q/k head
+])
+def test_gdn_prefill_longest_sequences_swept_as_halves(lengths, H, HV, halved, dtype):
+    """Ragged whole sequences with more than 128 chains and the offsets on the host: the last sweep runs the chains
+    of the longest sequences as two workgroups of 64 V columns each (the plan is host arithmetic and is asked for
+    here).  Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain
+    whole."""
+    import ctypes
+    from pla_amd import _lib
+    from pla_amd.workloads import gdn_prefill_packed
+    offs = [0]
+    for n in lengths:
+        offs.append(offs[-1] + n)
+    plan = _lib.load().pla_gdn_prefill_halved_sequences((ctypes.c_int32 * len(offs))(*offs), len(lengths), offs[-1] + 5, H, HV)
+    assert plan == halved
+    results = []
+    for with_raw in (True, False):
+        w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=4711, tail_pad=5, dtype=dtype)
+        assert w["raw_cu_seqlens"] == tuple(offs)
+        if with_raw:
+            _check(w, fast=True)
+            w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 3, seed=4711, tail_pad=5, dtype=dtype)
+        else:
+            w["raw_cu_seqlens"] = None
+        g_cum, _, o, _, final = _run_workload(w)
+        torch.cuda.synchronize()
+        results.append((o, g_cum.reshape(-1, HV)[:offs[-1]], final, w["initial_state"]))
+    for x, y in zip(*results):
+        assert torch.equal(x, y)
+
+
 @pytest.mark.parametrize("lengths,H,HV", [([1500, 2100, 900, 1500, 1300, 1100, 700, 1200], 4, 16), ([2600, 70], 2, 4)])
 def test_gdn_prefill_staged_pipeline_in_a_graph(lengths, H, HV):
     """The staged call forks to a side stream and joins again, so it can be captured: three replays with
