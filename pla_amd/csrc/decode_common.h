@@ -115,6 +115,10 @@ struct Tile {
   __amdgpu_buffer_rsrc_t rsrc;
   __device__ __forceinline__ explicit Tile(state_t* tile_base)
       : rsrc(__builtin_amdgcn_make_buffer_rsrc(tile_base, 0, 16384 * sizeof(state_t), 0x00020000)) {}
+  // present == false: a tile of no bytes, every load from it returns zero (the range check of the buffer
+  // instruction), so a kernel can issue the loads of an absent state without a branch
+  __device__ __forceinline__ Tile(state_t* tile_base, bool present)
+      : rsrc(__builtin_amdgcn_make_buffer_rsrc(tile_base, 0, present ? 16384 * (int)sizeof(state_t) : 0, 0x00020000)) {}
 };
 typedef int v2i_t __attribute__((ext_vector_type(2)));
 

@@ -62,6 +62,10 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   const int i_h = i_hv / (p.HV / p.H);
   const int rowbase = (blockIdx.y * 4 + wave) * RPW;
 
+  // the request's slot is requested together with its offsets: independent loads, one trip to memory instead of two
+  // on the path to the tile's address
+  int h0_direct = -1;
+  if (p.h0_indices != nullptr && p.stride_h0_indices_seq <= 0) h0_direct = p.h0_indices[i_n];
   int bos, T;
   if (p.cu_seqlens != nullptr) {
     bos = p.cu_seqlens[i_n];
@@ -70,7 +74,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     bos = i_n * p.T_max;
     T = p.T_max;
   }
-  // Empty requests touch nothing (no slot / accepted load either).
+  // Empty requests touch no tile and write nothing.
   if (bos < 0 || T <= 0 || T > p.T_max) return;
 
   act_t* const o_base = reinterpret_cast<act_t*>(p.o) + ((int64_t)bos * p.HV + i_hv) * 128 + rowbase;
@@ -81,7 +85,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       const int col = accepted > 0 ? accepted - 1 : 0;
       h0_idx = p.h0_indices[(int64_t)i_n * p.stride_h0_indices_seq + col];
     } else {
-      h0_idx = p.h0_indices[i_n];
+      h0_idx = h0_direct;
     }
     if (p.is_sglang ? (h0_idx < 0) : (h0_idx <= 0)) {
       float z[R];
@@ -95,7 +99,7 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   const bool have_state = p.h0 != nullptr && h0_idx >= 0;
   const int64_t tile_off = (int64_t)i_hv * 16384;                 // tile of this head inside a slot
   const int lane_off = ((rowbase + half) * 128 + 4 * c) * 4;      // bytes inside the tile
-  const Tile<state_t> h_tile(have_state ? pool + (int64_t)h0_idx * p.h0_slot_stride + tile_off : nullptr);
+  const Tile<state_t> h_tile(have_state ? pool + (int64_t)h0_idx * p.h0_slot_stride + tile_off : nullptr, have_state);
 
   int cidx = -1;
   if (MTP && p.cache != nullptr && p.cache_indices != nullptr) cidx = p.cache_indices[i_n];
@@ -178,15 +182,12 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         // contiguous bytes per instruction
         const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + (POOL_BF16 ? 8 : 4) * kb) * (int)sizeof(state_t);
         if constexpr (POOL_BF16) {
-          const v4i_t zero = {0, 0, 0, 0};
-          sb16[m][ks] = __builtin_bit_cast(bf16x8_t, have_state ? __builtin_bit_cast(v4i_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                                                      h_tile.rsrc, at, 0, kLoadPolicy)) : zero);
+          // (an absent state is a tile of no bytes: its loads return zero)
+          sb16[m][ks] = __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(h_tile.rsrc, at, 0, kLoadPolicy));
         } else {
 #pragma unroll
           for (int hf = 0; hf < 2; ++hf)
-            sa[m][ks][hf] = have_state ? __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                             h_tile.rsrc, at + 64 * hf, 0, kLoadPolicy))
-                                       : f32x4_t{0.f, 0.f, 0.f, 0.f};
+            sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(h_tile.rsrc, at + 64 * hf, 0, kLoadPolicy));
         }
       }
     // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one)
@@ -205,7 +206,13 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       for (int e = 0; e < 4; ++e) s[j][e] = 0.f;
   }
 
-  const float eA = log_decay ? 0.f : __expf(decode_scalar(alog_raw, p.alog_dtype));
+  // (decoded whether it is used or not, both halves named as used here: under `if (!log_decay)`, or for the half
+  // that only an FP32 A_log has, the compiler moves the load itself into that branch, behind the tile loads, where
+  // waiting for it means waiting for the whole tile)
+  RawScalar alog_here = alog_raw;
+  asm volatile("" : "+v"(alog_here.lo), "+v"(alog_here.hi));
+  const float eA_any = __expf(decode_scalar(alog_here, p.alog_dtype));
+  const float eA = log_decay ? 0.f : eA_any;
   float dt[4] = {0.f, 0.f, 0.f, 0.f};
   float dt_scalar = 0.f;
   if constexpr (IS_KDA) decode_k4<act_t>(dt_raw_k4, dt_wide || log_decay, dt);
@@ -317,8 +324,10 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       for (int ks = 0; ks < 4; ++ks) {
         const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 4 * kb]);
         const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 16 + 4 * kb]);
-        wq[ks][0] = w0.x * keep; wq[ks][1] = w0.y * keep; wq[ks][2] = w0.z * keep; wq[ks][3] = w0.w * keep;
-        wq[ks][4] = w1.x * keep; wq[ks][5] = w1.y * keep; wq[ks][6] = w1.z * keep; wq[ks][7] = w1.w * keep;
+        // (columns beyond the window repeat its last token: every column of the product depends on its own column
+        // of the queries only, and those columns are never stored)
+        wq[ks][0] = w0.x; wq[ks][1] = w0.y; wq[ks][2] = w0.z; wq[ks][3] = w0.w;
+        wq[ks][4] = w1.x; wq[ks][5] = w1.y; wq[ks][6] = w1.z; wq[ks][7] = w1.w;
       }
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks)
