@@ -135,8 +135,22 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
     xb[t] = qk_side ? p.x_k[tok * p.sx_k + ch] : p.g[tok * p.sg + ch];
     xc[t] = p.beta[tok * p.sbeta + h];
   }
-  const float eA = __expf(p.a_log[h]);
+  const float a_log_h = p.a_log[h];
   const float bias = p.dt_bias[ch];
+  // state tile, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]: requested before anything looks at
+  // the small inputs (the staging below waits for them, and would hold the tile back by one trip to memory)
+  const Tile<float> h_tile(p.h0 + slot * p.state_slot + (int64_t)h * 16384);
+  f32x4_t sa[2][4][2];
+#pragma unroll
+  for (int m = 0; m < 2; ++m)
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+        sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
+            h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
+
+  const float eA = __expf(a_log_h);
   if constexpr (STAGED) {
     if (staged) {
 #pragma unroll
@@ -151,18 +165,6 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
       }
     }
   }
-
-  // state tile, lane (r16, kb) holds S[32 w + 16 m + r16][32 ks + 8 kb .. + 7]
-  const Tile<float> h_tile(p.h0 + slot * p.state_slot + (int64_t)h * 16384);
-  f32x4_t sa[2][4][2];
-#pragma unroll
-  for (int m = 0; m < 2; ++m)
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int hf = 0; hf < 2; ++hf)
-        sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
-            h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
 
   const int64_t ring_row = ((p.native ? n : slot) * p.H + h) * p.L;   // first record of this (slot or request, head)
   if (qk_side) {
