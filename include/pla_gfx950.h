@@ -417,6 +417,27 @@ int pla_kda_prefill_launch(
     int H, int K, int V, int act_dtype, void* stream);
 
 /*
+ * pla_kda_prefill_launch with the sequence offsets on the host as well (N + 1 int32 values in HOST memory that
+ * equal cu_seqlens; NULL: exactly pla_kda_prefill_launch).  Replaces the `raw_cu_seqlens` argument of the reference's
+ * flashkda_fwd (pla/prefill/flashkdapro/ops.py: the trusted host copy of the offsets).  One host-side decision is
+ * taken from it and changes no bit of the results: a call of at most 64 ragged whole sequences with more than 128
+ * chains sweeps the chains of its longest sequences as two workgroups of 64 V columns each where idle CUs make that
+ * shorter (pla_kda_prefill_halved_sequences tells how many).  The values are read during the call and not kept.
+ */
+int pla_kda_prefill_launch_raw(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_g, int64_t stride_beta,
+    const float* A_log, const float* dt_bias, float lower_bound, float scale,
+    const int32_t* cu_seqlens, int N, int T,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    int H, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens);
+
+/* As pla_gdn_prefill_halved_sequences, for pla_kda_prefill_launch_raw.  Host arithmetic only. */
+int pla_kda_prefill_halved_sequences(const int32_t* raw_cu_seqlens, int N, int T, int H);
+
+/*
  * Rows of the 128-row state tile a wavefront owns (8, 16 or 32) that a k-last launch with
  * rows_per_wave = 0 takes for a shape: the row count the auto-tuner measured for the nearest batch size
  * of the same (kernel, heads, dtypes) if the built-in table holds the shape, else the size thresholds.

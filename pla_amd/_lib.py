@@ -98,6 +98,14 @@ SIGNATURES = {
         _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
         _c_p, _c_p, _c_i64,
         _c_int, _c_int, _c_int, _c_int, _c_p],
+    "pla_kda_prefill_launch_raw": [
+        _c_p, _c_p, _c_p, _c_p, _c_p,
+        _c_i64, _c_i64, _c_i64, _c_i64, _c_i64,
+        _c_p, _c_p, _c_f, _c_f,
+        _c_p, _c_int, _c_int,
+        _c_p, _c_p, _c_i64, _c_p, _c_p, _c_i64,
+        _c_p, _c_p, _c_i64,
+        _c_int, _c_int, _c_int, _c_int, _c_p, _c_p],
 }
 
 _lib = None
@@ -121,6 +129,8 @@ def load():
     lib.pla_gdn_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int, _c_int]
     lib.pla_gdn_prefill_halved_sequences.restype = _c_int
     lib.pla_gdn_prefill_halved_sequences.argtypes = [_c_p, _c_int, _c_int, _c_int, _c_int]
+    lib.pla_kda_prefill_halved_sequences.restype = _c_int
+    lib.pla_kda_prefill_halved_sequences.argtypes = [_c_p, _c_int, _c_int, _c_int]
     lib.pla_kda_prefill_workspace_bytes.restype = _c_i64
     lib.pla_kda_prefill_workspace_bytes.argtypes = [_c_int, _c_int, _c_int]
     lib.pla_tuned_rows_per_wave.restype = _c_int

@@ -242,7 +242,8 @@ bool try_flashkda_fwd(const Tensor& q, const Tensor& k, const Tensor& v, const T
   if (!(lower_bound >= -5.0 && lower_bound <= 0.0)) return false;
   if (!plain_offsets(cu_seqlens, q)) return false;
   const int64_t N = cu_seqlens->numel() - 1;
-  if (!plain_raw_offsets(raw_cu_seqlens, N, T)) return false;
+  std::vector<int32_t> host_offsets;
+  if (!plain_raw_offsets(raw_cu_seqlens, N, T, &host_offsets)) return false;
   const bool indexed = state_indices.has_value();
   if (indexed && (!plain_indices(*state_indices, q, N) || (!initial_state && !final_state))) return false;
   for (const OptTensor* t : {&initial_state, &final_state})
@@ -264,13 +265,14 @@ bool try_flashkda_fwd(const Tensor& q, const Tensor& k, const Tensor& v, const T
     }
   }
   const int32_t* idx = indexed ? state_indices->data_ptr<int32_t>() : nullptr;
-  launched(pla_kda_prefill_launch(
+  launched(pla_kda_prefill_launch_raw(
       q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(), q.stride(0), k.stride(0), v.stride(0), g.stride(0),
       beta.stride(0), A_log.data_ptr<float>(), dt_bias.data_ptr<float>(), (float)lower_bound, (float)scale,
       cu_seqlens->data_ptr<int32_t>(), (int)N, (int)T,
       initial_state ? initial_state->data_ptr<float>() : nullptr, idx, initial_state ? initial_state->stride(0) : 0,
       final_state ? final_state->data_ptr<float>() : nullptr, idx, final_state ? final_state->stride(0) : 0,
-      out.data_ptr(), ws.data_ptr(), ws_bytes, (int)H, 128, 128, PLA_BF16, stream_of(q)));
+      out.data_ptr(), ws.data_ptr(), ws_bytes, (int)H, 128, 128, PLA_BF16, stream_of(q),
+      host_offsets.empty() ? nullptr : host_offsets.data()));
   return true;
 }
 #endif  // PLA_BIND_FLASHKDAPRO

@@ -164,6 +164,14 @@ __device__ __forceinline__ void dma16(const char* gbase, uint32_t byte_offset, u
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :: "s"(lds_wave_base), "v"(byte_offset), "s"(gbase) : "memory", "m0");
 }
+// A pointer whose value is the same in every lane, as a scalar: where the compiler holds such a value in vector
+// registers (a value merged from two branches of one kernel, say) dma16 cannot take it as its base.
+template <typename T>
+__device__ __forceinline__ T* uniform_pointer(T* p) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return reinterpret_cast<T*>(((uint64_t)hi << 32) | lo);
+}
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
@@ -831,6 +839,45 @@ class SideStreamLease {
   }
   SideStream* taken_;
 };
+
+// Plan of a mixed sweep (gdn_fused_sweep_mixed_kernel, kda_sweep_mixed_kernel: the chains of the longest sequences as
+// two workgroups of 64 V columns each, first in the grid, the others whole, longest first, in one launch) for sequences that sweep `r[n]` chunks in one launch:
+// order[] receives the sequences longest first, the return value is the number of leading ones whose chains are swept
+// as two halves (0: sweep all chains whole).  The launch is priced in chunk times of a whole chain on an idle chip:
+// a half takes `half_cost` (0.9 measured for GDN) of that, the launch lasts as long as its longest chain (or as the whole chains need on the CUs the
+// halves leave them, or as all the work needs on all CUs), and a chunk takes up to `fill_cost` (17 % for GDN) longer as the chip fills (3.0
+// us with a third of the CUs busy, 3.5 us with all of them: the sweeps share the memory system).  The split is taken
+// where the price falls by 5 % or more.
+constexpr int CUS = 256;
+inline int mixed_sweep_plan(const int* r, int N, int HV, unsigned char* order, double half_cost = 0.9, double fill_cost = 0.17) {
+  for (int n = 0; n < N; ++n) {
+    int at = n;
+    for (; at > 0 && r[order[at - 1]] < r[n]; --at) order[at] = order[at - 1];
+    order[at] = (unsigned char)n;
+  }
+  double rest = 0, halves = 0;
+  for (int n = 0; n < N; ++n) rest += r[n];
+  if (rest == 0) return 0;
+  double whole_price = 0, best = 0;
+  int best_k = 0;
+  for (int k = 0; k <= N && 2 * k * HV <= CUS; ++k) {
+    if (k > 0) { halves += r[order[k - 1]]; rest -= r[order[k - 1]]; }
+    const double work = (2 * half_cost * halves + rest) * HV;
+    double span = std::max(k > 0 ? half_cost * r[order[0]] : 0.0, work / CUS);
+    if (k < N) {
+      span = std::max(span, (double)r[order[k]]);
+      if ((int64_t)(N + k) * HV > CUS) {          // whole chains wait for CUs: longest first on those the halves leave
+        const int free_cus = CUS - 2 * k * HV;
+        if (free_cus <= 0) break;
+        span = std::max(span, rest * HV / free_cus + 0.5 * r[order[N - 1]]);
+      }
+    }
+    const double price = span * (1.0 + fill_cost * std::min(1.0, work / (CUS * span)));
+    if (k == 0) whole_price = best = price;
+    else if (price < best) { best = price; best_k = k; }
+  }
+  return best <= 0.95 * whole_price ? best_k : 0;
+}
 
 // Stages for a call of whole sequences: two, where there are enough chains to fill the chip and 16 chunks per
 // sequence on average; the table kernel then keeps both only for chains of unequal length (stage_map).  Measured on

@@ -1354,44 +1354,6 @@ struct GdnWorkspaceLayout {
   size_t order, stage_begin, carry, total;
   int NC_max, seg_chunks, max_segments, stages;
 };
-// Plan of the mixed sweep (gdn_fused_sweep_mixed_kernel) for sequences that sweep `r[n]` chunks in one launch:
-// order[] receives the sequences longest first, the return value is the number of leading ones whose chains are swept
-// as two halves (0: sweep all chains whole).  The launch is priced in chunk times of a whole chain on an idle chip:
-// a half takes 0.9 of that, the launch lasts as long as its longest chain (or as the whole chains need on the CUs the
-// halves leave them, or as all the work needs on all CUs), and a chunk takes up to 17 % longer as the chip fills (3.0
-// us with a third of the CUs busy, 3.5 us with all of them: the sweeps share the memory system).  The split is taken
-// where the price falls by 5 % or more.
-constexpr int CUS = 256;
-static int mixed_sweep_plan(const int* r, int N, int HV, unsigned char* order) {
-  for (int n = 0; n < N; ++n) {
-    int at = n;
-    for (; at > 0 && r[order[at - 1]] < r[n]; --at) order[at] = order[at - 1];
-    order[at] = (unsigned char)n;
-  }
-  double rest = 0, halves = 0;
-  for (int n = 0; n < N; ++n) rest += r[n];
-  if (rest == 0) return 0;
-  double whole_price = 0, best = 0;
-  int best_k = 0;
-  for (int k = 0; k <= N && 2 * k * HV <= CUS; ++k) {
-    if (k > 0) { halves += r[order[k - 1]]; rest -= r[order[k - 1]]; }
-    const double work = (1.8 * halves + rest) * HV;
-    double span = std::max(k > 0 ? 0.9 * r[order[0]] : 0.0, work / CUS);
-    if (k < N) {
-      span = std::max(span, (double)r[order[k]]);
-      if ((int64_t)(N + k) * HV > CUS) {          // whole chains wait for CUs: longest first on those the halves leave
-        const int free_cus = CUS - 2 * k * HV;
-        if (free_cus <= 0) break;
-        span = std::max(span, rest * HV / free_cus + 0.5 * r[order[N - 1]]);
-      }
-    }
-    const double price = span * (1.0 + 0.17 * std::min(1.0, work / (CUS * span)));
-    if (k == 0) whole_price = best = price;
-    else if (price < best) { best = price; best_k = k; }
-  }
-  return best <= 0.95 * whole_price ? best_k : 0;
-}
-
 // The plan for a call of N <= INLINE_TABLE_SEQUENCES whole sequences run in `stages` stages (0: unstaged): *stage
 // receives the stage whose sweep is the last one.
 static int mixed_sweep_from_offsets(const int32_t* raw_cu_seqlens, int N, int HV, int stages, unsigned char* order, int* stage) {

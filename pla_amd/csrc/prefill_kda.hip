@@ -64,6 +64,10 @@ struct KdaPrefillParams {
   int pass;                                        // 0: whole sequences; 1, 2: the two sweeps over segments
   int stage;                                       // stage handled by this launch (prep kernel, passes 0 and 1)
   int H, NC_max;
+  // kda_sweep_mixed_kernel: the first `split_grid` workgroups sweep the chains of sequences seq_order[0 .. n_long) as
+  // two halves, the others those of seq_order[n_long .. N) whole
+  unsigned split_grid; int n_long;
+  unsigned char seq_order[INLINE_TABLE_SEQUENCES];
 };
 
 // 52 KB, so that three workgroups share a CU.  The normalised q never goes through LDS: the thread that
@@ -338,20 +342,30 @@ __global__ __launch_bounds__(256) void kda_prep_solve_kernel(const KdaPrefillPar
 //   barrier B   the tiles requested at A landed; V is free              copy V of c + 1
 //               O^T = S (scale Q e^G)^T + U^T P^T -> rows of o
 //               S^T = e^{G_last} (.) S^T + (K e^{G_last-G})^T U         (pairs: hi.lo + lo.hi + hi.hi)
+// LDS of one workgroup of kda_sweep
+constexpr int KDA_W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
+struct KdaSweepLds {
+  __align__(1024) uint16_t tK[2][TILE128_HALVES];       // swizzled operand tiles, as the preparation stored them
+  __align__(16) uint16_t tW[2][KDA_W_HALVES];           // [parity][hi blocks, lo blocks]
+  __align__(16) uint16_t tV[CHUNK * PITCH128];
+  __align__(1024) uint16_t tQ[TILE128_HALVES];
+  __align__(16) uint16_t tP[TRI_BLOCKS * 512];
+  __align__(1024) uint16_t tKt[2][TILE128_HALVES];      // hi, lo: the same layout, read transposed
+  __align__(16) float tE[128];
+};
+
+// The sweep of one workgroup.  `wide`: 2 / NB x the chain's logical index (sequence x H + head, or segment x H + head
+// in the second sweep over segments) plus, for NB = 1, the half of the V columns it takes.
 template <int NB>
-__global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_kernel(const KdaPrefillParams p) {
+__device__ __forceinline__ void kda_sweep(const KdaPrefillParams& p, KdaSweepLds& lds, const int wide) {
   constexpr int HALVES = 2 / NB;             // workgroups per chain: NB = 1 sweeps 64 of the 128 V columns
   constexpr int NCOPY = KDA_SWEEP_COPIERS;
   using CopyWide = TileCopy<CHUNK, 2 * PITCH128, 256, NCOPY>;  // 64 x 128 tile, its pieces dealt to the copying wavefronts
-  constexpr int W_HALVES = 2 * TRI_BLOCKS * 512;               // W: hi blocks, then lo blocks (six-block operand layout)
+  constexpr int W_HALVES = KDA_W_HALVES;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r16 = lane & 15, kb = lane >> 4;
-  // the two halves of a chain copy the same tiles: on one XCD they come from memory once (xcd_grouped_index)
-  const int wide = HALVES == 1 ? (int)blockIdx.x
-                               : xcd_grouped_index(blockIdx.x, HALVES, HALVES * (p.pass == 2 ? p.seg.max_segments : p.N) * p.H);
-  if (wide < 0) return;
   const int v_half = wide % HALVES;
   const SweepRole role = select_sweep(p.pass, p.H, p.N, p.seq_chunk_off, p.seg, p.stg, p.stage, p.h0, p.h0_indices, p.h0_slot_stride,
                                       p.ht, p.ht_indices, p.ht_slot_stride, wide / HALVES);
@@ -362,25 +376,19 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
   const int n_chunks = c_end - c_begin;
   auto chunk_len = [&](int c) { return min(CHUNK, seq_len - c * CHUNK); };
 
-  __shared__ __align__(1024) uint16_t tK[2][TILE128_HALVES];       // swizzled operand tiles, as the preparation stored them
-  __shared__ __align__(16) uint16_t tW[2][W_HALVES];                // [parity][hi blocks, lo blocks]
-  __shared__ __align__(16) uint16_t tV[CHUNK * PITCH128];
-  __shared__ __align__(1024) uint16_t tQ[TILE128_HALVES];
-  __shared__ __align__(16) uint16_t tP[TRI_BLOCKS * 512];
-  __shared__ __align__(1024) uint16_t tKt[2][TILE128_HALVES];      // hi, lo: the same layout, read transposed
-  __shared__ __align__(16) float tE[128];
+  auto& tK = lds.tK; auto& tW = lds.tW; auto& tV = lds.tV; auto& tQ = lds.tQ; auto& tP = lds.tP; auto& tKt = lds.tKt; auto& tE = lds.tE;
 
   if (wave >= 4) {
     const int cw = wave - 4;                         // which of the copying wavefronts
     // ---- the copying wavefront -------------------------------------------------------------
     const int64_t tile0 = (int64_t)c_begin * p.H + h;
-    const char* const kg_b = reinterpret_cast<const char*>(p.Kg) + tile0 * 16384;
-    const char* const qg_b = reinterpret_cast<const char*>(p.Qg) + tile0 * 16384;
-    const char* const kt_b = reinterpret_cast<const char*>(p.Kt) + tile0 * 32768;
-    const char* const w_b = reinterpret_cast<const char*>(p.W) + tile0 * (W_HALVES * 2);
-    const char* const pp_b = reinterpret_cast<const char*>(p.P) + tile0 * (TRI_BLOCKS * 1024);
-    const char* const eg_b = reinterpret_cast<const char*>(p.eGlast) + tile0 * 512;
-    const char* const v_b = reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2;
+    const char* const kg_b = uniform_pointer(reinterpret_cast<const char*>(p.Kg) + tile0 * 16384);
+    const char* const qg_b = uniform_pointer(reinterpret_cast<const char*>(p.Qg) + tile0 * 16384);
+    const char* const kt_b = uniform_pointer(reinterpret_cast<const char*>(p.Kt) + tile0 * 32768);
+    const char* const w_b = uniform_pointer(reinterpret_cast<const char*>(p.W) + tile0 * (W_HALVES * 2));
+    const char* const pp_b = uniform_pointer(reinterpret_cast<const char*>(p.P) + tile0 * (TRI_BLOCKS * 1024));
+    const char* const eg_b = uniform_pointer(reinterpret_cast<const char*>(p.eGlast) + tile0 * 512);
+    const char* const v_b = uniform_pointer(reinterpret_cast<const char*>(p.v) + ((int64_t)seq_start * p.stride_v + h * 128) * 2);
     const int64_t big_step = (int64_t)p.H * 16384, w_step = (int64_t)p.H * (W_HALVES * 2), p_step = (int64_t)p.H * (TRI_BLOCKS * 1024);
     const int64_t e_step = (int64_t)p.H * 512;
     CopyWide plan_v;
@@ -685,6 +693,35 @@ __global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_ker
       for (int mc = 0; mc < 8; ++mc)
         *reinterpret_cast<float4*>(dst + 16 * mc) = make_float4(St[nb][mc].x, St[nb][mc].y, St[nb][mc].z, St[nb][mc].w);
     }
+  }
+}
+
+// One workgroup per (sequence, head) or per (segment, head) in the second sweep over segments (NB = 2); NB = 1: two
+// per chain, 64 V columns each, on one XCD: they copy the same tiles, which then come from memory once.
+template <int NB>
+__global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_kernel(const KdaPrefillParams p) {
+  constexpr int HALVES = 2 / NB;
+  __shared__ KdaSweepLds lds;
+  const int wide = HALVES == 1 ? (int)blockIdx.x
+                               : xcd_grouped_index(blockIdx.x, HALVES, HALVES * (p.pass == 2 ? p.seg.max_segments : p.N) * p.H);
+  if (wide < 0) return;
+  kda_sweep<NB>(p, lds, wide);
+}
+
+// Ragged whole sequences: the chains of the longest sequences as two halves (first in the grid: workgroups are
+// dispatched in index order), those of the others whole, longest first (mixed_sweep_plan).
+__global__ __launch_bounds__(64 * (4 + KDA_SWEEP_COPIERS), 1) void kda_sweep_mixed_kernel(const KdaPrefillParams p) {
+  __shared__ KdaSweepLds lds;
+  if (blockIdx.x < p.split_grid) {
+    const int wide = xcd_grouped_index(blockIdx.x, 2, 2 * p.n_long * p.H);
+    if (wide < 0) return;
+    const int chain = wide >> 1, k = chain / p.H;
+    kda_sweep<1>(p, lds, __builtin_amdgcn_readfirstlane(2 * (p.seq_order[k] * p.H + chain - k * p.H) + (wide & 1)));
+  } else {
+    const int chain = blockIdx.x - p.split_grid;
+    if (chain >= (p.N - p.n_long) * p.H) return;
+    const int k = chain / p.H;
+    kda_sweep<2>(p, lds, __builtin_amdgcn_readfirstlane(p.seq_order[p.n_long + k] * p.H + chain - k * p.H));
   }
 }
 
@@ -1024,7 +1061,13 @@ extern "C" int64_t pla_kda_prefill_workspace_bytes(int T, int N, int H) {
   return (int64_t)kda_layout(T, N, H).total;
 }
 
-extern "C" int pla_kda_prefill_launch(
+// The share of a KDA chain's chunk time that one of its two half workgroups takes, and how much longer a chunk takes
+// on a full chip than on an idle one (mixed_sweep_plan).  Measured, ms per call of 32 heads without / with the plan
+// at (0.9, 0.17) / at (0.8, 0.05): 8000 + 7000 + 1000 + 2000 + 3000 tokens 0.793 / 0.749 / 0.701; eight ragged
+// sequences of 32 810 tokens 0.997 / - / 0.948; twelve of 700 to 6000 tokens 0.757 / 0.712 / 0.676.
+constexpr double KDA_HALF_COST = 0.8, KDA_FILL_COST = 0.05;
+
+static int kda_prefill_run(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
     int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_g, int64_t stride_beta,
     const float* A_log, const float* dt_bias, float lower_bound, float scale,
@@ -1032,7 +1075,7 @@ extern "C" int pla_kda_prefill_launch(
     const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
     float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
     void* o, void* workspace, int64_t workspace_bytes,
-    int H, int K, int V, int act_dtype, void* stream) {
+    int H, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens) {
   PLA_REQUIRE(K == 128 && V == 128, "KDA prefill requires head_dim K == V == 128, got K=%d, V=%d", K, V);
   PLA_REQUIRE(T > 0 && N > 0 && H > 0, "KDA prefill needs at least one token, sequence and head");
   PLA_REQUIRE(act_dtype == PLA_BF16, "KDA prefill takes bf16 activations (the MFMA operands are bf16)");
@@ -1085,6 +1128,16 @@ extern "C" int pla_kda_prefill_launch(
     p.seg.max_segments = L.max_segments;
   }
   const bool v_halves = !segmented && (int64_t)N * H <= 128;
+  // Ragged whole sequences whose offsets the host holds: the chains of the longest sequences run as two halves where
+  // that shortens the sweep (mixed_sweep_plan; the KDA path runs in one stage)
+  bool mixed = false;
+  if (!segmented && !v_halves && raw_cu_seqlens != nullptr && N <= INLINE_TABLE_SEQUENCES && L.stages == 0) {
+    int nc[INLINE_TABLE_SEQUENCES];
+    for (int n = 0; n < N; ++n) nc[n] = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+    p.n_long = mixed_sweep_plan(nc, N, H, p.seq_order, KDA_HALF_COST, KDA_FILL_COST);
+    mixed = p.n_long > 0;
+    if (mixed) p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * H, 2);
+  }
   const SideStreamLease lease(s, L.stages > 0);
   const int stages = lease.get() != nullptr ? L.stages : 0;
   if (stages > 0) {
@@ -1104,6 +1157,7 @@ extern "C" int pla_kda_prefill_launch(
         if (p.pass == 1) hipLaunchKernelGGL(kda_lean_sweep_kernel, dim3(grid / 2), dim3(512), 0, s, p);
         // Whole sequences that give at most 128 chains (few long ones are split into segments instead) leave half of the CUs idle: two
         // workgroups then sweep a chain, 64 V columns each (the columns of V are independent: the same bits).
+        else if (mixed) hipLaunchKernelGGL(kda_sweep_mixed_kernel, dim3(p.split_grid + (unsigned)(N - p.n_long) * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
         else if (v_halves) hipLaunchKernelGGL(kda_sweep_kernel<1>, dim3(xcd_grouped_grid(2 * grid, 2)), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
         else hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3(grid), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
       });
@@ -1120,4 +1174,42 @@ extern "C" int pla_kda_prefill_launch(
       hipLaunchKernelGGL(kda_sweep_kernel<2>, dim3((unsigned)L.max_segments * H), dim3(64 * (4 + KDA_SWEEP_COPIERS)), 0, s, p);
   }
   return check_launch("kda prefill launch");
+}
+
+extern "C" int pla_kda_prefill_launch(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_g, int64_t stride_beta,
+    const float* A_log, const float* dt_bias, float lower_bound, float scale,
+    const int32_t* cu_seqlens, int N, int T,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    int H, int K, int V, int act_dtype, void* stream) {
+  return kda_prefill_run(q, k, v, g, beta, stride_q, stride_k, stride_v, stride_g, stride_beta, A_log, dt_bias, lower_bound, scale,
+                         cu_seqlens, N, T, h0, h0_indices, h0_slot_stride, ht, ht_indices, ht_slot_stride, o, workspace,
+                         workspace_bytes, H, K, V, act_dtype, stream, nullptr);
+}
+
+extern "C" int pla_kda_prefill_launch_raw(
+    const void* q, const void* k, const void* v, const void* g, const void* beta,
+    int64_t stride_q, int64_t stride_k, int64_t stride_v, int64_t stride_g, int64_t stride_beta,
+    const float* A_log, const float* dt_bias, float lower_bound, float scale,
+    const int32_t* cu_seqlens, int N, int T,
+    const float* h0, const int32_t* h0_indices, int64_t h0_slot_stride,
+    float* ht, const int32_t* ht_indices, int64_t ht_slot_stride,
+    void* o, void* workspace, int64_t workspace_bytes,
+    int H, int K, int V, int act_dtype, void* stream, const int32_t* raw_cu_seqlens) {
+  return kda_prefill_run(q, k, v, g, beta, stride_q, stride_k, stride_v, stride_g, stride_beta, A_log, dt_bias, lower_bound, scale,
+                         cu_seqlens, N, T, h0, h0_indices, h0_slot_stride, ht, ht_indices, ht_slot_stride, o, workspace,
+                         workspace_bytes, H, K, V, act_dtype, stream, raw_cu_seqlens);
+}
+
+extern "C" int pla_kda_prefill_halved_sequences(const int32_t* raw_cu_seqlens, int N, int T, int H) {
+  if (raw_cu_seqlens == nullptr || N <= 0 || N > INLINE_TABLE_SEQUENCES || T <= 0 || H <= 0) return 0;
+  const KdaWorkspaceLayout L = kda_layout(T, N, H);
+  if (L.seg_chunks > 0 || L.stages > 0 || (int64_t)N * H <= 128) return 0;
+  int nc[INLINE_TABLE_SEQUENCES];
+  unsigned char order[INLINE_TABLE_SEQUENCES];
+  for (int n = 0; n < N; ++n) nc[n] = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
+  return mixed_sweep_plan(nc, N, H, order, KDA_HALF_COST, KDA_FILL_COST);
 }

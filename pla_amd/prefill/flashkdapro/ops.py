@@ -7,10 +7,12 @@ logits; ``state_pool`` + ``state_indices`` update an indexed pool in place.
 
 Differences that follow from the gfx950 design: chunk size 64; states are FP32 only and are NOT
 rounded to bf16 at the read / publish boundary (the reference's tc01 backend rounds them); chunk
-metadata is built on the device, so ``raw_cu_seqlens`` is validated and otherwise unused; there is
+metadata is built on the device, and ``raw_cu_seqlens`` is validated and used for one host-side
+decision that changes no bit of the results (``pla_kda_prefill_launch_raw``); there is
 one backend, so the ``PLA_FLASHKDA_*`` routing variables have no effect.
 """
 
+import ctypes
 from typing import Optional, Tuple
 
 import torch
@@ -139,10 +141,13 @@ def flashkda_fwd(
     N = cu32.numel() - 1
     if N <= 0:
         raise ValueError("cu_seqlens must describe at least one sequence")
+    raw_host = None
     if raw_cu_seqlens is not None:
         raw = tuple(int(x) for x in raw_cu_seqlens)
         if len(raw) != N + 1 or raw[0] != 0 or any(b < a for a, b in zip(raw, raw[1:])) or raw[-1] > T:
             raise ValueError("raw_cu_seqlens must be N+1 monotone offsets describing the same packed batch")
+        # host offsets, when the caller has them, go along (one decision is taken from them: see pla_kda_prefill_launch_raw)
+        raw_host = (ctypes.c_int32 * (N + 1))(*raw)
 
     indexed = state_indices is not None
     if indexed and (state_indices.dtype != torch.int32 or state_indices.dim() != 1 or state_indices.numel() != N
@@ -194,12 +199,12 @@ def flashkda_fwd(
                 final_state[:N].zero_()
     idx_ptr = _lib.ptr(state_indices) if indexed else None
     _lib.call(
-        "pla_kda_prefill_launch",
+        "pla_kda_prefill_launch_raw",
         q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), beta.data_ptr(),
         sq, sk, sv, sg, beta.stride(0),
         A_log.data_ptr(), dt_bias.data_ptr(), float(lower_bound), float(scale),
         cu32.data_ptr(), N, T,
         _lib.ptr(initial_state), idx_ptr, initial_state.stride(0) if initial_state is not None else 0,
         _lib.ptr(final_state), idx_ptr, final_state.stride(0) if final_state is not None else 0,
-        out.data_ptr(), ws.data_ptr(), nbytes, H, DK, DV, _lib.BF16, _lib.current_stream(q.device))
+        out.data_ptr(), ws.data_ptr(), nbytes, H, DK, DV, _lib.BF16, _lib.current_stream(q.device), raw_host)
     return None

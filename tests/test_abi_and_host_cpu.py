@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     assert {"pla_version", "pla_last_error", "pla_k_last_packed_launch", "pla_k_last_launch",
             "pla_kda_fold_launch", "pla_kda_fold_native_launch", "pla_kda_conv_native_launch", "pla_kda_commit_plan_launch", "pla_kda_decode_mega_launch", "pla_kda_verify_dspark_launch", "pla_kda_replay_verify_native_launch", "pla_conv_window_scatter_launch",
             "pla_gdn_prefill_launch", "pla_gdn_prefill_launch_raw", "pla_gdn_prefill_workspace_bytes", "pla_gdn_prefill_halved_sequences",
-            "pla_kda_prefill_launch", "pla_kda_prefill_workspace_bytes"} <= set(declared)
+            "pla_kda_prefill_launch", "pla_kda_prefill_launch_raw", "pla_kda_prefill_halved_sequences", "pla_kda_prefill_workspace_bytes"} <= set(declared)
     for name in declared:
         assert hasattr(lib, name), name
     lib.pla_version.restype = ctypes.c_char_p
@@ -76,6 +76,18 @@ def test_plan_of_the_halved_sequences_is_host_arithmetic():
     assert plan([3000, 100], 16, 32) == 0                              # at most 128 chains: every chain runs as halves anyway
     assert plan([100] * 65, 16, 32) == 0                               # more than 64 sequences: table kernel path
     assert lib.pla_gdn_prefill_halved_sequences(None, 5, 1000, 16, 32) == 0
+
+    def kda_plan(lengths, H):
+        offs = [0]
+        for n in lengths:
+            offs.append(offs[-1] + n)
+        return lib.pla_kda_prefill_halved_sequences((ctypes.c_int32 * len(offs))(*offs), len(lengths), offs[-1], H)
+    # a KDA half costs less of a whole chain's time and a full chip slows its chunks less: the plan splits more
+    assert kda_plan([8000, 7000, 1000, 2000, 3000], 32) == 2
+    assert kda_plan([2646, 6988, 1342, 6924, 3410, 2250, 1978, 7272], 32) == 3
+    assert kda_plan([4000] * 4 + [1000], 32) == 0                      # halves of all four would leave the fifth no CU
+    assert kda_plan([65536], 32) == 0 and kda_plan([3000, 100], 32) == 0 and kda_plan([100] * 65, 32) == 0
+    assert lib.pla_kda_prefill_halved_sequences(None, 5, 1000, 32) == 0
 
 
 def test_native_entry_points_reject_bad_arguments_without_a_gpu():

@@ -365,6 +365,43 @@ def test_kda_prefill_split_sequences_match_oracle(lengths, pad, H):
                 assert rel_l2(final[n, head], exp_final[n, head]) <= 1e-3, (n, head)
 
 
+@pytest.mark.parametrize("lengths,H,halved", [([1500, 1300, 300, 64, 0, 777, 500, 200, 900], 16, 2),
+                                              ([900, 800, 100, 64, 0, 300, 200, 150, 400, 130, 77, 60], 12, 2),
+                                              ([1500, 200, 300, 400, 700], 32, 1)])
+def test_kda_prefill_longest_sequences_swept_as_halves(lengths, H, halved):
+    """Ragged whole sequences with more than 128 chains and the offsets on the host: the chains of the longest
+    sequences run as two workgroups of 64 V columns each (the plan is host arithmetic and is asked for here).
+    Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain whole, through
+    both host layers."""
+    import ctypes
+    from pla_amd import _lib
+    from pla_amd.prefill.flashkdapro import flashkda_fwd, ops
+    q, k, v, raw, beta, A_log, dt_bias, offs, S0 = _inputs(lengths, H, seed=4711, pad=5)
+    plan = _lib.load().pla_kda_prefill_halved_sequences((ctypes.c_int32 * len(offs))(*offs), len(lengths), q.shape[0], H)
+    assert plan == halved
+    exp_o, exp_final = _oracle(q, k, v, raw, beta, A_log, dt_bias, offs, S0, fast=True)
+    dev = "cuda"
+    args = [t.to(dev) for t in (q, k, v, raw, beta, A_log, dt_bias)]
+    cu = torch.tensor(offs, dtype=torch.int32, device=dev)
+    results = []
+    for native in (False, True):
+        for host_offsets in (tuple(offs), None):
+            ops._native = None if native else False
+            out = torch.full((q.shape[0], H, 128), 7.0, dtype=torch.bfloat16, device=dev)
+            final = torch.empty_like(S0, device=dev)
+            flashkda_fwd(*args, out, initial_state=S0.to(dev), final_state=final, cu_seqlens=cu, raw_cu_seqlens=host_offsets)
+            torch.cuda.synchronize()
+            results.append((out, final))
+    ops._native = False
+    out, final = results[0]
+    torch.testing.assert_close(out[:offs[-1]].float().cpu(), exp_o[:offs[-1]].float(), atol=2e-2, rtol=2e-2)
+    assert torch.count_nonzero(out[offs[-1]:]) == 0
+    worst = max(rel_l2(final[n].cpu(), exp_final[n]) for n in range(len(lengths)))
+    assert worst <= 1e-3, worst
+    for other in results[1:]:
+        assert torch.equal(other[0], out) and torch.equal(other[1], final)
+
+
 def test_kda_prefill_many_chains_match_oracle_and_single_sequence_bits():
     """128 chains of ragged lengths (an empty sequence, sequences of one token and of one chunk) in one call, against
     the oracle; the short sequences run alone give the same bits.  (The shape is the one a pipelined call of
