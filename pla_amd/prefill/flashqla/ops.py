@@ -12,7 +12,8 @@ the bf16 high part of ``L^-1 diag(beta)`` per chunk, ``[chunks, H, 64, 64]``); t
 arguments ``auto_cp``, ``overlap_warmup_threshold`` and ``force_tc01_cp_candidate`` are accepted
 and have no effect because every sequence keeps its full history in one pass; chunk metadata is
 built on the device, so no call ever reads ``cu_seqlens`` back to the host (``raw_cu_seqlens`` is
-validated and otherwise unused).  States are FP32 and k-last ``[slots, H, DV, DK]``; the legacy
+validated and used for two host-side decisions that change no bit of the results:
+``pla_gdn_prefill_launch_raw``).  States are FP32 and k-last ``[slots, H, DV, DK]``; the legacy
 k-first ``[N, H, DK, DV]`` state form is not provided.
 """
 
