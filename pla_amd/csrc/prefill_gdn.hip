@@ -34,7 +34,10 @@
 //                            columns of S^T each, in MFMA accumulator layout, the chain K S^T -> X -> U -> S^T in
 //                            registers) and four feeding wavefronts that normalise the raw q / k rows into LDS
 //                            tiles, form P and issue the global -> LDS copies of V, W and the decay factors; two
-//                            barriers per chunk
+//                            barriers per chunk; with NB = 1 two workgroups per chain, 64 V columns each (calls
+//                            of at most 128 chains)
+//   gdn_fused_sweep_mixed_kernel  the same sweep for ragged whole sequences: the chains of the longest sequences as
+//                            two halves, the others whole, in one launch (plan from the host offsets)
 //   gdn_lean_sweep_kernel    first sweep over segments (no output): the zero-state and the identity sweep of a
 //                            segment side by side in one workgroup of eight wavefronts that share every tile
 

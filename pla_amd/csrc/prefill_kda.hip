@@ -25,7 +25,10 @@
 //                           inverse of I + L by 16 x 16 blocks, W and P (fp16)
 //   kda_sweep_kernel        one workgroup per (sequence, head) or second segment sweep: four computing
 //                           wavefronts x 32 V columns with a register-chained MFMA pipeline, two wavefronts
-//                           that issue the asynchronous global -> LDS tile copies; writes o
+//                           that issue the asynchronous global -> LDS tile copies; writes o; with NB = 1 two
+//                           workgroups per chain, 64 V columns each (calls of at most 128 chains)
+//   kda_sweep_mixed_kernel  the same sweep for ragged whole sequences: the chains of the longest sequences as two
+//                           halves, the others whole, in one launch (plan from the host offsets)
 //   kda_lean_sweep_kernel   first sweep over segments: the zero-state sweep and the transition-matrix
 //                           sweep of two segments in one workgroup of eight wavefronts, no output
 // The operands of every sweep product are fp16 (v_mfma_f32_16x16x32_f16): the decayed tiles hold factors in
