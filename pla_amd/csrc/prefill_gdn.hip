@@ -1564,11 +1564,14 @@ static int gdn_prefill_run(
   }
   // Ragged whole sequences whose offsets the host holds: the last (or only) sweep runs the chains of the longest
   // sequences as two halves where that shortens it (mixed_sweep_plan)
-  int mixed_stage = -1;
+  // More chains than CUs: every sweep of the call also starts its chains longest first (in the order of the
+  // sequences the last chain to find a CU may be the longest one, and the launch then ends that much later).
+  int mixed_stage = -1, halved = 0;
+  bool longest_first = false;
   if (!segmented && !v_halves && raw_cu_seqlens != nullptr && N <= INLINE_TABLE_SEQUENCES) {
-    p.n_long = mixed_sweep_from_offsets(raw_cu_seqlens, N, HV, stages, p.seq_order, &mixed_stage);
-    if (p.n_long > 0) p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * HV, 2 * (unsigned)(HV / H));
-    else mixed_stage = -1;
+    halved = mixed_sweep_from_offsets(raw_cu_seqlens, N, HV, stages, p.seq_order, &mixed_stage);
+    if (halved == 0) mixed_stage = -1;
+    longest_first = (int64_t)N * HV > CUS;
   }
   // At most 64 sequences: no table kernel runs ahead of the preparation, whose first launch also zeroes the padded
   // rows of o.  Whole sequences: every kernel works its chunks out by itself.  Segments: the
@@ -1604,7 +1607,9 @@ static int gdn_prefill_run(
           // workgroups then sweep a chain, 64 V columns each - the columns of V are independent, so the results are the
           // same bits.  A half costs 0.86 to 0.93 of a whole chain's chunk time (K, Q, W and P are fetched and formed once
           // per workgroup whatever its width): 4 x 4096 tokens of 32 value heads 0.248 -> 0.236 ms, 3 x 4096 0.227 -> 0.205.
-          if (p.stage == mixed_stage) {
+          if (p.stage == mixed_stage || longest_first) {
+            p.n_long = p.stage == mixed_stage ? halved : 0;
+            p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * HV, 2 * (unsigned)(HV / H));
             const unsigned g = p.split_grid + xcd_grouped_grid((unsigned)(N - p.n_long) * HV, (unsigned)(HV / H));
             if (half_act) hipLaunchKernelGGL(gdn_fused_sweep_mixed_kernel<f16_t>, dim3(g), dim3(512), 0, s, p);
             else hipLaunchKernelGGL(gdn_fused_sweep_mixed_kernel<bf16_t>, dim3(g), dim3(512), 0, s, p);

@@ -1138,8 +1138,10 @@ static int kda_prefill_run(
     int nc[INLINE_TABLE_SEQUENCES];
     for (int n = 0; n < N; ++n) nc[n] = (std::max(raw_cu_seqlens[n + 1] - raw_cu_seqlens[n], 0) + CHUNK - 1) / CHUNK;
     p.n_long = mixed_sweep_plan(nc, N, H, p.seq_order, KDA_HALF_COST, KDA_FILL_COST);
-    mixed = p.n_long > 0;
-    if (mixed) p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * H, 2);
+    // (more chains than CUs: the chains also start longest first - in the order of the sequences the last chain to
+    // find a CU may be the longest one -, with or without halves)
+    mixed = p.n_long > 0 || (int64_t)N * H > CUS;
+    p.split_grid = xcd_grouped_grid(2 * (unsigned)p.n_long * H, 2);
   }
   const SideStreamLease lease(s, L.stages > 0);
   const int stages = lease.get() != nullptr ? L.stages : 0;

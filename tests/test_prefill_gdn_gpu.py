@@ -353,11 +353,13 @@ def test_gdn_prefill_with_and_without_host_offsets_gives_the_same_bits():
     ([4000, 3500, 500, 1000, 1500], 16, 32, 1, torch.bfloat16),                         # two stages: the second sweep
     ([2000, 100, 200, 300, 2000, 64, 1, 0, 500], 16, 16, 2, torch.float16),             # as many value heads as q/k heads
     ([1800, 1750, 100, 64, 0, 300, 200, 150, 400, 130, 77], 4, 12, 2, torch.bfloat16),  # three value heads per q/k head
+    ([900, 100, 1500, 64, 0, 300, 2000, 150, 400, 130, 77, 700], 16, 32, 1, torch.bfloat16),     # more chains than CUs: longest first
+    ([1000, 1000, 1000, 990, 1010, 1000, 1000, 1000, 1000], 16, 32, 0, torch.bfloat16),          # the same without halves
 ])
 def test_gdn_prefill_longest_sequences_swept_as_halves(lengths, H, HV, halved, dtype):
     """Ragged whole sequences with more than 128 chains and the offsets on the host: the last sweep runs the chains
     of the longest sequences as two workgroups of 64 V columns each (the plan is host arithmetic and is asked for
-    here).  Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain
+    here); with more chains than CUs every sweep also starts its chains longest first.  Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain
     whole."""
     import ctypes
     from pla_amd import _lib

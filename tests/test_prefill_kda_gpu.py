@@ -367,11 +367,13 @@ def test_kda_prefill_split_sequences_match_oracle(lengths, pad, H):
 
 @pytest.mark.parametrize("lengths,H,halved", [([1500, 1300, 300, 64, 0, 777, 500, 200, 900], 16, 2),
                                               ([900, 800, 100, 64, 0, 300, 200, 150, 400, 130, 77, 60], 12, 2),
-                                              ([1500, 200, 300, 400, 700], 32, 1)])
+                                              ([1500, 200, 300, 400, 700], 32, 1),
+                                              ([900, 100, 1500, 64, 0, 300, 2000, 150, 400, 130, 77, 700], 32, 1),
+                                              ([500, 500, 500, 490, 510, 500, 500, 500, 500], 32, 0)])
 def test_kda_prefill_longest_sequences_swept_as_halves(lengths, H, halved):
     """Ragged whole sequences with more than 128 chains and the offsets on the host: the chains of the longest
-    sequences run as two workgroups of 64 V columns each (the plan is host arithmetic and is asked for here).
-    Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain whole, through
+    sequences run as two workgroups of 64 V columns each (the plan is host arithmetic and is asked for here); with
+    more chains than CUs the chains also start longest first.  Against the oracle, and bit for bit against the call without host offsets, which sweeps every chain whole, through
     both host layers."""
     import ctypes
     from pla_amd import _lib
