@@ -347,8 +347,8 @@ int pla_gdn_prefill_launch(
  * the device applies anyway, a call whose sequences are of nearly equal length runs in one stage, and with the offsets
  * at hand nothing is enqueued for a second one (two launches and four event operations less per call); and a call of
  * at most 64 ragged whole sequences with more than 128 chains sweeps the chains of its longest sequences as two
- * workgroups of 64 V columns each where idle CUs make that shorter (pla_gdn_prefill_halved_sequences).  The values
- * are read during the call and not kept.
+ * workgroups of 64 V columns each where idle CUs make that shorter (pla_gdn_prefill_halved_sequences) and, with
+ * more chains than CUs, starts its chains longest first.  The values are read during the call and not kept.
  */
 int pla_gdn_prefill_launch_raw(
     const void* q, const void* k, const void* v, int64_t stride_q, int64_t stride_k, int64_t stride_v,
@@ -422,7 +422,8 @@ int pla_kda_prefill_launch(
  * flashkda_fwd (pla/prefill/flashkdapro/ops.py: the trusted host copy of the offsets).  One host-side decision is
  * taken from it and changes no bit of the results: a call of at most 64 ragged whole sequences with more than 128
  * chains sweeps the chains of its longest sequences as two workgroups of 64 V columns each where idle CUs make that
- * shorter (pla_kda_prefill_halved_sequences tells how many).  The values are read during the call and not kept.
+ * shorter (pla_kda_prefill_halved_sequences tells how many) and, with more chains than CUs, starts its chains longest
+ * first.  The values are read during the call and not kept.
  */
 int pla_kda_prefill_launch_raw(
     const void* q, const void* k, const void* v, const void* g, const void* beta,
