@@ -385,11 +385,13 @@ def test_gdn_prefill_longest_sequences_swept_as_halves(lengths, H, HV, halved, d
         assert torch.equal(x, y)
 
 
-@pytest.mark.parametrize("lengths,H,HV", [([1500, 2100, 900, 1500, 1300, 1100, 700, 1200], 4, 16), ([2600, 70], 2, 4)])
+@pytest.mark.parametrize("lengths,H,HV", [([1500, 2100, 900, 1500, 1300, 1100, 700, 1200], 4, 16), ([2600, 70], 2, 4),
+                                          ([4000, 3500, 500, 1000, 1500], 8, 32)])
 def test_gdn_prefill_staged_pipeline_in_a_graph(lengths, H, HV):
     """The staged call forks to a side stream and joins again, so it can be captured: three replays with
     eager work and synchronisation in between reproduce the eager result bit for bit.  The second case is a call
-    split into segments (two sweeps and the combine step, tables written by the preparation's appended workgroup)."""
+    split into segments (two sweeps and the combine step, tables written by the preparation's appended workgroup),
+    the third a staged call whose last sweep runs the chains of its longest sequence as two workgroups each."""
     from pla_amd.workloads import gdn_prefill_packed
     w = gdn_prefill_packed(lengths, H=H, HV=HV, pool_slots=len(lengths) + 2, seed=31)
     pool0 = w["initial_state"].clone()

@@ -292,7 +292,7 @@ def test_config4_kda_prefill_full_size():
         assert rel_l2(call["final_state"][0, head], exp_final[0, i]) <= 1e-3, head
 
 
-@pytest.mark.parametrize("lengths,H", [([700, 0, 130, 64, 1], 24), ([4096, 40], 2)])
+@pytest.mark.parametrize("lengths,H", [([700, 0, 130, 64, 1], 24), ([4096, 40], 2), ([1500, 200, 300, 400, 700], 32)])
 def test_kda_prefill_in_a_graph(lengths, H):
     """flashkda_fwd allocates (workspace) and launches only, so it can be captured: a call of whole sequences (more
     than 64 chains) and a call that is split into segments (zero-state / identity sweeps, combine, second sweep),
@@ -307,7 +307,9 @@ def test_kda_prefill_in_a_graph(lengths, H):
     cu = torch.tensor(offs, dtype=torch.int32, device=dev)
 
     def run(out, final):
-        flashkda_fwd(dq, dk, dv, dg, db, dA, dD, out, initial_state=dS, final_state=final, cu_seqlens=cu)
+        # (with the host offsets: the third case then runs the chains of its longest sequence as two workgroups each)
+        flashkda_fwd(dq, dk, dv, dg, db, dA, dD, out, initial_state=dS, final_state=final, cu_seqlens=cu,
+                     raw_cu_seqlens=tuple(offs))
 
     o_eager = torch.empty(T, H, 128, dtype=torch.bfloat16, device=dev)
     f_eager = torch.empty(N, H, 128, 128, device=dev)
