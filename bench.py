@@ -220,27 +220,35 @@ def bench_prefill(steps, warmup, device, cpu_leg=False):
 REFERENCE_GDN_PREFILL_MS = (([2048] * 8, 1.4865), ([4096] * 4, 1.5035), ([16384], 2.241))
 
 
-def bench_prefill_reference_shapes(steps, device, only=None):
+def bench_prefill_reference_shapes(steps, device, only=None, host_offsets=True):
     """The batch x length shapes of the reference's own prefill report, next to its published times (other
     hardware: a ratio of two machines, not a like-for-like comparison).  only: a "BxL" string, that shape alone
-    (any batch and length, for profiling; without a published time unless it is one of the report's)."""
+    (any batch and length, for profiling; without a published time unless it is one of the report's), or ragged
+    lengths joined by "+" ("8000+7000+1000").  host_offsets False: the call goes without ``raw_cu_seqlens``."""
     import torch
     from pla_amd.prefill.flashqla import gdn_prefill_packed_qkv_fwd
     from pla_amd.workloads import gdn_prefill_packed
     rows = []
     shapes = REFERENCE_GDN_PREFILL_MS
     if only is not None:
-        batch, length = (int(x) for x in only.lower().split("x"))
-        published = dict(((len(l), l[0]), ms) for l, ms in REFERENCE_GDN_PREFILL_MS)
-        shapes = (([length] * batch, published.get((batch, length))),)
+        if "+" in only:
+            shapes = (([int(x) for x in only.split("+")], None),)
+        else:
+            batch, length = (int(x) for x in only.lower().split("x"))
+            published = dict(((len(l), l[0]), ms) for l, ms in REFERENCE_GDN_PREFILL_MS)
+            shapes = (([length] * batch, published.get((batch, length))),)
     for lengths, published_ms in shapes:
         w = gdn_prefill_packed(lengths, H=16, HV=32, pool_slots=len(lengths) + 2, seed=1, device=device)
         call = {k: v for k, v in w.items() if not k.startswith("_")}
         packed = call.pop("packed_qkv")
         a, b, A, dt, cu = (call.pop(n) for n in ("raw_gate_a", "raw_beta_b", "A_log", "dt_bias", "cu_seqlens"))
+        if not host_offsets:
+            call["raw_cu_seqlens"] = None
         run = lambda: gdn_prefill_packed_qkv_fwd(packed, a, b, A, dt, cu, **call)
         ms = time_calls(run, steps, 20, device)
-        rows.append({"shape": "%d x %d tokens" % (len(lengths), lengths[0]), "ms_per_call": round(ms, 4),
+        ragged = len(set(lengths)) > 1
+        rows.append({"shape": "+".join(str(n) for n in lengths) + " tokens" if ragged else "%d x %d tokens" % (len(lengths), lengths[0]),
+                     "host_offsets": bool(host_offsets), "ms_per_call": round(ms, 4),
                      "tokens_per_s": round(sum(lengths) / ms * 1e3, 1), "reference_ppu_ms": published_ms,
                      "reference_ms_over_ours": round(published_ms / ms, 2) if published_ms else None})
         del w, call, packed
@@ -580,7 +588,10 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the two prefill workloads (for rocprofv3 --pmc byte counters) and print their objects")
     ap.add_argument("--prefill-shape", metavar="BxL", default=None,
-                    help="run only the GDN prefill of B sequences of L tokens (H=16, HV=32), e.g. 1x16384, and print its row")
+                    help="run only the GDN prefill of B sequences of L tokens (H=16, HV=32), e.g. 1x16384, or of ragged "
+                         "lengths joined by +, e.g. 8000+7000+1000+2000+3000, and print its row")
+    ap.add_argument("--no-host-offsets", action="store_true",
+                    help="with --prefill-shape: call without raw_cu_seqlens (the host then plans nothing from the lengths)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch a 1 GiB device copy (reference for scaling rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -596,7 +607,8 @@ def main():
     torch.cuda.set_device(device)
     if args.prefill_shape:
         print(json.dumps({"prefill_reference_shapes": bench_prefill_reference_shapes(max(args.steps // 2, 10), device,
-                                                                                     only=args.prefill_shape)}))
+                                                                                     only=args.prefill_shape,
+                                                                                     host_offsets=not args.no_host_offsets)}))
         return
     if args.prefill_only:
         result = {"prefill": bench_prefill(max(args.steps, 50), 50, device)}
