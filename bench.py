@@ -636,7 +636,9 @@ def main():
         torch.cuda.empty_cache()
         extra["prefill"] = bench_prefill(max(args.steps, 50), 50, device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
-        extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 2, 10), device)
+        # (at least 50 timed calls per shape: the first calls of a process run 10-20 % slower, and ten calls of 0.2 ms
+        # after twenty warm-up calls still show it)
+        extra["prefill_reference_shapes"] = bench_prefill_reference_shapes(max(args.steps // 2, 50), device)
         extra["prefill_kda"] = bench_prefill_kda(max(args.steps // 4, 5), device, cpu_leg=not args.no_cpu_baseline)
         torch.cuda.empty_cache()
     d = time_decode(prep, args.steps, args.warmup)
