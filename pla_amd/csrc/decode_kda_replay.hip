@@ -147,8 +147,11 @@ __global__ __launch_bounds__(256) void kda_verify_dspark_kernel(const ReplayVeri
     for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf)
+        // (no non-temporal hint: the two loads of a contraction step take interleaved 16-byte pieces of the same
+        // 128-byte lines, and the second finds them in the vector cache; with the hint it fetched them from the L2
+        // again: 48.6 -> 42.2 us for 64 requests of 32 heads)
         sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(
-            h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, kLoadPolicy));
+            h_tile.rsrc, ((rowbase + 16 * m + r16) * 128 + 32 * ks + 8 * kb) * 4 + 16 * hf, 0, 0));
 
   const float eA = __expf(a_log_h);
   if constexpr (STAGED) {
