@@ -183,7 +183,8 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         const int at = ((rowbase + 16 * m + r16) * 128 + 32 * ks + (POOL_BF16 ? 8 : 4) * kb) * (int)sizeof(state_t);
         if constexpr (POOL_BF16) {
           // (an absent state is a tile of no bytes: its loads return zero)
-          sb16[m][ks] = __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(h_tile.rsrc, at, 0, kLoadPolicy));
+          // (no non-temporal hint, as for the FP32 tile below: consecutive contraction steps take pieces of the same lines)
+          sb16[m][ks] = __builtin_bit_cast(bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(h_tile.rsrc, at, 0, 0));
         } else {
 #pragma unroll
           for (int hf = 0; hf < 2; ++hf)
