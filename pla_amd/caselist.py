@@ -417,6 +417,8 @@ def main(argv=None):
     ap.add_argument("--limit", type=int, default=None)
     ap.add_argument("--start", type=int, default=0, help="skip this many cases of the list (a long list replayed in parts)")
     ap.add_argument("--csv", default=None)
+    ap.add_argument("--min-seqlen-q", type=int, default=0, metavar="N",
+                    help="decode lists: only the cases with at least N tokens per request (2: the verify shapes)")
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--check", type=int, default=0, metavar="N",
                     help="instead of timing, check N seeded small prefill shapes of the list: each case against itself "
@@ -447,6 +449,8 @@ def main(argv=None):
         writer.writeheader()
     try:
         for i, case in enumerate(read_caselist(args.caselist, args.limit)[args.start:]):
+            if args.min_seqlen_q and int(case.get("seqlen_q") or 1) < args.min_seqlen_q:
+                continue
             row = replay_case(case, reps=args.reps, device_inputs=args.device_inputs)
             if not args.quiet or i % 500 == 0:
                 print(args.start + i, row, flush=True)
