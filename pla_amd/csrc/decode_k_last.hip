@@ -156,6 +156,11 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
   // the K-vector algebra runs while the tile is in flight (memory returns in issue order).  Tokens the request
   // does not have repeat its last one (their results are never stored).
   constexpr int TM = READONCE > 0 ? READONCE : 1;      // draft tokens the read-once verify is built for
+  // Windows of more than four tokens keep fewer values in registers next to the tile in flight (each step's K-vectors
+  // re-read from LDS, the query operands read per contraction step, v requested after half of the products): 188 ->
+  // 120 registers, four wavefronts per SIMD instead of two (B = 64: 5 tokens 41.7 -> 37.7 us, 8 tokens 42.2 -> 38.8 us).
+  // The four-token kernel is faster as it is (31.5 us against 32.8).
+  constexpr bool LEAN = TM > 4;
   constexpr int NT = TM > 4 ? TM / 4 : 1;              // tokens per wavefront
   TokenIn mine[NT];
   if constexpr (READONCE > 0) {
@@ -193,13 +198,15 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
             sa[m][ks][hf] = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(h_tile.rsrc, at + 64 * hf, 0, 0));
         }
       }
-    // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one)
-#pragma unroll
-    for (int m = 0; m < 2; ++m)
-#pragma unroll
-      for (int t = 0; t < TM; ++t)
-        vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
-                                                   ((int64_t)bos + min(t, T - 1)) * p.stride_v);
+    if constexpr (!LEAN) {
+      // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one)
+  #pragma unroll
+      for (int m = 0; m < 2; ++m)
+  #pragma unroll
+        for (int t = 0; t < TM; ++t)
+          vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
+                                                     ((int64_t)bos + min(t, T - 1)) * p.stride_v);
+    }
   } else if (have_state) {
     load_state<R>(h_tile, lane_off, s);
   } else {
@@ -276,18 +283,38 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
         qn = fast_rsqrt(row32_allreduce(qs) + 1e-6f) * p.scale;
       }
       float w[4] = {q4[0] * qn, q4[1] * qn, q4[2] * qn, q4[3] * qn};
-      float kv[TM][4], dec[TM][4], beta[TM];
-#pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        // tokens after t do not enter w_t; the request's tokens before t are all present
-        const float4 k4 = j <= t ? *reinterpret_cast<const float4*>(&sK[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
-        const float4 d4 = j <= t ? *reinterpret_cast<const float4*>(&sD[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
-        kv[j][0] = k4.x; kv[j][1] = k4.y; kv[j][2] = k4.z; kv[j][3] = k4.w;
-        dec[j][0] = d4.x; dec[j][1] = d4.y; dec[j][2] = d4.z; dec[j][3] = d4.w;
-        beta[j] = j <= t ? sB[j] : 0.f;
-      }
       float cf[TM];
-      effective_query<TM>(t, w, kv, dec, beta, cf);
+      if constexpr (LEAN) {
+        // the recurrence of effective_query (readonce_verify.h), each step's key, decay and beta read from LDS when the
+        // step needs them: held in registers for the whole window they cost eight registers per token next to the tile
+        // in flight
+  #pragma unroll
+        for (int j = TM - 1; j >= 0; --j) {
+          cf[j] = 0.f;
+          if (j > t) continue;                       // tokens after t do not enter w_t
+          const float4 k4 = *reinterpret_cast<const float4*>(&sK[j][4 * c]);
+          const float4 d4 = *reinterpret_cast<const float4*>(&sD[j][4 * c]);
+          const float kj[4] = {k4.x, k4.y, k4.z, k4.w}, dj[4] = {d4.x, d4.y, d4.z, d4.w};
+          float dot = 0.f;
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) dot = fmaf(kj[e], w[e], dot);
+          cf[j] = sB[j] * row32_allreduce(dot);
+  #pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = dj[e] * fmaf(-cf[j], kj[e], w[e]);
+        }
+      } else {
+        float kv[TM][4], dec[TM][4], beta[TM];
+  #pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          // tokens after t do not enter w_t; the request's tokens before t are all present
+          const float4 k4 = j <= t ? *reinterpret_cast<const float4*>(&sK[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
+          const float4 d4 = j <= t ? *reinterpret_cast<const float4*>(&sD[j][4 * c]) : make_float4(0.f, 0.f, 0.f, 0.f);
+          kv[j][0] = k4.x; kv[j][1] = k4.y; kv[j][2] = k4.z; kv[j][3] = k4.w;
+          dec[j][0] = d4.x; dec[j][1] = d4.y; dec[j][2] = d4.z; dec[j][3] = d4.w;
+          beta[j] = j <= t ? sB[j] : 0.f;
+        }
+        effective_query<TM>(t, w, kv, dec, beta, cf);
+      }
       if (half == 0) *reinterpret_cast<float4*>(&sW[t][4 * c]) = make_float4(w[0], w[1], w[2], w[3]);
       if (lane == 0) {
 #pragma unroll
@@ -309,6 +336,14 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
     if constexpr (POOL_BF16) {
       HiLo wb[4];
       query_operands(sW, tcol, keep, kb, wb);
+      if constexpr (LEAN) {
+  #pragma unroll
+        for (int m = 0; m < 2; ++m)
+  #pragma unroll
+          for (int t = 0; t < TM; ++t)
+            vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
+                                                       ((int64_t)bos + min(t, T - 1)) * p.stride_v);
+      }
 #pragma unroll
       for (int m = 0; m < 2; ++m)
 #pragma unroll
@@ -322,25 +357,53 @@ __global__ __launch_bounds__(256) void k_last_kernel(const KLastParams p) {
       // tile nor the queries are split into 16-bit pairs: 64 matrix instructions per wavefront instead of 24, but
       // about 300 vector instructions fewer, and the products are exact.  The two row blocks alternate, so that
       // consecutive instructions never wait for the same accumulator.
-      float wq[4][8];
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 4 * kb]);
-        const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 16 + 4 * kb]);
-        // (columns beyond the window repeat its last token: every column of the product depends on its own column
-        // of the queries only, and those columns are never stored)
-        wq[ks][0] = w0.x; wq[ks][1] = w0.y; wq[ks][2] = w0.z; wq[ks][3] = w0.w;
-        wq[ks][4] = w1.x; wq[ks][5] = w1.y; wq[ks][6] = w1.z; wq[ks][7] = w1.w;
-      }
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-          for (int e = 0; e < 4; ++e)
-#pragma unroll
+      if constexpr (LEAN) {
+  #pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          // (columns beyond the window repeat its last token: every column of the product depends on its own column
+          // of the queries only, and those columns are never stored)
+          const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 4 * kb]);
+          const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 16 + 4 * kb]);
+          const float wq[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+  #pragma unroll
+          for (int hf = 0; hf < 2; ++hf)
+  #pragma unroll
+            for (int e = 0; e < 4; ++e)
+  #pragma unroll
+              for (int m = 0; m < 2; ++m)
+                accs[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[m][ks][hf][e], wq[4 * hf + e], accs[m], 0, 0, 0);
+          if (ks == 1) {
+            // v of every token for the lane's output rows 16 m + 4 kb .. + 3 (absent tokens repeat the last one), requested
+            // where half of the tile's registers are free again
+  #pragma unroll
             for (int m = 0; m < 2; ++m)
-              accs[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[m][ks][hf][e], wq[ks][4 * hf + e], accs[m], 0, 0, 0);
+  #pragma unroll
+              for (int t = 0; t < TM; ++t)
+                vq[m][t] = *reinterpret_cast<const uint2*>(reinterpret_cast<const act_t*>(p.v) + i_hv * 128 + rowbase + 16 * m + 4 * kb +
+                                                           ((int64_t)bos + min(t, T - 1)) * p.stride_v);
+          }
+        }
+      } else {
+        float wq[4][8];
+  #pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const float4 w0 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 4 * kb]);
+          const float4 w1 = *reinterpret_cast<const float4*>(&sW[tcol][32 * ks + 16 + 4 * kb]);
+          // (columns beyond the window repeat its last token: every column of the product depends on its own column
+          // of the queries only, and those columns are never stored)
+          wq[ks][0] = w0.x; wq[ks][1] = w0.y; wq[ks][2] = w0.z; wq[ks][3] = w0.w;
+          wq[ks][4] = w1.x; wq[ks][5] = w1.y; wq[ks][6] = w1.z; wq[ks][7] = w1.w;
+        }
+  #pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+  #pragma unroll
+          for (int hf = 0; hf < 2; ++hf)
+  #pragma unroll
+            for (int e = 0; e < 4; ++e)
+  #pragma unroll
+              for (int m = 0; m < 2; ++m)
+                accs[m] = __builtin_amdgcn_mfma_f32_16x16x4f32(sa[m][ks][hf][e], wq[ks][4 * hf + e], accs[m], 0, 0, 0);
+      }
     }
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
